@@ -1,0 +1,120 @@
+/* C ABI of libwarpctct_hip.so — the MI355X (gfx950) CTC-Transducer loss kernels.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream
+ * (passed as void*; NULL = the null stream), launches asynchronously on that
+ * stream, never synchronises with the host, never allocates, and returns 0
+ * or a WARPCTCT_E* code (never exits the process, unlike CHECK_KERNEL_STAT
+ * at csrc/core.h:5-12 of the reference).  The caller owns every buffer.
+ *
+ * Shapes use the reference's names: N lattices, T = max frames, U = max
+ * labels (the joint has U+1 contexts), V = vocabulary, blank = 0.  Tensors
+ * are dense row-major.  "units" are the three entries per cell (t,u) that
+ * the lattice uses: k=0 blank, k=1 label y[u-1], k=2 label y[u]
+ * (csrc/gather.cu:16-21 of the reference).
+ *
+ * Internally the lattice works on log2 values held in double ("units",
+ * alphas, betas below).  These intermediates are private to the library (the
+ * reference's alphas/betas are private too); unit gradients and costs are
+ * returned as fp32 in natural-log units exactly like the reference.
+ */
+#ifndef WARP_CTCT_HIP_H
+#define WARP_CTCT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    WARPCTCT_OK = 0,
+    WARPCTCT_EINVAL = 1,     /* null pointer, negative size, size limit exceeded */
+    WARPCTCT_ELAUNCH = 2,    /* hipGetLastError() reported a failed launch */
+    WARPCTCT_EWORKSPACE = 3, /* workspace smaller than warpctct_workspace_bytes() */
+    WARPCTCT_ENODEVICE = 4   /* no usable HIP device */
+};
+
+/* Human-readable text for a return code (static storage). */
+const char *warpctct_error_string(int code);
+
+/* Library version, "major.minor.patch". */
+const char *warpctct_version(void);
+
+/* Bytes of device workspace the two *_forward orchestrators need
+ * (units, alpha and beta lattices, all double).  Replaces the
+ * allocations of csrc/binding.cpp:70-77 (alphas, betas, counts); needs no
+ * host sync because it does not depend on max(lx-ly) (binding.cpp:68). */
+size_t warpctct_workspace_bytes(int N, int T, int U);
+
+/* ---- stage entry points (each replaces one reference stage) ------------ */
+
+/* Gather of the three units per live cell out of the joint tensor, scaled
+ * to log2 units.  Replaces warp_ctct/__init__.py:124-131 (index build +
+ * torch.gather).  joint (N,T,U+1,V) f32, ys (N,U) i32, lx/ly (N) i32,
+ * units_out (N,T,U+1,3) f64.  Cells with t>=lx[n] or u>ly[n] are not read
+ * and not written. */
+int warpctct_gather_units_f32(const float *joint, const int *ys, const int *lx, const int *ly,
+                              double *units_out, int N, int T, int U, int V, void *stream);
+
+/* Same for an already gathered (N,T,U+1,3) natural-log tensor, i.e. the
+ * `log_probs` argument of _C.ctct_loss_fwd (csrc/binding.cpp:31-35). */
+int warpctct_scale_units_f32(const float *units_nat, const int *lx, const int *ly,
+                             double *units_out, int N, int T, int U, void *stream);
+
+/* Units of the log-add joiner, LP = f + g - den (den may be NULL for the
+ * unnormalised variant).  Replaces the LOGPROBY/LOGPROBB macros of
+ * csrc/simple.cu:20-26 and csrc/simple_unnorm.cu:20-25.
+ * f_g (N,T,U+1), g_g (N,U+1,3), den (N,T,U+1) or NULL. */
+int warpctct_simple_units_f32(const float *f_g, const float *g_g, const float *den,
+                              const int *lx, const int *ly, double *units_out,
+                              int N, int T, int U, void *stream);
+
+/* Alpha and beta lattices of all N samples, concurrently, one wavefront per
+ * (sample, direction).  Replaces run_warp_ctct (csrc/core.h:14-16,
+ * csrc/gather.cu:293-309: k_warp_alphas + k_warp_betas).
+ * units (N,T,U+1,3) f64 log2 domain; alphas, betas (N,T+1,U+1,2) f64 =
+ * {state 2u-1, state 2u} (only t<=lx[n], u<=ly[n] is written); costs (N) f32
+ * = -beta(0,0) in natural-log units (csrc/binding.cpp:86).
+ * beta_only != 0 skips alpha (alphas may be NULL), as binding.cpp:84. */
+int warpctct_lattice_f32(const double *units, const int *ys, const int *lx, const int *ly,
+                         double *alphas, double *betas, float *costs, int N, int T, int U,
+                         int beta_only, void *stream);
+
+/* d(cost)/d(unit) for every cell, natural-log units, zero outside
+ * t<lx[n], u<=ly[n].  Replaces run_fill_grad + the zeros_like before it
+ * (csrc/core.h:18-20, csrc/gather.cu:311-387, csrc/binding.cpp:89).
+ * unit_grads (N,T,U+1,3). */
+int warpctct_unit_grads_f32(const double *units, const int *ys, const int *lx, const int *ly,
+                            const double *alphas, const double *betas, float *unit_grads, int N,
+                            int T, int U, void *stream);
+
+/* Dense gradient wrt the joint: every element of dense (N,T,U+1,V) is written
+ * exactly once — zero, or grad_out[n] * unit gradient at columns 0, y[u-1],
+ * y[u] (coincident columns add).  Replaces CTCTLoss.backward
+ * (warp_ctct/__init__.py:30-33) and autograd's gather backward (zeros +
+ * scatter_add).  grad_out (N) f32 or NULL (= ones). */
+int warpctct_dense_grad_f32(const float *unit_grads, const int *ys, const int *lx, const int *ly,
+                            const float *grad_out, float *dense, int N, int T, int U, int V,
+                            void *stream);
+
+/* ---- orchestrators ----------------------------------------------------- */
+
+/* ctct_loss forward on the un-gathered joint: gather, lattice, unit grads.
+ * Replaces warp_ctct/__init__.py:124-136 + _C.ctct_loss_fwd
+ * (csrc/binding.cpp:31-100).  unit_grads may be NULL (no-grad mode). */
+int warpctct_loss_forward_f32(const float *joint, const int *ys, const int *lx, const int *ly,
+                              int N, int T, int U, int V, void *workspace,
+                              size_t workspace_bytes, float *costs, float *unit_grads,
+                              void *stream);
+
+/* _C.ctct_loss_fwd proper: the input is already gathered (N,T,U+1,3). */
+int warpctct_loss_forward_units_f32(const float *units_nat, const int *ys, const int *lx,
+                                    const int *ly, int N, int T, int U, void *workspace,
+                                    size_t workspace_bytes, float *costs, float *unit_grads,
+                                    void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WARP_CTCT_HIP_H */

@@ -1,0 +1,51 @@
+"""CPU-side checks of the C-ABI library: it loads without a GPU, exports every
+symbol the header declares, and rejects bad arguments without touching a
+device."""
+import ctypes
+
+import hip_lib
+
+
+def test_library_exports_every_declared_symbol():
+    lib = hip_lib.lib()
+    names = hip_lib.declared_symbols()
+    assert "warpctct_loss_forward_f32" in names and "warpctct_dense_grad_f32" in names
+    for name in names:
+        assert hasattr(lib, name), name
+
+
+def test_version_and_error_strings():
+    lib = hip_lib.lib()
+    assert lib.warpctct_version().decode().count(".") == 2
+    assert lib.warpctct_error_string(0) == b"ok"
+    for code in range(1, 5):
+        assert len(lib.warpctct_error_string(code)) > 3
+
+
+def test_workspace_size_is_monotone_and_covers_buffers():
+    lib = hip_lib.lib()
+    N, T, U = 32, 250, 60
+    need = lib.warpctct_workspace_bytes(N, T, U)
+    floor = 8 * N * T * (U + 1) * 3 + 2 * 8 * N * (T + 1) * (U + 1) * 2
+    assert need >= floor and need < floor + 3 * 256
+    assert lib.warpctct_workspace_bytes(N, T + 1, U) > need
+    assert lib.warpctct_workspace_bytes(-1, T, U) == 0
+
+
+def test_invalid_arguments_are_rejected_on_the_host():
+    lib = hip_lib.lib()
+    null = ctypes.c_void_p(0)
+    EINVAL, EWORKSPACE = 1, 3
+    # negative size / null pointers: refused before any launch
+    assert lib.warpctct_gather_units_f32(null, null, null, null, null, -1, 4, 2, 8, null) == EINVAL
+    assert lib.warpctct_gather_units_f32(null, null, null, null, null, 2, 4, 2, 8, null) == EINVAL
+    assert lib.warpctct_dense_grad_f32(null, null, null, null, null, null, 2, 4, 2, 8, null) == EINVAL
+    # more contexts than a wavefront can hold
+    buf = (ctypes.c_float * 16)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    assert lib.warpctct_lattice_f32(p, p, p, p, p, p, p, 1, 1, 512, 0, null) == EINVAL
+    assert lib.warpctct_loss_forward_f32(p, p, p, p, 1, 1, 1, 8, p, ctypes.c_size_t(16), p, p,
+                                         null) == EWORKSPACE
+    # empty batch is a no-op
+    assert lib.warpctct_loss_forward_f32(null, null, null, null, 0, 4, 2, 8, null,
+                                         ctypes.c_size_t(0), null, null, null) == 0

@@ -1,0 +1,328 @@
+"""GPU parity tests of the ctct_loss path: HIP kernels (through the C ABI and
+through the warp_ctct Python API) against the float64 oracle on identical
+seeded inputs.
+
+Tolerances (from the build's north star): loss relative error <= 1e-5,
+gradient absolute error <= 1e-4, both in fp32 against the float64 oracle.
+Integer/structural facts (which cells are -inf, which gradient entries are
+exactly zero) are compared exactly."""
+import ctypes
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import hip_lib
+from ctct_cases import make_joint_case
+from oracle import c_oracle as C
+from oracle import ctct_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+LOSS_RTOL = 1e-5
+GRAD_ATOL = 1e-4
+LN2 = math.log(2.0)
+LOG2E = np.float64(1.4426950408889634074)
+
+
+def assert_support(got, ref, what):
+    """Structural zeros of the oracle are exact zeros here; an exact zero here
+    is either structural or an fp32 underflow of a negligible value."""
+    assert np.all(got[ref == 0] == 0), what + ": non-zero where the oracle has a structural zero"
+    assert np.all(np.abs(ref[got == 0]) < 1e-30), what + ": zero where the oracle has mass"
+
+
+def dev(a, dtype=None):
+    t = torch.as_tensor(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.cuda()
+
+
+def run_stages(joint, ys, lx, ly, beta_only=False):
+    """Call every stage through the C ABI; returns numpy views of all buffers."""
+    lib = hip_lib.lib()
+    N, T, U1, V = joint.shape
+    U = U1 - 1
+    s = hip_lib.stream_ptr()
+    d_joint, d_ys, d_lx, d_ly = dev(joint), dev(ys), dev(lx), dev(ly)
+    f64 = dict(device="cuda", dtype=torch.float64)
+    units = torch.full((N, T, U1, 3), float("nan"), **f64)
+    alphas = torch.full((N, T + 1, U1, 2), float("nan"), **f64)
+    betas = torch.full((N, T + 1, U1, 2), float("nan"), **f64)
+    costs = torch.full((N,), float("nan"), device="cuda")
+    ug = torch.full((N, T, U1, 3), float("nan"), device="cuda")
+    p = hip_lib.ptr
+    hip_lib.check(lib.warpctct_gather_units_f32(p(d_joint), p(d_ys), p(d_lx), p(d_ly), p(units),
+                                                N, T, U, V, s))
+    hip_lib.check(lib.warpctct_lattice_f32(p(units), p(d_ys), p(d_lx), p(d_ly),
+                                           p(None if beta_only else alphas), p(betas), p(costs),
+                                           N, T, U, int(beta_only), s))
+    if not beta_only:
+        hip_lib.check(lib.warpctct_unit_grads_f32(p(units), p(d_ys), p(d_lx), p(d_ly), p(alphas),
+                                                  p(betas), p(ug), N, T, U, s))
+    torch.cuda.synchronize()
+    out = dict(units=units, alphas=alphas, betas=betas, costs=costs, unit_grads=ug)
+    return {k: v.cpu().numpy() for k, v in out.items()}
+
+
+def check_lattice(name, stored, ref, lx, ly):
+    """stored (N,T+1,U+1,2) {o,e} in log2 units; ref[n] (lx+1, 2ly+1) natural
+    log.  Same -inf cells ("identical lattice paths"), finite cells within
+    2e-5 absolute (the values are O(1000))."""
+    for n in range(stored.shape[0]):
+        t, u = int(lx[n]), int(ly[n])
+        got = np.full((t + 1, 2 * u + 1), np.nan)
+        val = stored[n, :t + 1, :u + 1] * LN2
+        got[:, 0::2] = val[:, :, 1]
+        got[:, 1::2] = val[:, 1:, 0]
+        assert np.all(np.isneginf(stored[n, :t + 1, 0, 0])), name + ": state -1 must be -inf"
+        r = ref[n]
+        assert np.array_equal(np.isneginf(got), np.isneginf(r)), name + ": live-cell pattern differs"
+        fin = np.isfinite(r)
+        np.testing.assert_allclose(got[fin], r[fin], rtol=0, atol=2e-5, err_msg=name)
+
+
+CASES = [
+    # name, seed, N, T, U, V, lx, ly, sigma
+    ("c1_reference_config", 1, 2, 40, 10, 32, None, None, 1.0),
+    ("ragged_small", 2, 5, 23, 7, 16, range(9, 24), range(1, 8), 1.0),
+    ("single_label", 3, 3, 6, 1, 5, [6, 3, 1], [1, 1, 1], 1.0),
+    ("lx_equals_ly", 4, 2, 9, 9, 12, [9, 9], [9, 9], 1.0),
+    ("two_contexts_per_lane", 5, 3, 150, 100, 48, range(120, 151), range(64, 101), 1.0),
+    ("three_contexts_per_lane", 6, 2, 200, 160, 24, range(180, 201), range(129, 161), 2.0),
+    ("five_contexts_per_lane", 7, 2, 340, 300, 12, [340, 331], [300, 257], 1.0),
+    ("odd_vocab_scalar_stores", 8, 3, 17, 5, 37, range(8, 18), range(2, 6), 1.0),
+    ("vocab_1024_vector_stores", 9, 2, 30, 12, 1024, [30, 21], [12, 7], 1.0),
+    ("peaky", 10, 4, 60, 20, 64, range(40, 61), range(10, 21), 4.0),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
+def test_stages_against_oracle(case):
+    name, seed, N, T, U, V, lx, ly, sigma = case
+    joint, ys, lx, ly = make_joint_case(seed, N, T, U, V, lx=lx, ly=ly, sigma=sigma)
+    got = run_stages(joint, ys, lx, ly)
+    # gather: exact (the gathered fp32 value times log2(e), in double)
+    lp3 = O.gather_units(joint, ys)
+    for n in range(N):
+        t, u = int(lx[n]), int(ly[n])
+        exp = lp3[n, :t, :u + 1].astype(np.float64) * LOG2E
+        g = got["units"][n, :t, :u + 1]
+        np.testing.assert_array_equal(g[..., 0], exp[..., 0])
+        np.testing.assert_array_equal(g[:, 1:, 1], exp[:, 1:, 1])
+        np.testing.assert_array_equal(g[:, :u, 2], exp[:, :u, 2])
+        # padding is never written
+        assert np.all(np.isnan(got["units"][n, t:])) and np.all(np.isnan(got["units"][n, :, u + 1:]))
+    # lattices
+    ref_a, ref_b = [], []
+    for n in range(N):
+        t, u = int(lx[n]), int(ly[n])
+        a, ll_a = O.alpha_lattice(lp3[n, :t, :u + 1], ys[n, :u])
+        b, ll_b = O.beta_lattice(lp3[n, :t, :u + 1], ys[n, :u])
+        ref_a.append(a)
+        ref_b.append(b)
+    check_lattice("alpha", got["alphas"], ref_a, lx, ly)
+    check_lattice("beta", got["betas"], ref_b, lx, ly)
+    # costs and unit gradients
+    costs, grads = O.ctct_loss_fwd(lp3, ys, lx, ly)
+    np.testing.assert_allclose(got["costs"], costs, rtol=LOSS_RTOL)
+    np.testing.assert_allclose(got["unit_grads"], grads, atol=GRAD_ATOL, rtol=0)
+    assert_support(got["unit_grads"], grads, "unit grads")
+    # beta-only mode gives the same costs bit for bit
+    again = run_stages(joint, ys, lx, ly, beta_only=True)
+    np.testing.assert_array_equal(again["costs"], got["costs"])
+
+
+@pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
+def test_public_api_loss_and_dense_grad(case):
+    import warp_ctct
+    name, seed, N, T, U, V, lx, ly, sigma = case
+    joint, ys, lx, ly = make_joint_case(seed, N, T, U, V, lx=lx, ly=ly, sigma=sigma)
+    rng = np.random.default_rng(seed)
+    w = rng.standard_normal(N)
+    ref_loss, ref_dense, ref_costs = O.ctct_loss(joint, ys, lx, ly, reduction="none", grad_output=w)
+    x = dev(joint).requires_grad_(True)
+    costs = warp_ctct.ctct_loss(x, dev(ys), dev(lx), dev(ly), reduction="none")
+    (costs * dev(w, torch.float32)).sum().backward()
+    np.testing.assert_allclose(costs.detach().cpu().numpy(), ref_costs, rtol=LOSS_RTOL)
+    g = x.grad.cpu().numpy()
+    assert g.shape == joint.shape and x.grad.dtype == torch.float32
+    np.testing.assert_allclose(g, ref_dense, atol=GRAD_ATOL * max(1.0, np.abs(w).max()), rtol=0)
+    assert_support(g, ref_dense, "dense gradient")
+
+
+def test_repeated_label_columns_add():
+    """y[u-1] == y[u]: units k=1 and k=2 of context u land in the same column."""
+    joint, ys, lx, ly = make_joint_case(12, 1, 8, 3, 8, force_repeat=False)
+    ys[0] = [3, 3, 5]
+    import warp_ctct
+    x = dev(joint).requires_grad_(True)
+    loss = warp_ctct.ctct_loss(x, dev(ys), dev(lx), dev(ly), reduction="sum")
+    loss.backward()
+    _, dense, _ = O.ctct_loss(joint, ys, lx, ly, reduction="sum")
+    lp3 = O.gather_units(joint, ys)
+    _, ug = O.ctct_loss_fwd(lp3, ys, lx, ly)
+    # context 1 has current label 3 and next label 3
+    np.testing.assert_allclose(dense[0, :, 1, 3], ug[0, :, 1, 1] + ug[0, :, 1, 2], rtol=1e-12)
+    assert np.any(ug[0, :, 1, 1] != 0) and np.any(ug[0, :, 1, 2] != 0)
+    np.testing.assert_allclose(x.grad.cpu().numpy(), dense, atol=GRAD_ATOL, rtol=0)
+
+
+@pytest.mark.parametrize("reduction", ["none", "sum", "mean", None])
+@pytest.mark.parametrize("average_frames", [False, True])
+def test_reduction_and_average_frames(reduction, average_frames):
+    import warp_ctct
+    joint, ys, lx, ly = make_joint_case(13, 4, 19, 6, 11, lx=range(10, 20), ly=range(2, 7))
+    ref_loss, ref_dense, _ = O.ctct_loss(joint, ys, lx, ly, reduction=reduction,
+                                         average_frames=average_frames)
+    x = dev(joint).requires_grad_(True)
+    loss = warp_ctct.ctct_loss(x, dev(ys), dev(lx), dev(ly), reduction=reduction,
+                               average_frames=average_frames)
+    np.testing.assert_allclose(loss.detach().cpu().numpy(), ref_loss, rtol=LOSS_RTOL)
+    if reduction in ("none", None):
+        assert loss.shape == (4,)
+        loss.sum().backward()
+    else:
+        assert loss.dim() == 0
+        loss.backward()
+    np.testing.assert_allclose(x.grad.cpu().numpy(), ref_dense, atol=GRAD_ATOL, rtol=0)
+
+
+def test_no_grad_and_int64_lengths_and_half_input():
+    import warp_ctct
+    joint, ys, lx, ly = make_joint_case(14, 3, 21, 5, 9, lx=range(11, 22), ly=range(2, 6))
+    _, _, ref_costs = O.ctct_loss(joint, ys, lx, ly, reduction="none")
+    x = dev(joint)
+    c1 = warp_ctct.ctct_loss(x, dev(ys).long(), dev(lx).long(), dev(ly).long(), reduction="none")
+    assert not c1.requires_grad
+    np.testing.assert_allclose(c1.cpu().numpy(), ref_costs, rtol=LOSS_RTOL)
+    xr = dev(joint).requires_grad_(True)
+    with torch.no_grad():
+        c2 = warp_ctct.ctct_loss(xr, dev(ys), dev(lx), dev(ly), reduction="none")
+    assert not c2.requires_grad
+    np.testing.assert_array_equal(c2.cpu().numpy(), c1.cpu().numpy())
+    # a half-precision joint is computed in fp32 and gets a half gradient back
+    xh = dev(joint).half().requires_grad_(True)
+    _, _, ref_h = O.ctct_loss(xh.detach().float().cpu().numpy(), ys, lx, ly, reduction="none")
+    ch = warp_ctct.ctct_loss(xh, dev(ys), dev(lx), dev(ly), reduction="none")
+    assert ch.dtype == torch.float32
+    np.testing.assert_allclose(ch.detach().cpu().numpy(), ref_h, rtol=LOSS_RTOL)
+    ch.sum().backward()
+    assert xh.grad.dtype == torch.float16 and xh.grad.shape == xh.shape
+
+
+def test_operator_surface_on_gathered_units():
+    """_C.ctct_loss_fwd keeps the reference's contract: gathered (N,T,U+1,3)
+    input, (costs, grads) output, grads zero in padding, costs twice when
+    requires_grad is False."""
+    from warp_ctct import _C
+    joint, ys, lx, ly = make_joint_case(15, 4, 26, 8, 13, lx=range(12, 27), ly=range(3, 9))
+    lp3 = O.gather_units(joint, ys).astype(np.float32)
+    costs_ref, grads_ref = O.ctct_loss_fwd(lp3, ys, lx, ly)
+    costs, grads = _C.ctct_loss_fwd(dev(lp3), dev(ys), dev(lx), dev(ly), True)
+    np.testing.assert_allclose(costs.cpu().numpy(), costs_ref, rtol=LOSS_RTOL)
+    np.testing.assert_allclose(grads.cpu().numpy(), grads_ref, atol=GRAD_ATOL, rtol=0)
+    assert_support(grads.cpu().numpy(), grads_ref, "unit grads")
+    c2, same = _C.ctct_loss_fwd(dev(lp3), dev(ys), dev(lx), dev(ly), False)
+    assert same.data_ptr() == c2.data_ptr()
+    np.testing.assert_array_equal(c2.cpu().numpy(), costs.cpu().numpy())
+
+
+def test_binding_rejects_bad_tensors():
+    from warp_ctct import _C
+    joint, ys, lx, ly = make_joint_case(16, 2, 6, 2, 5)
+    lp3 = dev(O.gather_units(joint, ys).astype(np.float32))
+    d_ys, d_lx, d_ly = dev(ys), dev(lx), dev(ly)
+    with pytest.raises(RuntimeError):
+        _C.ctct_loss_fwd(lp3.double(), d_ys, d_lx, d_ly, True)          # dtype
+    with pytest.raises(RuntimeError):
+        _C.ctct_loss_fwd(lp3, d_ys.long(), d_lx, d_ly, True)            # label dtype
+    with pytest.raises(RuntimeError):
+        _C.ctct_loss_fwd(lp3.cpu(), d_ys, d_lx, d_ly, True)             # device
+    with pytest.raises(RuntimeError):
+        _C.ctct_loss_fwd(lp3.transpose(1, 2), d_ys, d_lx, d_ly, True)   # layout
+    with pytest.raises(RuntimeError):
+        _C.ctct_loss_fwd(lp3[..., :2].contiguous(), d_ys, d_lx, d_ly, True)   # not gathered
+    with pytest.raises(RuntimeError):
+        _C.ctct_loss_fwd(lp3, d_ys, d_lx[:1], d_ly, True)               # batch mismatch
+    import warp_ctct
+    with pytest.raises(AssertionError):
+        warp_ctct.ctct_loss(dev(joint), d_ys[:, :1], d_lx, d_ly)
+    with pytest.raises(AssertionError):
+        warp_ctct.ctct_loss(dev(joint), d_ys, d_lx, d_ly, reduction="avg")
+
+
+def test_infeasible_sample_has_infinite_cost():
+    import warp_ctct
+    joint, ys, lx, ly = make_joint_case(17, 2, 6, 3, 5, force_repeat=False)
+    ys[0] = [2, 2, 2]
+    lx = np.array([4, 6], dtype=np.int32)          # sample 0 needs 5 frames
+    ly = np.array([3, 3], dtype=np.int32)
+    c = warp_ctct.ctct_loss(dev(joint), dev(ys), dev(lx), dev(ly), reduction="none").cpu().numpy()
+    _, _, ref = O.ctct_loss(joint, ys, lx, ly, reduction="none")
+    assert np.isposinf(c[0]) and np.isposinf(ref[0])
+    np.testing.assert_allclose(c[1], ref[1], rtol=LOSS_RTOL)
+
+
+def test_full_size_typical_asr_batch():
+    """N=32, T<=250, U<=60, V=1024: costs and unit gradients against the C
+    oracle in float64; the 2 GB dense gradient is checked on the GPU through
+    size-independent properties (support, per-frame mass -1, gathered values)."""
+    import warp_ctct
+    N, T, U, V = 32, 250, 60, 1024
+    g = torch.Generator(device="cuda").manual_seed(1234)
+    logits = torch.randn(N, T, U + 1, V, device="cuda", generator=g)
+    joint = logits.log_softmax(-1)
+    del logits
+    rng = np.random.default_rng(1234)
+    lx = rng.integers(150, 251, N).astype(np.int32)
+    ly = rng.integers(30, 61, N).astype(np.int32)
+    lx[3], ly[5] = 250, 60
+    ys = rng.integers(1, V, (N, U)).astype(np.int32)
+    ys[:, 7] = ys[:, 6]
+    d_ys, d_lx, d_ly = dev(ys), dev(lx), dev(ly)
+    t_idx = torch.arange(T, device="cuda")[None, :, None, None]
+    u_idx = torch.arange(U + 1, device="cuda")[None, None, :, None]
+    pad = (t_idx >= d_lx[:, None, None, None]) | (u_idx > d_ly[:, None, None, None])
+    joint.masked_fill_(pad, 0.0)
+    joint.requires_grad_(True)
+    w = torch.tensor(rng.standard_normal(N), dtype=torch.float32, device="cuda")
+    costs = warp_ctct.ctct_loss(joint, d_ys, d_lx, d_ly, reduction="none")
+    (costs * w).sum().backward()
+    dense = joint.grad
+    # reference from the gathered units (exactly what the reference's gather yields)
+    index = torch.zeros(N, U + 1, 3, dtype=torch.long, device="cuda")
+    index[:, 1:, 1] = d_ys
+    index[:, :U, 2] = d_ys
+    index = index[:, None].expand(-1, T, -1, -1)
+    lp3 = joint.detach().gather(-1, index).cpu().numpy()
+    costs_ref, ug_ref = C.ctct_loss_fwd(lp3, ys, lx, ly, dtype=np.float64)
+    np.testing.assert_allclose(costs.detach().cpu().numpy(), costs_ref, rtol=LOSS_RTOL)
+    ug_ref_w = ug_ref * w.cpu().numpy().astype(np.float64)[:, None, None, None]
+    # values on the gathered columns (context 7 has coincident columns k=1,k=2)
+    got = dense.gather(-1, index).cpu().numpy().astype(np.float64)
+    exp = ug_ref_w.copy()
+    assert (ys[:, 6] == ys[:, 7]).all()
+    for n in range(N):
+        for u in range(1, U):
+            if ys[n, u - 1] == ys[n, u]:
+                both = ug_ref_w[n, :, u, 1] + ug_ref_w[n, :, u, 2]
+                exp[n, :, u, 1] = both
+                exp[n, :, u, 2] = both
+    exp[:, :, 0, 1] = exp[:, :, 0, 0]          # u=0,k=1 and u=U,k=2 gather column 0
+    exp[:, :, U, 2] = exp[:, :, U, 0]
+    scale = max(1.0, float(w.abs().max()))
+    np.testing.assert_allclose(got, exp, atol=GRAD_ATOL * scale, rtol=0)
+    # support: every non-zero sits on a gathered column
+    mask = torch.zeros_like(dense, dtype=torch.bool)
+    mask.scatter_(-1, index, True)
+    assert int((dense != 0).sum()) == int(((dense != 0) & mask).sum())
+    assert int((dense[pad.expand_as(dense)] != 0).sum()) == 0
+    # per-frame mass: sum over (u, v) = -w[n] for t < lx[n], 0 beyond
+    mass = dense.double().sum((2, 3)).cpu().numpy()
+    wn = w.cpu().numpy().astype(np.float64)
+    for n in range(N):
+        np.testing.assert_allclose(mass[n, :lx[n]], -wn[n], rtol=1e-4, atol=1e-5)
+        assert np.all(mass[n, lx[n]:] == 0)

@@ -1,0 +1,71 @@
+// Device-side helpers shared by the gfx950 kernels: log2-domain semiring
+// arithmetic (double state, native fp32 transcendentals) and 64-lane
+// wavefront data movement through DPP.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+namespace wctct {
+
+constexpr int kWave = 64;
+constexpr double kLog2e = 1.4426950408889634074;
+constexpr double kLn2 = 0.6931471805599453094;
+// Finite stand-in used only to form differences against a maximum that may be
+// -inf:  (-inf) - max(-inf, kFloor) = -inf  instead of NaN.
+constexpr double kFloor = -1.0e300;
+
+__device__ __forceinline__ double neg_inf() { return -__builtin_huge_val(); }
+
+// 2^x and log2(x) straight on the transcendental unit (v_exp_f32, v_log_f32;
+// no denormal fix-up: a result below 2^-126 flushes to 0, which is what a
+// log-semiring sum wants).
+__device__ __forceinline__ float exp2_hw(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float log2_hw(float x) { return __builtin_amdgcn_logf(x); }
+
+// The lattice keeps its log2 values in double (gfx950 issues v_add_f64 /
+// v_max_f64 at the fp32 rate), so sums of hundreds of log-probabilities lose
+// nothing; only the bounded correction term log2(1 + 2^d), d <= 0, goes
+// through the fp32 transcendental unit.  The absolute error of one (+) is
+// ~1e-7 whatever the magnitude of the operands, where plain fp32 arithmetic
+// on values near -2000 would lose ~1e-4 per operation.
+
+// log2(2^x + 2^y); -inf (+) -inf = -inf, never NaN for non-NaN inputs.
+// Same value as logaddexpf_ of the reference (csrc/gather.cu:23-34) up to the
+// change of base: larger + log(1 + exp(smaller - larger)).
+__device__ __forceinline__ double lse2(double x, double y) {
+    const double mx = __builtin_fmax(x, y);
+    const double mn = __builtin_fmin(x, y);
+    const float d = (float)(mn - __builtin_fmax(mx, kFloor));
+    return mx + (double)log2_hw(1.0f + exp2_hw(d));
+}
+
+// log2(2^x + 2^y + 2^z).  All three -inf: the sum of exponentials is 0, its
+// log2 is -inf, the result is -inf.
+__device__ __forceinline__ double lse3(double x, double y, double z) {
+    const double mx = __builtin_fmax(__builtin_fmax(x, y), z);
+    const double ms = __builtin_fmax(mx, kFloor);
+    const float s =
+        exp2_hw((float)(x - ms)) + exp2_hw((float)(y - ms)) + exp2_hw((float)(z - ms));
+    return ms + (double)log2_hw(s);
+}
+
+// Lane l receives x of lane l-1; lane 0 receives `fill`.  Two DPP moves
+// (wave_shr:1), no LDS traffic.
+__device__ __forceinline__ double wave_shift_up(double x, double fill) {
+    const int lo = __builtin_amdgcn_update_dpp(__double2loint(fill), __double2loint(x),
+                                               0x138 /* wave_shr:1 */, 0xf, 0xf, false);
+    const int hi = __builtin_amdgcn_update_dpp(__double2hiint(fill), __double2hiint(x), 0x138,
+                                               0xf, 0xf, false);
+    return __hiloint2double(hi, lo);
+}
+
+// Lane l receives x of lane l+1; lane 63 receives `fill` (wave_shl:1).
+__device__ __forceinline__ double wave_shift_down(double x, double fill) {
+    const int lo = __builtin_amdgcn_update_dpp(__double2loint(fill), __double2loint(x),
+                                               0x130 /* wave_shl:1 */, 0xf, 0xf, false);
+    const int hi = __builtin_amdgcn_update_dpp(__double2hiint(fill), __double2hiint(x), 0x130,
+                                               0xf, 0xf, false);
+    return __hiloint2double(hi, lo);
+}
+
+}  // namespace wctct

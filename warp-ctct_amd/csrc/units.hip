@@ -1,0 +1,173 @@
+// Per-cell "units" of the CTC-Transducer lattice and their gradients.
+//
+// A unit is one of the three log-probabilities a cell (t,u) contributes:
+//   k=0 blank, k=1 label y[u-1] ("current"), k=2 label y[u] ("next")
+// (csrc/gather.cu:16-21 of the reference).  The kernels here
+//   * pull the units out of the (N,T,U+1,V) joint tensor (replaces the index
+//     build + torch.gather of warp_ctct/__init__.py:124-131),
+//   * or form them from the log-add joiner operands f, g, den (replaces the
+//     LOGPROBY/LOGPROBB macros of csrc/simple.cu:20-26, simple_unnorm.cu:20-25),
+//   * and turn alpha/beta into d(cost)/d(unit) (replaces k_fill_grad,
+//     csrc/gather.cu:311-374).
+// Units are stored as doubles scaled to log2, the lattice's working format
+// (v_exp_f32 / v_log_f32 are base 2, and the lattice sums in double).  One
+// thread per cell; cells of padding (t >= lx[n] or u > ly[n]) are never read.
+#include "device_utils.h"
+#include "launch.h"
+
+namespace wctct {
+
+namespace {
+
+constexpr int kCellBlock = 256;
+
+struct Cell {
+    int n, t, u, Tn, Un;
+    bool in_range, live;
+};
+
+__device__ __forceinline__ Cell locate_cell(const int *lx, const int *ly, int T, int U) {
+    Cell c;
+    const int U1 = U + 1;
+    c.n = blockIdx.y;
+    const int cell = blockIdx.x * kCellBlock + threadIdx.x;
+    c.in_range = cell < T * U1;
+    c.t = cell / U1;
+    c.u = cell - c.t * U1;
+    c.Tn = min(max(lx[c.n], 0), T);
+    c.Un = min(max(ly[c.n], 0), U);
+    c.live = c.in_range && c.t < c.Tn && c.u <= c.Un;
+    return c;
+}
+
+__device__ __forceinline__ void store_units(double *units, const Cell &c, int T, int U, double b,
+                                            double cur, double nxt) {
+    double *o = units + (((size_t)c.n * T + c.t) * (U + 1) + c.u) * 3;
+    o[0] = b * kLog2e;
+    o[1] = cur * kLog2e;
+    o[2] = nxt * kLog2e;
+}
+
+__global__ __launch_bounds__(kCellBlock) void gather_units_kernel(
+    const float *__restrict__ joint, const int *__restrict__ ys, const int *__restrict__ lx,
+    const int *__restrict__ ly, double *__restrict__ units, int T, int U, int V) {
+    const Cell c = locate_cell(lx, ly, T, U);
+    if (!c.live) return;
+    const float *row = joint + (((size_t)c.n * T + c.t) * (U + 1) + c.u) * (size_t)V;
+    const int *y = ys + (size_t)c.n * U;
+    const float b = row[0];
+    float cur = b, nxt = b;   // the reference gathers index 0 where no label exists
+    // labels are clamped into [0,V) so that a corrupt label cannot fault
+    if (c.u >= 1) cur = row[min(max(y[c.u - 1], 0), V - 1)];
+    if (c.u < c.Un) nxt = row[min(max(y[c.u], 0), V - 1)];
+    store_units(units, c, T, U, b, cur, nxt);
+}
+
+__global__ __launch_bounds__(kCellBlock) void scale_units_kernel(
+    const float *__restrict__ units_nat, const int *__restrict__ lx, const int *__restrict__ ly,
+    double *__restrict__ units, int T, int U) {
+    const Cell c = locate_cell(lx, ly, T, U);
+    if (!c.live) return;
+    const float *i = units_nat + (((size_t)c.n * T + c.t) * (U + 1) + c.u) * 3;
+    store_units(units, c, T, U, i[0], i[1], i[2]);
+}
+
+// LP(t,u,0) = f_g[t,0]   + g_g[u,0] - den[t,u]
+// LP(t,u,k) = f_g[t,u+k-1] + g_g[u,k] - den[t,u],  k = 1 (u >= 1), 2 (u < U)
+__global__ __launch_bounds__(kCellBlock) void simple_units_kernel(
+    const float *__restrict__ f_g, const float *__restrict__ g_g, const float *__restrict__ den,
+    const int *__restrict__ lx, const int *__restrict__ ly, double *__restrict__ units, int T,
+    int U) {
+    const Cell c = locate_cell(lx, ly, T, U);
+    if (!c.live) return;
+    const int U1 = U + 1;
+    const float *fr = f_g + ((size_t)c.n * T + c.t) * U1;
+    const float *gr = g_g + ((size_t)c.n * U1 + c.u) * 3;
+    const double d = den ? (double)den[((size_t)c.n * T + c.t) * U1 + c.u] : 0.0;
+    const double b = (double)fr[0] + (double)gr[0] - d;
+    const double cur = (c.u >= 1) ? (double)fr[c.u] + (double)gr[1] - d : b;
+    const double nxt = (c.u < c.Un) ? (double)fr[c.u + 1] + (double)gr[2] - d : b;
+    store_units(units, c, T, U, b, cur, nxt);
+}
+
+// g0 = -[2^(a_e+LP0+b_e-ll) + 2^(a_o+LP0+b_e-ll)]
+// g1 = - 2^(a_o+LP1+b_o-ll)
+// g2 = -[2^(a_e+LP2+b_o'-ll) + [y[u-1]!=y[u]] 2^(a_o+LP2+b_o'-ll)]       (u < U)
+// with a_* = alpha(t,.) of context u, b_* = beta(t+1,.) of context u,
+// b_o' = beta(t+1, 2u+1) (context u+1), ll = beta(0,0), all in log2 units.
+// alpha(t, 2u-1) of context 0 is stored as -inf, which zeroes the u >= 1 terms.
+// The exponent is summed in double and rounded once.
+__global__ __launch_bounds__(kCellBlock) void unit_grads_kernel(
+    const double *__restrict__ units, const int *__restrict__ ys, const int *__restrict__ lx,
+    const int *__restrict__ ly, const double *__restrict__ alphas,
+    const double *__restrict__ betas, float *__restrict__ unit_grads, int T, int U) {
+    const Cell c = locate_cell(lx, ly, T, U);
+    if (!c.in_range) return;
+    const int U1 = U + 1;
+    float *go = unit_grads + (((size_t)c.n * T + c.t) * U1 + c.u) * 3;
+    if (!c.live) {
+        go[0] = 0.0f;
+        go[1] = 0.0f;
+        go[2] = 0.0f;
+        return;
+    }
+    const size_t lat = (size_t)(T + 1) * U1 * 2;
+    const double *an = alphas + (size_t)c.n * lat;
+    const double *bn = betas + (size_t)c.n * lat;
+    const double ll = bn[1];   // beta(0, state 0): pair {o,e} of context 0 at t = 0
+    const double2 a = *reinterpret_cast<const double2 *>(an + ((size_t)c.t * U1 + c.u) * 2);
+    const double2 b = *reinterpret_cast<const double2 *>(bn + ((size_t)(c.t + 1) * U1 + c.u) * 2);
+    const double *lp = units + (((size_t)c.n * T + c.t) * U1 + c.u) * 3;
+    const double lp0 = lp[0] - ll, lp1 = lp[1] - ll, lp2 = lp[2] - ll;
+    const float g0 = -(exp2_hw((float)(a.y + lp0 + b.y)) + exp2_hw((float)(a.x + lp0 + b.y)));
+    const float g1 = -exp2_hw((float)(a.x + lp1 + b.x));
+    float g2 = 0.0f;
+    if (c.u < c.Un) {
+        const double bo_next = bn[((size_t)(c.t + 1) * U1 + c.u + 1) * 2];
+        g2 = -exp2_hw((float)(a.y + lp2 + bo_next));
+        const int *y = ys + (size_t)c.n * U;
+        if (c.u >= 1 && y[c.u - 1] != y[c.u]) g2 -= exp2_hw((float)(a.x + lp2 + bo_next));
+    }
+    go[0] = g0;
+    go[1] = (c.u >= 1) ? g1 : 0.0f;
+    go[2] = g2;
+}
+
+inline dim3 cell_grid(int N, int T, int U) {
+    const long cells = (long)T * (U + 1);
+    return dim3((unsigned)((cells + kCellBlock - 1) / kCellBlock), (unsigned)N);
+}
+
+}  // namespace
+
+hipError_t launch_gather_units(const float *joint, const int *ys, const int *lx, const int *ly,
+                               double *units, int N, int T, int U, int V, hipStream_t stream) {
+    hipLaunchKernelGGL(gather_units_kernel, cell_grid(N, T, U), dim3(kCellBlock), 0, stream,
+                       joint, ys, lx, ly, units, T, U, V);
+    return hipGetLastError();
+}
+
+hipError_t launch_scale_units(const float *units_nat, const int *lx, const int *ly, double *units,
+                              int N, int T, int U, hipStream_t stream) {
+    hipLaunchKernelGGL(scale_units_kernel, cell_grid(N, T, U), dim3(kCellBlock), 0, stream,
+                       units_nat, lx, ly, units, T, U);
+    return hipGetLastError();
+}
+
+hipError_t launch_simple_units(const float *f_g, const float *g_g, const float *den,
+                               const int *lx, const int *ly, double *units, int N, int T, int U,
+                               hipStream_t stream) {
+    hipLaunchKernelGGL(simple_units_kernel, cell_grid(N, T, U), dim3(kCellBlock), 0, stream, f_g,
+                       g_g, den, lx, ly, units, T, U);
+    return hipGetLastError();
+}
+
+hipError_t launch_unit_grads(const double *units, const int *ys, const int *lx, const int *ly,
+                             const double *alphas, const double *betas, float *unit_grads, int N,
+                             int T, int U, hipStream_t stream) {
+    hipLaunchKernelGGL(unit_grads_kernel, cell_grid(N, T, U), dim3(kCellBlock), 0, stream, units,
+                       ys, lx, ly, alphas, betas, unit_grads, T, U);
+    return hipGetLastError();
+}
+
+}  // namespace wctct

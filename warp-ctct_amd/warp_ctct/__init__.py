@@ -1,0 +1,124 @@
+"""CTC-Transducer loss for AMD MI355X (gfx950) with the warp_ctct API.
+
+Drop-in for ``warp_ctct`` of maxwellzh/warp-ctct: the public functions
+``ctct_loss`` and ``ctct_simple_loss`` keep the reference's signatures,
+assertions, reduction / average_frames semantics and autograd contract
+(warp_ctct/__init__.py:88-147 and :150-236 of the reference); blank = 0.
+
+All device work is done by hand-written HIP kernels in libwarpctct_hip.so,
+reached through the torch binding ``warp_ctct._C``.  There is no CPU or eager
+fallback: importing this package without the built extension raises.
+"""
+from typing import Optional
+
+import torch
+
+try:
+    from . import _C as core
+except ImportError as exc:  # pragma: no cover - exercised only on a broken install
+    raise ImportError(
+        "warp_ctct._C (the HIP extension) is not built; run "
+        "`python setup.py build_ext --inplace` in warp-ctct_amd/ "
+        "(needs hipcc, --offload-arch=gfx950)"
+    ) from exc
+
+__all__ = ["ctct_loss", "ctct_simple_loss"]
+__version__ = core.library_version()
+
+
+def _no_autocast():
+    return torch.autocast(device_type="cuda", enabled=False)
+
+
+def _as_int(x: torch.Tensor) -> torch.Tensor:
+    return x.to(torch.int).contiguous()
+
+
+class _CTCTLoss(torch.autograd.Function):
+    """ctct_loss on the un-gathered joint.
+
+    Counterpart of the reference's gather (warp_ctct/__init__.py:124-131) +
+    CTCTLoss (:20-33).  Forward runs gather, lattice and unit gradients on the
+    GPU and stashes the (N,T,U+1,3) unit gradients; backward writes the dense
+    gradient in one pass, scaled by grad_output[n]."""
+
+    @staticmethod
+    def forward(ctx, joint, labels, lx, ly, requires_grad):
+        costs, unit_grads = core.ctct_loss_joint_fwd(joint, labels, lx, ly, requires_grad)
+        if requires_grad:
+            ctx.save_for_backward(unit_grads, labels, lx, ly)
+            ctx.vocab = joint.size(3)
+        return costs
+
+    @staticmethod
+    def backward(ctx, grad_outputs):
+        unit_grads, labels, lx, ly = ctx.saved_tensors
+        grad_outputs = grad_outputs.reshape(-1).float().contiguous()
+        dense = core.ctct_loss_joint_bwd(unit_grads, labels, lx, ly, grad_outputs, ctx.vocab)
+        return dense, None, None, None, None
+
+
+def _reduce(costs, frames_lengths, reduction, average_frames):
+    # warp_ctct/__init__.py:138-147 of the reference
+    if average_frames:
+        costs = costs / frames_lengths
+    if reduction == "none" or reduction is None:
+        return costs
+    if reduction == "sum":
+        return costs.sum()
+    if reduction == "mean":
+        return costs.mean()
+    return costs
+
+
+def ctct_loss(log_probs: torch.Tensor,
+              labels: torch.Tensor,
+              frames_lengths: torch.Tensor,
+              labels_lengths: torch.Tensor,
+              reduction: Optional[str] = "mean",
+              average_frames: bool = False) -> torch.Tensor:
+    """The CTC-Transducer loss.
+
+    Args:
+        log_probs: (N, T, U, V) joint log-probabilities, where N is the batch
+            size, T the maximum number of frames, U the maximum number of
+            labels + 1 and V the vocabulary size including the blank (index 0).
+        labels: (N, U-1) reference labels.
+        frames_lengths: (N,) number of frames of each sample.
+        labels_lengths: (N,) number of labels of each sample.
+        reduction: 'none' | 'mean' | 'sum' (None behaves like 'none').
+        average_frames: divide each sample's loss by its number of frames.
+    """
+    assert average_frames is None or isinstance(average_frames, bool)
+    assert reduction is None or reduction in ("none", "mean", "sum")
+    assert log_probs.dim() == 4
+    assert labels.dim() == 2
+    assert log_probs.size(2) == labels.size(1) + 1
+    assert log_probs.size(0) == labels.size(0) == frames_lengths.size(0) == labels_lengths.size(0)
+
+    enable_grad = log_probs.requires_grad and torch.is_grad_enabled()
+    with _no_autocast():
+        costs = _CTCTLoss.apply(log_probs.float().contiguous(), _as_int(labels),
+                                _as_int(frames_lengths), _as_int(labels_lengths), enable_grad)
+    return _reduce(costs, frames_lengths, reduction, average_frames)
+
+
+def ctct_simple_loss(f: torch.Tensor,
+                     g: torch.Tensor,
+                     labels: torch.Tensor,
+                     frames_lengths: torch.Tensor,
+                     labels_lengths: torch.Tensor,
+                     reduction: Optional[str] = "mean",
+                     average_frames: bool = False,
+                     normalized: bool = True) -> torch.Tensor:
+    """The CTC-Transducer loss with the log-add joiner  joint = f (+) g.
+
+    Args:
+        f: (N, T, V) encoder scores.
+        g: (N, U, V) predictor scores, U = maximum number of labels + 1.
+        labels, frames_lengths, labels_lengths, reduction, average_frames: as
+            in :func:`ctct_loss`.
+        normalized: subtract logsumexp_v(f + g) per (t, u) (a proper
+            distribution); False scores paths with the raw sums.
+    """
+    raise NotImplementedError("ctct_simple_loss: HIP path not built yet")
