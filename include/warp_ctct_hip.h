@@ -114,6 +114,87 @@ int warpctct_loss_forward_units_f32(const float *units_nat, const int *ys, const
                                     size_t workspace_bytes, float *costs, float *unit_grads,
                                     void *stream);
 
+/* ---- log-add joiner path (ctct_simple_loss) ------------------------------ */
+
+/* Units straight from the un-gathered operands: f (N,T,V), g (N,U+1,V),
+ * den (N,T,U+1) or NULL.  Replaces the two torch.gather calls of
+ * warp_ctct/__init__.py:204-215 plus the LOGPROB macros of csrc/simple.cu:20-26. */
+int warpctct_simple_gather_units_f32(const float *f, const float *g, const float *den,
+                                     const int *ys, const int *lx, const int *ly,
+                                     double *units_out, int N, int T, int U, int V, void *stream);
+
+/* Reductions of unit gradients (N,T,U+1,3) that csrc/binding.cpp:198-219 does
+ * with ATen: grad_f (N,T,U+1), grad_g (N,U+1,3), grad_den (N,T,U+1) or NULL. */
+int warpctct_simple_reduce_f32(const float *unit_grads, float *grad_f, float *grad_g,
+                               float *grad_den, int N, int T, int U, void *stream);
+
+/* Backward of the two gathers: dense_f (N,T,V) += grad_out[n]*grad_f at columns
+ * [0, y0..y_{U-1}], dense_g (N,U+1,V) += grad_out[n]*grad_g at [0, y[u-1], y[u]]
+ * (atomic adds into buffers the caller has initialised).  Either dense pointer
+ * may be NULL.  Replaces SimpleCTCTLoss.backward (warp_ctct/__init__.py:76-85)
+ * and autograd's gather backward. */
+int warpctct_simple_scatter_f32(const float *grad_f, const float *grad_g, const int *ys,
+                                const int *lx, const int *ly, const float *grad_out,
+                                float *dense_f, float *dense_g, int N, int T, int U, int V,
+                                void *stream);
+
+/* p[0..n) = 0 with a kernel (safe to capture in a HIP graph). */
+int warpctct_zero_fill_f32(float *p, size_t n, void *stream);
+
+/* Bytes of workspace for the two simple_forward orchestrators. */
+size_t warpctct_simple_workspace_bytes(int N, int T, int U);
+
+/* ctct_simple_loss forward on f (N,T,V), g (N,U+1,V): den (if normalized),
+ * units, lattice, unit gradients and their reductions.  Replaces
+ * warp_ctct/__init__.py:195-225 + _C.ctct_loss_simple_fwd
+ * (csrc/binding.cpp:103-222).  den (N,T,U+1) is an output when normalized != 0
+ * (only t<lx[n], u<=ly[n] is written) and ignored otherwise.  grad_f/grad_g/
+ * grad_den may all be NULL (no-grad mode). */
+int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, const int *lx,
+                                const int *ly, int N, int T, int U, int V, int normalized,
+                                void *workspace, size_t workspace_bytes, float *den, float *costs,
+                                float *grad_f, float *grad_g, float *grad_den, void *stream);
+
+/* _C.ctct_loss_simple_fwd proper: f_g (N,T,U+1), g_g (N,U+1,3) already
+ * gathered, den (N,T,U+1) or NULL (unnormalised, csrc/simple_unnorm.cu). */
+int warpctct_simple_forward_units_f32(const float *f_g, const float *g_g, const float *den,
+                                      const int *ys, const int *lx, const int *ly, int N, int T,
+                                      int U, void *workspace, size_t workspace_bytes, float *costs,
+                                      float *grad_f, float *grad_g, float *grad_den, void *stream);
+
+/* Dense gradients of ctct_simple_loss: dense_f (N,T,V), dense_g (N,U+1,V),
+ * every element written.  With den != NULL the den-path
+ * (LogMMExp.backward, warp_ctct/__init__.py:45-52) is included:
+ * dense_f[t,v] = sum_u w*grad_den[t,u]*exp(f[t,v]+g[u,v]-den[t,u]) + scatter,
+ * dense_g likewise summed over t.  Either dense pointer may be NULL. */
+int warpctct_simple_backward_f32(const float *f, const float *g, const float *den,
+                                 const float *grad_f, const float *grad_g, const float *grad_den,
+                                 const int *ys, const int *lx, const int *ly,
+                                 const float *grad_out, int N, int T, int U, int V,
+                                 float *dense_f, float *dense_g, void *stream);
+
+/* ---- log-semiring matmul -------------------------------------------------- */
+
+/* Bytes of workspace for warpctct_logmm_fwd_f32 (row and column maxima). */
+size_t warpctct_logmm_workspace_bytes(int B, int M, int Nn);
+
+/* res[b,i,j] = log sum_k exp(lhs[b,i,k] + rhs[b,k,j]); operands strided in
+ * elements (lhs[b,i,k] at lhs[b*lsb + i*lsm + k*lsk], rhs[b,k,j] at
+ * rhs[b*rsb + k*rsk + j*rsn]), res contiguous (B,M,Nn).  Replaces
+ * log_matmul_cuda (csrc/binding.cpp:224-245, csrc/logmatmul.cu:148-181). */
+int warpctct_logmm_fwd_f32(const float *lhs, long lsb, long lsm, long lsk, const float *rhs,
+                           long rsb, long rsk, long rsn, int B, int M, int K, int Nn,
+                           void *workspace, size_t workspace_bytes, float *res, void *stream);
+
+/* grad_lhs[b,i,k] = sum_j go*exp(lhs+rhs-res), grad_rhs[b,k,j] = sum_i (same);
+ * grad_out and res contiguous (B,M,Nn); the gradients use the given element
+ * strides; either may be NULL.  Replaces log_matmul_backward
+ * (csrc/binding.cpp:247-324). */
+int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, long lsm, long lsk,
+                           const float *rhs, long rsb, long rsk, long rsn, const float *res, int B,
+                           int M, int K, int Nn, float *grad_lhs, long glsb, long glsm, long glsk,
+                           float *grad_rhs, long grsb, long grsk, long grsn, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

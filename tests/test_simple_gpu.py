@@ -1,0 +1,299 @@
+"""GPU parity tests of the log-add joiner path: log-semiring matmul (forward
+and backward), the reference's _C.ctct_loss_simple_fwd surface, and the public
+ctct_simple_loss with its autograd, against the float64 oracle.
+
+Tolerances: loss relative error <= 1e-5, gradient absolute error <= 1e-4."""
+import numpy as np
+import pytest
+import torch
+
+from ctct_cases import make_simple_case
+from oracle import c_oracle as C
+from oracle import ctct_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+LOSS_RTOL = 1e-5
+GRAD_ATOL = 1e-4
+
+
+def dev(a, dtype=None):
+    t = torch.as_tensor(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.cuda()
+
+
+# ------------------------------------------------------------------ log matmul
+@pytest.mark.parametrize("B,M,K,Nn", [(1, 1, 1, 1), (2, 5, 7, 3), (3, 70, 100, 33), (2, 130, 257, 81)])
+@pytest.mark.parametrize("layout", ["contiguous", "transposed_view"])
+def test_log_matmul_forward(B, M, K, Nn, layout):
+    from warp_ctct import _C
+    rng = np.random.default_rng(B * 1000 + M)
+    lhs = (rng.standard_normal((B, M, K)) * 3).astype(np.float32)
+    rhs = (rng.standard_normal((B, K, Nn)) * 3).astype(np.float32)
+    ref = C.log_matmul(lhs, rhs)
+    d_lhs = dev(lhs)
+    if layout == "contiguous":
+        d_rhs = dev(rhs)
+    else:   # what ctct_simple_loss passes: g (B,Nn,K) viewed as (B,K,Nn)
+        d_rhs = dev(np.ascontiguousarray(rhs.transpose(0, 2, 1))).transpose(1, 2)
+        assert not d_rhs.is_contiguous() or K == 1 or Nn == 1
+    out = _C.log_matmul(d_lhs, d_rhs)
+    assert out.shape == (B, M, Nn) and out.is_contiguous()
+    np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=1e-5, atol=1e-5)
+
+
+def test_log_matmul_infinities_and_far_apart_maxima():
+    from warp_ctct import _C
+    rng = np.random.default_rng(3)
+    B, M, K, Nn = 2, 9, 40, 6
+    lhs = rng.standard_normal((B, M, K)).astype(np.float32)
+    rhs = rng.standard_normal((B, K, Nn)).astype(np.float32)
+    lhs[0, 1, :] = -np.inf            # whole row -inf -> -inf outputs
+    rhs[1, :, 2] = -np.inf            # whole column -inf
+    lhs[0, 3, 5:] = -np.inf           # partly -inf
+    # row maximum at k=0, column maximum at k=7, 300 apart: the shifted sum
+    # underflows and the exact path must take over
+    lhs[1, 4, 0] = 300.0
+    rhs[1, 7, 4] = 300.0
+    ref = C.log_matmul(lhs, rhs)
+    out = _C.log_matmul(dev(lhs), dev(rhs)).cpu().numpy()
+    assert np.all(np.isneginf(out[0, 1])) and np.all(np.isneginf(out[1, :, 2]))
+    assert np.array_equal(np.isneginf(out), np.isneginf(ref))
+    fin = np.isfinite(ref)
+    np.testing.assert_allclose(out[fin], ref[fin], rtol=1e-5, atol=1e-5)
+    assert abs(out[1, 4, 4] - ref[1, 4, 4]) < 1e-3 and ref[1, 4, 4] > 290
+
+
+def test_log_matmul_rejects_bad_arguments():
+    from warp_ctct import _C
+    a = torch.zeros(2, 3, 4, device="cuda")
+    with pytest.raises(RuntimeError):
+        _C.log_matmul(a, torch.zeros(2, 5, 3, device="cuda"))      # inner sizes differ
+    with pytest.raises(RuntimeError):
+        _C.log_matmul(a.double(), torch.zeros(2, 4, 3, device="cuda").double())
+    with pytest.raises(RuntimeError):
+        _C.log_matmul(a.cpu(), torch.zeros(2, 4, 3))
+    with pytest.raises(RuntimeError):
+        _C.log_matmul(a[0], torch.zeros(4, 3, device="cuda"))
+
+
+@pytest.mark.parametrize("B,M,K,Nn", [(2, 5, 7, 3), (2, 45, 130, 40), (1, 33, 65, 17)])
+@pytest.mark.parametrize("mask", [(True, True), (True, False), (False, True)])
+def test_log_matmul_backward(B, M, K, Nn, mask):
+    from warp_ctct import _C
+    rng = np.random.default_rng(M + K)
+    lhs = rng.standard_normal((B, M, K)).astype(np.float32)
+    rhs_t = rng.standard_normal((B, Nn, K)).astype(np.float32)
+    rhs = rhs_t.transpose(0, 2, 1)
+    go = rng.standard_normal((B, M, Nn)).astype(np.float32)       # signed
+    go[0, 0, :] = 0.0
+    res = O.log_matmul(lhs, rhs)
+    gl, gr = O.log_matmul_backward(go, lhs, rhs, res)
+    d_rhs = dev(rhs_t).transpose(1, 2)
+    d_res = _C.log_matmul(dev(lhs), d_rhs)
+    out_l, out_r = _C.log_matmul_backward(dev(go), dev(lhs), d_rhs, d_res, list(mask))
+    if mask[0]:
+        assert out_l.shape == lhs.shape
+        np.testing.assert_allclose(out_l.cpu().numpy(), gl, atol=2e-5, rtol=1e-4)
+    else:
+        assert out_l is None
+    if mask[1]:
+        assert out_r.shape == (B, K, Nn)
+        np.testing.assert_allclose(out_r.cpu().numpy(), gr, atol=2e-5, rtol=1e-4)
+    else:
+        assert out_r is None
+
+
+# ------------------------------------------------ reference operator surface
+SIMPLE_CASES = [
+    # name, seed, N, T, U, V, lx, ly
+    ("small", 1, 3, 12, 4, 9, [12, 9, 7], [4, 2, 3]),
+    ("ragged", 2, 5, 40, 11, 33, range(20, 41), range(3, 12)),
+    ("two_contexts_per_lane", 3, 2, 140, 90, 50, [140, 120], [90, 70]),
+    ("single_label", 4, 2, 5, 1, 6, [5, 2], [1, 1]),
+]
+
+
+@pytest.mark.parametrize("case", SIMPLE_CASES, ids=[c[0] for c in SIMPLE_CASES])
+@pytest.mark.parametrize("normalized", [True, False])
+def test_operator_surface_simple_fwd(case, normalized):
+    """_C.ctct_loss_simple_fwd(f_g, g_g, ys, den, lx, ly, requires_grad)."""
+    from warp_ctct import _C
+    name, seed, N, T, U, V, lx, ly = case
+    f, g, ys, lx, ly = make_simple_case(seed, N, T, U, V, lx=lx, ly=ly, normalized=normalized)
+    f_g, g_g = O.gather_separate(f, g, ys)
+    den = O.log_matmul(f, np.swapaxes(g, 1, 2)).astype(np.float32) if normalized else None
+    costs, gf, gg, gd = O.ctct_loss_simple_fwd(f_g, g_g, ys, den, lx, ly)
+    d_den = dev(den) if normalized else torch.empty(1)       # the reference's own stand-in
+    out = _C.ctct_loss_simple_fwd(dev(f_g), dev(g_g), dev(ys), d_den, dev(lx), dev(ly), True)
+    np.testing.assert_allclose(out[0].cpu().numpy(), costs, rtol=LOSS_RTOL)
+    np.testing.assert_allclose(out[1].cpu().numpy(), gf, atol=GRAD_ATOL, rtol=0)
+    # grad_g sums T gradients: scale the bound by what was summed
+    np.testing.assert_allclose(out[2].cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
+    if normalized:
+        np.testing.assert_allclose(out[3].cpu().numpy(), gd, atol=GRAD_ATOL, rtol=0)
+    else:
+        assert out[3] is None
+    nog = _C.ctct_loss_simple_fwd(dev(f_g), dev(g_g), dev(ys), d_den, dev(lx), dev(ly), False)
+    np.testing.assert_array_equal(nog[0].cpu().numpy(), out[0].cpu().numpy())
+    assert nog[1] is None and nog[2] is None and nog[3] is None
+
+
+# ----------------------------------------------------------------- public API
+@pytest.mark.parametrize("case", SIMPLE_CASES, ids=[c[0] for c in SIMPLE_CASES])
+@pytest.mark.parametrize("normalized", [True, False])
+def test_public_simple_loss_and_grads(case, normalized):
+    import warp_ctct
+    name, seed, N, T, U, V, lx, ly = case
+    f, g, ys, lx, ly = make_simple_case(seed, N, T, U, V, lx=lx, ly=ly, normalized=normalized)
+    w = np.random.default_rng(seed).standard_normal(N)
+    loss, gf, gg, costs = O.ctct_simple_loss(f, g, ys, lx, ly, reduction="none",
+                                             normalized=normalized, grad_output=w)
+    tf = dev(f).requires_grad_(True)
+    tg = dev(g).requires_grad_(True)
+    out = warp_ctct.ctct_simple_loss(tf, tg, dev(ys), dev(lx), dev(ly), reduction="none",
+                                     normalized=normalized)
+    np.testing.assert_allclose(out.detach().cpu().numpy(), costs, rtol=LOSS_RTOL)
+    (out * dev(w, torch.float32)).sum().backward()
+    scale = max(1.0, float(np.abs(w).max()))
+    # dense gradients sum up to T (resp. U+1) unit gradients per entry
+    np.testing.assert_allclose(tf.grad.cpu().numpy(), gf, atol=GRAD_ATOL * scale, rtol=1e-5)
+    np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=GRAD_ATOL * scale, rtol=1e-5)
+    assert tf.grad.shape == f.shape and tg.grad.shape == g.shape
+    for n in range(N):
+        assert np.all(tf.grad[n, lx[n]:].cpu().numpy() == 0)
+        assert np.all(tg.grad[n, ly[n] + 1:].cpu().numpy() == 0)
+
+
+@pytest.mark.parametrize("track", [(True, False), (False, True), (False, False)])
+def test_simple_loss_partial_tracking_and_reduction(track):
+    import warp_ctct
+    f, g, ys, lx, ly = make_simple_case(7, 3, 15, 5, 12, lx=[15, 11, 8], ly=[5, 3, 4])
+    loss, gf, gg, _ = O.ctct_simple_loss(f, g, ys, lx, ly, reduction="mean", average_frames=True)
+    tf = dev(f).requires_grad_(track[0])
+    tg = dev(g).requires_grad_(track[1])
+    out = warp_ctct.ctct_simple_loss(tf, tg, dev(ys).long(), dev(lx).long(), dev(ly).long(),
+                                     reduction="mean", average_frames=True)
+    np.testing.assert_allclose(float(out.detach()), loss, rtol=LOSS_RTOL)
+    if not any(track):
+        assert not out.requires_grad
+        return
+    out.backward()
+    if track[0]:
+        np.testing.assert_allclose(tf.grad.cpu().numpy(), gf, atol=GRAD_ATOL, rtol=1e-5)
+    else:
+        assert tf.grad is None
+    if track[1]:
+        np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
+    else:
+        assert tg.grad is None
+
+
+def test_simple_loss_assertions():
+    import warp_ctct
+    f, g, ys, lx, ly = make_simple_case(8, 2, 6, 2, 5)
+    with pytest.raises(AssertionError):
+        warp_ctct.ctct_simple_loss(dev(f), dev(g)[:, :2], dev(ys), dev(lx), dev(ly))
+    with pytest.raises(AssertionError):
+        warp_ctct.ctct_simple_loss(dev(f)[0], dev(g), dev(ys), dev(lx), dev(ly))
+    with pytest.raises(AssertionError):
+        warp_ctct.ctct_simple_loss(dev(f), dev(g), dev(ys), dev(lx), dev(ly), reduction="max")
+
+
+def _identity_check(N, T, U, V, lx_rng, ly_rng, normalized, seed):
+    """ctct_simple_loss(f, g) == ctct_loss(joiner(f, g)) with the joint
+    materialised on the GPU, losses and gradients (through torch autograd of
+    the broadcast add / log_softmax)."""
+    import warp_ctct
+    rng = np.random.default_rng(seed)
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    f = torch.randn(N, T, V, device="cuda", generator=gen)
+    g = torch.randn(N, U + 1, V, device="cuda", generator=gen)
+    if normalized:
+        f = f.log_softmax(-1)
+        g = g.log_softmax(-1)
+    lx = rng.integers(lx_rng[0], lx_rng[1] + 1, N).astype(np.int32)
+    ly = rng.integers(ly_rng[0], ly_rng[1] + 1, N).astype(np.int32)
+    lx[0], ly[-1] = lx_rng[1], ly_rng[1]
+    ys = rng.integers(1, V, (N, U)).astype(np.int32)
+    ys[:, 5] = ys[:, 4]
+    d_ys, d_lx, d_ly = dev(ys), dev(lx), dev(ly)
+    w = torch.tensor(rng.standard_normal(N), dtype=torch.float32, device="cuda")
+    f1 = f.clone().requires_grad_(True)
+    g1 = g.clone().requires_grad_(True)
+    c1 = warp_ctct.ctct_simple_loss(f1, g1, d_ys, d_lx, d_ly, reduction="none",
+                                    normalized=normalized)
+    (c1 * w).sum().backward()
+    f2 = f.clone().requires_grad_(True)
+    g2 = g.clone().requires_grad_(True)
+    joint = f2[:, :, None, :] + g2[:, None, :, :]
+    if normalized:
+        joint = joint.log_softmax(-1)
+    c2 = warp_ctct.ctct_loss(joint, d_ys, d_lx, d_ly, reduction="none")
+    (c2 * w).sum().backward()
+    np.testing.assert_allclose(c1.detach().cpu().numpy(), c2.detach().cpu().numpy(), rtol=LOSS_RTOL)
+    scale = max(1.0, float(w.abs().max()))
+    # torch sums fp32 gradients over u (resp. t) in the reference side: allow for that
+    np.testing.assert_allclose(f1.grad.cpu().numpy(), f2.grad.cpu().numpy(),
+                               atol=2 * GRAD_ATOL * scale, rtol=1e-4)
+    np.testing.assert_allclose(g1.grad.cpu().numpy(), g2.grad.cpu().numpy(),
+                               atol=2 * GRAD_ATOL * scale, rtol=1e-4)
+    return c1
+
+
+def test_full_size_log_add_joiner_normalized():
+    """N=32, T<=400, U<=80, V=2048, normalized."""
+    c = _identity_check(32, 400, 80, 2048, (300, 400), (50, 80), True, 404)
+    assert torch.isfinite(c).all()
+
+
+def test_deep_lattice_unnormalized():
+    """The long-utterance shape (T<=1500, U<=300) at a vocabulary that lets the
+    joint be materialised for the identity check."""
+    c = _identity_check(2, 1500, 300, 256, (1200, 1500), (250, 300), False, 505)
+    assert torch.isfinite(c).all()
+
+
+def test_full_size_unnormalized_stress_against_c_oracle():
+    """N=4, T<=1500, U<=300, V=8192 raw scores: costs and compact gradients
+    against the C oracle in float64 on the gathered operands; dense gradients
+    through their scatter structure."""
+    import warp_ctct
+    from warp_ctct import _C
+    N, T, U, V = 4, 1500, 300, 8192
+    rng = np.random.default_rng(606)
+    gen = torch.Generator(device="cuda").manual_seed(606)
+    f = torch.randn(N, T, V, device="cuda", generator=gen)
+    g = torch.randn(N, U + 1, V, device="cuda", generator=gen)
+    lx = rng.integers(1200, 1501, N).astype(np.int32)
+    ly = rng.integers(250, 301, N).astype(np.int32)
+    lx[1], ly[2] = 1500, 300
+    ys = rng.integers(1, V, (N, U)).astype(np.int32)
+    ys[:, 9] = ys[:, 8]
+    d_ys, d_lx, d_ly = dev(ys), dev(lx), dev(ly)
+    f.requires_grad_(True)
+    g.requires_grad_(True)
+    costs = warp_ctct.ctct_simple_loss(f, g, d_ys, d_lx, d_ly, reduction="none", normalized=False)
+    costs.sum().backward()
+    # oracle on gathered operands
+    fi = torch.zeros(N, T, U + 1, dtype=torch.long, device="cuda")
+    fi[..., 1:] = d_ys.long()[:, None, :]
+    gi = torch.zeros(N, U + 1, 3, dtype=torch.long, device="cuda")
+    gi[:, 1:, 1] = d_ys
+    gi[:, :U, 2] = d_ys
+    f_g = f.detach().gather(-1, fi).cpu().numpy()
+    g_g = g.detach().gather(-1, gi).cpu().numpy()
+    lp3 = O.simple_units(f_g, g_g, None)
+    c_ref, ug = C.ctct_loss_fwd(lp3, ys, lx, ly, dtype=np.float64)
+    np.testing.assert_allclose(costs.detach().cpu().numpy(), c_ref, rtol=LOSS_RTOL)
+    gf_ref, gg_ref, _ = O.simple_unit_grad_reduce(ug, False)
+    # dense grad_f at the gathered columns: labels repeat, so compare column sums
+    dense_f = f.grad
+    exp_f = torch.zeros_like(dense_f, dtype=torch.float64)
+    exp_f.scatter_add_(-1, fi, torch.as_tensor(gf_ref).cuda())
+    np.testing.assert_allclose(dense_f.cpu().numpy(), exp_f.cpu().numpy(), atol=GRAD_ATOL, rtol=1e-5)
+    exp_g = torch.zeros_like(g.grad, dtype=torch.float64)
+    exp_g.scatter_add_(-1, gi, torch.as_tensor(gg_ref).cuda())
+    np.testing.assert_allclose(g.grad.cpu().numpy(), exp_g.cpu().numpy(), atol=GRAD_ATOL, rtol=1e-5)

@@ -63,6 +63,38 @@ int forward_from_units(const Workspace &w, const int *ys, const int *lx, const i
                                   stream));
 }
 
+struct SimpleWorkspace {
+    Workspace lattice;
+    float *unit_grads;   // (N,T,U+1,3)
+    float *fmax;         // (N,T)   row maxima of f
+    float *gmax;         // (N,U+1) row maxima of g
+    size_t bytes;
+};
+
+SimpleWorkspace carve_simple(void *base, int N, int T, int U) {
+    SimpleWorkspace w;
+    w.lattice = carve(base, N, T, U);
+    const uintptr_t p = reinterpret_cast<uintptr_t>(base) + w.lattice.bytes;
+    const size_t ug_b = align256((size_t)N * T * (U + 1) * 3 * sizeof(float));
+    const size_t fm_b = align256((size_t)N * T * sizeof(float));
+    const size_t gm_b = align256((size_t)N * (U + 1) * sizeof(float));
+    w.unit_grads = reinterpret_cast<float *>(p);
+    w.fmax = reinterpret_cast<float *>(p + ug_b);
+    w.gmax = reinterpret_cast<float *>(p + ug_b + fm_b);
+    w.bytes = w.lattice.bytes + ug_b + fm_b + gm_b;
+    return w;
+}
+
+// lattice + unit gradients + reductions, shared by the two simple forwards
+int simple_from_units(const SimpleWorkspace &w, const int *ys, const int *lx, const int *ly, int N,
+                      int T, int U, float *costs, float *grad_f, float *grad_g, float *grad_den,
+                      bool want_grad, hipStream_t stream) {
+    int rc = forward_from_units(w.lattice, ys, lx, ly, N, T, U, costs,
+                                want_grad ? w.unit_grads : nullptr, stream);
+    if (rc != WARPCTCT_OK || !want_grad) return rc;
+    return done(launch_simple_reduce(w.unit_grads, grad_f, grad_g, grad_den, N, T, U, stream));
+}
+
 }  // namespace
 
 extern "C" {
@@ -190,6 +222,189 @@ int warpctct_loss_forward_units_f32(const float *units_nat, const int *ys, const
     }
     return forward_from_units(w, ys, lx, ly, N, T, U, costs, T > 0 ? unit_grads : nullptr,
                               as_stream(stream));
+}
+
+int warpctct_simple_gather_units_f32(const float *f, const float *g, const float *den,
+                                     const int *ys, const int *lx, const int *ly,
+                                     double *units_out, int N, int T, int U, int V, void *stream) {
+    if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
+    if (N == 0 || T == 0) return WARPCTCT_OK;
+    if (!f || !g || !lx || !ly || !units_out || (U > 0 && !ys)) return WARPCTCT_EINVAL;
+    return done(launch_simple_gather_units(f, g, den, ys, lx, ly, units_out, N, T, U, V,
+                                           as_stream(stream)));
+}
+
+int warpctct_simple_reduce_f32(const float *unit_grads, float *grad_f, float *grad_g,
+                               float *grad_den, int N, int T, int U, void *stream) {
+    if (!dims_ok(N, T, U)) return WARPCTCT_EINVAL;
+    if (N == 0) return WARPCTCT_OK;
+    if (!grad_g || (T > 0 && (!unit_grads || !grad_f))) return WARPCTCT_EINVAL;
+    return done(launch_simple_reduce(unit_grads, grad_f, grad_g, grad_den, N, T, U,
+                                     as_stream(stream)));
+}
+
+int warpctct_simple_scatter_f32(const float *grad_f, const float *grad_g, const int *ys,
+                                const int *lx, const int *ly, const float *grad_out,
+                                float *dense_f, float *dense_g, int N, int T, int U, int V,
+                                void *stream) {
+    if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
+    if (N == 0) return WARPCTCT_OK;
+    if (!lx || !ly || (U > 0 && !ys) || (dense_f && !grad_f) || (dense_g && !grad_g))
+        return WARPCTCT_EINVAL;
+    return done(launch_simple_scatter(grad_f, grad_g, ys, lx, ly, grad_out, T > 0 ? dense_f : nullptr,
+                                      dense_g, N, T, U, V, as_stream(stream)));
+}
+
+int warpctct_zero_fill_f32(float *p, size_t n, void *stream) {
+    if (n == 0) return WARPCTCT_OK;
+    if (!p) return WARPCTCT_EINVAL;
+    return done(launch_zero_fill(p, n, as_stream(stream)));
+}
+
+size_t warpctct_simple_workspace_bytes(int N, int T, int U) {
+    if (N < 0 || T < 0 || U < 0) return 0;
+    return carve_simple(nullptr, N, T, U).bytes;
+}
+
+int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, const int *lx,
+                                const int *ly, int N, int T, int U, int V, int normalized,
+                                void *workspace, size_t workspace_bytes, float *den, float *costs,
+                                float *grad_f, float *grad_g, float *grad_den, void *stream) {
+    if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
+    if (N == 0) return WARPCTCT_OK;
+    const bool want_grad = grad_f || grad_g || grad_den;
+    if (!g || !lx || !ly || !costs || !workspace || (T > 0 && !f) || (U > 0 && !ys))
+        return WARPCTCT_EINVAL;
+    if (want_grad && (!grad_f || !grad_g || (normalized && !grad_den))) return WARPCTCT_EINVAL;
+    if (normalized && T > 0 && !den) return WARPCTCT_EINVAL;
+    const SimpleWorkspace w = carve_simple(workspace, N, T, U);
+    if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
+    hipStream_t st = as_stream(stream);
+    if (T > 0) {
+        if (normalized) {
+            // den[n,t,u] = logsumexp_v(f[n,t,v] + g[n,u,v]):  lhs = f, rhs[b,k,j] = g[b,j,k]
+            const LogmmOperand lhs = {f, (long)T * V, (long)V, 1L};
+            const LogmmOperand rhs = {g, (long)(U + 1) * V, 1L, (long)V};
+            int rc = done(launch_logmm_fwd(lhs, rhs, w.fmax, w.gmax, den, N, T, V, U + 1, lx, ly, st));
+            if (rc != WARPCTCT_OK) return rc;
+        }
+        int rc = done(launch_simple_gather_units(f, g, normalized ? den : nullptr, ys, lx, ly,
+                                                 w.lattice.units, N, T, U, V, st));
+        if (rc != WARPCTCT_OK) return rc;
+    }
+    return simple_from_units(w, ys, lx, ly, N, T, U, costs, grad_f, grad_g,
+                             normalized ? grad_den : nullptr, want_grad && T > 0, st);
+}
+
+int warpctct_simple_forward_units_f32(const float *f_g, const float *g_g, const float *den,
+                                      const int *ys, const int *lx, const int *ly, int N, int T,
+                                      int U, void *workspace, size_t workspace_bytes, float *costs,
+                                      float *grad_f, float *grad_g, float *grad_den, void *stream) {
+    if (!dims_ok(N, T, U)) return WARPCTCT_EINVAL;
+    if (N == 0) return WARPCTCT_OK;
+    const bool want_grad = grad_f || grad_g || grad_den;
+    if (!g_g || !lx || !ly || !costs || !workspace || (T > 0 && !f_g) || (U > 0 && !ys))
+        return WARPCTCT_EINVAL;
+    if (want_grad && (!grad_f || !grad_g || (den && !grad_den))) return WARPCTCT_EINVAL;
+    const SimpleWorkspace w = carve_simple(workspace, N, T, U);
+    if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
+    hipStream_t st = as_stream(stream);
+    if (T > 0) {
+        int rc = done(launch_simple_units(f_g, g_g, den, lx, ly, w.lattice.units, N, T, U, st));
+        if (rc != WARPCTCT_OK) return rc;
+    }
+    return simple_from_units(w, ys, lx, ly, N, T, U, costs, grad_f, grad_g,
+                             den ? grad_den : nullptr, want_grad && T > 0, st);
+}
+
+int warpctct_simple_backward_f32(const float *f, const float *g, const float *den,
+                                 const float *grad_f, const float *grad_g, const float *grad_den,
+                                 const int *ys, const int *lx, const int *ly,
+                                 const float *grad_out, int N, int T, int U, int V,
+                                 float *dense_f, float *dense_g, void *stream) {
+    if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
+    if (N == 0) return WARPCTCT_OK;
+    if (!lx || !ly || (U > 0 && !ys) || (dense_f && !grad_f) || (dense_g && !grad_g))
+        return WARPCTCT_EINVAL;
+    if (den && (!f || !g || !grad_den)) return WARPCTCT_EINVAL;
+    hipStream_t st = as_stream(stream);
+    const int U1 = U + 1;
+    if (T == 0) dense_f = nullptr;
+    if (den) {
+        const LogmmOperand lhs = {f, (long)T * V, (long)V, 1L};
+        const LogmmOperand rhs = {g, (long)U1 * V, 1L, (long)V};
+        if (dense_f) {
+            const LogmmGrad gl = {dense_f, (long)T * V, (long)V, 1L};
+            int rc = done(launch_logmm_bwd_lhs(lhs, rhs, grad_den, den, gl, N, T, V, U1, lx, ly,
+                                               grad_out, st));
+            if (rc != WARPCTCT_OK) return rc;
+        }
+        if (dense_g) {
+            // gradient of rhs[b,k,j] = g[b,j,k] stored straight into the (N,U+1,V) layout
+            const LogmmGrad gr = {dense_g, (long)U1 * V, 1L, (long)V};
+            int rc = done(launch_logmm_bwd_rhs(lhs, rhs, grad_den, den, gr, N, T, V, U1, lx, ly,
+                                               grad_out, st));
+            if (rc != WARPCTCT_OK) return rc;
+        }
+    } else {
+        if (dense_f) {
+            int rc = done(launch_zero_fill(dense_f, (size_t)N * T * V, st));
+            if (rc != WARPCTCT_OK) return rc;
+        }
+        if (dense_g) {
+            int rc = done(launch_zero_fill(dense_g, (size_t)N * U1 * V, st));
+            if (rc != WARPCTCT_OK) return rc;
+        }
+    }
+    return done(launch_simple_scatter(grad_f, grad_g, ys, lx, ly, grad_out, dense_f, dense_g, N, T,
+                                      U, V, st));
+}
+
+size_t warpctct_logmm_workspace_bytes(int B, int M, int Nn) {
+    if (B < 0 || M < 0 || Nn < 0) return 0;
+    return align256((size_t)B * M * sizeof(float)) + align256((size_t)B * Nn * sizeof(float));
+}
+
+int warpctct_logmm_fwd_f32(const float *lhs, long lsb, long lsm, long lsk, const float *rhs,
+                           long rsb, long rsk, long rsn, int B, int M, int K, int Nn,
+                           void *workspace, size_t workspace_bytes, float *res, void *stream) {
+    if (B < 0 || M < 0 || K < 0 || Nn < 0 || B > kMaxGrid || Nn > kMaxGrid * 32)
+        return WARPCTCT_EINVAL;
+    if (B == 0 || M == 0 || Nn == 0) return WARPCTCT_OK;
+    if (!res || !workspace || (K > 0 && (!lhs || !rhs))) return WARPCTCT_EINVAL;
+    if (workspace_bytes < warpctct_logmm_workspace_bytes(B, M, Nn)) return WARPCTCT_EWORKSPACE;
+    float *lmax = static_cast<float *>(workspace);
+    float *rmax = reinterpret_cast<float *>(static_cast<char *>(workspace) +
+                                            align256((size_t)B * M * sizeof(float)));
+    const LogmmOperand l = {lhs, lsb, lsm, lsk};
+    const LogmmOperand r = {rhs, rsb, rsk, rsn};
+    return done(launch_logmm_fwd(l, r, lmax, rmax, res, B, M, K, Nn, nullptr, nullptr,
+                                 as_stream(stream)));
+}
+
+int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, long lsm, long lsk,
+                           const float *rhs, long rsb, long rsk, long rsn, const float *res, int B,
+                           int M, int K, int Nn, float *grad_lhs, long glsb, long glsm, long glsk,
+                           float *grad_rhs, long grsb, long grsk, long grsn, void *stream) {
+    if (B < 0 || M < 0 || K < 0 || Nn < 0 || B > kMaxGrid || K > kMaxGrid * 64)
+        return WARPCTCT_EINVAL;
+    if (B == 0 || K == 0) return WARPCTCT_OK;
+    if (!lhs || !rhs || ((M > 0 && Nn > 0) && (!grad_out || !res))) return WARPCTCT_EINVAL;
+    const LogmmOperand l = {lhs, lsb, lsm, lsk};
+    const LogmmOperand r = {rhs, rsb, rsk, rsn};
+    if (grad_lhs) {
+        const LogmmGrad g = {grad_lhs, glsb, glsm, glsk};
+        int rc = done(launch_logmm_bwd_lhs(l, r, grad_out, res, g, B, M, K, Nn, nullptr, nullptr,
+                                           nullptr, as_stream(stream)));
+        if (rc != WARPCTCT_OK) return rc;
+    }
+    if (grad_rhs) {
+        const LogmmGrad g = {grad_rhs, grsb, grsk, grsn};
+        int rc = done(launch_logmm_bwd_rhs(l, r, grad_out, res, g, B, M, K, Nn, nullptr, nullptr,
+                                           nullptr, as_stream(stream)));
+        if (rc != WARPCTCT_OK) return rc;
+    }
+    return WARPCTCT_OK;
 }
 
 }  // extern "C"

@@ -149,6 +149,221 @@ torch::Tensor ctct_loss_joint_bwd(const torch::Tensor &unit_grads, const torch::
     return dense;
 }
 
+torch::Tensor make_bytes(const torch::Tensor &like, size_t bytes) {
+    return torch::empty({static_cast<int64_t>(bytes)}, like.options().dtype(at::ScalarType::Byte));
+}
+
+// Reference surface: _C.ctct_loss_simple_fwd (csrc/binding.cpp:103-222).
+// f (N,T,U+1) and g (N,U+1,3) are already gathered; den is (N,T,U+1), or any
+// tensor that is not 3-d to select the unnormalised variant (binding.cpp:144).
+// Returns (costs, grad_f, grad_g, grad_den); the gradients are undefined
+// (None in Python) when requires_grad is false, grad_den also when
+// unnormalised.
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> ctct_loss_simple_fwd(
+    const torch::Tensor &f, const torch::Tensor &g, const torch::Tensor &ys,
+    const torch::Tensor &den, const torch::Tensor &lx, const torch::Tensor &ly,
+    const bool requires_grad) {
+    CHECK_CONTIGUOUS(f);
+    CHECK_CONTIGUOUS(g);
+    CHECK_FLOAT(f);
+    CHECK_FLOAT(g);
+    CHECK_DEVICE(f);
+    CHECK_DEVICE(g);
+    TORCH_CHECK(f.dim() == 3, "f must have 3 dims.");
+    TORCH_CHECK(g.dim() == 3, "g must have 3 dims.");
+    TORCH_CHECK(f.size(2) == g.size(1),
+                "f should be gathered at last dim to length U matching the g at dim 1.");
+    TORCH_CHECK(g.size(2) == 3, "g should be first gathered to length 3 at last dim.");
+    const int N = f.size(0), T = f.size(1), U = g.size(1) - 1;
+    TORCH_CHECK(g.size(0) == N, "input args should match at dim 0 (batch N)");
+    check_lengths(ys, lx, ly, N, U);
+    const bool normalized = (den.dim() == 3);
+    if (normalized) {
+        CHECK_CONTIGUOUS(den);
+        CHECK_DEVICE(den);
+        CHECK_FLOAT(den);
+        TORCH_CHECK(den.size(0) == N && den.size(1) == T && den.size(2) == U + 1,
+                    "den must be (N,T,U+1)");
+    }
+    const DeviceGuard device_guard(device_of(f));
+    auto ws = make_bytes(f, warpctct_simple_workspace_bytes(N, T, U));
+    auto costs = torch::empty({N}, f.options());
+    torch::Tensor grad_f, grad_g, grad_den;
+    if (requires_grad) {
+        grad_f = torch::empty_like(f);
+        grad_g = torch::empty_like(g);
+        if (normalized) grad_den = torch::empty_like(den);
+    }
+    check_rc(warpctct_simple_forward_units_f32(
+                 f.data_ptr<float>(), g.data_ptr<float>(),
+                 normalized ? den.data_ptr<float>() : nullptr, ys.data_ptr<int>(),
+                 lx.data_ptr<int>(), ly.data_ptr<int>(), N, T, U, ws.data_ptr(), ws.numel(),
+                 costs.data_ptr<float>(), requires_grad ? grad_f.data_ptr<float>() : nullptr,
+                 requires_grad ? grad_g.data_ptr<float>() : nullptr,
+                 (requires_grad && normalized) ? grad_den.data_ptr<float>() : nullptr,
+                 current_stream()),
+             "ctct_loss_simple_fwd");
+    return std::make_tuple(costs, grad_f, grad_g, grad_den);
+}
+
+// Fused entry for ctct_simple_loss: un-gathered f (N,T,V), g (N,U+1,V).
+// Returns (costs, den, grad_f_g, grad_g_g, grad_den); den is defined when
+// normalized, the three compact gradients when requires_grad.
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor>
+ctct_simple_fwd(const torch::Tensor &f, const torch::Tensor &g, const torch::Tensor &ys,
+                const torch::Tensor &lx, const torch::Tensor &ly, const bool normalized,
+                const bool requires_grad) {
+    CHECK_CONTIGUOUS(f);
+    CHECK_CONTIGUOUS(g);
+    CHECK_FLOAT(f);
+    CHECK_FLOAT(g);
+    CHECK_DEVICE(f);
+    CHECK_DEVICE(g);
+    TORCH_CHECK(f.dim() == 3, "f must have 3 dims.");
+    TORCH_CHECK(g.dim() == 3, "g must have 3 dims.");
+    TORCH_CHECK(f.size(2) == g.size(2), "f and g must share the vocabulary dim");
+    const int N = f.size(0), T = f.size(1), U = g.size(1) - 1, V = f.size(2);
+    TORCH_CHECK(g.size(0) == N, "input args should match at dim 0 (batch N)");
+    check_lengths(ys, lx, ly, N, U);
+    const DeviceGuard device_guard(device_of(f));
+    auto ws = make_bytes(f, warpctct_simple_workspace_bytes(N, T, U));
+    auto costs = torch::empty({N}, f.options());
+    torch::Tensor den, grad_f, grad_g, grad_den;
+    if (normalized) den = torch::empty({N, T, U + 1}, f.options());
+    if (requires_grad) {
+        grad_f = torch::empty({N, T, U + 1}, f.options());
+        grad_g = torch::empty({N, U + 1, 3}, f.options());
+        if (normalized) grad_den = torch::empty({N, T, U + 1}, f.options());
+    }
+    check_rc(warpctct_simple_forward_f32(
+                 f.data_ptr<float>(), g.data_ptr<float>(), ys.data_ptr<int>(), lx.data_ptr<int>(),
+                 ly.data_ptr<int>(), N, T, U, V, normalized ? 1 : 0, ws.data_ptr(), ws.numel(),
+                 normalized ? den.data_ptr<float>() : nullptr, costs.data_ptr<float>(),
+                 requires_grad ? grad_f.data_ptr<float>() : nullptr,
+                 requires_grad ? grad_g.data_ptr<float>() : nullptr,
+                 (requires_grad && normalized) ? grad_den.data_ptr<float>() : nullptr,
+                 current_stream()),
+             "ctct_simple_fwd");
+    return std::make_tuple(costs, den, grad_f, grad_g, grad_den);
+}
+
+// Dense gradients (N,T,V) and (N,U+1,V) of the fused entry, scaled by
+// grad_out[n]; den / grad_den undefined selects the unnormalised variant.
+std::tuple<torch::Tensor, torch::Tensor> ctct_simple_bwd(
+    const torch::Tensor &f, const torch::Tensor &g, const c10::optional<torch::Tensor> &den,
+    const torch::Tensor &grad_f_g, const torch::Tensor &grad_g_g,
+    const c10::optional<torch::Tensor> &grad_den, const torch::Tensor &ys, const torch::Tensor &lx,
+    const torch::Tensor &ly, const torch::Tensor &grad_out, const bool want_f, const bool want_g) {
+    CHECK_CONTIGUOUS(f);
+    CHECK_CONTIGUOUS(g);
+    CHECK_FLOAT(f);
+    CHECK_FLOAT(g);
+    CHECK_DEVICE(f);
+    CHECK_DEVICE(g);
+    CHECK_CONTIGUOUS(grad_f_g);
+    CHECK_CONTIGUOUS(grad_g_g);
+    CHECK_FLOAT(grad_f_g);
+    CHECK_FLOAT(grad_g_g);
+    CHECK_CONTIGUOUS(grad_out);
+    CHECK_FLOAT(grad_out);
+    CHECK_DEVICE(grad_out);
+    TORCH_CHECK(f.dim() == 3 && g.dim() == 3 && f.size(2) == g.size(2), "f (N,T,V), g (N,U+1,V)");
+    const int N = f.size(0), T = f.size(1), U = g.size(1) - 1, V = f.size(2);
+    check_lengths(ys, lx, ly, N, U);
+    TORCH_CHECK(grad_out.dim() == 1 && grad_out.size(0) == N, "grad_out must be (N,)");
+    TORCH_CHECK(grad_f_g.dim() == 3 && grad_f_g.size(0) == N && grad_f_g.size(1) == T &&
+                    grad_f_g.size(2) == U + 1, "grad_f must be (N,T,U+1)");
+    TORCH_CHECK(grad_g_g.dim() == 3 && grad_g_g.size(0) == N && grad_g_g.size(1) == U + 1 &&
+                    grad_g_g.size(2) == 3, "grad_g must be (N,U+1,3)");
+    const bool normalized = den.has_value() && den->defined();
+    if (normalized) {
+        TORCH_CHECK(grad_den.has_value() && grad_den->defined(), "grad_den is required with den");
+        CHECK_CONTIGUOUS(*den);
+        CHECK_FLOAT(*den);
+        CHECK_DEVICE(*den);
+        CHECK_CONTIGUOUS(*grad_den);
+        CHECK_FLOAT(*grad_den);
+        TORCH_CHECK(den->numel() == (int64_t)N * T * (U + 1) && grad_den->numel() == den->numel(),
+                    "den and grad_den must be (N,T,U+1)");
+    }
+    const DeviceGuard device_guard(device_of(f));
+    torch::Tensor dense_f, dense_g;
+    if (want_f) dense_f = torch::empty_like(f);
+    if (want_g) dense_g = torch::empty_like(g);
+    check_rc(warpctct_simple_backward_f32(
+                 f.data_ptr<float>(), g.data_ptr<float>(),
+                 normalized ? den->data_ptr<float>() : nullptr, grad_f_g.data_ptr<float>(),
+                 grad_g_g.data_ptr<float>(), normalized ? grad_den->data_ptr<float>() : nullptr,
+                 ys.data_ptr<int>(), lx.data_ptr<int>(), ly.data_ptr<int>(),
+                 grad_out.data_ptr<float>(), N, T, U, V,
+                 want_f ? dense_f.data_ptr<float>() : nullptr,
+                 want_g ? dense_g.data_ptr<float>() : nullptr, current_stream()),
+             "ctct_simple_bwd");
+    return std::make_tuple(dense_f, dense_g);
+}
+
+long batch_stride(const torch::Tensor &t, int64_t B) {
+    return (t.size(0) == 1 && B > 1) ? 0L : static_cast<long>(t.stride(0));
+}
+
+// Reference surface: _C.log_matmul (csrc/binding.cpp:224-245).  Strided
+// operands are accepted as they are (the reference passes a transposed view).
+torch::Tensor log_matmul(const torch::Tensor &self, const torch::Tensor &other) {
+    CHECK_FLOAT(self);
+    CHECK_FLOAT(other);
+    TORCH_CHECK(self.is_cuda(), "need cuda tensors");
+    TORCH_CHECK(self.device() == other.device(), "need tensors on same GPU");
+    TORCH_CHECK(self.dim() == 3 && other.dim() == 3, "invalid sizes");
+    TORCH_CHECK(self.size(2) == other.size(1), "invalid sizes");
+    TORCH_CHECK(other.size(0) == self.size(0) || other.size(0) == 1, "invalid sizes");
+    const DeviceGuard device_guard(device_of(self));
+    const int B = self.size(0), M = self.size(1), K = self.size(2), Nn = other.size(2);
+    auto out = torch::empty({B, M, Nn}, self.options());
+    auto ws = make_bytes(self, warpctct_logmm_workspace_bytes(B, M, Nn));
+    check_rc(warpctct_logmm_fwd_f32(self.data_ptr<float>(), self.stride(0), self.stride(1),
+                                    self.stride(2), other.data_ptr<float>(),
+                                    batch_stride(other, B), other.stride(1), other.stride(2), B, M,
+                                    K, Nn, ws.data_ptr(), ws.numel(), out.data_ptr<float>(),
+                                    current_stream()),
+             "log_matmul");
+    return out;
+}
+
+// Reference surface: _C.log_matmul_backward (csrc/binding.cpp:247-324).
+std::tuple<torch::Tensor, torch::Tensor> log_matmul_backward(
+    const torch::Tensor &grad_out, const torch::Tensor &lhs, const torch::Tensor &rhs,
+    const torch::Tensor &result, const std::array<bool, 2> grad_input_mask) {
+    torch::Tensor grad_lhs, grad_rhs;
+    if (!grad_out.defined()) return std::make_tuple(grad_lhs, grad_rhs);
+    CHECK_FLOAT(grad_out);
+    CHECK_FLOAT(lhs);
+    CHECK_FLOAT(rhs);
+    CHECK_FLOAT(result);
+    TORCH_CHECK(lhs.is_cuda() && rhs.is_cuda() && result.is_cuda() && grad_out.is_cuda(),
+                "need cuda tensors");
+    TORCH_CHECK(lhs.dim() == 3 && rhs.dim() == 3 && result.dim() == 3 && grad_out.dim() == 3,
+                "invalid sizes");
+    const int B = lhs.size(0), M = lhs.size(1), K = lhs.size(2), Nn = rhs.size(2);
+    TORCH_CHECK(rhs.size(0) == B && rhs.size(1) == K, "invalid sizes (batch broadcast is not "
+                "supported in the backward)");
+    TORCH_CHECK(result.size(0) == B && result.size(1) == M && result.size(2) == Nn &&
+                    grad_out.sizes() == result.sizes(), "invalid sizes");
+    const DeviceGuard device_guard(device_of(lhs));
+    auto go = grad_out.contiguous();
+    auto res = result.contiguous();
+    if (grad_input_mask[0]) grad_lhs = torch::empty({B, M, K}, lhs.options());
+    if (grad_input_mask[1]) grad_rhs = torch::empty({B, K, Nn}, rhs.options());
+    check_rc(warpctct_logmm_bwd_f32(
+                 go.data_ptr<float>(), lhs.data_ptr<float>(), lhs.stride(0), lhs.stride(1),
+                 lhs.stride(2), rhs.data_ptr<float>(), rhs.stride(0), rhs.stride(1), rhs.stride(2),
+                 res.data_ptr<float>(), B, M, K, Nn,
+                 grad_input_mask[0] ? grad_lhs.data_ptr<float>() : nullptr, (long)M * K, (long)K, 1L,
+                 grad_input_mask[1] ? grad_rhs.data_ptr<float>() : nullptr, (long)K * Nn, (long)Nn,
+                 1L, current_stream()),
+             "log_matmul_backward");
+    return std::make_tuple(grad_lhs, grad_rhs);
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -163,5 +378,23 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           "Dense gradient wrt the joint from unit gradients.", pybind11::arg("unit_grads"),
           pybind11::arg("ys"), pybind11::arg("lx"), pybind11::arg("ly"),
           pybind11::arg("grad_out"), pybind11::arg("V"));
+    m.def("ctct_loss_simple_fwd", &ctct_loss_simple_fwd,
+          "CTC-Transducer loss with the log-add joiner on gathered operands (forward).",
+          pybind11::arg("f"), pybind11::arg("g"), pybind11::arg("ys"), pybind11::arg("den"),
+          pybind11::arg("lx"), pybind11::arg("ly"), pybind11::arg("requires_grad"));
+    m.def("ctct_simple_fwd", &ctct_simple_fwd,
+          "CTC-Transducer loss with the log-add joiner on un-gathered f, g (forward).",
+          pybind11::arg("f"), pybind11::arg("g"), pybind11::arg("ys"), pybind11::arg("lx"),
+          pybind11::arg("ly"), pybind11::arg("normalized"), pybind11::arg("requires_grad"));
+    m.def("ctct_simple_bwd", &ctct_simple_bwd, "Dense gradients wrt f and g.", pybind11::arg("f"),
+          pybind11::arg("g"), pybind11::arg("den"), pybind11::arg("grad_f"),
+          pybind11::arg("grad_g"), pybind11::arg("grad_den"), pybind11::arg("ys"),
+          pybind11::arg("lx"), pybind11::arg("ly"), pybind11::arg("grad_out"),
+          pybind11::arg("want_f"), pybind11::arg("want_g"));
+    m.def("log_matmul", &log_matmul, "Log matrix multiplication", pybind11::arg("lhs"),
+          pybind11::arg("rhs"));
+    m.def("log_matmul_backward", &log_matmul_backward, "Log matrix multiplication backward",
+          pybind11::arg("grad_out"), pybind11::arg("lhs"), pybind11::arg("rhs"),
+          pybind11::arg("res"), pybind11::arg("grad_masks"));
     m.def("library_version", []() { return std::string(warpctct_version()); });
 }

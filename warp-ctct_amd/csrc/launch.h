@@ -36,4 +36,42 @@ hipError_t launch_dense_grad(const float *unit_grads, const int *ys, const int *
                              const float *grad_out, float *dense, int N, int T, int U, int V,
                              hipStream_t stream);
 
+// ---- log-add joiner path -------------------------------------------------
+hipError_t launch_simple_gather_units(const float *f, const float *g, const float *den,
+                                      const int *ys, const int *lx, const int *ly, double *units,
+                                      int N, int T, int U, int V, hipStream_t stream);
+hipError_t launch_simple_reduce(const float *unit_grads, float *grad_f, float *grad_g,
+                                float *grad_den, int N, int T, int U, hipStream_t stream);
+hipError_t launch_simple_scatter(const float *grad_f, const float *grad_g, const int *ys,
+                                 const int *lx, const int *ly, const float *grad_out,
+                                 float *dense_f, float *dense_g, int N, int T, int U, int V,
+                                 hipStream_t stream);
+hipError_t launch_zero_fill(float *p, size_t n, hipStream_t stream);
+
+// ---- log-semiring matmul -------------------------------------------------
+// A strided 3-d operand: element [b, i1, i2] lives at p[b*sb + i1*s1 + i2*s2].
+// lhs is (B,M,K), rhs is (B,K,Nn); a gradient uses the layout of its operand.
+struct LogmmOperand {
+    const float *p;
+    long sb, s1, s2;
+};
+struct LogmmGrad {
+    float *p;
+    long sb, s1, s2;
+};
+
+// row_len / col_len (may be null): per-batch number of valid rows of lhs and
+// index of the last valid column of rhs; outputs outside are not computed.
+hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs, float *lmax,
+                            float *rmax, float *res, int B, int M, int K, int Nn,
+                            const int *row_len, const int *col_len, hipStream_t stream);
+hipError_t launch_logmm_bwd_lhs(const LogmmOperand &lhs, const LogmmOperand &rhs, const float *go,
+                                const float *res, const LogmmGrad &grad, int B, int M, int K,
+                                int Nn, const int *row_len, const int *col_len,
+                                const float *batch_scale, hipStream_t stream);
+hipError_t launch_logmm_bwd_rhs(const LogmmOperand &lhs, const LogmmOperand &rhs, const float *go,
+                                const float *res, const LogmmGrad &grad, int B, int M, int K,
+                                int Nn, const int *row_len, const int *col_len,
+                                const float *batch_scale, hipStream_t stream);
+
 }  // namespace wctct

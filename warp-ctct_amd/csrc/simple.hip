@@ -1,0 +1,217 @@
+// Kernels of the log-add joiner path (ctct_simple_loss): joint = f (+) g,
+// optionally normalised by den = logsumexp_v(f + g).
+//
+//  * units straight from f (N,T,V), g (N,U+1,V), den (N,T,U+1): the two
+//    torch.gather calls of warp_ctct/__init__.py:204-215 and the
+//    LOGPROBY/LOGPROBB macros of csrc/simple.cu:20-26 in one pass;
+//  * the reductions of the unit gradients that csrc/binding.cpp:198-219 does
+//    with ATen ops: grad_den = -sum_k, grad_g = sum_t, grad_f[...,0] = sum_u g0,
+//    grad_f[...,u>=1] = g1[u] + g2[u-1];
+//  * the backward of the two gathers: scatter-add of those compact gradients
+//    into the dense (N,T,V) and (N,U+1,V) tensors, scaled by grad_output[n]
+//    (SimpleCTCTLoss.backward, warp_ctct/__init__.py:76-85).
+#include "device_utils.h"
+#include "launch.h"
+
+namespace wctct {
+
+namespace {
+
+constexpr int kBlock = 256;
+
+__device__ __forceinline__ int clampi(int v, int lo, int hi) { return min(max(v, lo), hi); }
+
+// One thread per cell (t,u) of sample blockIdx.y.
+__global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
+    const float *__restrict__ f, const float *__restrict__ g, const float *__restrict__ den,
+    const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
+    double *__restrict__ units, int T, int U, int V) {
+    const int U1 = U + 1;
+    const int n = blockIdx.y;
+    const int cell = blockIdx.x * kBlock + threadIdx.x;
+    if (cell >= T * U1) return;
+    const int t = cell / U1, u = cell - t * U1;
+    const int Tn = clampi(lx[n], 0, T), Un = clampi(ly[n], 0, U);
+    if (t >= Tn || u > Un) return;
+    const float *fr = f + ((size_t)n * T + t) * V;
+    const float *gr = g + ((size_t)n * U1 + u) * V;
+    const int *y = ys + (size_t)n * U;
+    const double d = den ? (double)den[((size_t)n * T + t) * U1 + u] : 0.0;
+    const double b = (double)fr[0] + (double)gr[0] - d;
+    double cur = b, nxt = b;
+    if (u >= 1) {
+        const int c = clampi(y[u - 1], 0, V - 1);
+        cur = (double)fr[c] + (double)gr[c] - d;
+    }
+    if (u < Un) {
+        const int c = clampi(y[u], 0, V - 1);
+        nxt = (double)fr[c] + (double)gr[c] - d;
+    }
+    double *o = units + (((size_t)n * T + t) * U1 + u) * 3;
+    o[0] = b * kLog2e;
+    o[1] = cur * kLog2e;
+    o[2] = nxt * kLog2e;
+}
+
+// Per frame: grad_den[t,u] = -(g0+g1+g2), grad_f[t,u>=1] = g1[t,u] + g2[t,u-1],
+// grad_f[t,0] = sum_u g0[t,u].  One wavefront per (n,t); unit gradients are zero
+// in padding already.
+__global__ __launch_bounds__(kBlock) void simple_reduce_frames_kernel(
+    const float *__restrict__ ug, float *__restrict__ grad_f, float *__restrict__ grad_den, int T,
+    int U) {
+    const int U1 = U + 1;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int t = blockIdx.x * 4 + wave;
+    const int n = blockIdx.y;
+    if (t >= T) return;
+    const float *row = ug + ((size_t)n * T + t) * U1 * 3;
+    float *gf = grad_f + ((size_t)n * T + t) * U1;
+    float blank = 0.0f;
+    for (int u = lane; u < U1; u += 64) {
+        const float g0 = row[u * 3], g1 = row[u * 3 + 1], g2 = row[u * 3 + 2];
+        blank += g0;
+        if (grad_den) grad_den[((size_t)n * T + t) * U1 + u] = -(g0 + g1 + g2);
+        if (u >= 1) gf[u] = g1 + row[(u - 1) * 3 + 2];
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) blank += __shfl_xor(blank, off, 64);
+    if (lane == 0) gf[0] = blank;
+}
+
+// Per context: grad_g[u,k] = sum_t g_k[t,u].  One wavefront per (n,u).
+__global__ __launch_bounds__(kBlock) void simple_reduce_contexts_kernel(
+    const float *__restrict__ ug, float *__restrict__ grad_g, int T, int U) {
+    const int U1 = U + 1;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int u = blockIdx.x * 4 + wave;
+    const int n = blockIdx.y;
+    if (u >= U1) return;
+    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f;
+    for (int t = lane; t < T; t += 64) {
+        const float *p = ug + (((size_t)n * T + t) * U1 + u) * 3;
+        s0 += p[0];
+        s1 += p[1];
+        s2 += p[2];
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        s0 += __shfl_xor(s0, off, 64);
+        s1 += __shfl_xor(s1, off, 64);
+        s2 += __shfl_xor(s2, off, 64);
+    }
+    if (lane == 0) {
+        float *o = grad_g + ((size_t)n * U1 + u) * 3;
+        o[0] = s0;
+        o[1] = s1;
+        o[2] = s2;
+    }
+}
+
+// dense_f[n,t,idx(u)] += w[n] * grad_f[n,t,u],  idx = [0, y0 .. y_{U-1}]: the
+// backward of f.gather (warp_ctct/__init__.py:205-208).  The same label may
+// occur at several u, so the adds are atomic.  Padding holds zeros: skipped.
+__global__ __launch_bounds__(kBlock) void simple_scatter_f_kernel(
+    const float *__restrict__ grad_f, const int *__restrict__ ys, const int *__restrict__ lx,
+    const int *__restrict__ ly, const float *__restrict__ grad_out, float *__restrict__ dense_f,
+    int T, int U, int V) {
+    const int U1 = U + 1;
+    const int n = blockIdx.y;
+    const int cell = blockIdx.x * kBlock + threadIdx.x;
+    if (cell >= T * U1) return;
+    const int t = cell / U1, u = cell - t * U1;
+    const int Tn = clampi(lx[n], 0, T), Un = clampi(ly[n], 0, U);
+    if (t >= Tn || u > Un) return;
+    const float w = grad_out ? grad_out[n] : 1.0f;
+    const int col = (u == 0) ? 0 : clampi(ys[(size_t)n * U + u - 1], 0, V - 1);
+    atomicAdd(dense_f + ((size_t)n * T + t) * V + col, w * grad_f[((size_t)n * T + t) * U1 + u]);
+}
+
+// dense_g[n,u,{0,y[u-1],y[u]}] += w[n] * grad_g[n,u,k]: backward of g.gather
+// (warp_ctct/__init__.py:211-215).  One thread per (n,u,k).
+__global__ __launch_bounds__(kBlock) void simple_scatter_g_kernel(
+    const float *__restrict__ grad_g, const int *__restrict__ ys, const int *__restrict__ ly,
+    const float *__restrict__ grad_out, float *__restrict__ dense_g, int U, int V) {
+    const int U1 = U + 1;
+    const int n = blockIdx.y;
+    const int e = blockIdx.x * kBlock + threadIdx.x;
+    if (e >= U1 * 3) return;
+    const int u = e / 3, k = e - u * 3;
+    const int Un = clampi(ly[n], 0, U);
+    if (u > Un || (k == 1 && u == 0) || (k == 2 && u >= Un)) return;
+    const float w = grad_out ? grad_out[n] : 1.0f;
+    int col = 0;
+    if (k == 1) col = clampi(ys[(size_t)n * U + u - 1], 0, V - 1);
+    if (k == 2) col = clampi(ys[(size_t)n * U + u], 0, V - 1);
+    atomicAdd(dense_g + ((size_t)n * U1 + u) * V + col, w * grad_g[((size_t)n * U1 + u) * 3 + k]);
+}
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// n4 = number of leading 16-byte groups to store as vectors (0 if p is not
+// 16-byte aligned); the rest goes out as single floats.
+__global__ __launch_bounds__(kBlock) void zero_fill_kernel(float *__restrict__ p, size_t n,
+                                                           size_t n4) {
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    v4f *p4 = reinterpret_cast<v4f *>(p);
+    const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n4; i += stride) p4[i] = z;
+    for (size_t i = (n4 << 2) + (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride)
+        p[i] = 0.0f;
+}
+
+inline dim3 cell_grid(int N, int T, int U) {
+    const long cells = (long)T * (U + 1);
+    return dim3((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N);
+}
+
+}  // namespace
+
+hipError_t launch_simple_gather_units(const float *f, const float *g, const float *den,
+                                      const int *ys, const int *lx, const int *ly, double *units,
+                                      int N, int T, int U, int V, hipStream_t stream) {
+    hipLaunchKernelGGL(simple_gather_units_kernel, cell_grid(N, T, U), dim3(kBlock), 0, stream, f,
+                       g, den, ys, lx, ly, units, T, U, V);
+    return hipGetLastError();
+}
+
+hipError_t launch_simple_reduce(const float *unit_grads, float *grad_f, float *grad_g,
+                                float *grad_den, int N, int T, int U, hipStream_t stream) {
+    hipLaunchKernelGGL(simple_reduce_frames_kernel, dim3((T + 3) / 4, N), dim3(kBlock), 0, stream,
+                       unit_grads, grad_f, grad_den, T, U);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(simple_reduce_contexts_kernel, dim3((U + 1 + 3) / 4, N), dim3(kBlock), 0,
+                       stream, unit_grads, grad_g, T, U);
+    return hipGetLastError();
+}
+
+hipError_t launch_simple_scatter(const float *grad_f, const float *grad_g, const int *ys,
+                                 const int *lx, const int *ly, const float *grad_out,
+                                 float *dense_f, float *dense_g, int N, int T, int U, int V,
+                                 hipStream_t stream) {
+    if (dense_f) {
+        hipLaunchKernelGGL(simple_scatter_f_kernel, cell_grid(N, T, U), dim3(kBlock), 0, stream,
+                           grad_f, ys, lx, ly, grad_out, dense_f, T, U, V);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    if (dense_g) {
+        hipLaunchKernelGGL(simple_scatter_g_kernel, dim3(((U + 1) * 3 + kBlock - 1) / kBlock, N),
+                           dim3(kBlock), 0, stream, grad_g, ys, ly, grad_out, dense_g, U, V);
+        return hipGetLastError();
+    }
+    return hipSuccess;
+}
+
+hipError_t launch_zero_fill(float *p, size_t n, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    size_t blocks = (n / 4 + kBlock - 1) / kBlock;
+    if (blocks > 16384) blocks = 16384;
+    if (blocks == 0) blocks = 1;
+    const size_t n4 = (reinterpret_cast<uintptr_t>(p) & 15u) ? 0 : n / 4;
+    hipLaunchKernelGGL(zero_fill_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream, p, n,
+                       n4);
+    return hipGetLastError();
+}
+
+}  // namespace wctct

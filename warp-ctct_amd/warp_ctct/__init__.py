@@ -26,6 +26,25 @@ __all__ = ["ctct_loss", "ctct_simple_loss"]
 __version__ = core.library_version()
 
 
+# Optional observer for profiling: called as observer(kernel_name, fn) and must
+# return fn().  bench.py uses it to bracket single kernels with HIP events on
+# the stream they are launched on; it is None in normal use.
+_kernel_observer = None
+
+
+def set_kernel_observer(observer):
+    """Install (or clear, with None) a callable ``observer(name, fn)`` that
+    runs ``fn()`` and returns its result; used to time individual kernels."""
+    global _kernel_observer
+    _kernel_observer = observer
+
+
+def _run(name, fn):
+    if _kernel_observer is None:
+        return fn()
+    return _kernel_observer(name, fn)
+
+
 def _no_autocast():
     return torch.autocast(device_type="cuda", enabled=False)
 
@@ -44,7 +63,8 @@ class _CTCTLoss(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, joint, labels, lx, ly, requires_grad):
-        costs, unit_grads = core.ctct_loss_joint_fwd(joint, labels, lx, ly, requires_grad)
+        costs, unit_grads = _run("loss_forward", lambda: core.ctct_loss_joint_fwd(
+            joint, labels, lx, ly, requires_grad))
         if requires_grad:
             ctx.save_for_backward(unit_grads, labels, lx, ly)
             ctx.vocab = joint.size(3)
@@ -54,8 +74,38 @@ class _CTCTLoss(torch.autograd.Function):
     def backward(ctx, grad_outputs):
         unit_grads, labels, lx, ly = ctx.saved_tensors
         grad_outputs = grad_outputs.reshape(-1).float().contiguous()
-        dense = core.ctct_loss_joint_bwd(unit_grads, labels, lx, ly, grad_outputs, ctx.vocab)
+        dense = _run("dense_grad", lambda: core.ctct_loss_joint_bwd(
+            unit_grads, labels, lx, ly, grad_outputs, ctx.vocab))
         return dense, None, None, None, None
+
+
+class _SimpleCTCTLoss(torch.autograd.Function):
+    """ctct_simple_loss on the un-gathered f (N,T,V) and g (N,U+1,V).
+
+    Counterpart of the reference's LogMMExp (warp_ctct/__init__.py:36-52), the
+    two gathers (:204-215) and SimpleCTCTLoss (:55-85).  Forward computes den
+    (if normalized), the lattice and the compact gradients wrt the gathered f,
+    g and den; backward expands them to dense gradients wrt f and g, including
+    the path through den, scaled by grad_output[n]."""
+
+    @staticmethod
+    def forward(ctx, f, g, labels, lx, ly, normalized, track_f, track_g):
+        need_grad = track_f or track_g
+        costs, den, grad_f, grad_g, grad_den = _run("simple_forward", lambda: core.ctct_simple_fwd(
+            f, g, labels, lx, ly, normalized, need_grad))
+        if need_grad:
+            ctx.save_for_backward(f, g, den, grad_f, grad_g, grad_den, labels, lx, ly)
+            ctx.track = (track_f, track_g)
+        return costs
+
+    @staticmethod
+    def backward(ctx, grad_outputs):
+        f, g, den, grad_f, grad_g, grad_den, labels, lx, ly = ctx.saved_tensors
+        grad_outputs = grad_outputs.reshape(-1).float().contiguous()
+        dense_f, dense_g = _run("simple_backward", lambda: core.ctct_simple_bwd(
+            f, g, den, grad_f, grad_g, grad_den, labels, lx, ly, grad_outputs,
+            ctx.track[0], ctx.track[1]))
+        return dense_f, dense_g, None, None, None, None, None, None
 
 
 def _reduce(costs, frames_lengths, reduction, average_frames):
@@ -121,4 +171,17 @@ def ctct_simple_loss(f: torch.Tensor,
         normalized: subtract logsumexp_v(f + g) per (t, u) (a proper
             distribution); False scores paths with the raw sums.
     """
-    raise NotImplementedError("ctct_simple_loss: HIP path not built yet")
+    assert average_frames is None or isinstance(average_frames, bool)
+    assert reduction is None or reduction in ("none", "mean", "sum")
+    assert f.dim() == 3 and g.dim() == 3
+    assert labels.dim() == 2
+    assert g.size(1) == labels.size(1) + 1
+    assert f.size(0) == g.size(0) == labels.size(0) == frames_lengths.size(0) == labels_lengths.size(0)
+
+    track_f = f.requires_grad and torch.is_grad_enabled()
+    track_g = g.requires_grad and torch.is_grad_enabled()
+    with _no_autocast():
+        costs = _SimpleCTCTLoss.apply(f.float().contiguous(), g.float().contiguous(),
+                                      _as_int(labels), _as_int(frames_lengths),
+                                      _as_int(labels_lengths), bool(normalized), track_f, track_g)
+    return _reduce(costs, frames_lengths, reduction, average_frames)
