@@ -13,9 +13,11 @@
  * (csrc/gather.cu:16-21 of the reference).
  *
  * Internally the lattice works on log2 values held in double ("units",
- * alphas, betas below).  These intermediates are private to the library (the
- * reference's alphas/betas are private too); unit gradients and costs are
- * returned as fp32 in natural-log units exactly like the reference.
+ * alphas, betas below), in work buffers whose context dimension is padded to
+ * P = warpctct_padded_contexts(U), a multiple of the 64-lane wavefront.  These
+ * intermediates are private to the library (the reference's alphas/betas are
+ * private too); unit gradients and costs are returned as fp32 in natural-log
+ * units exactly like the reference.
  */
 #ifndef WARP_CTCT_HIP_H
 #define WARP_CTCT_HIP_H
@@ -41,6 +43,10 @@ const char *warpctct_error_string(int code);
 /* Library version, "major.minor.patch". */
 const char *warpctct_version(void);
 
+/* Contexts per frame in the work buffers: the smallest multiple of 64 that is
+ * >= U+1. */
+int warpctct_padded_contexts(int U);
+
 /* Bytes of device workspace the two *_forward orchestrators need
  * (units, alpha and beta lattices, all double).  Replaces the
  * allocations of csrc/binding.cpp:70-77 (alphas, betas, counts); needs no
@@ -52,8 +58,9 @@ size_t warpctct_workspace_bytes(int N, int T, int U);
 /* Gather of the three units per live cell out of the joint tensor, scaled
  * to log2 units.  Replaces warp_ctct/__init__.py:124-131 (index build +
  * torch.gather).  joint (N,T,U+1,V) f32, ys (N,U) i32, lx/ly (N) i32,
- * units_out (N,T,U+1,3) f64.  Cells with t>=lx[n] or u>ly[n] are not read
- * and not written. */
+ * units_out (N,T,P,3) f64.  Cells with t>=lx[n] or u>ly[n] are not read;
+ * for t<lx[n] the contexts u>ly[n] (up to P-1) receive the neutral units
+ * {0,0,-inf}; frames t>=lx[n] are not written. */
 int warpctct_gather_units_f32(const float *joint, const int *ys, const int *lx, const int *ly,
                               double *units_out, int N, int T, int U, int V, void *stream);
 
@@ -73,8 +80,8 @@ int warpctct_simple_units_f32(const float *f_g, const float *g_g, const float *d
 /* Alpha and beta lattices of all N samples, concurrently, one wavefront per
  * (sample, direction).  Replaces run_warp_ctct (csrc/core.h:14-16,
  * csrc/gather.cu:293-309: k_warp_alphas + k_warp_betas).
- * units (N,T,U+1,3) f64 log2 domain; alphas, betas (N,T+1,U+1,2) f64 =
- * {state 2u-1, state 2u} (only t<=lx[n], u<=ly[n] is written); costs (N) f32
+ * units (N,T,P,3) f64 log2 domain; alphas, betas (N,T+1,P,2) f64 =
+ * {state 2u-1, state 2u} (only t<=lx[n] is written); costs (N) f32
  * = -beta(0,0) in natural-log units (csrc/binding.cpp:86).
  * beta_only != 0 skips alpha (alphas may be NULL), as binding.cpp:84. */
 int warpctct_lattice_f32(const double *units, const int *ys, const int *lx, const int *ly,
@@ -89,14 +96,22 @@ int warpctct_unit_grads_f32(const double *units, const int *ys, const int *lx, c
                             const double *alphas, const double *betas, float *unit_grads, int N,
                             int T, int U, void *stream);
 
-/* Dense gradient wrt the joint: every element of dense (N,T,U+1,V) is written
- * exactly once — zero, or grad_out[n] * unit gradient at columns 0, y[u-1],
- * y[u] (coincident columns add).  Replaces CTCTLoss.backward
+/* Dense gradient wrt the joint: dense (N,T,U+1,V) = zeros, except
+ * grad_out[n] * unit gradient at columns 0, y[u-1], y[u] of every live row
+ * (coincident columns add).  Replaces CTCTLoss.backward
  * (warp_ctct/__init__.py:30-33) and autograd's gather backward (zeros +
- * scatter_add).  grad_out (N) f32 or NULL (= ones). */
+ * scatter_add).  grad_out (N) f32 or NULL (= ones).  Two launches: a pure
+ * zero-fill at full HBM write bandwidth, then the sparse patch. */
 int warpctct_dense_grad_f32(const float *unit_grads, const int *ys, const int *lx, const int *ly,
                             const float *grad_out, float *dense, int N, int T, int U, int V,
                             void *stream);
+
+/* The sparse half of warpctct_dense_grad_f32 alone: dense must already hold
+ * zeros (e.g. from warpctct_zero_fill_f32 run earlier on another stream, since
+ * the fill does not depend on the lattice). */
+int warpctct_dense_patch_f32(const float *unit_grads, const int *ys, const int *lx, const int *ly,
+                             const float *grad_out, float *dense, int N, int T, int U, int V,
+                             void *stream);
 
 /* ---- orchestrators ----------------------------------------------------- */
 
@@ -138,7 +153,8 @@ int warpctct_simple_scatter_f32(const float *grad_f, const float *grad_g, const 
                                 float *dense_f, float *dense_g, int N, int T, int U, int V,
                                 void *stream);
 
-/* p[0..n) = 0 with a kernel (safe to capture in a HIP graph). */
+/* p[0..n) = 0 with a kernel (one 16-byte store per thread; safe to capture in
+ * a HIP graph). */
 int warpctct_zero_fill_f32(float *p, size_t n, void *stream);
 
 /* Bytes of workspace for the two simple_forward orchestrators. */

@@ -26,7 +26,9 @@ def test_workspace_size_is_monotone_and_covers_buffers():
     lib = hip_lib.lib()
     N, T, U = 32, 250, 60
     need = lib.warpctct_workspace_bytes(N, T, U)
-    floor = 8 * N * T * (U + 1) * 3 + 2 * 8 * N * (T + 1) * (U + 1) * 2
+    P = lib.warpctct_padded_contexts(U)
+    assert P == 64 and lib.warpctct_padded_contexts(64) == 128 and lib.warpctct_padded_contexts(0) == 64
+    floor = 8 * N * T * P * 3 + 2 * 8 * N * (T + 1) * P * 2
     assert need >= floor and need < floor + 3 * 256
     assert lib.warpctct_workspace_bytes(N, T + 1, U) > need
     assert lib.warpctct_workspace_bytes(-1, T, U) == 0

@@ -48,9 +48,11 @@ def run_stages(joint, ys, lx, ly, beta_only=False):
     s = hip_lib.stream_ptr()
     d_joint, d_ys, d_lx, d_ly = dev(joint), dev(ys), dev(lx), dev(ly)
     f64 = dict(device="cuda", dtype=torch.float64)
-    units = torch.full((N, T, U1, 3), float("nan"), **f64)
-    alphas = torch.full((N, T + 1, U1, 2), float("nan"), **f64)
-    betas = torch.full((N, T + 1, U1, 2), float("nan"), **f64)
+    P = lib.warpctct_padded_contexts(U)           # contexts per frame in the work buffers
+    assert P % 64 == 0 and U1 <= P < U1 + 64
+    units = torch.full((N, T, P, 3), float("nan"), **f64)
+    alphas = torch.full((N, T + 1, P, 2), float("nan"), **f64)
+    betas = torch.full((N, T + 1, P, 2), float("nan"), **f64)
     costs = torch.full((N,), float("nan"), device="cuda")
     ug = torch.full((N, T, U1, 3), float("nan"), device="cuda")
     p = hip_lib.ptr
@@ -113,8 +115,12 @@ def test_stages_against_oracle(case):
         np.testing.assert_array_equal(g[..., 0], exp[..., 0])
         np.testing.assert_array_equal(g[:, 1:, 1], exp[:, 1:, 1])
         np.testing.assert_array_equal(g[:, :u, 2], exp[:, :u, 2])
-        # padding is never written
-        assert np.all(np.isnan(got["units"][n, t:])) and np.all(np.isnan(got["units"][n, :, u + 1:]))
+        # no label follows the last one; padding contexts are neutral; frames
+        # beyond lx are never written
+        assert np.all(np.isneginf(g[:, u, 2]))
+        pad = got["units"][n, :t, u + 1:]
+        assert np.all(pad[..., :2] == 0) and np.all(np.isneginf(pad[..., 2]))
+        assert np.all(np.isnan(got["units"][n, t:]))
     # lattices
     ref_a, ref_b = [], []
     for n in range(N):

@@ -19,21 +19,22 @@ inline int done(hipError_t e) { return e == hipSuccess ? WARPCTCT_OK : WARPCTCT_
 
 inline bool dims_ok(int N, int T, int U) {
     return N >= 0 && T >= 0 && U >= 0 && N <= kMaxGrid && T <= kMaxGrid &&
-           (U + 1) <= lattice_max_contexts() && (long)T * (U + 1) < (1L << 31);
+           (U + 1) <= lattice_max_contexts() && (long)T * padded_contexts(U) < (1L << 31);
 }
 
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct Workspace {
-    double *units;    // (N,T,U+1,3)
-    double *alphas;   // (N,T+1,U+1,2)
-    double *betas;    // (N,T+1,U+1,2)
+    double *units;    // (N,T,P,3),   P = padded_contexts(U)
+    double *alphas;   // (N,T+1,P,2)
+    double *betas;    // (N,T+1,P,2)
     size_t bytes;
 };
 
 Workspace carve(void *base, int N, int T, int U) {
-    const size_t units_b = align256((size_t)N * T * (U + 1) * 3 * sizeof(double));
-    const size_t lat_b = align256((size_t)N * (T + 1) * (U + 1) * 2 * sizeof(double));
+    const size_t P = (size_t)padded_contexts(U);
+    const size_t units_b = align256((size_t)N * T * P * 3 * sizeof(double));
+    const size_t lat_b = align256((size_t)N * (T + 1) * P * 2 * sizeof(double));
     const uintptr_t p = reinterpret_cast<uintptr_t>(base);
     Workspace w;
     w.units = reinterpret_cast<double *>(p);
@@ -114,6 +115,8 @@ const char *warpctct_error_string(int code) {
 
 const char *warpctct_version(void) { return "0.1.0"; }
 
+int warpctct_padded_contexts(int U) { return U < 0 ? 0 : padded_contexts(U); }
+
 size_t warpctct_workspace_bytes(int N, int T, int U) {
     if (N < 0 || T < 0 || U < 0) return 0;
     return carve(nullptr, N, T, U).bytes;
@@ -186,6 +189,16 @@ int warpctct_dense_grad_f32(const float *unit_grads, const int *ys, const int *l
     if (!unit_grads || !lx || !ly || !dense || (U > 0 && !ys)) return WARPCTCT_EINVAL;
     return done(launch_dense_grad(unit_grads, ys, lx, ly, grad_out, dense, N, T, U, V,
                                   as_stream(stream)));
+}
+
+int warpctct_dense_patch_f32(const float *unit_grads, const int *ys, const int *lx, const int *ly,
+                             const float *grad_out, float *dense, int N, int T, int U, int V,
+                             void *stream) {
+    if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
+    if (N == 0 || T == 0) return WARPCTCT_OK;
+    if (!unit_grads || !lx || !ly || !dense || (U > 0 && !ys)) return WARPCTCT_EINVAL;
+    return done(launch_dense_patch(unit_grads, ys, lx, ly, grad_out, dense, N, T, U, V,
+                                   as_stream(stream)));
 }
 
 int warpctct_loss_forward_f32(const float *joint, const int *ys, const int *lx, const int *ly,

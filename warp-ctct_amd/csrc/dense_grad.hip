@@ -3,14 +3,21 @@
 // The reference obtains it in two steps: CTCTLoss.backward scales the saved
 // unit gradients by grad_output (warp_ctct/__init__.py:30-33) and autograd's
 // gather backward zero-fills an (N,T,U+1,V) tensor and scatter-adds into it.
-// Here one streaming pass writes every element exactly once: a row (n,t,u) of
-// V floats is all zeros except columns 0, y[u-1], y[u], which receive
-// grad_out[n] * g0 / g1 / g2 (coincident columns add, as scatter_add does).
-// The pass is pure HBM write traffic (4*N*T*(U+1)*V bytes) and decides the
-// throughput of the whole loss: stores are 16 bytes per lane, 1 KiB contiguous
-// per wavefront instruction, non-temporal (the data is not read again by this
-// library), and a 256-column chunk that holds none of the three columns takes
-// a branch-free all-zero path.
+// The result is all zeros except, in row (n,t,u), columns 0, y[u-1], y[u],
+// which hold grad_out[n] * g0 / g1 / g2 (coincident columns add).
+//
+// The zero-fill is pure HBM write traffic (4*N*T*(U+1)*V bytes) and decides
+// the throughput of the whole loss, so it is kept free of everything else:
+//  * zero_fill_vec_kernel: a 256-thread workgroup issues ONE 16-byte store
+//    per thread (4 KiB contiguous per workgroup) and retires.  On MI355X this
+//    finest-grained launch gives the highest write bandwidth (~6.8 TB/s);
+//    workgroups that loop over 16-64 KiB or use non-temporal stores lose
+//    10-20 %, and a workgroup that first has to fetch per-row data (labels,
+//    unit gradients) before it can store loses 25-35 %.  The fill does not
+//    depend on the lattice, so a caller may run it on another stream while
+//    the lattice is computed.
+//  * patch_kernel: one thread per live cell (t,u) overwrites the <= 3
+//    non-zero entries of its row.
 #include "device_utils.h"
 #include "launch.h"
 
@@ -20,90 +27,103 @@ namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kRowsPerBlock = 16;
-constexpr int kWavesPerBlock = 4;
+constexpr int kBlock = 256;
 
-template <bool VEC4>
-__global__ __launch_bounds__(kWavesPerBlock * 64) void dense_grad_kernel(
+// p4[i] = 0 for i < n4: one store per thread, no loop.
+__global__ __launch_bounds__(kBlock) void zero_fill_vec_kernel(v4f *__restrict__ p4, size_t n4) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (i < n4) p4[i] = z;
+}
+
+__global__ __launch_bounds__(kBlock) void zero_fill_scalar_kernel(float *__restrict__ p,
+                                                                  size_t n) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) p[i] = 0.0f;
+}
+
+// One thread per cell (t,u) of sample blockIdx.y.  Writes (not adds) the
+// non-zero entries of row (n,t,u); columns that coincide are summed first so
+// that every element is written by exactly one store.
+__global__ __launch_bounds__(kBlock) void patch_kernel(
     const float *__restrict__ unit_grads, const int *__restrict__ ys,
     const int *__restrict__ lx, const int *__restrict__ ly, const float *__restrict__ grad_out,
     float *__restrict__ dense, int T, int U, int V) {
-    const int n = blockIdx.z;
-    const int t = blockIdx.y;
     const int U1 = U + 1;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int lane = threadIdx.x & 63;
+    const int n = blockIdx.y;
+    const int cell = blockIdx.x * kBlock + threadIdx.x;
+    if (cell >= T * U1) return;
+    const int t = cell / U1, u = cell - t * U1;
     const int Tn = min(max(lx[n], 0), T);
     const int Un = min(max(ly[n], 0), U);
+    if (t >= Tn || u > Un) return;
+    const size_t row = ((size_t)n * T + t) * U1 + u;
+    const float *g = unit_grads + row * 3;
     const float w = grad_out ? grad_out[n] : 1.0f;
     const int *y = ys + (size_t)n * U;
-
-    for (int r = wave; r < kRowsPerBlock; r += kWavesPerBlock) {
-        const int u = blockIdx.x * kRowsPerBlock + r;
-        if (u > U) break;
-        const size_t row = ((size_t)n * T + t) * U1 + u;
-        float *out = dense + row * (size_t)V;
-        const bool live = (t < Tn) && (u <= Un);
-        float g0 = 0.0f, g1 = 0.0f, g2 = 0.0f;
-        int c1 = 0, c2 = 0;
-        if (live) {
-            const float *g = unit_grads + row * 3;
-            g0 = g[0] * w;
-            if (u >= 1) {
-                g1 = g[1] * w;
-                c1 = min(max(y[u - 1], 0), V - 1);
-            }
-            if (u < Un) {
-                g2 = g[2] * w;
-                c2 = min(max(y[u], 0), V - 1);
-            }
-        }
-        if (VEC4) {
-            v4f *out4 = reinterpret_cast<v4f *>(out);
-            const int nvec = V >> 2;
-            for (int base = 0; base < nvec; base += 64) {
-                const int fi = base + lane;
-                // does this 256-column chunk hold any of the three columns?
-                const int chunk = base >> 6;
-                const bool hit = live && (chunk == 0 || (c1 >> 8) == chunk || (c2 >> 8) == chunk);
-                v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
-                if (hit) {
-                    const int col = fi << 2;
-                    const int d1 = c1 - col;
-                    const int d2 = c2 - col;
-                    v.x = (col == 0 ? g0 : 0.0f) + (d1 == 0 ? g1 : 0.0f) + (d2 == 0 ? g2 : 0.0f);
-                    v.y = (d1 == 1 ? g1 : 0.0f) + (d2 == 1 ? g2 : 0.0f);
-                    v.z = (d1 == 2 ? g1 : 0.0f) + (d2 == 2 ? g2 : 0.0f);
-                    v.w = (d1 == 3 ? g1 : 0.0f) + (d2 == 3 ? g2 : 0.0f);
-                }
-                if (fi < nvec) __builtin_nontemporal_store(v, out4 + fi);
-            }
-        } else {
-            for (int col = lane; col < V; col += 64) {
-                float v = 0.0f;
-                if (live)
-                    v = (col == 0 ? g0 : 0.0f) + (col == c1 ? g1 : 0.0f) + (col == c2 ? g2 : 0.0f);
-                out[col] = v;
-            }
-        }
+    const bool has1 = (u >= 1), has2 = (u < Un);
+    const int c1 = has1 ? min(max(y[u - 1], 0), V - 1) : -1;
+    const int c2 = has2 ? min(max(y[u], 0), V - 1) : -2;
+    float v0 = g[0] * w;
+    float v1 = has1 ? g[1] * w : 0.0f;
+    float v2 = has2 ? g[2] * w : 0.0f;
+    if (c2 == c1) {   // y[u-1] == y[u]: both label units land in one column
+        v1 += v2;
+        v2 = 0.0f;
     }
+    if (c1 == 0) v0 += v1;   // a label equal to the blank index
+    if (c2 == 0) v0 += v2;
+    float *out = dense + row * (size_t)V;
+    out[0] = v0;
+    if (c1 > 0) out[c1] = v1;
+    if (c2 > 0 && c2 != c1) out[c2] = v2;
 }
 
 }  // namespace
 
+hipError_t launch_zero_fill(float *p, size_t n, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    // leading floats up to the first 16-byte boundary, then vectors, then the tail
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(p);
+    size_t head = ((16 - (addr & 15u)) & 15u) / sizeof(float);
+    if ((addr & 3u) != 0) head = n;   // not even float-aligned: all scalar
+    if (head > n) head = n;
+    const size_t n4 = (n - head) / 4;
+    const size_t tail = n - head - n4 * 4;
+    if (head) {
+        hipLaunchKernelGGL(zero_fill_scalar_kernel, dim3((unsigned)((head + kBlock - 1) / kBlock)),
+                           dim3(kBlock), 0, stream, p, head);
+    }
+    if (n4) {
+        const size_t blocks = (n4 + kBlock - 1) / kBlock;
+        if (blocks > 0x7fffffffUL) return hipErrorInvalidValue;
+        hipLaunchKernelGGL(zero_fill_vec_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream,
+                           reinterpret_cast<v4f *>(p + head), n4);
+    }
+    if (tail) {
+        hipLaunchKernelGGL(zero_fill_scalar_kernel, dim3(1), dim3(kBlock), 0, stream,
+                           p + head + n4 * 4, tail);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_dense_patch(const float *unit_grads, const int *ys, const int *lx,
+                              const int *ly, const float *grad_out, float *dense, int N, int T,
+                              int U, int V, hipStream_t stream) {
+    const long cells = (long)T * (U + 1);
+    if (cells == 0 || N == 0) return hipSuccess;
+    dim3 grid((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N);
+    hipLaunchKernelGGL(patch_kernel, grid, dim3(kBlock), 0, stream, unit_grads, ys, lx, ly,
+                       grad_out, dense, T, U, V);
+    return hipGetLastError();
+}
+
 hipError_t launch_dense_grad(const float *unit_grads, const int *ys, const int *lx, const int *ly,
                              const float *grad_out, float *dense, int N, int T, int U, int V,
                              hipStream_t stream) {
-    dim3 grid((unsigned)((U + 1 + kRowsPerBlock - 1) / kRowsPerBlock), (unsigned)T, (unsigned)N);
-    dim3 block(kWavesPerBlock * 64);
-    const bool vec4 = (V % 4 == 0) && ((reinterpret_cast<uintptr_t>(dense) & 15u) == 0);
-    if (vec4)
-        hipLaunchKernelGGL(dense_grad_kernel<true>, grid, block, 0, stream, unit_grads, ys, lx, ly,
-                           grad_out, dense, T, U, V);
-    else
-        hipLaunchKernelGGL(dense_grad_kernel<false>, grid, block, 0, stream, unit_grads, ys, lx,
-                           ly, grad_out, dense, T, U, V);
-    return hipGetLastError();
+    hipError_t e = launch_zero_fill(dense, (size_t)N * T * (U + 1) * V, stream);
+    if (e != hipSuccess) return e;
+    return launch_dense_patch(unit_grads, ys, lx, ly, grad_out, dense, N, T, U, V, stream);
 }
 
 }  // namespace wctct

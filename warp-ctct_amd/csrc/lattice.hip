@@ -26,14 +26,18 @@ struct Front {
     double o[K];
 };
 
+// Work buffers are padded to P = 64*K contexts per frame so that every lane
+// loads and stores unconditionally: no exec-mask branches in the sweep, which
+// lets the compiler count outstanding loads exactly and keep the prefetch of
+// the next chunk in flight while the current one is consumed.
+//   units  (N, T,   P, 3)  {blank, cur, next}; for u > Un: {0, 0, -inf},
+//                          and next = -inf at u = Un (no label follows)
+//   alpha, beta (N, T+1, P, 2) pairs {o, e}
 template <int K>
-__device__ __forceinline__ void front_store(double *dst, const Front<K> &f, int u0, int Un) {
-    // dst points at [t][u0][0]; pairs {o, e}
+__device__ __forceinline__ void front_store(double *dst, const Front<K> &f) {
 #pragma unroll
-    for (int j = 0; j < K; ++j) {
-        if (u0 + j <= Un)
-            *reinterpret_cast<double2 *>(dst + 2 * j) = make_double2(f.o[j], f.e[j]);
-    }
+    for (int j = 0; j < K; ++j)
+        *reinterpret_cast<double2 *>(dst + 2 * j) = make_double2(f.o[j], f.e[j]);
 }
 
 template <int K, int R>
@@ -41,30 +45,21 @@ struct Chunk {
     double lp[R][K][3];
 };
 
-// Load the units of frames t_first + dir*r, r in [0,R), for this lane's
-// contexts.  Frames outside [0,Tn) and contexts beyond Un are not touched in
-// memory; their units read as 0, and the "next label" unit of context Un (and
-// beyond) reads as -inf so that no mass flows past the last label.
+// Units of frames t_first + dir*r, r in [0,R); the frame index is clamped into
+// [0, Tn-1] so that a prefetch past the end re-reads a valid row (its values
+// are then not used).
 template <int K, int R>
-__device__ __forceinline__ void chunk_load(Chunk<K, R> &c, const double *units_n, int U1, int u0,
-                                           int Un, int Tn, int t_first, int dir) {
+__device__ __forceinline__ void chunk_load(Chunk<K, R> &c, const double *units_lane, size_t row,
+                                           int Tn, int t_first, int dir) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int t = t_first + dir * r;
-        const bool t_ok = (t >= 0) && (t < Tn);
+        const int t = min(max(t_first + dir * r, 0), Tn - 1);
+        const double *p = units_lane + (size_t)t * row;
 #pragma unroll
         for (int j = 0; j < K; ++j) {
-            const int u = u0 + j;
-            double b = 0.0, cur = 0.0, nxt = 0.0;
-            if (t_ok && u <= Un) {
-                const double *p = units_n + ((size_t)t * U1 + u) * 3;
-                b = p[0];
-                cur = p[1];
-                nxt = p[2];
-            }
-            c.lp[r][j][0] = b;
-            c.lp[r][j][1] = cur;
-            c.lp[r][j][2] = (u < Un) ? nxt : neg_inf();
+            c.lp[r][j][0] = p[3 * j];
+            c.lp[r][j][1] = p[3 * j + 1];
+            c.lp[r][j][2] = p[3 * j + 2];
         }
     }
 }
@@ -74,8 +69,10 @@ __device__ __forceinline__ void chunk_load(Chunk<K, R> &c, const double *units_n
 // alpha(t+1, 2u-1) =  alpha(t,2u-1) + LP(t,u,1)
 //                 (+) alpha(t,2u-2) + LP(t,u-1,2)
 //                 (+) [y[u-1] != y[u-2]] alpha(t,2u-3) + LP(t,u-1,2)
+// skip_mask[j] is 0 where the third arc exists and -inf where it does not.
 template <int K>
-__device__ __forceinline__ void alpha_step(Front<K> &f, const double (*lp)[3], const bool *skip) {
+__device__ __forceinline__ void alpha_step(Front<K> &f, const double (*lp)[3],
+                                           const double *skip_mask) {
     double from_e[K], from_o[K];
 #pragma unroll
     for (int j = 0; j < K; ++j) {
@@ -89,22 +86,23 @@ __device__ __forceinline__ void alpha_step(Front<K> &f, const double (*lp)[3], c
         const double pe = (j == 0) ? in_e : from_e[j - 1];
         const double po = (j == 0) ? in_o : from_o[j - 1];
         const double ne = lse2(f.e[j], f.o[j]) + lp[j][0];
-        const double no = lse3(f.o[j] + lp[j][1], pe, skip[j] ? po : neg_inf());
+        const double no = lse3(f.o[j] + lp[j][1], pe, po + skip_mask[j]);
         f.e[j] = ne;
         f.o[j] = no;
     }
 }
 
 template <int K, int R>
-__device__ void alpha_sweep(const double *units_n, const int *y, int Tn, int Un, int U1,
+__device__ void alpha_sweep(const double *units_n, const int *y, int Tn, int Un, int P,
                             double *alpha_n) {
     const int lane = threadIdx.x;
     const int u0 = lane * K;
-    bool skip[K];
+    double skip_mask[K];
 #pragma unroll
     for (int j = 0; j < K; ++j) {
         const int u = u0 + j;
-        skip[j] = (u >= 2) && (u <= Un) && (y[u - 1] != y[u - 2]);
+        const bool skip = (u >= 2) && (u <= Un) && (y[u - 1] != y[u - 2]);
+        skip_mask[j] = skip ? 0.0 : neg_inf();
     }
     Front<K> f;
 #pragma unroll
@@ -113,30 +111,45 @@ __device__ void alpha_sweep(const double *units_n, const int *y, int Tn, int Un,
         f.o[j] = neg_inf();
     }
     if (lane == 0) f.e[0] = 0.0;
-    const size_t row = (size_t)U1 * 2;
+    const size_t srow = (size_t)P * 2;       // doubles per frame of alpha
+    const size_t urow = (size_t)P * 3;       // doubles per frame of units
     double *out = alpha_n + (size_t)u0 * 2;
-    front_store<K>(out, f, u0, Un);
+    const double *in = units_n + (size_t)u0 * 3;
+    front_store<K>(out, f);
+    if (Tn == 0) return;
 
     Chunk<K, R> a, b;
-    chunk_load<K, R>(a, units_n, U1, u0, Un, Tn, 0, 1);
-    for (int t0 = 0; t0 < Tn; t0 += 2 * R) {
-        chunk_load<K, R>(b, units_n, U1, u0, Un, Tn, t0 + R, 1);
+    int t0 = 0;
+    chunk_load<K, R>(a, in, urow, Tn, 0, 1);
+    while (t0 + 2 * R <= Tn) {
+        chunk_load<K, R>(b, in, urow, Tn, t0 + R, 1);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int t = t0 + r;
-            if (t < Tn) {
-                alpha_step<K>(f, a.lp[r], skip);
-                front_store<K>(out + (size_t)(t + 1) * row, f, u0, Un);
-            }
+            alpha_step<K>(f, a.lp[r], skip_mask);
+            front_store<K>(out + (size_t)(t0 + r + 1) * srow, f);
         }
-        chunk_load<K, R>(a, units_n, U1, u0, Un, Tn, t0 + 2 * R, 1);
+        chunk_load<K, R>(a, in, urow, Tn, t0 + 2 * R, 1);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int t = t0 + R + r;
-            if (t < Tn) {
-                alpha_step<K>(f, b.lp[r], skip);
-                front_store<K>(out + (size_t)(t + 1) * row, f, u0, Un);
-            }
+            alpha_step<K>(f, b.lp[r], skip_mask);
+            front_store<K>(out + (size_t)(t0 + R + r + 1) * srow, f);
+        }
+        t0 += 2 * R;
+    }
+    // fewer than 2R frames left
+    chunk_load<K, R>(b, in, urow, Tn, t0 + R, 1);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (t0 + r < Tn) {
+            alpha_step<K>(f, a.lp[r], skip_mask);
+            front_store<K>(out + (size_t)(t0 + r + 1) * srow, f);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (t0 + R + r < Tn) {
+            alpha_step<K>(f, b.lp[r], skip_mask);
+            front_store<K>(out + (size_t)(t0 + R + r + 1) * srow, f);
         }
     }
 }
@@ -145,9 +158,10 @@ __device__ void alpha_sweep(const double *units_n, const int *y, int Tn, int Un,
 // beta(t, 2u)   = beta(t+1,2u) + LP(t,u,0)  (+) [u<U] beta(t+1,2u+1) + LP(t,u,2)
 // beta(t, 2u-1) = beta(t+1,2u-1) + LP(t,u,1) (+) beta(t+1,2u) + LP(t,u,0)
 //              (+) [u<U, y[u-1] != y[u]] beta(t+1,2u+1) + LP(t,u,2)
+// o_mask[j] is 0 for contexts that have a state 2u-1 (1 <= u <= Un), else -inf.
 template <int K>
-__device__ __forceinline__ void beta_step(Front<K> &f, const double (*lp)[3], const bool *skip,
-                                          const bool *has_o) {
+__device__ __forceinline__ void beta_step(Front<K> &f, const double (*lp)[3],
+                                          const double *skip_mask, const double *o_mask) {
     const double in_o = wave_shift_down(f.o[0], neg_inf());
 #pragma unroll
     for (int j = 0; j < K; ++j) {
@@ -155,23 +169,24 @@ __device__ __forceinline__ void beta_step(Front<K> &f, const double (*lp)[3], co
         const double nxt = nb + lp[j][2];
         const double stay_e = f.e[j] + lp[j][0];
         const double ne = lse2(stay_e, nxt);
-        const double no = lse3(f.o[j] + lp[j][1], stay_e, skip[j] ? nxt : neg_inf());
+        const double no = lse3(f.o[j] + lp[j][1], stay_e, nxt + skip_mask[j]);
         f.e[j] = ne;
-        f.o[j] = has_o[j] ? no : neg_inf();
+        f.o[j] = no + o_mask[j];
     }
 }
 
 template <int K, int R>
-__device__ void beta_sweep(const double *units_n, const int *y, int Tn, int Un, int U1,
+__device__ void beta_sweep(const double *units_n, const int *y, int Tn, int Un, int P,
                            double *beta_n, float *cost_n) {
     const int lane = threadIdx.x;
     const int u0 = lane * K;
-    bool skip[K], has_o[K];
+    double skip_mask[K], o_mask[K];
 #pragma unroll
     for (int j = 0; j < K; ++j) {
         const int u = u0 + j;
-        has_o[j] = (u >= 1) && (u <= Un);
-        skip[j] = (u >= 1) && (u < Un) && (y[u - 1] != y[u]);
+        const bool skip = (u >= 1) && (u < Un) && (y[u - 1] != y[u]);
+        skip_mask[j] = skip ? 0.0 : neg_inf();
+        o_mask[j] = ((u >= 1) && (u <= Un)) ? 0.0 : neg_inf();
     }
     Front<K> f;
 #pragma unroll
@@ -180,29 +195,45 @@ __device__ void beta_sweep(const double *units_n, const int *y, int Tn, int Un, 
         f.e[j] = (u == Un) ? 0.0 : neg_inf();
         f.o[j] = (u == Un && Un >= 1) ? 0.0 : neg_inf();
     }
-    const size_t row = (size_t)U1 * 2;
+    const size_t srow = (size_t)P * 2;
+    const size_t urow = (size_t)P * 3;
     double *out = beta_n + (size_t)u0 * 2;
-    front_store<K>(out + (size_t)Tn * row, f, u0, Un);
+    const double *in = units_n + (size_t)u0 * 3;
+    front_store<K>(out + (size_t)Tn * srow, f);
 
-    Chunk<K, R> a, b;
-    chunk_load<K, R>(a, units_n, U1, u0, Un, Tn, Tn - 1, -1);
-    for (int s0 = 0; s0 < Tn; s0 += 2 * R) {
-        chunk_load<K, R>(b, units_n, U1, u0, Un, Tn, Tn - 1 - (s0 + R), -1);
+    if (Tn > 0) {
+        Chunk<K, R> a, b;
+        int t1 = Tn - 1;                      // frame consumed by the next step
+        chunk_load<K, R>(a, in, urow, Tn, t1, -1);
+        while (t1 - 2 * R + 1 >= 0) {
+            chunk_load<K, R>(b, in, urow, Tn, t1 - R, -1);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                beta_step<K>(f, a.lp[r], skip_mask, o_mask);
+                front_store<K>(out + (size_t)(t1 - r) * srow, f);
+            }
+            chunk_load<K, R>(a, in, urow, Tn, t1 - 2 * R, -1);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                beta_step<K>(f, b.lp[r], skip_mask, o_mask);
+                front_store<K>(out + (size_t)(t1 - R - r) * srow, f);
+            }
+            t1 -= 2 * R;
+        }
+        // fewer than 2R frames left: t1, t1-1, .., 0
+        chunk_load<K, R>(b, in, urow, Tn, t1 - R, -1);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int t = Tn - 1 - (s0 + r);
-            if (t >= 0) {
-                beta_step<K>(f, a.lp[r], skip, has_o);
-                front_store<K>(out + (size_t)t * row, f, u0, Un);
+            if (t1 - r >= 0) {
+                beta_step<K>(f, a.lp[r], skip_mask, o_mask);
+                front_store<K>(out + (size_t)(t1 - r) * srow, f);
             }
         }
-        chunk_load<K, R>(a, units_n, U1, u0, Un, Tn, Tn - 1 - (s0 + 2 * R), -1);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int t = Tn - 1 - (s0 + R + r);
-            if (t >= 0) {
-                beta_step<K>(f, b.lp[r], skip, has_o);
-                front_store<K>(out + (size_t)t * row, f, u0, Un);
+            if (t1 - R - r >= 0) {
+                beta_step<K>(f, b.lp[r], skip_mask, o_mask);
+                front_store<K>(out + (size_t)(t1 - R - r) * srow, f);
             }
         }
     }
@@ -221,18 +252,18 @@ __global__ __launch_bounds__(64) void lattice_kernel(const double *__restrict__ 
                                                      double *__restrict__ betas,
                                                      float *__restrict__ costs, int T, int U) {
     const int n = blockIdx.x;
-    const int U1 = U + 1;
+    constexpr int P = 64 * K;
     // lengths outside the allocation are clamped: nothing is ever read or
     // written beyond (T, U), whatever the length tensors hold
     const int Tn = min(max(lx[n], 0), T);
     const int Un = min(max(ly[n], 0), U);
-    const double *units_n = units + (size_t)n * T * U1 * 3;
+    const double *units_n = units + (size_t)n * T * P * 3;
     const int *y = ys + (size_t)n * U;
-    const size_t lat = (size_t)(T + 1) * U1 * 2;
+    const size_t lat = (size_t)(T + 1) * P * 2;
     if (blockIdx.y == 0)
-        beta_sweep<K, R>(units_n, y, Tn, Un, U1, betas + (size_t)n * lat, costs + n);
+        beta_sweep<K, R>(units_n, y, Tn, Un, P, betas + (size_t)n * lat, costs + n);
     else
-        alpha_sweep<K, R>(units_n, y, Tn, Un, U1, alphas + (size_t)n * lat);
+        alpha_sweep<K, R>(units_n, y, Tn, Un, P, alphas + (size_t)n * lat);
 }
 
 template <int K, int R>

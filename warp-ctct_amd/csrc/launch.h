@@ -7,13 +7,18 @@
 
 namespace wctct {
 
+// Work buffers (units, alphas, betas) hold P = padded_contexts(U) contexts per
+// frame, a multiple of the wavefront size, so that the lattice sweep loads and
+// stores without lane masks.
+inline int padded_contexts(int U) { return ((U + 1 + 63) / 64) * 64; }
+
 struct LatticeArgs {
-    const double *units;  // (N,T,U+1,3) log2 units
+    const double *units;  // (N,T,P,3) log2 units, neutral values in the padding
     const int *ys;        // (N,U)
     const int *lx;        // (N)
     const int *ly;        // (N)
-    double *alphas;       // (N,T+1,U+1,2) log2 units, or null if beta_only
-    double *betas;        // (N,T+1,U+1,2) log2 units
+    double *alphas;       // (N,T+1,P,2) log2 units, or null if beta_only
+    double *betas;        // (N,T+1,P,2) log2 units
     float *costs;         // (N)
     int N, T, U;
     bool beta_only;
@@ -32,9 +37,14 @@ hipError_t launch_simple_units(const float *f_g, const float *g_g, const float *
 hipError_t launch_unit_grads(const double *units, const int *ys, const int *lx, const int *ly,
                              const double *alphas, const double *betas, float *unit_grads, int N,
                              int T, int U, hipStream_t stream);
+// dense = zeros, then the patch (two launches on the same stream)
 hipError_t launch_dense_grad(const float *unit_grads, const int *ys, const int *lx, const int *ly,
                              const float *grad_out, float *dense, int N, int T, int U, int V,
                              hipStream_t stream);
+// only the <= 3 non-zero entries per live row, into a tensor that holds zeros
+hipError_t launch_dense_patch(const float *unit_grads, const int *ys, const int *lx,
+                              const int *ly, const float *grad_out, float *dense, int N, int T,
+                              int U, int V, hipStream_t stream);
 
 // ---- log-add joiner path -------------------------------------------------
 hipError_t launch_simple_gather_units(const float *f, const float *g, const float *den,

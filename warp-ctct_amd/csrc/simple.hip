@@ -25,32 +25,38 @@ __device__ __forceinline__ int clampi(int v, int lo, int hi) { return min(max(v,
 __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     const float *__restrict__ f, const float *__restrict__ g, const float *__restrict__ den,
     const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
-    double *__restrict__ units, int T, int U, int V) {
+    double *__restrict__ units, int T, int U, int V, int P) {
     const int U1 = U + 1;
     const int n = blockIdx.y;
     const int cell = blockIdx.x * kBlock + threadIdx.x;
-    if (cell >= T * U1) return;
-    const int t = cell / U1, u = cell - t * U1;
+    if (cell >= T * P) return;
+    const int t = cell / P, u = cell - t * P;
     const int Tn = clampi(lx[n], 0, T), Un = clampi(ly[n], 0, U);
-    if (t >= Tn || u > Un) return;
+    if (t >= Tn) return;
+    double *o = units + (((size_t)n * T + t) * P + u) * 3;
+    if (u > Un) {   // padding context of a live frame: neutral units
+        o[0] = 0.0;
+        o[1] = 0.0;
+        o[2] = neg_inf();
+        return;
+    }
     const float *fr = f + ((size_t)n * T + t) * V;
     const float *gr = g + ((size_t)n * U1 + u) * V;
     const int *y = ys + (size_t)n * U;
     const double d = den ? (double)den[((size_t)n * T + t) * U1 + u] : 0.0;
     const double b = (double)fr[0] + (double)gr[0] - d;
-    double cur = b, nxt = b;
+    double cur = b, nxt = neg_inf();
     if (u >= 1) {
         const int c = clampi(y[u - 1], 0, V - 1);
         cur = (double)fr[c] + (double)gr[c] - d;
     }
     if (u < Un) {
         const int c = clampi(y[u], 0, V - 1);
-        nxt = (double)fr[c] + (double)gr[c] - d;
+        nxt = ((double)fr[c] + (double)gr[c] - d) * kLog2e;
     }
-    double *o = units + (((size_t)n * T + t) * U1 + u) * 3;
     o[0] = b * kLog2e;
     o[1] = cur * kLog2e;
-    o[2] = nxt * kLog2e;
+    o[2] = nxt;
 }
 
 // Per frame: grad_den[t,u] = -(g0+g1+g2), grad_f[t,u>=1] = g1[t,u] + g2[t,u-1],
@@ -145,20 +151,6 @@ __global__ __launch_bounds__(kBlock) void simple_scatter_g_kernel(
     atomicAdd(dense_g + ((size_t)n * U1 + u) * V + col, w * grad_g[((size_t)n * U1 + u) * 3 + k]);
 }
 
-typedef float v4f __attribute__((ext_vector_type(4)));
-
-// n4 = number of leading 16-byte groups to store as vectors (0 if p is not
-// 16-byte aligned); the rest goes out as single floats.
-__global__ __launch_bounds__(kBlock) void zero_fill_kernel(float *__restrict__ p, size_t n,
-                                                           size_t n4) {
-    const size_t stride = (size_t)gridDim.x * kBlock;
-    v4f *p4 = reinterpret_cast<v4f *>(p);
-    const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < n4; i += stride) p4[i] = z;
-    for (size_t i = (n4 << 2) + (size_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride)
-        p[i] = 0.0f;
-}
-
 inline dim3 cell_grid(int N, int T, int U) {
     const long cells = (long)T * (U + 1);
     return dim3((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N);
@@ -169,8 +161,11 @@ inline dim3 cell_grid(int N, int T, int U) {
 hipError_t launch_simple_gather_units(const float *f, const float *g, const float *den,
                                       const int *ys, const int *lx, const int *ly, double *units,
                                       int N, int T, int U, int V, hipStream_t stream) {
-    hipLaunchKernelGGL(simple_gather_units_kernel, cell_grid(N, T, U), dim3(kBlock), 0, stream, f,
-                       g, den, ys, lx, ly, units, T, U, V);
+    const int P = padded_contexts(U);
+    const long cells = (long)T * P;
+    hipLaunchKernelGGL(simple_gather_units_kernel,
+                       dim3((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N), dim3(kBlock),
+                       0, stream, f, g, den, ys, lx, ly, units, T, U, V, P);
     return hipGetLastError();
 }
 
@@ -201,17 +196,6 @@ hipError_t launch_simple_scatter(const float *grad_f, const float *grad_g, const
         return hipGetLastError();
     }
     return hipSuccess;
-}
-
-hipError_t launch_zero_fill(float *p, size_t n, hipStream_t stream) {
-    if (n == 0) return hipSuccess;
-    size_t blocks = (n / 4 + kBlock - 1) / kBlock;
-    if (blocks > 16384) blocks = 16384;
-    if (blocks == 0) blocks = 1;
-    const size_t n4 = (reinterpret_cast<uintptr_t>(p) & 15u) ? 0 : n / 4;
-    hipLaunchKernelGGL(zero_fill_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream, p, n,
-                       n4);
-    return hipGetLastError();
 }
 
 }  // namespace wctct

@@ -10,8 +10,11 @@
 //   * and turn alpha/beta into d(cost)/d(unit) (replaces k_fill_grad,
 //     csrc/gather.cu:311-374).
 // Units are stored as doubles scaled to log2, the lattice's working format
-// (v_exp_f32 / v_log_f32 are base 2, and the lattice sums in double).  One
-// thread per cell; cells of padding (t >= lx[n] or u > ly[n]) are never read.
+// (v_exp_f32 / v_log_f32 are base 2, and the lattice sums in double), in a
+// buffer of P = padded_contexts(U) contexts per frame.  One thread per cell;
+// cells of padding (t >= lx[n] or u > ly[n]) are never read from the inputs.
+// For t < lx[n] the padding contexts u > ly[n] get the neutral units
+// {0, 0, -inf}, and "next" is -inf at u = ly[n]: no mass can flow there.
 #include "device_utils.h"
 #include "launch.h"
 
@@ -26,33 +29,47 @@ struct Cell {
     bool in_range, live;
 };
 
-__device__ __forceinline__ Cell locate_cell(const int *lx, const int *ly, int T, int U) {
+// Cell of a (T x W) grid of sample blockIdx.y, W = U+1 (tensors of the
+// interface) or W = P (work buffers).
+__device__ __forceinline__ Cell locate_cell(const int *lx, const int *ly, int T, int U, int W) {
     Cell c;
-    const int U1 = U + 1;
     c.n = blockIdx.y;
     const int cell = blockIdx.x * kCellBlock + threadIdx.x;
-    c.in_range = cell < T * U1;
-    c.t = cell / U1;
-    c.u = cell - c.t * U1;
+    c.in_range = cell < T * W;
+    c.t = cell / W;
+    c.u = cell - c.t * W;
     c.Tn = min(max(lx[c.n], 0), T);
     c.Un = min(max(ly[c.n], 0), U);
     c.live = c.in_range && c.t < c.Tn && c.u <= c.Un;
     return c;
 }
 
-__device__ __forceinline__ void store_units(double *units, const Cell &c, int T, int U, double b,
+// b, cur, nxt in natural-log units; nxt is only meaningful for u < Un.
+__device__ __forceinline__ void store_units(double *units, const Cell &c, int T, int P, double b,
                                             double cur, double nxt) {
-    double *o = units + (((size_t)c.n * T + c.t) * (U + 1) + c.u) * 3;
+    double *o = units + (((size_t)c.n * T + c.t) * P + c.u) * 3;
     o[0] = b * kLog2e;
     o[1] = cur * kLog2e;
-    o[2] = nxt * kLog2e;
+    o[2] = (c.u < c.Un) ? nxt * kLog2e : neg_inf();
+}
+
+// Padding context of a live frame: neutral units.  Returns true if handled.
+__device__ __forceinline__ bool store_padding(double *units, const Cell &c, int T, int P) {
+    if (c.live) return false;
+    if (c.in_range && c.t < c.Tn) {
+        double *o = units + (((size_t)c.n * T + c.t) * P + c.u) * 3;
+        o[0] = 0.0;
+        o[1] = 0.0;
+        o[2] = neg_inf();
+    }
+    return true;
 }
 
 __global__ __launch_bounds__(kCellBlock) void gather_units_kernel(
     const float *__restrict__ joint, const int *__restrict__ ys, const int *__restrict__ lx,
-    const int *__restrict__ ly, double *__restrict__ units, int T, int U, int V) {
-    const Cell c = locate_cell(lx, ly, T, U);
-    if (!c.live) return;
+    const int *__restrict__ ly, double *__restrict__ units, int T, int U, int V, int P) {
+    const Cell c = locate_cell(lx, ly, T, U, P);
+    if (store_padding(units, c, T, P)) return;
     const float *row = joint + (((size_t)c.n * T + c.t) * (U + 1) + c.u) * (size_t)V;
     const int *y = ys + (size_t)c.n * U;
     const float b = row[0];
@@ -60,16 +77,16 @@ __global__ __launch_bounds__(kCellBlock) void gather_units_kernel(
     // labels are clamped into [0,V) so that a corrupt label cannot fault
     if (c.u >= 1) cur = row[min(max(y[c.u - 1], 0), V - 1)];
     if (c.u < c.Un) nxt = row[min(max(y[c.u], 0), V - 1)];
-    store_units(units, c, T, U, b, cur, nxt);
+    store_units(units, c, T, P, b, cur, nxt);
 }
 
 __global__ __launch_bounds__(kCellBlock) void scale_units_kernel(
     const float *__restrict__ units_nat, const int *__restrict__ lx, const int *__restrict__ ly,
-    double *__restrict__ units, int T, int U) {
-    const Cell c = locate_cell(lx, ly, T, U);
-    if (!c.live) return;
+    double *__restrict__ units, int T, int U, int P) {
+    const Cell c = locate_cell(lx, ly, T, U, P);
+    if (store_padding(units, c, T, P)) return;
     const float *i = units_nat + (((size_t)c.n * T + c.t) * (U + 1) + c.u) * 3;
-    store_units(units, c, T, U, i[0], i[1], i[2]);
+    store_units(units, c, T, P, i[0], i[1], i[2]);
 }
 
 // LP(t,u,0) = f_g[t,0]   + g_g[u,0] - den[t,u]
@@ -77,9 +94,9 @@ __global__ __launch_bounds__(kCellBlock) void scale_units_kernel(
 __global__ __launch_bounds__(kCellBlock) void simple_units_kernel(
     const float *__restrict__ f_g, const float *__restrict__ g_g, const float *__restrict__ den,
     const int *__restrict__ lx, const int *__restrict__ ly, double *__restrict__ units, int T,
-    int U) {
-    const Cell c = locate_cell(lx, ly, T, U);
-    if (!c.live) return;
+    int U, int P) {
+    const Cell c = locate_cell(lx, ly, T, U, P);
+    if (store_padding(units, c, T, P)) return;
     const int U1 = U + 1;
     const float *fr = f_g + ((size_t)c.n * T + c.t) * U1;
     const float *gr = g_g + ((size_t)c.n * U1 + c.u) * 3;
@@ -87,7 +104,7 @@ __global__ __launch_bounds__(kCellBlock) void simple_units_kernel(
     const double b = (double)fr[0] + (double)gr[0] - d;
     const double cur = (c.u >= 1) ? (double)fr[c.u] + (double)gr[1] - d : b;
     const double nxt = (c.u < c.Un) ? (double)fr[c.u + 1] + (double)gr[2] - d : b;
-    store_units(units, c, T, U, b, cur, nxt);
+    store_units(units, c, T, P, b, cur, nxt);
 }
 
 // g0 = -[2^(a_e+LP0+b_e-ll) + 2^(a_o+LP0+b_e-ll)]
@@ -100,8 +117,8 @@ __global__ __launch_bounds__(kCellBlock) void simple_units_kernel(
 __global__ __launch_bounds__(kCellBlock) void unit_grads_kernel(
     const double *__restrict__ units, const int *__restrict__ ys, const int *__restrict__ lx,
     const int *__restrict__ ly, const double *__restrict__ alphas,
-    const double *__restrict__ betas, float *__restrict__ unit_grads, int T, int U) {
-    const Cell c = locate_cell(lx, ly, T, U);
+    const double *__restrict__ betas, float *__restrict__ unit_grads, int T, int U, int P) {
+    const Cell c = locate_cell(lx, ly, T, U, U + 1);
     if (!c.in_range) return;
     const int U1 = U + 1;
     float *go = unit_grads + (((size_t)c.n * T + c.t) * U1 + c.u) * 3;
@@ -111,19 +128,19 @@ __global__ __launch_bounds__(kCellBlock) void unit_grads_kernel(
         go[2] = 0.0f;
         return;
     }
-    const size_t lat = (size_t)(T + 1) * U1 * 2;
+    const size_t lat = (size_t)(T + 1) * P * 2;
     const double *an = alphas + (size_t)c.n * lat;
     const double *bn = betas + (size_t)c.n * lat;
     const double ll = bn[1];   // beta(0, state 0): pair {o,e} of context 0 at t = 0
-    const double2 a = *reinterpret_cast<const double2 *>(an + ((size_t)c.t * U1 + c.u) * 2);
-    const double2 b = *reinterpret_cast<const double2 *>(bn + ((size_t)(c.t + 1) * U1 + c.u) * 2);
-    const double *lp = units + (((size_t)c.n * T + c.t) * U1 + c.u) * 3;
+    const double2 a = *reinterpret_cast<const double2 *>(an + ((size_t)c.t * P + c.u) * 2);
+    const double2 b = *reinterpret_cast<const double2 *>(bn + ((size_t)(c.t + 1) * P + c.u) * 2);
+    const double *lp = units + (((size_t)c.n * T + c.t) * P + c.u) * 3;
     const double lp0 = lp[0] - ll, lp1 = lp[1] - ll, lp2 = lp[2] - ll;
     const float g0 = -(exp2_hw((float)(a.y + lp0 + b.y)) + exp2_hw((float)(a.x + lp0 + b.y)));
     const float g1 = -exp2_hw((float)(a.x + lp1 + b.x));
     float g2 = 0.0f;
     if (c.u < c.Un) {
-        const double bo_next = bn[((size_t)(c.t + 1) * U1 + c.u + 1) * 2];
+        const double bo_next = bn[((size_t)(c.t + 1) * P + c.u + 1) * 2];
         g2 = -exp2_hw((float)(a.y + lp2 + bo_next));
         const int *y = ys + (size_t)c.n * U;
         if (c.u >= 1 && y[c.u - 1] != y[c.u]) g2 -= exp2_hw((float)(a.x + lp2 + bo_next));
@@ -133,8 +150,8 @@ __global__ __launch_bounds__(kCellBlock) void unit_grads_kernel(
     go[2] = g2;
 }
 
-inline dim3 cell_grid(int N, int T, int U) {
-    const long cells = (long)T * (U + 1);
+inline dim3 cell_grid(int N, int T, int W) {
+    const long cells = (long)T * W;
     return dim3((unsigned)((cells + kCellBlock - 1) / kCellBlock), (unsigned)N);
 }
 
@@ -142,31 +159,34 @@ inline dim3 cell_grid(int N, int T, int U) {
 
 hipError_t launch_gather_units(const float *joint, const int *ys, const int *lx, const int *ly,
                                double *units, int N, int T, int U, int V, hipStream_t stream) {
-    hipLaunchKernelGGL(gather_units_kernel, cell_grid(N, T, U), dim3(kCellBlock), 0, stream,
-                       joint, ys, lx, ly, units, T, U, V);
+    const int P = padded_contexts(U);
+    hipLaunchKernelGGL(gather_units_kernel, cell_grid(N, T, P), dim3(kCellBlock), 0, stream,
+                       joint, ys, lx, ly, units, T, U, V, P);
     return hipGetLastError();
 }
 
 hipError_t launch_scale_units(const float *units_nat, const int *lx, const int *ly, double *units,
                               int N, int T, int U, hipStream_t stream) {
-    hipLaunchKernelGGL(scale_units_kernel, cell_grid(N, T, U), dim3(kCellBlock), 0, stream,
-                       units_nat, lx, ly, units, T, U);
+    const int P = padded_contexts(U);
+    hipLaunchKernelGGL(scale_units_kernel, cell_grid(N, T, P), dim3(kCellBlock), 0, stream,
+                       units_nat, lx, ly, units, T, U, P);
     return hipGetLastError();
 }
 
 hipError_t launch_simple_units(const float *f_g, const float *g_g, const float *den,
                                const int *lx, const int *ly, double *units, int N, int T, int U,
                                hipStream_t stream) {
-    hipLaunchKernelGGL(simple_units_kernel, cell_grid(N, T, U), dim3(kCellBlock), 0, stream, f_g,
-                       g_g, den, lx, ly, units, T, U);
+    const int P = padded_contexts(U);
+    hipLaunchKernelGGL(simple_units_kernel, cell_grid(N, T, P), dim3(kCellBlock), 0, stream, f_g,
+                       g_g, den, lx, ly, units, T, U, P);
     return hipGetLastError();
 }
 
 hipError_t launch_unit_grads(const double *units, const int *ys, const int *lx, const int *ly,
                              const double *alphas, const double *betas, float *unit_grads, int N,
                              int T, int U, hipStream_t stream) {
-    hipLaunchKernelGGL(unit_grads_kernel, cell_grid(N, T, U), dim3(kCellBlock), 0, stream, units,
-                       ys, lx, ly, alphas, betas, unit_grads, T, U);
+    hipLaunchKernelGGL(unit_grads_kernel, cell_grid(N, T, U + 1), dim3(kCellBlock), 0, stream,
+                       units, ys, lx, ly, alphas, betas, unit_grads, T, U, padded_contexts(U));
     return hipGetLastError();
 }
 
