@@ -272,20 +272,29 @@ def test_infeasible_sample_has_infinite_cost():
     np.testing.assert_allclose(c[1], ref[1], rtol=LOSS_RTOL)
 
 
-def test_full_size_typical_asr_batch():
-    """N=32, T<=250, U<=60, V=1024: costs and unit gradients against the C
-    oracle in float64; the 2 GB dense gradient is checked on the GPU through
-    size-independent properties (support, per-frame mass -1, gathered values)."""
+FULL_SIZE = [
+    # name, N, T, U, V, lx range, ly range, sigma
+    ("typical_asr_batch", 32, 250, 60, 1024, (150, 250), (30, 60), 1.0),
+    ("large_vocab_long_lattice", 8, 500, 120, 4096, (400, 500), (80, 120), 2.0),
+]
+
+
+@pytest.mark.parametrize("cfg", FULL_SIZE, ids=[c[0] for c in FULL_SIZE])
+def test_full_size(cfg):
+    """Full-size batches of the benchmark configurations: costs and unit
+    gradients against the C oracle in float64; the 2 GB / 7.9 GB dense gradient
+    is checked on the GPU through size-independent properties (support,
+    per-frame mass -1, gathered values)."""
     import warp_ctct
-    N, T, U, V = 32, 250, 60, 1024
+    name, N, T, U, V, lx_rng, ly_rng, sigma = cfg
     g = torch.Generator(device="cuda").manual_seed(1234)
-    logits = torch.randn(N, T, U + 1, V, device="cuda", generator=g)
+    logits = torch.randn(N, T, U + 1, V, device="cuda", generator=g).mul_(sigma)
     joint = logits.log_softmax(-1)
     del logits
     rng = np.random.default_rng(1234)
-    lx = rng.integers(150, 251, N).astype(np.int32)
-    ly = rng.integers(30, 61, N).astype(np.int32)
-    lx[3], ly[5] = 250, 60
+    lx = rng.integers(lx_rng[0], lx_rng[1] + 1, N).astype(np.int32)
+    ly = rng.integers(ly_rng[0], ly_rng[1] + 1, N).astype(np.int32)
+    lx[3], ly[5] = lx_rng[1], ly_rng[1]
     ys = rng.integers(1, V, (N, U)).astype(np.int32)
     ys[:, 7] = ys[:, 6]
     d_ys, d_lx, d_ly = dev(ys), dev(lx), dev(ly)
@@ -327,7 +336,7 @@ def test_full_size_typical_asr_batch():
     assert int((dense != 0).sum()) == int(((dense != 0) & mask).sum())
     assert int((dense[pad.expand_as(dense)] != 0).sum()) == 0
     # per-frame mass: sum over (u, v) = -w[n] for t < lx[n], 0 beyond
-    mass = dense.double().sum((2, 3)).cpu().numpy()
+    mass = dense.sum((2, 3), dtype=torch.float64).cpu().numpy()
     wn = w.cpu().numpy().astype(np.float64)
     for n in range(N):
         np.testing.assert_allclose(mass[n, :lx[n]], -wn[n], rtol=1e-4, atol=1e-5)

@@ -122,8 +122,48 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_loss_joint_fwd(const torch::Tensor
     return std::make_tuple(costs, costs);
 }
 
+// The two halves of ctct_loss_joint_bwd as separate operators, so that a
+// caller (bench.py) can bracket the zero-fill kernel alone with HIP events.
+torch::Tensor dense_zero_fill(const torch::Tensor &like, const int64_t N, const int64_t T,
+                              const int64_t U1, const int64_t V) {
+    CHECK_DEVICE(like);
+    CHECK_FLOAT(like);
+    TORCH_CHECK(N >= 0 && T >= 0 && U1 >= 1 && V >= 1, "invalid sizes");
+    const DeviceGuard device_guard(device_of(like));
+    auto dense = torch::empty({N, T, U1, V}, like.options());
+    check_rc(warpctct_zero_fill_f32(dense.data_ptr<float>(), static_cast<size_t>(dense.numel()),
+                                    current_stream()),
+             "dense_zero_fill");
+    return dense;
+}
+
+void dense_patch(const torch::Tensor &unit_grads, const torch::Tensor &ys, const torch::Tensor &lx,
+                 const torch::Tensor &ly, const torch::Tensor &grad_out, torch::Tensor &dense) {
+    CHECK_CONTIGUOUS(unit_grads);
+    CHECK_FLOAT(unit_grads);
+    CHECK_DEVICE(unit_grads);
+    CHECK_CONTIGUOUS(grad_out);
+    CHECK_FLOAT(grad_out);
+    CHECK_DEVICE(grad_out);
+    CHECK_CONTIGUOUS(dense);
+    CHECK_FLOAT(dense);
+    CHECK_DEVICE(dense);
+    TORCH_CHECK(unit_grads.dim() == 4 && unit_grads.size(3) == 3, "unit_grads must be (N,T,U+1,3)");
+    const int N = unit_grads.size(0), T = unit_grads.size(1), U = unit_grads.size(2) - 1;
+    TORCH_CHECK(dense.dim() == 4 && dense.size(0) == N && dense.size(1) == T &&
+                    dense.size(2) == U + 1, "dense must be (N,T,U+1,V)");
+    TORCH_CHECK(grad_out.dim() == 1 && grad_out.size(0) == N, "grad_out must be (N,)");
+    check_lengths(ys, lx, ly, N, U);
+    const DeviceGuard device_guard(device_of(unit_grads));
+    check_rc(warpctct_dense_patch_f32(unit_grads.data_ptr<float>(), ys.data_ptr<int>(),
+                                      lx.data_ptr<int>(), ly.data_ptr<int>(),
+                                      grad_out.data_ptr<float>(), dense.data_ptr<float>(), N, T, U,
+                                      static_cast<int>(dense.size(3)), current_stream()),
+             "dense_patch");
+}
+
 // Backward of the fused entry: CTCTLoss.backward (warp_ctct/__init__.py:30-33)
-// and the gather backward in one pass.  grad_out (N) scales sample n.
+// and the gather backward.  grad_out (N) scales sample n.
 torch::Tensor ctct_loss_joint_bwd(const torch::Tensor &unit_grads, const torch::Tensor &ys,
                                   const torch::Tensor &lx, const torch::Tensor &ly,
                                   const torch::Tensor &grad_out, const int64_t V) {
@@ -378,6 +418,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           "Dense gradient wrt the joint from unit gradients.", pybind11::arg("unit_grads"),
           pybind11::arg("ys"), pybind11::arg("lx"), pybind11::arg("ly"),
           pybind11::arg("grad_out"), pybind11::arg("V"));
+    m.def("dense_zero_fill", &dense_zero_fill, "Zero-filled (N,T,U+1,V) gradient tensor.",
+          pybind11::arg("like"), pybind11::arg("N"), pybind11::arg("T"), pybind11::arg("U1"),
+          pybind11::arg("V"));
+    m.def("dense_patch", &dense_patch, "Write the non-zero entries of the dense gradient.",
+          pybind11::arg("unit_grads"), pybind11::arg("ys"), pybind11::arg("lx"),
+          pybind11::arg("ly"), pybind11::arg("grad_out"), pybind11::arg("dense"));
     m.def("ctct_loss_simple_fwd", &ctct_loss_simple_fwd,
           "CTC-Transducer loss with the log-add joiner on gathered operands (forward).",
           pybind11::arg("f"), pybind11::arg("g"), pybind11::arg("ys"), pybind11::arg("den"),

@@ -7,17 +7,22 @@
 // which hold grad_out[n] * g0 / g1 / g2 (coincident columns add).
 //
 // The zero-fill is pure HBM write traffic (4*N*T*(U+1)*V bytes) and decides
-// the throughput of the whole loss, so it is kept free of everything else:
-//  * zero_fill_vec_kernel: a 256-thread workgroup issues ONE 16-byte store
-//    per thread (4 KiB contiguous per workgroup) and retires.  On MI355X this
-//    finest-grained launch gives the highest write bandwidth (~6.8 TB/s);
-//    workgroups that loop over 16-64 KiB or use non-temporal stores lose
-//    10-20 %, and a workgroup that first has to fetch per-row data (labels,
-//    unit gradients) before it can store loses 25-35 %.  The fill does not
-//    depend on the lattice, so a caller may run it on another stream while
-//    the lattice is computed.
-//  * patch_kernel: one thread per live cell (t,u) overwrites the <= 3
-//    non-zero entries of its row.
+// the throughput of the whole loss, so it is kept free of everything else.
+// Measurements on MI355X (N=32, T=250, U=60, V=1024; 2.0 GB) behind this:
+//  * zero_fill_vec_kernel — a 256-thread workgroup issues ONE 16-byte store
+//    per thread (4 KiB contiguous per workgroup) and retires — reaches
+//    ~6.7 TB/s (295 us); workgroups that loop over 16-64 KiB, persistent
+//    grid-stride loops and non-temporal stores all lose 10-35 %;
+//  * a fused kernel whose workgroups also fetch their row's labels and unit
+//    gradients (before the store, or after it with the non-zero lanes storing
+//    a second time) takes 370-480 us: a wave that waits for a load keeps its
+//    slot, and the fill lives off instant wave turnover;
+//  * the separate sparse pass (patch_kernel, one thread per live cell, <= 3
+//    scattered 4-byte stores) costs ~40 us; 64-byte aligned group stores
+//    instead of 4-byte ones gain little;
+//  * running the fill on a second stream next to the gather / lattice kernels
+//    is slower than running everything back to back.
+// Hence two launches on one stream: fill, then patch.
 #include "device_utils.h"
 #include "launch.h"
 

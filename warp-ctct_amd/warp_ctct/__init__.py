@@ -74,8 +74,9 @@ class _CTCTLoss(torch.autograd.Function):
     def backward(ctx, grad_outputs):
         unit_grads, labels, lx, ly = ctx.saved_tensors
         grad_outputs = grad_outputs.reshape(-1).float().contiguous()
-        dense = _run("dense_grad", lambda: core.ctct_loss_joint_bwd(
-            unit_grads, labels, lx, ly, grad_outputs, ctx.vocab))
+        n, t, u1, _ = unit_grads.shape
+        dense = _run("dense_zero_fill", lambda: core.dense_zero_fill(unit_grads, n, t, u1, ctx.vocab))
+        _run("dense_patch", lambda: core.dense_patch(unit_grads, labels, lx, ly, grad_outputs, dense))
         return dense, None, None, None, None
 
 
