@@ -123,6 +123,32 @@ int warpctct_loss_forward_f32(const float *joint, const int *ys, const int *lx, 
                               size_t workspace_bytes, float *costs, float *unit_grads,
                               void *stream);
 
+/* The same without unit gradients: gather + lattices only.  The workspace then
+ * holds everything the dense gradient needs (units, alpha, beta) and must be
+ * kept until warpctct_dense_grad_lattice_f32 has run.  want_alpha == 0 is the
+ * no-grad mode (beta only). */
+int warpctct_loss_lattice_f32(const float *joint, const int *ys, const int *lx, const int *ly,
+                              int N, int T, int U, int V, void *workspace, size_t workspace_bytes,
+                              float *costs, int want_alpha, void *stream);
+
+/* Dense gradient straight from that workspace: zero-fill, then per live cell
+ * the unit gradients are computed on the fly and written to columns 0, y[u-1],
+ * y[u].  Sample n is weighted by grad_out[n*grad_out_stride] * scale
+ * (/ lx[n] if average_frames): stride 0 with scale 1/N is the backward of
+ * reduction='mean', stride 1 with scale 1 of reduction='none'
+ * (warp_ctct/__init__.py:138-147 differentiated; CTCTLoss.backward :30-33;
+ * gather backward).  grad_out NULL = ones. */
+int warpctct_dense_grad_lattice_f32(const void *workspace, size_t workspace_bytes, const int *ys,
+                                    const int *lx, const int *ly, const float *grad_out,
+                                    int grad_out_stride, float scale, int average_frames,
+                                    float *dense, int N, int T, int U, int V, void *stream);
+
+/* Its sparse half alone, into a tensor that already holds zeros. */
+int warpctct_dense_patch_lattice_f32(const void *workspace, size_t workspace_bytes, const int *ys,
+                                     const int *lx, const int *ly, const float *grad_out,
+                                     int grad_out_stride, float scale, int average_frames,
+                                     float *dense, int N, int T, int U, int V, void *stream);
+
 /* _C.ctct_loss_fwd proper: the input is already gathered (N,T,U+1,3). */
 int warpctct_loss_forward_units_f32(const float *units_nat, const int *ys, const int *lx,
                                     const int *ly, int N, int T, int U, void *workspace,
@@ -163,13 +189,15 @@ size_t warpctct_simple_workspace_bytes(int N, int T, int U);
 /* ctct_simple_loss forward on f (N,T,V), g (N,U+1,V): den (if normalized),
  * units, lattice, unit gradients and their reductions.  Replaces
  * warp_ctct/__init__.py:195-225 + _C.ctct_loss_simple_fwd
- * (csrc/binding.cpp:103-222).  den (N,T,U+1) is an output when normalized != 0
- * (only t<lx[n], u<=ly[n] is written) and ignored otherwise.  grad_f/grad_g/
- * grad_den may all be NULL (no-grad mode). */
+ * (csrc/binding.cpp:103-222).  When normalized != 0, den (N,T,U+1; only
+ * t<lx[n], u<=ly[n] is written), fmax (N,T) = max_v f and gmax (N,U+1) =
+ * max_v g are outputs (the backward needs them); otherwise they are ignored.
+ * grad_f/grad_g/grad_den may all be NULL (no-grad mode). */
 int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, const int *lx,
                                 const int *ly, int N, int T, int U, int V, int normalized,
-                                void *workspace, size_t workspace_bytes, float *den, float *costs,
-                                float *grad_f, float *grad_g, float *grad_den, void *stream);
+                                void *workspace, size_t workspace_bytes, float *den, float *fmax,
+                                float *gmax, float *costs, float *grad_f, float *grad_g,
+                                float *grad_den, void *stream);
 
 /* _C.ctct_loss_simple_fwd proper: f_g (N,T,U+1), g_g (N,U+1,3) already
  * gathered, den (N,T,U+1) or NULL (unnormalised, csrc/simple_unnorm.cu). */
@@ -182,16 +210,19 @@ int warpctct_simple_forward_units_f32(const float *f_g, const float *g_g, const 
  * every element written.  With den != NULL the den-path
  * (LogMMExp.backward, warp_ctct/__init__.py:45-52) is included:
  * dense_f[t,v] = sum_u w*grad_den[t,u]*exp(f[t,v]+g[u,v]-den[t,u]) + scatter,
- * dense_g likewise summed over t.  Either dense pointer may be NULL. */
+ * dense_g likewise summed over t; fmax/gmax are the forward's row maxima.
+ * Either dense pointer may be NULL. */
 int warpctct_simple_backward_f32(const float *f, const float *g, const float *den,
-                                 const float *grad_f, const float *grad_g, const float *grad_den,
+                                 const float *fmax, const float *gmax, const float *grad_f,
+                                 const float *grad_g, const float *grad_den,
                                  const int *ys, const int *lx, const int *ly,
                                  const float *grad_out, int N, int T, int U, int V,
                                  float *dense_f, float *dense_g, void *stream);
 
 /* ---- log-semiring matmul -------------------------------------------------- */
 
-/* Bytes of workspace for warpctct_logmm_fwd_f32 (row and column maxima). */
+/* Bytes of workspace for warpctct_logmm_fwd_f32 / _bwd_f32 (row and column
+ * maxima, by which the operands are shifted before they are exponentiated). */
 size_t warpctct_logmm_workspace_bytes(int B, int M, int Nn);
 
 /* res[b,i,j] = log sum_k exp(lhs[b,i,k] + rhs[b,k,j]); operands strided in
@@ -208,8 +239,9 @@ int warpctct_logmm_fwd_f32(const float *lhs, long lsb, long lsm, long lsk, const
  * (csrc/binding.cpp:247-324). */
 int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, long lsm, long lsk,
                            const float *rhs, long rsb, long rsk, long rsn, const float *res, int B,
-                           int M, int K, int Nn, float *grad_lhs, long glsb, long glsm, long glsk,
-                           float *grad_rhs, long grsb, long grsk, long grsn, void *stream);
+                           int M, int K, int Nn, void *workspace, size_t workspace_bytes,
+                           float *grad_lhs, long glsb, long glsm, long glsk, float *grad_rhs,
+                           long grsb, long grsk, long grsn, void *stream);
 
 #ifdef __cplusplus
 }

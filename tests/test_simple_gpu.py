@@ -64,6 +64,16 @@ def test_log_matmul_infinities_and_far_apart_maxima():
     fin = np.isfinite(ref)
     np.testing.assert_allclose(out[fin], ref[fin], rtol=1e-5, atol=1e-5)
     assert abs(out[1, 4, 4] - ref[1, 4, 4]) < 1e-3 and ref[1, 4, 4] > 290
+    # backward over the same operands: -inf rows have no gradient, and the pair
+    # (4,4) whose maxima are 300 apart takes the exact per-term path
+    go = rng.standard_normal((B, M, Nn)).astype(np.float32)
+    gl, gr = O.log_matmul_backward(go, lhs, rhs, ref)
+    d_lhs, d_rhs = dev(lhs), dev(rhs)
+    d_res = _C.log_matmul(d_lhs, d_rhs)
+    out_l, out_r = _C.log_matmul_backward(dev(go), d_lhs, d_rhs, d_res, [True, True])
+    np.testing.assert_allclose(out_l.cpu().numpy(), gl, atol=2e-5, rtol=1e-4)
+    np.testing.assert_allclose(out_r.cpu().numpy(), gr, atol=2e-5, rtol=1e-4)
+    assert abs(gl[1, 4, 0]) + abs(gl[1, 4, 7]) > 1e-3      # the far-apart pair carries gradient
 
 
 def test_log_matmul_rejects_bad_arguments():

@@ -67,8 +67,6 @@ int forward_from_units(const Workspace &w, const int *ys, const int *lx, const i
 struct SimpleWorkspace {
     Workspace lattice;
     float *unit_grads;   // (N,T,U+1,3)
-    float *fmax;         // (N,T)   row maxima of f
-    float *gmax;         // (N,U+1) row maxima of g
     size_t bytes;
 };
 
@@ -77,12 +75,8 @@ SimpleWorkspace carve_simple(void *base, int N, int T, int U) {
     w.lattice = carve(base, N, T, U);
     const uintptr_t p = reinterpret_cast<uintptr_t>(base) + w.lattice.bytes;
     const size_t ug_b = align256((size_t)N * T * (U + 1) * 3 * sizeof(float));
-    const size_t fm_b = align256((size_t)N * T * sizeof(float));
-    const size_t gm_b = align256((size_t)N * (U + 1) * sizeof(float));
     w.unit_grads = reinterpret_cast<float *>(p);
-    w.fmax = reinterpret_cast<float *>(p + ug_b);
-    w.gmax = reinterpret_cast<float *>(p + ug_b + fm_b);
-    w.bytes = w.lattice.bytes + ug_b + fm_b + gm_b;
+    w.bytes = w.lattice.bytes + ug_b;
     return w;
 }
 
@@ -201,6 +195,63 @@ int warpctct_dense_patch_f32(const float *unit_grads, const int *ys, const int *
                                    as_stream(stream)));
 }
 
+int warpctct_loss_lattice_f32(const float *joint, const int *ys, const int *lx, const int *ly,
+                              int N, int T, int U, int V, void *workspace, size_t workspace_bytes,
+                              float *costs, int want_alpha, void *stream) {
+    if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
+    if (N == 0) return WARPCTCT_OK;
+    if (!lx || !ly || !costs || !workspace || (T > 0 && !joint) || (U > 0 && !ys))
+        return WARPCTCT_EINVAL;
+    const Workspace w = carve(workspace, N, T, U);
+    if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
+    if (T > 0) {
+        int rc = done(launch_gather_units(joint, ys, lx, ly, w.units, N, T, U, V,
+                                          as_stream(stream)));
+        if (rc != WARPCTCT_OK) return rc;
+    }
+    LatticeArgs a;
+    a.units = w.units;
+    a.ys = ys;
+    a.lx = lx;
+    a.ly = ly;
+    a.alphas = w.alphas;
+    a.betas = w.betas;
+    a.costs = costs;
+    a.N = N;
+    a.T = T;
+    a.U = U;
+    a.beta_only = (want_alpha == 0);
+    return done(launch_lattice(a, as_stream(stream)));
+}
+
+int warpctct_dense_patch_lattice_f32(const void *workspace, size_t workspace_bytes, const int *ys,
+                                     const int *lx, const int *ly, const float *grad_out,
+                                     int grad_out_stride, float scale, int average_frames,
+                                     float *dense, int N, int T, int U, int V, void *stream) {
+    if (!dims_ok(N, T, U) || V < 1 || grad_out_stride < 0) return WARPCTCT_EINVAL;
+    if (N == 0 || T == 0) return WARPCTCT_OK;
+    if (!workspace || !lx || !ly || !dense || (U > 0 && !ys)) return WARPCTCT_EINVAL;
+    const Workspace w = carve(const_cast<void *>(workspace), N, T, U);
+    if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
+    return done(launch_dense_patch_lattice(w.units, w.alphas, w.betas, ys, lx, ly, grad_out,
+                                           grad_out_stride, scale, average_frames, dense, N, T, U,
+                                           V, as_stream(stream)));
+}
+
+int warpctct_dense_grad_lattice_f32(const void *workspace, size_t workspace_bytes, const int *ys,
+                                    const int *lx, const int *ly, const float *grad_out,
+                                    int grad_out_stride, float scale, int average_frames,
+                                    float *dense, int N, int T, int U, int V, void *stream) {
+    if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
+    if (N == 0 || T == 0) return WARPCTCT_OK;
+    if (!dense) return WARPCTCT_EINVAL;
+    int rc = done(launch_zero_fill(dense, (size_t)N * T * (U + 1) * V, as_stream(stream)));
+    if (rc != WARPCTCT_OK) return rc;
+    return warpctct_dense_patch_lattice_f32(workspace, workspace_bytes, ys, lx, ly, grad_out,
+                                            grad_out_stride, scale, average_frames, dense, N, T, U,
+                                            V, stream);
+}
+
 int warpctct_loss_forward_f32(const float *joint, const int *ys, const int *lx, const int *ly,
                               int N, int T, int U, int V, void *workspace, size_t workspace_bytes,
                               float *costs, float *unit_grads, void *stream) {
@@ -281,15 +332,16 @@ size_t warpctct_simple_workspace_bytes(int N, int T, int U) {
 
 int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, const int *lx,
                                 const int *ly, int N, int T, int U, int V, int normalized,
-                                void *workspace, size_t workspace_bytes, float *den, float *costs,
-                                float *grad_f, float *grad_g, float *grad_den, void *stream) {
+                                void *workspace, size_t workspace_bytes, float *den, float *fmax,
+                                float *gmax, float *costs, float *grad_f, float *grad_g,
+                                float *grad_den, void *stream) {
     if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
     if (N == 0) return WARPCTCT_OK;
     const bool want_grad = grad_f || grad_g || grad_den;
     if (!g || !lx || !ly || !costs || !workspace || (T > 0 && !f) || (U > 0 && !ys))
         return WARPCTCT_EINVAL;
     if (want_grad && (!grad_f || !grad_g || (normalized && !grad_den))) return WARPCTCT_EINVAL;
-    if (normalized && T > 0 && !den) return WARPCTCT_EINVAL;
+    if (normalized && T > 0 && (!den || !fmax || !gmax)) return WARPCTCT_EINVAL;
     const SimpleWorkspace w = carve_simple(workspace, N, T, U);
     if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
     hipStream_t st = as_stream(stream);
@@ -298,7 +350,7 @@ int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, c
             // den[n,t,u] = logsumexp_v(f[n,t,v] + g[n,u,v]):  lhs = f, rhs[b,k,j] = g[b,j,k]
             const LogmmOperand lhs = {f, (long)T * V, (long)V, 1L};
             const LogmmOperand rhs = {g, (long)(U + 1) * V, 1L, (long)V};
-            int rc = done(launch_logmm_fwd(lhs, rhs, w.fmax, w.gmax, den, N, T, V, U + 1, lx, ly, st));
+            int rc = done(launch_logmm_fwd(lhs, rhs, fmax, gmax, den, N, T, V, U + 1, lx, ly, st));
             if (rc != WARPCTCT_OK) return rc;
         }
         int rc = done(launch_simple_gather_units(f, g, normalized ? den : nullptr, ys, lx, ly,
@@ -331,7 +383,8 @@ int warpctct_simple_forward_units_f32(const float *f_g, const float *g_g, const 
 }
 
 int warpctct_simple_backward_f32(const float *f, const float *g, const float *den,
-                                 const float *grad_f, const float *grad_g, const float *grad_den,
+                                 const float *fmax, const float *gmax, const float *grad_f,
+                                 const float *grad_g, const float *grad_den,
                                  const int *ys, const int *lx, const int *ly,
                                  const float *grad_out, int N, int T, int U, int V,
                                  float *dense_f, float *dense_g, void *stream) {
@@ -339,7 +392,7 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
     if (N == 0) return WARPCTCT_OK;
     if (!lx || !ly || (U > 0 && !ys) || (dense_f && !grad_f) || (dense_g && !grad_g))
         return WARPCTCT_EINVAL;
-    if (den && (!f || !g || !grad_den)) return WARPCTCT_EINVAL;
+    if (den && (!f || !g || !grad_den || !fmax || !gmax)) return WARPCTCT_EINVAL;
     hipStream_t st = as_stream(stream);
     const int U1 = U + 1;
     if (T == 0) dense_f = nullptr;
@@ -348,14 +401,14 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
         const LogmmOperand rhs = {g, (long)U1 * V, 1L, (long)V};
         if (dense_f) {
             const LogmmGrad gl = {dense_f, (long)T * V, (long)V, 1L};
-            int rc = done(launch_logmm_bwd_lhs(lhs, rhs, grad_den, den, gl, N, T, V, U1, lx, ly,
+            int rc = done(launch_logmm_bwd_lhs(lhs, rhs, fmax, gmax, grad_den, den, gl, N, T, V, U1, lx, ly,
                                                grad_out, st));
             if (rc != WARPCTCT_OK) return rc;
         }
         if (dense_g) {
             // gradient of rhs[b,k,j] = g[b,j,k] stored straight into the (N,U+1,V) layout
             const LogmmGrad gr = {dense_g, (long)U1 * V, 1L, (long)V};
-            int rc = done(launch_logmm_bwd_rhs(lhs, rhs, grad_den, den, gr, N, T, V, U1, lx, ly,
+            int rc = done(launch_logmm_bwd_rhs(lhs, rhs, fmax, gmax, grad_den, den, gr, N, T, V, U1, lx, ly,
                                                grad_out, st));
             if (rc != WARPCTCT_OK) return rc;
         }
@@ -397,24 +450,34 @@ int warpctct_logmm_fwd_f32(const float *lhs, long lsb, long lsm, long lsk, const
 
 int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, long lsm, long lsk,
                            const float *rhs, long rsb, long rsk, long rsn, const float *res, int B,
-                           int M, int K, int Nn, float *grad_lhs, long glsb, long glsm, long glsk,
-                           float *grad_rhs, long grsb, long grsk, long grsn, void *stream) {
+                           int M, int K, int Nn, void *workspace, size_t workspace_bytes,
+                           float *grad_lhs, long glsb, long glsm, long glsk, float *grad_rhs,
+                           long grsb, long grsk, long grsn, void *stream) {
     if (B < 0 || M < 0 || K < 0 || Nn < 0 || B > kMaxGrid || K > kMaxGrid * 64)
         return WARPCTCT_EINVAL;
     if (B == 0 || K == 0) return WARPCTCT_OK;
-    if (!lhs || !rhs || ((M > 0 && Nn > 0) && (!grad_out || !res))) return WARPCTCT_EINVAL;
+    if (!lhs || !rhs || !workspace || ((M > 0 && Nn > 0) && (!grad_out || !res)))
+        return WARPCTCT_EINVAL;
+    if (workspace_bytes < warpctct_logmm_workspace_bytes(B, M, Nn)) return WARPCTCT_EWORKSPACE;
+    float *lmax = static_cast<float *>(workspace);
+    float *rmax = reinterpret_cast<float *>(static_cast<char *>(workspace) +
+                                            align256((size_t)B * M * sizeof(float)));
     const LogmmOperand l = {lhs, lsb, lsm, lsk};
     const LogmmOperand r = {rhs, rsb, rsk, rsn};
+    {
+        int rc = done(launch_logmm_max(l, r, lmax, rmax, B, M, K, Nn, as_stream(stream)));
+        if (rc != WARPCTCT_OK) return rc;
+    }
     if (grad_lhs) {
         const LogmmGrad g = {grad_lhs, glsb, glsm, glsk};
-        int rc = done(launch_logmm_bwd_lhs(l, r, grad_out, res, g, B, M, K, Nn, nullptr, nullptr,
-                                           nullptr, as_stream(stream)));
+        int rc = done(launch_logmm_bwd_lhs(l, r, lmax, rmax, grad_out, res, g, B, M, K, Nn, nullptr,
+                                           nullptr, nullptr, as_stream(stream)));
         if (rc != WARPCTCT_OK) return rc;
     }
     if (grad_rhs) {
         const LogmmGrad g = {grad_rhs, grsb, grsk, grsn};
-        int rc = done(launch_logmm_bwd_rhs(l, r, grad_out, res, g, B, M, K, Nn, nullptr, nullptr,
-                                           nullptr, as_stream(stream)));
+        int rc = done(launch_logmm_bwd_rhs(l, r, lmax, rmax, grad_out, res, g, B, M, K, Nn, nullptr,
+                                           nullptr, nullptr, as_stream(stream)));
         if (rc != WARPCTCT_OK) return rc;
     }
     return WARPCTCT_OK;

@@ -95,6 +95,9 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_loss_fwd(const torch::Tensor &log_
 
 // Fused entry for ctct_loss: takes the un-gathered joint (N,T,U+1,V), so the
 // index build + torch.gather of warp_ctct/__init__.py:124-131 happens inside.
+// Returns (costs, workspace): the workspace (units, alpha, beta) is what
+// dense_patch_lattice needs in backward; without requires_grad only beta runs
+// and costs is returned twice (as the reference does, binding.cpp:98).
 std::tuple<torch::Tensor, torch::Tensor> ctct_loss_joint_fwd(const torch::Tensor &joint,
                                                              const torch::Tensor &ys,
                                                              const torch::Tensor &lx,
@@ -110,20 +113,17 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_loss_joint_fwd(const torch::Tensor
 
     auto ws = make_workspace(joint, N, T, U);
     auto costs = torch::empty({N}, joint.options());
-    torch::Tensor grads;
-    if (requires_grad) grads = torch::empty({N, T, U + 1, 3}, joint.options());
-    check_rc(warpctct_loss_forward_f32(joint.data_ptr<float>(), ys.data_ptr<int>(),
+    check_rc(warpctct_loss_lattice_f32(joint.data_ptr<float>(), ys.data_ptr<int>(),
                                        lx.data_ptr<int>(), ly.data_ptr<int>(), N, T, U, V,
                                        ws.data_ptr(), ws.numel(), costs.data_ptr<float>(),
-                                       requires_grad ? grads.data_ptr<float>() : nullptr,
-                                       current_stream()),
+                                       requires_grad ? 1 : 0, current_stream()),
              "ctct_loss_joint_fwd");
-    if (requires_grad) return std::make_tuple(costs, grads);
+    if (requires_grad) return std::make_tuple(costs, ws);
     return std::make_tuple(costs, costs);
 }
 
-// The two halves of ctct_loss_joint_bwd as separate operators, so that a
-// caller (bench.py) can bracket the zero-fill kernel alone with HIP events.
+// The two halves of the dense gradient as separate operators, so that a caller
+// can bracket the zero-fill kernel alone with HIP events.
 torch::Tensor dense_zero_fill(const torch::Tensor &like, const int64_t N, const int64_t T,
                               const int64_t U1, const int64_t V) {
     CHECK_DEVICE(like);
@@ -137,29 +137,33 @@ torch::Tensor dense_zero_fill(const torch::Tensor &like, const int64_t N, const 
     return dense;
 }
 
-void dense_patch(const torch::Tensor &unit_grads, const torch::Tensor &ys, const torch::Tensor &lx,
-                 const torch::Tensor &ly, const torch::Tensor &grad_out, torch::Tensor &dense) {
-    CHECK_CONTIGUOUS(unit_grads);
-    CHECK_FLOAT(unit_grads);
-    CHECK_DEVICE(unit_grads);
+// grad_out: (N,) per-sample upstream gradients, or a 0-dim / 1-element tensor
+// that is broadcast; every sample is further scaled by `scale` and, with
+// average_frames, divided by lx[n].
+void dense_patch_lattice(const torch::Tensor &workspace, const torch::Tensor &ys,
+                         const torch::Tensor &lx, const torch::Tensor &ly,
+                         const torch::Tensor &grad_out, const double scale,
+                         const bool average_frames, torch::Tensor &dense) {
+    CHECK_CONTIGUOUS(workspace);
+    CHECK_DEVICE(workspace);
+    TORCH_CHECK(workspace.scalar_type() == at::ScalarType::Byte, "workspace must be a byte tensor");
     CHECK_CONTIGUOUS(grad_out);
     CHECK_FLOAT(grad_out);
     CHECK_DEVICE(grad_out);
     CHECK_CONTIGUOUS(dense);
     CHECK_FLOAT(dense);
     CHECK_DEVICE(dense);
-    TORCH_CHECK(unit_grads.dim() == 4 && unit_grads.size(3) == 3, "unit_grads must be (N,T,U+1,3)");
-    const int N = unit_grads.size(0), T = unit_grads.size(1), U = unit_grads.size(2) - 1;
-    TORCH_CHECK(dense.dim() == 4 && dense.size(0) == N && dense.size(1) == T &&
-                    dense.size(2) == U + 1, "dense must be (N,T,U+1,V)");
-    TORCH_CHECK(grad_out.dim() == 1 && grad_out.size(0) == N, "grad_out must be (N,)");
+    TORCH_CHECK(dense.dim() == 4, "dense must be (N,T,U+1,V)");
+    const int N = dense.size(0), T = dense.size(1), U = dense.size(2) - 1, V = dense.size(3);
+    TORCH_CHECK(grad_out.numel() == N || grad_out.numel() == 1, "grad_out must have N or 1 elements");
     check_lengths(ys, lx, ly, N, U);
-    const DeviceGuard device_guard(device_of(unit_grads));
-    check_rc(warpctct_dense_patch_f32(unit_grads.data_ptr<float>(), ys.data_ptr<int>(),
-                                      lx.data_ptr<int>(), ly.data_ptr<int>(),
-                                      grad_out.data_ptr<float>(), dense.data_ptr<float>(), N, T, U,
-                                      static_cast<int>(dense.size(3)), current_stream()),
-             "dense_patch");
+    const DeviceGuard device_guard(device_of(dense));
+    const int stride = (grad_out.numel() == 1 && N > 1) ? 0 : 1;
+    check_rc(warpctct_dense_patch_lattice_f32(
+                 workspace.data_ptr(), workspace.numel(), ys.data_ptr<int>(), lx.data_ptr<int>(),
+                 ly.data_ptr<int>(), grad_out.data_ptr<float>(), stride, static_cast<float>(scale),
+                 average_frames ? 1 : 0, dense.data_ptr<float>(), N, T, U, V, current_stream()),
+             "dense_patch_lattice");
 }
 
 // Backward of the fused entry: CTCTLoss.backward (warp_ctct/__init__.py:30-33)
@@ -247,9 +251,11 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> ctct_loss
 }
 
 // Fused entry for ctct_simple_loss: un-gathered f (N,T,V), g (N,U+1,V).
-// Returns (costs, den, grad_f_g, grad_g_g, grad_den); den is defined when
-// normalized, the three compact gradients when requires_grad.
-std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor>
+// Returns (costs, den, fmax, gmax, grad_f_g, grad_g_g, grad_den); den and the
+// row maxima fmax (N,T), gmax (N,U+1) are defined when normalized, the three
+// compact gradients when requires_grad.
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+           torch::Tensor, torch::Tensor>
 ctct_simple_fwd(const torch::Tensor &f, const torch::Tensor &g, const torch::Tensor &ys,
                 const torch::Tensor &lx, const torch::Tensor &ly, const bool normalized,
                 const bool requires_grad) {
@@ -268,8 +274,12 @@ ctct_simple_fwd(const torch::Tensor &f, const torch::Tensor &g, const torch::Ten
     const DeviceGuard device_guard(device_of(f));
     auto ws = make_bytes(f, warpctct_simple_workspace_bytes(N, T, U));
     auto costs = torch::empty({N}, f.options());
-    torch::Tensor den, grad_f, grad_g, grad_den;
-    if (normalized) den = torch::empty({N, T, U + 1}, f.options());
+    torch::Tensor den, fmax, gmax, grad_f, grad_g, grad_den;
+    if (normalized) {
+        den = torch::empty({N, T, U + 1}, f.options());
+        fmax = torch::empty({N, T}, f.options());
+        gmax = torch::empty({N, U + 1}, f.options());
+    }
     if (requires_grad) {
         grad_f = torch::empty({N, T, U + 1}, f.options());
         grad_g = torch::empty({N, U + 1, 3}, f.options());
@@ -278,19 +288,22 @@ ctct_simple_fwd(const torch::Tensor &f, const torch::Tensor &g, const torch::Ten
     check_rc(warpctct_simple_forward_f32(
                  f.data_ptr<float>(), g.data_ptr<float>(), ys.data_ptr<int>(), lx.data_ptr<int>(),
                  ly.data_ptr<int>(), N, T, U, V, normalized ? 1 : 0, ws.data_ptr(), ws.numel(),
-                 normalized ? den.data_ptr<float>() : nullptr, costs.data_ptr<float>(),
+                 normalized ? den.data_ptr<float>() : nullptr,
+                 normalized ? fmax.data_ptr<float>() : nullptr,
+                 normalized ? gmax.data_ptr<float>() : nullptr, costs.data_ptr<float>(),
                  requires_grad ? grad_f.data_ptr<float>() : nullptr,
                  requires_grad ? grad_g.data_ptr<float>() : nullptr,
                  (requires_grad && normalized) ? grad_den.data_ptr<float>() : nullptr,
                  current_stream()),
              "ctct_simple_fwd");
-    return std::make_tuple(costs, den, grad_f, grad_g, grad_den);
+    return std::make_tuple(costs, den, fmax, gmax, grad_f, grad_g, grad_den);
 }
 
 // Dense gradients (N,T,V) and (N,U+1,V) of the fused entry, scaled by
 // grad_out[n]; den / grad_den undefined selects the unnormalised variant.
 std::tuple<torch::Tensor, torch::Tensor> ctct_simple_bwd(
     const torch::Tensor &f, const torch::Tensor &g, const c10::optional<torch::Tensor> &den,
+    const c10::optional<torch::Tensor> &fmax, const c10::optional<torch::Tensor> &gmax,
     const torch::Tensor &grad_f_g, const torch::Tensor &grad_g_g,
     const c10::optional<torch::Tensor> &grad_den, const torch::Tensor &ys, const torch::Tensor &lx,
     const torch::Tensor &ly, const torch::Tensor &grad_out, const bool want_f, const bool want_g) {
@@ -325,6 +338,16 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_simple_bwd(
         CHECK_FLOAT(*grad_den);
         TORCH_CHECK(den->numel() == (int64_t)N * T * (U + 1) && grad_den->numel() == den->numel(),
                     "den and grad_den must be (N,T,U+1)");
+        TORCH_CHECK(fmax.has_value() && fmax->defined() && gmax.has_value() && gmax->defined(),
+                    "fmax and gmax are required with den");
+        CHECK_CONTIGUOUS(*fmax);
+        CHECK_FLOAT(*fmax);
+        CHECK_DEVICE(*fmax);
+        CHECK_CONTIGUOUS(*gmax);
+        CHECK_FLOAT(*gmax);
+        CHECK_DEVICE(*gmax);
+        TORCH_CHECK(fmax->numel() == (int64_t)N * T && gmax->numel() == (int64_t)N * (U + 1),
+                    "fmax must be (N,T), gmax (N,U+1)");
     }
     const DeviceGuard device_guard(device_of(f));
     torch::Tensor dense_f, dense_g;
@@ -332,7 +355,9 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_simple_bwd(
     if (want_g) dense_g = torch::empty_like(g);
     check_rc(warpctct_simple_backward_f32(
                  f.data_ptr<float>(), g.data_ptr<float>(),
-                 normalized ? den->data_ptr<float>() : nullptr, grad_f_g.data_ptr<float>(),
+                 normalized ? den->data_ptr<float>() : nullptr,
+                 normalized ? fmax->data_ptr<float>() : nullptr,
+                 normalized ? gmax->data_ptr<float>() : nullptr, grad_f_g.data_ptr<float>(),
                  grad_g_g.data_ptr<float>(), normalized ? grad_den->data_ptr<float>() : nullptr,
                  ys.data_ptr<int>(), lx.data_ptr<int>(), ly.data_ptr<int>(),
                  grad_out.data_ptr<float>(), N, T, U, V,
@@ -393,10 +418,11 @@ std::tuple<torch::Tensor, torch::Tensor> log_matmul_backward(
     auto res = result.contiguous();
     if (grad_input_mask[0]) grad_lhs = torch::empty({B, M, K}, lhs.options());
     if (grad_input_mask[1]) grad_rhs = torch::empty({B, K, Nn}, rhs.options());
+    auto ws = make_bytes(lhs, warpctct_logmm_workspace_bytes(B, M, Nn));
     check_rc(warpctct_logmm_bwd_f32(
                  go.data_ptr<float>(), lhs.data_ptr<float>(), lhs.stride(0), lhs.stride(1),
                  lhs.stride(2), rhs.data_ptr<float>(), rhs.stride(0), rhs.stride(1), rhs.stride(2),
-                 res.data_ptr<float>(), B, M, K, Nn,
+                 res.data_ptr<float>(), B, M, K, Nn, ws.data_ptr(), ws.numel(),
                  grad_input_mask[0] ? grad_lhs.data_ptr<float>() : nullptr, (long)M * K, (long)K, 1L,
                  grad_input_mask[1] ? grad_rhs.data_ptr<float>() : nullptr, (long)K * Nn, (long)Nn,
                  1L, current_stream()),
@@ -421,9 +447,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("dense_zero_fill", &dense_zero_fill, "Zero-filled (N,T,U+1,V) gradient tensor.",
           pybind11::arg("like"), pybind11::arg("N"), pybind11::arg("T"), pybind11::arg("U1"),
           pybind11::arg("V"));
-    m.def("dense_patch", &dense_patch, "Write the non-zero entries of the dense gradient.",
-          pybind11::arg("unit_grads"), pybind11::arg("ys"), pybind11::arg("lx"),
-          pybind11::arg("ly"), pybind11::arg("grad_out"), pybind11::arg("dense"));
+    m.def("dense_patch_lattice", &dense_patch_lattice,
+          "Write the non-zero entries of the dense gradient from the lattice workspace.",
+          pybind11::arg("workspace"), pybind11::arg("ys"), pybind11::arg("lx"),
+          pybind11::arg("ly"), pybind11::arg("grad_out"), pybind11::arg("scale"),
+          pybind11::arg("average_frames"), pybind11::arg("dense"));
     m.def("ctct_loss_simple_fwd", &ctct_loss_simple_fwd,
           "CTC-Transducer loss with the log-add joiner on gathered operands (forward).",
           pybind11::arg("f"), pybind11::arg("g"), pybind11::arg("ys"), pybind11::arg("den"),
@@ -433,7 +461,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           pybind11::arg("f"), pybind11::arg("g"), pybind11::arg("ys"), pybind11::arg("lx"),
           pybind11::arg("ly"), pybind11::arg("normalized"), pybind11::arg("requires_grad"));
     m.def("ctct_simple_bwd", &ctct_simple_bwd, "Dense gradients wrt f and g.", pybind11::arg("f"),
-          pybind11::arg("g"), pybind11::arg("den"), pybind11::arg("grad_f"),
+          pybind11::arg("g"), pybind11::arg("den"), pybind11::arg("fmax"), pybind11::arg("gmax"),
+          pybind11::arg("grad_f"),
           pybind11::arg("grad_g"), pybind11::arg("grad_den"), pybind11::arg("ys"),
           pybind11::arg("lx"), pybind11::arg("ly"), pybind11::arg("grad_out"),
           pybind11::arg("want_f"), pybind11::arg("want_g"));

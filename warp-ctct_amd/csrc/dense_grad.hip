@@ -18,13 +18,15 @@
 //    a second time) takes 370-480 us: a wave that waits for a load keeps its
 //    slot, and the fill lives off instant wave turnover;
 //  * the separate sparse pass (patch_kernel, one thread per live cell, <= 3
-//    scattered 4-byte stores) costs ~40 us; 64-byte aligned group stores
+//    scattered 4-byte stores) costs ~40 us, whether it reads ready-made unit
+//    gradients or computes them on the fly from alpha / beta; 64-byte aligned group stores
 //    instead of 4-byte ones gain little;
 //  * running the fill on a second stream next to the gather / lattice kernels
 //    is slower than running everything back to back.
 // Hence two launches on one stream: fill, then patch.
 #include "device_utils.h"
 #include "launch.h"
+#include "unit_grad.h"
 
 namespace wctct {
 
@@ -47,41 +49,78 @@ __global__ __launch_bounds__(kBlock) void zero_fill_scalar_kernel(float *__restr
     if (i < n) p[i] = 0.0f;
 }
 
-// One thread per cell (t,u) of sample blockIdx.y.  Writes (not adds) the
-// non-zero entries of row (n,t,u); columns that coincide are summed first so
-// that every element is written by exactly one store.
-__global__ __launch_bounds__(kBlock) void patch_kernel(
-    const float *__restrict__ unit_grads, const int *__restrict__ ys,
-    const int *__restrict__ lx, const int *__restrict__ ly, const float *__restrict__ grad_out,
-    float *__restrict__ dense, int T, int U, int V) {
-    const int U1 = U + 1;
-    const int n = blockIdx.y;
-    const int cell = blockIdx.x * kBlock + threadIdx.x;
-    if (cell >= T * U1) return;
-    const int t = cell / U1, u = cell - t * U1;
-    const int Tn = min(max(lx[n], 0), T);
-    const int Un = min(max(ly[n], 0), U);
-    if (t >= Tn || u > Un) return;
-    const size_t row = ((size_t)n * T + t) * U1 + u;
-    const float *g = unit_grads + row * 3;
-    const float w = grad_out ? grad_out[n] : 1.0f;
-    const int *y = ys + (size_t)n * U;
+// Per-sample weight of the upstream gradient: grad_out[n * stride] (stride 0
+// broadcasts a scalar), times `scale` (1/N for reduction='mean'), divided by
+// lx[n] when the loss was averaged over frames (warp_ctct/__init__.py:138-147
+// of the reference, differentiated).
+struct Weight {
+    const float *grad_out;   // null = ones
+    int stride;
+    float scale;
+    int average_frames;
+};
+
+__device__ __forceinline__ float sample_weight(const Weight &w, int n, int lxn) {
+    float v = w.grad_out ? w.grad_out[(size_t)n * w.stride] : 1.0f;
+    v *= w.scale;
+    if (w.average_frames) v /= (float)lxn;
+    return v;
+}
+
+// Writes (not adds) the non-zero entries of row (n,t,u) of the dense gradient:
+// columns 0, y[u-1], y[u]; columns that coincide are summed first so that
+// every element is written by exactly one store.
+__device__ __forceinline__ void patch_row(float *out, const int *y, int u, int Un, int V, float v0,
+                                          float v1, float v2) {
     const bool has1 = (u >= 1), has2 = (u < Un);
     const int c1 = has1 ? min(max(y[u - 1], 0), V - 1) : -1;
     const int c2 = has2 ? min(max(y[u], 0), V - 1) : -2;
-    float v0 = g[0] * w;
-    float v1 = has1 ? g[1] * w : 0.0f;
-    float v2 = has2 ? g[2] * w : 0.0f;
+    if (!has1) v1 = 0.0f;
+    if (!has2) v2 = 0.0f;
     if (c2 == c1) {   // y[u-1] == y[u]: both label units land in one column
         v1 += v2;
         v2 = 0.0f;
     }
     if (c1 == 0) v0 += v1;   // a label equal to the blank index
     if (c2 == 0) v0 += v2;
-    float *out = dense + row * (size_t)V;
     out[0] = v0;
     if (c1 > 0) out[c1] = v1;
     if (c2 > 0 && c2 != c1) out[c2] = v2;
+}
+
+// One thread per cell (t,u) of sample blockIdx.y; FROM_LATTICE computes the
+// unit gradients on the fly from units / alpha / beta (work-buffer layout, P
+// contexts per frame), otherwise they are read from the (N,T,U+1,3) tensor.
+template <bool FROM_LATTICE>
+__global__ __launch_bounds__(kBlock) void patch_kernel(
+    const float *__restrict__ unit_grads, const double *__restrict__ units,
+    const double *__restrict__ alphas, const double *__restrict__ betas,
+    const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
+    Weight weight, float *__restrict__ dense, int T, int U, int V, int P) {
+    const int U1 = U + 1;
+    const int n = blockIdx.y;
+    const int cell = blockIdx.x * kBlock + threadIdx.x;
+    if (cell >= T * U1) return;
+    const int t = cell / U1, u = cell - t * U1;
+    const int lxn = lx[n];
+    const int Tn = min(max(lxn, 0), T);
+    const int Un = min(max(ly[n], 0), U);
+    if (t >= Tn || u > Un) return;
+    const size_t row = ((size_t)n * T + t) * U1 + u;
+    const int *y = ys + (size_t)n * U;
+    UnitGrad g;
+    if (FROM_LATTICE) {
+        const size_t lat = (size_t)(T + 1) * P * 2;
+        g = unit_grad_cell(units + (size_t)n * T * P * 3, alphas + (size_t)n * lat,
+                           betas + (size_t)n * lat, y, t, u, Un, P);
+    } else {
+        const float *p = unit_grads + row * 3;
+        g.g0 = p[0];
+        g.g1 = p[1];
+        g.g2 = p[2];
+    }
+    const float w = sample_weight(weight, n, lxn);
+    patch_row(dense + row * (size_t)V, y, u, Un, V, g.g0 * w, g.g1 * w, g.g2 * w);
 }
 
 }  // namespace
@@ -118,8 +157,23 @@ hipError_t launch_dense_patch(const float *unit_grads, const int *ys, const int 
     const long cells = (long)T * (U + 1);
     if (cells == 0 || N == 0) return hipSuccess;
     dim3 grid((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N);
-    hipLaunchKernelGGL(patch_kernel, grid, dim3(kBlock), 0, stream, unit_grads, ys, lx, ly,
-                       grad_out, dense, T, U, V);
+    const Weight w = {grad_out, 1, 1.0f, 0};
+    hipLaunchKernelGGL(patch_kernel<false>, grid, dim3(kBlock), 0, stream, unit_grads, nullptr,
+                       nullptr, nullptr, ys, lx, ly, w, dense, T, U, V, 0);
+    return hipGetLastError();
+}
+
+hipError_t launch_dense_patch_lattice(const double *units, const double *alphas,
+                                      const double *betas, const int *ys, const int *lx,
+                                      const int *ly, const float *grad_out, int grad_out_stride,
+                                      float scale, int average_frames, float *dense, int N, int T,
+                                      int U, int V, hipStream_t stream) {
+    const long cells = (long)T * (U + 1);
+    if (cells == 0 || N == 0) return hipSuccess;
+    dim3 grid((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N);
+    const Weight w = {grad_out, grad_out_stride, scale, average_frames};
+    hipLaunchKernelGGL(patch_kernel<true>, grid, dim3(kBlock), 0, stream, nullptr, units, alphas,
+                       betas, ys, lx, ly, w, dense, T, U, V, padded_contexts(U));
     return hipGetLastError();
 }
 

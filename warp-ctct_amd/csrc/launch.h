@@ -46,6 +46,14 @@ hipError_t launch_dense_patch(const float *unit_grads, const int *ys, const int 
                               const int *ly, const float *grad_out, float *dense, int N, int T,
                               int U, int V, hipStream_t stream);
 
+// the same with the unit gradients computed on the fly from the work buffers
+// and the upstream gradient given as grad_out[n*stride] * scale (/ lx[n])
+hipError_t launch_dense_patch_lattice(const double *units, const double *alphas,
+                                      const double *betas, const int *ys, const int *lx,
+                                      const int *ly, const float *grad_out, int grad_out_stride,
+                                      float scale, int average_frames, float *dense, int N, int T,
+                                      int U, int V, hipStream_t stream);
+
 // ---- log-add joiner path -------------------------------------------------
 hipError_t launch_simple_gather_units(const float *f, const float *g, const float *den,
                                       const int *ys, const int *lx, const int *ly, double *units,
@@ -70,16 +78,23 @@ struct LogmmGrad {
     long sb, s1, s2;
 };
 
+// lmax (B,M) / rmax (B,Nn): maxima of every lhs row and rhs column over k; the
+// forward computes them, the backward takes them as inputs (launch_logmm_max
+// recomputes them when they were not kept).
 // row_len / col_len (may be null): per-batch number of valid rows of lhs and
 // index of the last valid column of rhs; outputs outside are not computed.
+hipError_t launch_logmm_max(const LogmmOperand &lhs, const LogmmOperand &rhs, float *lmax,
+                            float *rmax, int B, int M, int K, int Nn, hipStream_t stream);
 hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs, float *lmax,
                             float *rmax, float *res, int B, int M, int K, int Nn,
                             const int *row_len, const int *col_len, hipStream_t stream);
-hipError_t launch_logmm_bwd_lhs(const LogmmOperand &lhs, const LogmmOperand &rhs, const float *go,
+hipError_t launch_logmm_bwd_lhs(const LogmmOperand &lhs, const LogmmOperand &rhs,
+                                const float *lmax, const float *rmax, const float *go,
                                 const float *res, const LogmmGrad &grad, int B, int M, int K,
                                 int Nn, const int *row_len, const int *col_len,
                                 const float *batch_scale, hipStream_t stream);
-hipError_t launch_logmm_bwd_rhs(const LogmmOperand &lhs, const LogmmOperand &rhs, const float *go,
+hipError_t launch_logmm_bwd_rhs(const LogmmOperand &lhs, const LogmmOperand &rhs,
+                                const float *lmax, const float *rmax, const float *go,
                                 const float *res, const LogmmGrad &grad, int B, int M, int K,
                                 int Nn, const int *row_len, const int *col_len,
                                 const float *batch_scale, hipStream_t stream);

@@ -1,0 +1,44 @@
+// d(cost)/d(unit) of one live cell from the stored lattices; shared by the
+// kernel that writes the (N,T,U+1,3) unit-gradient tensor and by the kernel
+// that writes the non-zero entries of the dense gradient directly.
+#pragma once
+
+#include "device_utils.h"
+
+namespace wctct {
+
+struct UnitGrad {
+    float g0, g1, g2;   // blank, current label (u >= 1), next label (u < Un)
+};
+
+// g0 = -[2^(a_e+LP0+b_e-ll) + 2^(a_o+LP0+b_e-ll)]
+// g1 = - 2^(a_o+LP1+b_o-ll)
+// g2 = -[2^(a_e+LP2+b_o'-ll) + [y[u-1]!=y[u]] 2^(a_o+LP2+b_o'-ll)]       (u < Un)
+// with a_* = alpha(t,.) of context u, b_* = beta(t+1,.) of context u,
+// b_o' = beta(t+1, 2u+1) (context u+1), ll = beta(0,0), all in log2 units
+// (csrc/gather.cu:311-374 of the reference in natural coordinates).
+// alpha(t, 2u-1) of context 0 is stored as -inf, which zeroes the u >= 1 terms.
+// The exponent is summed in double and rounded once.
+// units_n / alpha_n / beta_n point at sample n; P contexts per frame.
+__device__ __forceinline__ UnitGrad unit_grad_cell(const double *units_n, const double *alpha_n,
+                                                   const double *beta_n, const int *y, int t,
+                                                   int u, int Un, int P) {
+    const double ll = beta_n[1];   // beta(0, state 0): pair {o,e} of context 0 at t = 0
+    const double2 a = *reinterpret_cast<const double2 *>(alpha_n + ((size_t)t * P + u) * 2);
+    const double2 b = *reinterpret_cast<const double2 *>(beta_n + ((size_t)(t + 1) * P + u) * 2);
+    const double *lp = units_n + ((size_t)t * P + u) * 3;
+    const double lp0 = lp[0] - ll, lp1 = lp[1] - ll;
+    UnitGrad r;
+    r.g0 = -(exp2_hw((float)(a.y + lp0 + b.y)) + exp2_hw((float)(a.x + lp0 + b.y)));
+    r.g1 = (u >= 1) ? -exp2_hw((float)(a.x + lp1 + b.x)) : 0.0f;
+    r.g2 = 0.0f;
+    if (u < Un) {
+        const double lp2 = lp[2] - ll;
+        const double bo_next = beta_n[((size_t)(t + 1) * P + u + 1) * 2];
+        r.g2 = -exp2_hw((float)(a.y + lp2 + bo_next));
+        if (u >= 1 && y[u - 1] != y[u]) r.g2 -= exp2_hw((float)(a.x + lp2 + bo_next));
+    }
+    return r;
+}
+
+}  // namespace wctct

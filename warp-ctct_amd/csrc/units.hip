@@ -17,6 +17,7 @@
 // {0, 0, -inf}, and "next" is -inf at u = ly[n]: no mass can flow there.
 #include "device_utils.h"
 #include "launch.h"
+#include "unit_grad.h"
 
 namespace wctct {
 
@@ -107,47 +108,23 @@ __global__ __launch_bounds__(kCellBlock) void simple_units_kernel(
     store_units(units, c, T, P, b, cur, nxt);
 }
 
-// g0 = -[2^(a_e+LP0+b_e-ll) + 2^(a_o+LP0+b_e-ll)]
-// g1 = - 2^(a_o+LP1+b_o-ll)
-// g2 = -[2^(a_e+LP2+b_o'-ll) + [y[u-1]!=y[u]] 2^(a_o+LP2+b_o'-ll)]       (u < U)
-// with a_* = alpha(t,.) of context u, b_* = beta(t+1,.) of context u,
-// b_o' = beta(t+1, 2u+1) (context u+1), ll = beta(0,0), all in log2 units.
-// alpha(t, 2u-1) of context 0 is stored as -inf, which zeroes the u >= 1 terms.
-// The exponent is summed in double and rounded once.
+// One thread per cell of the (N,T,U+1,3) unit-gradient tensor; zeros in padding.
 __global__ __launch_bounds__(kCellBlock) void unit_grads_kernel(
     const double *__restrict__ units, const int *__restrict__ ys, const int *__restrict__ lx,
     const int *__restrict__ ly, const double *__restrict__ alphas,
     const double *__restrict__ betas, float *__restrict__ unit_grads, int T, int U, int P) {
     const Cell c = locate_cell(lx, ly, T, U, U + 1);
     if (!c.in_range) return;
-    const int U1 = U + 1;
-    float *go = unit_grads + (((size_t)c.n * T + c.t) * U1 + c.u) * 3;
-    if (!c.live) {
-        go[0] = 0.0f;
-        go[1] = 0.0f;
-        go[2] = 0.0f;
-        return;
+    float *go = unit_grads + (((size_t)c.n * T + c.t) * (U + 1) + c.u) * 3;
+    UnitGrad g = {0.0f, 0.0f, 0.0f};
+    if (c.live) {
+        const size_t lat = (size_t)(T + 1) * P * 2;
+        g = unit_grad_cell(units + (size_t)c.n * T * P * 3, alphas + (size_t)c.n * lat,
+                           betas + (size_t)c.n * lat, ys + (size_t)c.n * U, c.t, c.u, c.Un, P);
     }
-    const size_t lat = (size_t)(T + 1) * P * 2;
-    const double *an = alphas + (size_t)c.n * lat;
-    const double *bn = betas + (size_t)c.n * lat;
-    const double ll = bn[1];   // beta(0, state 0): pair {o,e} of context 0 at t = 0
-    const double2 a = *reinterpret_cast<const double2 *>(an + ((size_t)c.t * P + c.u) * 2);
-    const double2 b = *reinterpret_cast<const double2 *>(bn + ((size_t)(c.t + 1) * P + c.u) * 2);
-    const double *lp = units + (((size_t)c.n * T + c.t) * P + c.u) * 3;
-    const double lp0 = lp[0] - ll, lp1 = lp[1] - ll, lp2 = lp[2] - ll;
-    const float g0 = -(exp2_hw((float)(a.y + lp0 + b.y)) + exp2_hw((float)(a.x + lp0 + b.y)));
-    const float g1 = -exp2_hw((float)(a.x + lp1 + b.x));
-    float g2 = 0.0f;
-    if (c.u < c.Un) {
-        const double bo_next = bn[((size_t)(c.t + 1) * P + c.u + 1) * 2];
-        g2 = -exp2_hw((float)(a.y + lp2 + bo_next));
-        const int *y = ys + (size_t)c.n * U;
-        if (c.u >= 1 && y[c.u - 1] != y[c.u]) g2 -= exp2_hw((float)(a.x + lp2 + bo_next));
-    }
-    go[0] = g0;
-    go[1] = (c.u >= 1) ? g1 : 0.0f;
-    go[2] = g2;
+    go[0] = g.g0;
+    go[1] = g.g1;
+    go[2] = g.g2;
 }
 
 inline dim3 cell_grid(int N, int T, int W) {

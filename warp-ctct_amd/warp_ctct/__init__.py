@@ -53,31 +53,51 @@ def _as_int(x: torch.Tensor) -> torch.Tensor:
     return x.to(torch.int).contiguous()
 
 
-class _CTCTLoss(torch.autograd.Function):
-    """ctct_loss on the un-gathered joint.
+def _reduce(costs, frames_lengths, reduction, average_frames):
+    # warp_ctct/__init__.py:138-147 of the reference
+    if average_frames:
+        costs = costs / frames_lengths
+    if reduction == "none" or reduction is None:
+        return costs
+    if reduction == "sum":
+        return costs.sum()
+    if reduction == "mean":
+        return costs.mean()
+    return costs
 
-    Counterpart of the reference's gather (warp_ctct/__init__.py:124-131) +
-    CTCTLoss (:20-33).  Forward runs gather, lattice and unit gradients on the
-    GPU and stashes the (N,T,U+1,3) unit gradients; backward writes the dense
-    gradient in one pass, scaled by grad_output[n]."""
+
+class _CTCTLoss(torch.autograd.Function):
+    """ctct_loss on the un-gathered joint, reduction included.
+
+    Counterpart of the reference's gather (warp_ctct/__init__.py:124-131),
+    CTCTLoss (:20-33) and the reduction (:138-147).  Forward runs gather and
+    both lattices on the GPU and keeps their workspace; backward zero-fills
+    the dense gradient at full HBM write bandwidth and then writes the <= 3
+    non-zero entries per live row, already weighted by the upstream gradient
+    and by the reduction's own factor (1/N, 1/lx[n]), so autograd launches
+    nothing else."""
 
     @staticmethod
-    def forward(ctx, joint, labels, lx, ly, requires_grad):
-        costs, unit_grads = _run("loss_forward", lambda: core.ctct_loss_joint_fwd(
+    def forward(ctx, joint, labels, lx, ly, frames_lengths, requires_grad, reduction,
+                average_frames):
+        costs, workspace = _run("loss_forward", lambda: core.ctct_loss_joint_fwd(
             joint, labels, lx, ly, requires_grad))
         if requires_grad:
-            ctx.save_for_backward(unit_grads, labels, lx, ly)
-            ctx.vocab = joint.size(3)
-        return costs
+            ctx.save_for_backward(workspace, labels, lx, ly)
+            ctx.shape = tuple(joint.shape)
+            ctx.scale = 1.0 / joint.size(0) if reduction == "mean" else 1.0
+            ctx.average_frames = bool(average_frames)
+        return _reduce(costs, frames_lengths, reduction, average_frames)
 
     @staticmethod
     def backward(ctx, grad_outputs):
-        unit_grads, labels, lx, ly = ctx.saved_tensors
+        workspace, labels, lx, ly = ctx.saved_tensors
+        n, t, u1, v = ctx.shape
         grad_outputs = grad_outputs.reshape(-1).float().contiguous()
-        n, t, u1, _ = unit_grads.shape
-        dense = _run("dense_zero_fill", lambda: core.dense_zero_fill(unit_grads, n, t, u1, ctx.vocab))
-        _run("dense_patch", lambda: core.dense_patch(unit_grads, labels, lx, ly, grad_outputs, dense))
-        return dense, None, None, None, None
+        dense = _run("dense_zero_fill", lambda: core.dense_zero_fill(grad_outputs, n, t, u1, v))
+        _run("dense_patch", lambda: core.dense_patch_lattice(
+            workspace, labels, lx, ly, grad_outputs, ctx.scale, ctx.average_frames, dense))
+        return dense, None, None, None, None, None, None, None
 
 
 class _SimpleCTCTLoss(torch.autograd.Function):
@@ -92,34 +112,22 @@ class _SimpleCTCTLoss(torch.autograd.Function):
     @staticmethod
     def forward(ctx, f, g, labels, lx, ly, normalized, track_f, track_g):
         need_grad = track_f or track_g
-        costs, den, grad_f, grad_g, grad_den = _run("simple_forward", lambda: core.ctct_simple_fwd(
-            f, g, labels, lx, ly, normalized, need_grad))
+        costs, den, fmax, gmax, grad_f, grad_g, grad_den = _run(
+            "simple_forward", lambda: core.ctct_simple_fwd(f, g, labels, lx, ly, normalized,
+                                                           need_grad))
         if need_grad:
-            ctx.save_for_backward(f, g, den, grad_f, grad_g, grad_den, labels, lx, ly)
+            ctx.save_for_backward(f, g, den, fmax, gmax, grad_f, grad_g, grad_den, labels, lx, ly)
             ctx.track = (track_f, track_g)
         return costs
 
     @staticmethod
     def backward(ctx, grad_outputs):
-        f, g, den, grad_f, grad_g, grad_den, labels, lx, ly = ctx.saved_tensors
+        f, g, den, fmax, gmax, grad_f, grad_g, grad_den, labels, lx, ly = ctx.saved_tensors
         grad_outputs = grad_outputs.reshape(-1).float().contiguous()
         dense_f, dense_g = _run("simple_backward", lambda: core.ctct_simple_bwd(
-            f, g, den, grad_f, grad_g, grad_den, labels, lx, ly, grad_outputs,
+            f, g, den, fmax, gmax, grad_f, grad_g, grad_den, labels, lx, ly, grad_outputs,
             ctx.track[0], ctx.track[1]))
         return dense_f, dense_g, None, None, None, None, None, None
-
-
-def _reduce(costs, frames_lengths, reduction, average_frames):
-    # warp_ctct/__init__.py:138-147 of the reference
-    if average_frames:
-        costs = costs / frames_lengths
-    if reduction == "none" or reduction is None:
-        return costs
-    if reduction == "sum":
-        return costs.sum()
-    if reduction == "mean":
-        return costs.mean()
-    return costs
 
 
 def ctct_loss(log_probs: torch.Tensor,
@@ -149,9 +157,9 @@ def ctct_loss(log_probs: torch.Tensor,
 
     enable_grad = log_probs.requires_grad and torch.is_grad_enabled()
     with _no_autocast():
-        costs = _CTCTLoss.apply(log_probs.float().contiguous(), _as_int(labels),
-                                _as_int(frames_lengths), _as_int(labels_lengths), enable_grad)
-    return _reduce(costs, frames_lengths, reduction, average_frames)
+        return _CTCTLoss.apply(log_probs.float().contiguous(), _as_int(labels),
+                               _as_int(frames_lengths), _as_int(labels_lengths), frames_lengths,
+                               enable_grad, reduction, bool(average_frames))
 
 
 def ctct_simple_loss(f: torch.Tensor,
