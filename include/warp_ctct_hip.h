@@ -206,23 +206,30 @@ int warpctct_simple_forward_units_f32(const float *f_g, const float *g_g, const 
                                       int U, void *workspace, size_t workspace_bytes, float *costs,
                                       float *grad_f, float *grad_g, float *grad_den, void *stream);
 
+/* Bytes of workspace for warpctct_simple_backward_f32 (the factors
+ * w*grad_den*exp(fmax+gmax-den) shared by both gradients of the den-path). */
+size_t warpctct_simple_backward_workspace_bytes(int N, int T, int U);
+
 /* Dense gradients of ctct_simple_loss: dense_f (N,T,V), dense_g (N,U+1,V),
  * every element written.  With den != NULL the den-path
  * (LogMMExp.backward, warp_ctct/__init__.py:45-52) is included:
  * dense_f[t,v] = sum_u w*grad_den[t,u]*exp(f[t,v]+g[u,v]-den[t,u]) + scatter,
  * dense_g likewise summed over t; fmax/gmax are the forward's row maxima.
- * Either dense pointer may be NULL. */
+ * Either dense pointer may be NULL; workspace is only used with den. */
 int warpctct_simple_backward_f32(const float *f, const float *g, const float *den,
                                  const float *fmax, const float *gmax, const float *grad_f,
                                  const float *grad_g, const float *grad_den,
                                  const int *ys, const int *lx, const int *ly,
                                  const float *grad_out, int N, int T, int U, int V,
-                                 float *dense_f, float *dense_g, void *stream);
+                                 void *workspace, size_t workspace_bytes, float *dense_f,
+                                 float *dense_g, void *stream);
 
 /* ---- log-semiring matmul -------------------------------------------------- */
 
 /* Bytes of workspace for warpctct_logmm_fwd_f32 / _bwd_f32 (row and column
- * maxima, by which the operands are shifted before they are exponentiated). */
+ * maxima, by which the operands are shifted before they are exponentiated, and
+ * the per-pair factors go*exp(lmax+rmax-res) that both gradients share).
+ * Offsets inside one batch of an operand must fit 31 bits (else EINVAL). */
 size_t warpctct_logmm_workspace_bytes(int B, int M, int Nn);
 
 /* res[b,i,j] = log sum_k exp(lhs[b,i,k] + rhs[b,k,j]); operands strided in

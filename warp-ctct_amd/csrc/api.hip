@@ -15,7 +15,10 @@ constexpr int kMaxGrid = 65535;
 
 inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
 
-inline int done(hipError_t e) { return e == hipSuccess ? WARPCTCT_OK : WARPCTCT_ELAUNCH; }
+inline int done(hipError_t e) {
+    if (e == hipSuccess) return WARPCTCT_OK;
+    return e == hipErrorInvalidValue ? WARPCTCT_EINVAL : WARPCTCT_ELAUNCH;
+}
 
 inline bool dims_ok(int N, int T, int U) {
     return N >= 0 && T >= 0 && U >= 0 && N <= kMaxGrid && T <= kMaxGrid &&
@@ -80,6 +83,22 @@ SimpleWorkspace carve_simple(void *base, int N, int T, int U) {
     return w;
 }
 
+// Work buffers of the log-matmul backward: pair factors (B,M,Nn) and row flags (B,M).
+struct PairWorkspace {
+    float *factors;
+    int *flags;
+    size_t bytes;
+};
+
+PairWorkspace carve_pairs(void *base, int B, int M, int Nn) {
+    PairWorkspace w;
+    const size_t fb = align256((size_t)B * M * Nn * sizeof(float));
+    w.factors = reinterpret_cast<float *>(base);
+    w.flags = reinterpret_cast<int *>(reinterpret_cast<uintptr_t>(base) + fb);
+    w.bytes = fb + align256((size_t)B * M * sizeof(int));
+    return w;
+}
+
 // lattice + unit gradients + reductions, shared by the two simple forwards
 int simple_from_units(const SimpleWorkspace &w, const int *ys, const int *lx, const int *ly, int N,
                       int T, int U, float *costs, float *grad_f, float *grad_g, float *grad_den,
@@ -121,7 +140,8 @@ int warpctct_gather_units_f32(const float *joint, const int *ys, const int *lx, 
     if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
     if (N == 0 || T == 0) return WARPCTCT_OK;
     if (!joint || !lx || !ly || !units_out || (U > 0 && !ys)) return WARPCTCT_EINVAL;
-    return done(launch_gather_units(joint, ys, lx, ly, units_out, N, T, U, V, as_stream(stream)));
+    return done(launch_gather_units(joint, ys, lx, ly, units_out, N, T, U, V, false,
+                                    as_stream(stream)));
 }
 
 int warpctct_scale_units_f32(const float *units_nat, const int *lx, const int *ly,
@@ -205,7 +225,7 @@ int warpctct_loss_lattice_f32(const float *joint, const int *ys, const int *lx, 
     const Workspace w = carve(workspace, N, T, U);
     if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
     if (T > 0) {
-        int rc = done(launch_gather_units(joint, ys, lx, ly, w.units, N, T, U, V,
+        int rc = done(launch_gather_units(joint, ys, lx, ly, w.units, N, T, U, V, true,
                                           as_stream(stream)));
         if (rc != WARPCTCT_OK) return rc;
     }
@@ -262,7 +282,7 @@ int warpctct_loss_forward_f32(const float *joint, const int *ys, const int *lx, 
     const Workspace w = carve(workspace, N, T, U);
     if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
     if (T > 0) {
-        int rc = done(launch_gather_units(joint, ys, lx, ly, w.units, N, T, U, V,
+        int rc = done(launch_gather_units(joint, ys, lx, ly, w.units, N, T, U, V, true,
                                           as_stream(stream)));
         if (rc != WARPCTCT_OK) return rc;
     }
@@ -382,34 +402,48 @@ int warpctct_simple_forward_units_f32(const float *f_g, const float *g_g, const 
                              den ? grad_den : nullptr, want_grad && T > 0, st);
 }
 
+size_t warpctct_simple_backward_workspace_bytes(int N, int T, int U) {
+    if (N < 0 || T < 0 || U < 0) return 0;
+    return carve_pairs(nullptr, N, T, U + 1).bytes;
+}
+
 int warpctct_simple_backward_f32(const float *f, const float *g, const float *den,
                                  const float *fmax, const float *gmax, const float *grad_f,
                                  const float *grad_g, const float *grad_den,
                                  const int *ys, const int *lx, const int *ly,
                                  const float *grad_out, int N, int T, int U, int V,
-                                 float *dense_f, float *dense_g, void *stream) {
+                                 void *workspace, size_t workspace_bytes, float *dense_f,
+                                 float *dense_g, void *stream) {
     if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
     if (N == 0) return WARPCTCT_OK;
     if (!lx || !ly || (U > 0 && !ys) || (dense_f && !grad_f) || (dense_g && !grad_g))
         return WARPCTCT_EINVAL;
-    if (den && (!f || !g || !grad_den || !fmax || !gmax)) return WARPCTCT_EINVAL;
+    if (den && (!f || !g || !grad_den || !fmax || !gmax || !workspace)) return WARPCTCT_EINVAL;
+    if (den && workspace_bytes < warpctct_simple_backward_workspace_bytes(N, T, U))
+        return WARPCTCT_EWORKSPACE;
     hipStream_t st = as_stream(stream);
     const int U1 = U + 1;
     if (T == 0) dense_f = nullptr;
     if (den) {
         const LogmmOperand lhs = {f, (long)T * V, (long)V, 1L};
         const LogmmOperand rhs = {g, (long)U1 * V, 1L, (long)V};
+        const PairWorkspace pw = carve_pairs(workspace, N, T, U1);
+        if (T > 0) {
+            int rc = done(launch_logmm_pair_factor(grad_den, den, fmax, gmax, grad_out, lx, ly,
+                                                   pw.factors, pw.flags, N, T, U1, st));
+            if (rc != WARPCTCT_OK) return rc;
+        }
         if (dense_f) {
             const LogmmGrad gl = {dense_f, (long)T * V, (long)V, 1L};
-            int rc = done(launch_logmm_bwd_lhs(lhs, rhs, fmax, gmax, grad_den, den, gl, N, T, V, U1, lx, ly,
-                                               grad_out, st));
+            int rc = done(launch_logmm_bwd_lhs(lhs, rhs, fmax, gmax, grad_den, den, pw.factors,
+                                               pw.flags, gl, N, T, V, U1, lx, ly, grad_out, st));
             if (rc != WARPCTCT_OK) return rc;
         }
         if (dense_g) {
             // gradient of rhs[b,k,j] = g[b,j,k] stored straight into the (N,U+1,V) layout
             const LogmmGrad gr = {dense_g, (long)U1 * V, 1L, (long)V};
-            int rc = done(launch_logmm_bwd_rhs(lhs, rhs, fmax, gmax, grad_den, den, gr, N, T, V, U1, lx, ly,
-                                               grad_out, st));
+            int rc = done(launch_logmm_bwd_rhs(lhs, rhs, fmax, gmax, grad_den, den, pw.factors,
+                                               pw.flags, gr, N, T, V, U1, lx, ly, grad_out, st));
             if (rc != WARPCTCT_OK) return rc;
         }
     } else {
@@ -428,7 +462,8 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
 
 size_t warpctct_logmm_workspace_bytes(int B, int M, int Nn) {
     if (B < 0 || M < 0 || Nn < 0) return 0;
-    return align256((size_t)B * M * sizeof(float)) + align256((size_t)B * Nn * sizeof(float));
+    return align256((size_t)B * M * sizeof(float)) + align256((size_t)B * Nn * sizeof(float)) +
+           carve_pairs(nullptr, B, M, Nn).bytes;
 }
 
 int warpctct_logmm_fwd_f32(const float *lhs, long lsb, long lsm, long lsk, const float *rhs,
@@ -464,20 +499,29 @@ int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, lo
                                             align256((size_t)B * M * sizeof(float)));
     const LogmmOperand l = {lhs, lsb, lsm, lsk};
     const LogmmOperand r = {rhs, rsb, rsk, rsn};
+    const PairWorkspace pw = carve_pairs(
+        static_cast<char *>(workspace) + align256((size_t)B * M * sizeof(float)) +
+            align256((size_t)B * Nn * sizeof(float)),
+        B, M, Nn);
     {
         int rc = done(launch_logmm_max(l, r, lmax, rmax, B, M, K, Nn, as_stream(stream)));
+        if (rc != WARPCTCT_OK) return rc;
+        rc = done(launch_logmm_pair_factor(grad_out, res, lmax, rmax, nullptr, nullptr, nullptr,
+                                           pw.factors, pw.flags, B, M, Nn, as_stream(stream)));
         if (rc != WARPCTCT_OK) return rc;
     }
     if (grad_lhs) {
         const LogmmGrad g = {grad_lhs, glsb, glsm, glsk};
-        int rc = done(launch_logmm_bwd_lhs(l, r, lmax, rmax, grad_out, res, g, B, M, K, Nn, nullptr,
-                                           nullptr, nullptr, as_stream(stream)));
+        int rc = done(launch_logmm_bwd_lhs(l, r, lmax, rmax, grad_out, res, pw.factors, pw.flags, g,
+                                           B, M, K, Nn, nullptr, nullptr, nullptr,
+                                           as_stream(stream)));
         if (rc != WARPCTCT_OK) return rc;
     }
     if (grad_rhs) {
         const LogmmGrad g = {grad_rhs, grsb, grsk, grsn};
-        int rc = done(launch_logmm_bwd_rhs(l, r, lmax, rmax, grad_out, res, g, B, M, K, Nn, nullptr,
-                                           nullptr, nullptr, as_stream(stream)));
+        int rc = done(launch_logmm_bwd_rhs(l, r, lmax, rmax, grad_out, res, pw.factors, pw.flags, g,
+                                           B, M, K, Nn, nullptr, nullptr, nullptr,
+                                           as_stream(stream)));
         if (rc != WARPCTCT_OK) return rc;
     }
     return WARPCTCT_OK;

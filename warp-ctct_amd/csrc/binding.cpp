@@ -353,6 +353,7 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_simple_bwd(
     torch::Tensor dense_f, dense_g;
     if (want_f) dense_f = torch::empty_like(f);
     if (want_g) dense_g = torch::empty_like(g);
+    auto ws = make_bytes(f, normalized ? warpctct_simple_backward_workspace_bytes(N, T, U) : 0);
     check_rc(warpctct_simple_backward_f32(
                  f.data_ptr<float>(), g.data_ptr<float>(),
                  normalized ? den->data_ptr<float>() : nullptr,
@@ -360,7 +361,7 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_simple_bwd(
                  normalized ? gmax->data_ptr<float>() : nullptr, grad_f_g.data_ptr<float>(),
                  grad_g_g.data_ptr<float>(), normalized ? grad_den->data_ptr<float>() : nullptr,
                  ys.data_ptr<int>(), lx.data_ptr<int>(), ly.data_ptr<int>(),
-                 grad_out.data_ptr<float>(), N, T, U, V,
+                 grad_out.data_ptr<float>(), N, T, U, V, ws.data_ptr(), ws.numel(),
                  want_f ? dense_f.data_ptr<float>() : nullptr,
                  want_g ? dense_g.data_ptr<float>() : nullptr, current_stream()),
              "ctct_simple_bwd");

@@ -106,6 +106,8 @@ __global__ __launch_bounds__(kBlock) void patch_kernel(
     const int Tn = min(max(lxn, 0), T);
     const int Un = min(max(ly[n], 0), U);
     if (t >= Tn || u > Un) return;
+    // outside the band the gradient is exactly zero: the fill wrote it already
+    if (FROM_LATTICE && outside_band(t, u, Tn, Un)) return;
     const size_t row = ((size_t)n * T + t) * U1 + u;
     const int *y = ys + (size_t)n * U;
     UnitGrad g;

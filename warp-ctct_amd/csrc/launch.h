@@ -27,8 +27,11 @@ struct LatticeArgs {
 int lattice_max_contexts();
 hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream);
 
+// band_only: cells outside the band of complete alignments get neutral units
+// (same costs and gradients; alpha / beta of dead cells are not the oracle's)
 hipError_t launch_gather_units(const float *joint, const int *ys, const int *lx, const int *ly,
-                               double *units, int N, int T, int U, int V, hipStream_t stream);
+                               double *units, int N, int T, int U, int V, bool band_only,
+                               hipStream_t stream);
 hipError_t launch_scale_units(const float *units_nat, const int *lx, const int *ly, double *units,
                               int N, int T, int U, hipStream_t stream);
 hipError_t launch_simple_units(const float *f_g, const float *g_g, const float *den,
@@ -88,15 +91,24 @@ hipError_t launch_logmm_max(const LogmmOperand &lhs, const LogmmOperand &rhs, fl
 hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs, float *lmax,
                             float *rmax, float *res, int B, int M, int K, int Nn,
                             const int *row_len, const int *col_len, hipStream_t stream);
+// C (B,M,Nn) and flags (B,M): the pair factors go * exp(lmax + rmax - res) that
+// both gradients share, and per row whether a pair was left to the exact pass;
+// batch_scale (may be null) multiplies grad_out per batch.
+hipError_t launch_logmm_pair_factor(const float *go, const float *res, const float *lmax,
+                                    const float *rmax, const float *batch_scale,
+                                    const int *row_len, const int *col_len, float *C, int *flags,
+                                    int B, int M, int Nn, hipStream_t stream);
 hipError_t launch_logmm_bwd_lhs(const LogmmOperand &lhs, const LogmmOperand &rhs,
                                 const float *lmax, const float *rmax, const float *go,
-                                const float *res, const LogmmGrad &grad, int B, int M, int K,
-                                int Nn, const int *row_len, const int *col_len,
-                                const float *batch_scale, hipStream_t stream);
+                                const float *res, const float *C, const int *flags,
+                                const LogmmGrad &grad, int B, int M, int K, int Nn,
+                                const int *row_len, const int *col_len, const float *batch_scale,
+                                hipStream_t stream);
 hipError_t launch_logmm_bwd_rhs(const LogmmOperand &lhs, const LogmmOperand &rhs,
                                 const float *lmax, const float *rmax, const float *go,
-                                const float *res, const LogmmGrad &grad, int B, int M, int K,
-                                int Nn, const int *row_len, const int *col_len,
-                                const float *batch_scale, hipStream_t stream);
+                                const float *res, const float *C, const int *flags,
+                                const LogmmGrad &grad, int B, int M, int K, int Nn,
+                                const int *row_len, const int *col_len, const float *batch_scale,
+                                hipStream_t stream);
 
 }  // namespace wctct

@@ -7,6 +7,17 @@
 
 namespace wctct {
 
+// Every frame consumes exactly one unit and a label needs at least one frame,
+// so a complete alignment of Tn frames and Un labels can only use cell (t,u)
+// if u labels fit into the t frames before it (t >= u) and the Un - u labels
+// still missing fit into the Tn - t frames from t on.  Outside this band alpha
+// is -inf, or every successor's beta is, whatever the units are, and the
+// gradient is exactly zero (the reference skips the same cells through its
+// shifted storage, csrc/gather.cu:333-336, :354-357).
+__device__ __forceinline__ bool outside_band(int t, int u, int Tn, int Un) {
+    return t < u || Tn - t < Un - u;
+}
+
 struct UnitGrad {
     float g0, g1, g2;   // blank, current label (u >= 1), next label (u < Un)
 };

@@ -66,10 +66,17 @@ __device__ __forceinline__ bool store_padding(double *units, const Cell &c, int 
     return true;
 }
 
+// BAND_ONLY: cells that no complete alignment can pass through (see
+// outside_band in unit_grad.h) get neutral units instead of a gather.  Costs
+// and gradients do not change: such a cell is entered with alpha = -inf or
+// left towards beta = -inf whatever its units are; only the alpha / beta values
+// of dead cells themselves differ from a full gather's.
+template <bool BAND_ONLY>
 __global__ __launch_bounds__(kCellBlock) void gather_units_kernel(
     const float *__restrict__ joint, const int *__restrict__ ys, const int *__restrict__ lx,
     const int *__restrict__ ly, double *__restrict__ units, int T, int U, int V, int P) {
-    const Cell c = locate_cell(lx, ly, T, U, P);
+    Cell c = locate_cell(lx, ly, T, U, P);
+    if (BAND_ONLY && c.live && outside_band(c.t, c.u, c.Tn, c.Un)) c.live = false;
     if (store_padding(units, c, T, P)) return;
     const float *row = joint + (((size_t)c.n * T + c.t) * (U + 1) + c.u) * (size_t)V;
     const int *y = ys + (size_t)c.n * U;
@@ -135,10 +142,16 @@ inline dim3 cell_grid(int N, int T, int W) {
 }  // namespace
 
 hipError_t launch_gather_units(const float *joint, const int *ys, const int *lx, const int *ly,
-                               double *units, int N, int T, int U, int V, hipStream_t stream) {
+                               double *units, int N, int T, int U, int V, bool band_only,
+                               hipStream_t stream) {
     const int P = padded_contexts(U);
-    hipLaunchKernelGGL(gather_units_kernel, cell_grid(N, T, P), dim3(kCellBlock), 0, stream,
-                       joint, ys, lx, ly, units, T, U, V, P);
+    if (band_only) {
+        hipLaunchKernelGGL(gather_units_kernel<true>, cell_grid(N, T, P), dim3(kCellBlock), 0,
+                           stream, joint, ys, lx, ly, units, T, U, V, P);
+    } else {
+        hipLaunchKernelGGL(gather_units_kernel<false>, cell_grid(N, T, P), dim3(kCellBlock), 0,
+                           stream, joint, ys, lx, ly, units, T, U, V, P);
+    }
     return hipGetLastError();
 }
 
