@@ -189,15 +189,17 @@ size_t warpctct_simple_workspace_bytes(int N, int T, int U);
 /* ctct_simple_loss forward on f (N,T,V), g (N,U+1,V): den (if normalized),
  * units, lattice, unit gradients and their reductions.  Replaces
  * warp_ctct/__init__.py:195-225 + _C.ctct_loss_simple_fwd
- * (csrc/binding.cpp:103-222).  When normalized != 0, den (N,T,U+1; only
- * t<lx[n], u<=ly[n] is written), fmax (N,T) = max_v f and gmax (N,U+1) =
- * max_v g are outputs (the backward needs them); otherwise they are ignored.
+ * (csrc/binding.cpp:103-222).  When normalized != 0, these are outputs that
+ * the backward needs (otherwise they are ignored): den (N,T,U+1; only
+ * t<lx[n], u<=ly[n] is written), fmax (N,T) = max_v f, gmax (N,U+1) = max_v g,
+ * fexp (N,T,Vp) = exp(f - fmax) and gexp (N,U+1,Vp) = exp(g - gmax) with
+ * Vp = warpctct_logmm_padded_reduction(V), zero in the padding.
  * grad_f/grad_g/grad_den may all be NULL (no-grad mode). */
 int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, const int *lx,
                                 const int *ly, int N, int T, int U, int V, int normalized,
                                 void *workspace, size_t workspace_bytes, float *den, float *fmax,
-                                float *gmax, float *costs, float *grad_f, float *grad_g,
-                                float *grad_den, void *stream);
+                                float *gmax, float *fexp, float *gexp, float *costs,
+                                float *grad_f, float *grad_g, float *grad_den, void *stream);
 
 /* _C.ctct_loss_simple_fwd proper: f_g (N,T,U+1), g_g (N,U+1,3) already
  * gathered, den (N,T,U+1) or NULL (unnormalised, csrc/simple_unnorm.cu). */
@@ -214,10 +216,11 @@ size_t warpctct_simple_backward_workspace_bytes(int N, int T, int U);
  * every element written.  With den != NULL the den-path
  * (LogMMExp.backward, warp_ctct/__init__.py:45-52) is included:
  * dense_f[t,v] = sum_u w*grad_den[t,u]*exp(f[t,v]+g[u,v]-den[t,u]) + scatter,
- * dense_g likewise summed over t; fmax/gmax are the forward's row maxima.
+ * dense_g likewise summed over t; fmax/gmax/fexp/gexp are the forward's.
  * Either dense pointer may be NULL; workspace is only used with den. */
 int warpctct_simple_backward_f32(const float *f, const float *g, const float *den,
-                                 const float *fmax, const float *gmax, const float *grad_f,
+                                 const float *fmax, const float *gmax, const float *fexp,
+                                 const float *gexp, const float *grad_f,
                                  const float *grad_g, const float *grad_den,
                                  const int *ys, const int *lx, const int *ly,
                                  const float *grad_out, int N, int T, int U, int V,
@@ -226,11 +229,16 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
 
 /* ---- log-semiring matmul -------------------------------------------------- */
 
-/* Bytes of workspace for warpctct_logmm_fwd_f32 / _bwd_f32 (row and column
- * maxima, by which the operands are shifted before they are exponentiated, and
- * the per-pair factors go*exp(lmax+rmax-res) that both gradients share).
- * Offsets inside one batch of an operand must fit 31 bits (else EINVAL). */
-size_t warpctct_logmm_workspace_bytes(int B, int M, int Nn);
+/* Row length of the shifted exponentials: K rounded up to the chunk (32) of
+ * the matrix-core GEMMs. */
+int warpctct_logmm_padded_reduction(int K);
+
+/* Bytes of workspace for warpctct_logmm_fwd_f32 / _bwd_f32: row and column
+ * maxima, the operands shifted by them and exponentiated ((B,M,Kp) and
+ * (B,Nn,Kp) floats), and the per-pair factors go*exp(lmax+rmax-res) that both
+ * gradients share.  Offsets inside one batch of an operand must fit 31 bits
+ * (else EINVAL). */
+size_t warpctct_logmm_workspace_bytes(int B, int M, int K, int Nn);
 
 /* res[b,i,j] = log sum_k exp(lhs[b,i,k] + rhs[b,k,j]); operands strided in
  * elements (lhs[b,i,k] at lhs[b*lsb + i*lsm + k*lsk], rhs[b,k,j] at

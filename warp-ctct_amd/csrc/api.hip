@@ -99,6 +99,31 @@ PairWorkspace carve_pairs(void *base, int B, int M, int Nn) {
     return w;
 }
 
+// Work buffers of the standalone log-matmul: maxima, shifted exponentials, pairs.
+struct LogmmWorkspace {
+    LogmmShifted sh;
+    PairWorkspace pw;
+    size_t bytes;
+};
+
+LogmmWorkspace carve_logmm(void *base, int B, int M, int K, int Nn) {
+    LogmmWorkspace w;
+    const size_t Kp = (size_t)logmm_padded_reduction(K);
+    uintptr_t p = reinterpret_cast<uintptr_t>(base);
+    const uintptr_t p0 = p;
+    w.sh.lmax = reinterpret_cast<float *>(p);
+    p += align256((size_t)B * M * sizeof(float));
+    w.sh.rmax = reinterpret_cast<float *>(p);
+    p += align256((size_t)B * Nn * sizeof(float));
+    w.sh.El = reinterpret_cast<float *>(p);
+    p += align256((size_t)B * M * Kp * sizeof(float));
+    w.sh.Er = reinterpret_cast<float *>(p);
+    p += align256((size_t)B * Nn * Kp * sizeof(float));
+    w.pw = carve_pairs(reinterpret_cast<void *>(p), B, M, Nn);
+    w.bytes = (p - p0) + w.pw.bytes;
+    return w;
+}
+
 // lattice + unit gradients + reductions, shared by the two simple forwards
 int simple_from_units(const SimpleWorkspace &w, const int *ys, const int *lx, const int *ly, int N,
                       int T, int U, float *costs, float *grad_f, float *grad_g, float *grad_den,
@@ -353,15 +378,15 @@ size_t warpctct_simple_workspace_bytes(int N, int T, int U) {
 int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, const int *lx,
                                 const int *ly, int N, int T, int U, int V, int normalized,
                                 void *workspace, size_t workspace_bytes, float *den, float *fmax,
-                                float *gmax, float *costs, float *grad_f, float *grad_g,
-                                float *grad_den, void *stream) {
+                                float *gmax, float *fexp, float *gexp, float *costs,
+                                float *grad_f, float *grad_g, float *grad_den, void *stream) {
     if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
     if (N == 0) return WARPCTCT_OK;
     const bool want_grad = grad_f || grad_g || grad_den;
     if (!g || !lx || !ly || !costs || !workspace || (T > 0 && !f) || (U > 0 && !ys))
         return WARPCTCT_EINVAL;
     if (want_grad && (!grad_f || !grad_g || (normalized && !grad_den))) return WARPCTCT_EINVAL;
-    if (normalized && T > 0 && (!den || !fmax || !gmax)) return WARPCTCT_EINVAL;
+    if (normalized && T > 0 && (!den || !fmax || !gmax || !fexp || !gexp)) return WARPCTCT_EINVAL;
     const SimpleWorkspace w = carve_simple(workspace, N, T, U);
     if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
     hipStream_t st = as_stream(stream);
@@ -370,7 +395,10 @@ int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, c
             // den[n,t,u] = logsumexp_v(f[n,t,v] + g[n,u,v]):  lhs = f, rhs[b,k,j] = g[b,j,k]
             const LogmmOperand lhs = {f, (long)T * V, (long)V, 1L};
             const LogmmOperand rhs = {g, (long)(U + 1) * V, 1L, (long)V};
-            int rc = done(launch_logmm_fwd(lhs, rhs, fmax, gmax, den, N, T, V, U + 1, lx, ly, st));
+            const LogmmShifted sh = {fmax, gmax, fexp, gexp};
+            int rc = done(launch_logmm_shift_exp(lhs, rhs, sh, N, T, V, U + 1, lx, ly, st));
+            if (rc != WARPCTCT_OK) return rc;
+            rc = done(launch_logmm_fwd(lhs, rhs, sh, den, N, T, V, U + 1, lx, ly, st));
             if (rc != WARPCTCT_OK) return rc;
         }
         int rc = done(launch_simple_gather_units(f, g, normalized ? den : nullptr, ys, lx, ly,
@@ -408,7 +436,8 @@ size_t warpctct_simple_backward_workspace_bytes(int N, int T, int U) {
 }
 
 int warpctct_simple_backward_f32(const float *f, const float *g, const float *den,
-                                 const float *fmax, const float *gmax, const float *grad_f,
+                                 const float *fmax, const float *gmax, const float *fexp,
+                                 const float *gexp, const float *grad_f,
                                  const float *grad_g, const float *grad_den,
                                  const int *ys, const int *lx, const int *ly,
                                  const float *grad_out, int N, int T, int U, int V,
@@ -418,7 +447,8 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
     if (N == 0) return WARPCTCT_OK;
     if (!lx || !ly || (U > 0 && !ys) || (dense_f && !grad_f) || (dense_g && !grad_g))
         return WARPCTCT_EINVAL;
-    if (den && (!f || !g || !grad_den || !fmax || !gmax || !workspace)) return WARPCTCT_EINVAL;
+    if (den && (!f || !g || !grad_den || !fmax || !gmax || !fexp || !gexp || !workspace))
+        return WARPCTCT_EINVAL;
     if (den && workspace_bytes < warpctct_simple_backward_workspace_bytes(N, T, U))
         return WARPCTCT_EWORKSPACE;
     hipStream_t st = as_stream(stream);
@@ -428,6 +458,8 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
         const LogmmOperand lhs = {f, (long)T * V, (long)V, 1L};
         const LogmmOperand rhs = {g, (long)U1 * V, 1L, (long)V};
         const PairWorkspace pw = carve_pairs(workspace, N, T, U1);
+        const LogmmShifted sh = {const_cast<float *>(fmax), const_cast<float *>(gmax),
+                                 const_cast<float *>(fexp), const_cast<float *>(gexp)};
         if (T > 0) {
             int rc = done(launch_logmm_pair_factor(grad_den, den, fmax, gmax, grad_out, lx, ly,
                                                    pw.factors, pw.flags, N, T, U1, st));
@@ -435,15 +467,15 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
         }
         if (dense_f) {
             const LogmmGrad gl = {dense_f, (long)T * V, (long)V, 1L};
-            int rc = done(launch_logmm_bwd_lhs(lhs, rhs, fmax, gmax, grad_den, den, pw.factors,
-                                               pw.flags, gl, N, T, V, U1, lx, ly, grad_out, st));
+            int rc = done(launch_logmm_bwd_lhs(lhs, rhs, sh, grad_den, den, pw.factors, pw.flags,
+                                               gl, N, T, V, U1, lx, ly, grad_out, st));
             if (rc != WARPCTCT_OK) return rc;
         }
         if (dense_g) {
             // gradient of rhs[b,k,j] = g[b,j,k] stored straight into the (N,U+1,V) layout
             const LogmmGrad gr = {dense_g, (long)U1 * V, 1L, (long)V};
-            int rc = done(launch_logmm_bwd_rhs(lhs, rhs, fmax, gmax, grad_den, den, pw.factors,
-                                               pw.flags, gr, N, T, V, U1, lx, ly, grad_out, st));
+            int rc = done(launch_logmm_bwd_rhs(lhs, rhs, sh, grad_den, den, pw.factors, pw.flags,
+                                               gr, N, T, V, U1, lx, ly, grad_out, st));
             if (rc != WARPCTCT_OK) return rc;
         }
     } else {
@@ -460,10 +492,11 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
                                       U, V, st));
 }
 
-size_t warpctct_logmm_workspace_bytes(int B, int M, int Nn) {
-    if (B < 0 || M < 0 || Nn < 0) return 0;
-    return align256((size_t)B * M * sizeof(float)) + align256((size_t)B * Nn * sizeof(float)) +
-           carve_pairs(nullptr, B, M, Nn).bytes;
+int warpctct_logmm_padded_reduction(int K) { return K < 0 ? 0 : logmm_padded_reduction(K); }
+
+size_t warpctct_logmm_workspace_bytes(int B, int M, int K, int Nn) {
+    if (B < 0 || M < 0 || K < 0 || Nn < 0) return 0;
+    return carve_logmm(nullptr, B, M, K, Nn).bytes;
 }
 
 int warpctct_logmm_fwd_f32(const float *lhs, long lsb, long lsm, long lsk, const float *rhs,
@@ -473,13 +506,14 @@ int warpctct_logmm_fwd_f32(const float *lhs, long lsb, long lsm, long lsk, const
         return WARPCTCT_EINVAL;
     if (B == 0 || M == 0 || Nn == 0) return WARPCTCT_OK;
     if (!res || !workspace || (K > 0 && (!lhs || !rhs))) return WARPCTCT_EINVAL;
-    if (workspace_bytes < warpctct_logmm_workspace_bytes(B, M, Nn)) return WARPCTCT_EWORKSPACE;
-    float *lmax = static_cast<float *>(workspace);
-    float *rmax = reinterpret_cast<float *>(static_cast<char *>(workspace) +
-                                            align256((size_t)B * M * sizeof(float)));
+    const LogmmWorkspace w = carve_logmm(workspace, B, M, K, Nn);
+    if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
     const LogmmOperand l = {lhs, lsb, lsm, lsk};
     const LogmmOperand r = {rhs, rsb, rsk, rsn};
-    return done(launch_logmm_fwd(l, r, lmax, rmax, res, B, M, K, Nn, nullptr, nullptr,
+    int rc = done(launch_logmm_shift_exp(l, r, w.sh, B, M, K, Nn, nullptr, nullptr,
+                                         as_stream(stream)));
+    if (rc != WARPCTCT_OK) return rc;
+    return done(launch_logmm_fwd(l, r, w.sh, res, B, M, K, Nn, nullptr, nullptr,
                                  as_stream(stream)));
 }
 
@@ -493,35 +527,28 @@ int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, lo
     if (B == 0 || K == 0) return WARPCTCT_OK;
     if (!lhs || !rhs || !workspace || ((M > 0 && Nn > 0) && (!grad_out || !res)))
         return WARPCTCT_EINVAL;
-    if (workspace_bytes < warpctct_logmm_workspace_bytes(B, M, Nn)) return WARPCTCT_EWORKSPACE;
-    float *lmax = static_cast<float *>(workspace);
-    float *rmax = reinterpret_cast<float *>(static_cast<char *>(workspace) +
-                                            align256((size_t)B * M * sizeof(float)));
+    const LogmmWorkspace w = carve_logmm(workspace, B, M, K, Nn);
+    if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
     const LogmmOperand l = {lhs, lsb, lsm, lsk};
     const LogmmOperand r = {rhs, rsb, rsk, rsn};
-    const PairWorkspace pw = carve_pairs(
-        static_cast<char *>(workspace) + align256((size_t)B * M * sizeof(float)) +
-            align256((size_t)B * Nn * sizeof(float)),
-        B, M, Nn);
+    hipStream_t st = as_stream(stream);
     {
-        int rc = done(launch_logmm_max(l, r, lmax, rmax, B, M, K, Nn, as_stream(stream)));
+        int rc = done(launch_logmm_shift_exp(l, r, w.sh, B, M, K, Nn, nullptr, nullptr, st));
         if (rc != WARPCTCT_OK) return rc;
-        rc = done(launch_logmm_pair_factor(grad_out, res, lmax, rmax, nullptr, nullptr, nullptr,
-                                           pw.factors, pw.flags, B, M, Nn, as_stream(stream)));
+        rc = done(launch_logmm_pair_factor(grad_out, res, w.sh.lmax, w.sh.rmax, nullptr, nullptr,
+                                           nullptr, w.pw.factors, w.pw.flags, B, M, Nn, st));
         if (rc != WARPCTCT_OK) return rc;
     }
     if (grad_lhs) {
         const LogmmGrad g = {grad_lhs, glsb, glsm, glsk};
-        int rc = done(launch_logmm_bwd_lhs(l, r, lmax, rmax, grad_out, res, pw.factors, pw.flags, g,
-                                           B, M, K, Nn, nullptr, nullptr, nullptr,
-                                           as_stream(stream)));
+        int rc = done(launch_logmm_bwd_lhs(l, r, w.sh, grad_out, res, w.pw.factors, w.pw.flags, g,
+                                           B, M, K, Nn, nullptr, nullptr, nullptr, st));
         if (rc != WARPCTCT_OK) return rc;
     }
     if (grad_rhs) {
         const LogmmGrad g = {grad_rhs, grsb, grsk, grsn};
-        int rc = done(launch_logmm_bwd_rhs(l, r, lmax, rmax, grad_out, res, pw.factors, pw.flags, g,
-                                           B, M, K, Nn, nullptr, nullptr, nullptr,
-                                           as_stream(stream)));
+        int rc = done(launch_logmm_bwd_rhs(l, r, w.sh, grad_out, res, w.pw.factors, w.pw.flags, g,
+                                           B, M, K, Nn, nullptr, nullptr, nullptr, st));
         if (rc != WARPCTCT_OK) return rc;
     }
     return WARPCTCT_OK;

@@ -251,11 +251,13 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> ctct_loss
 }
 
 // Fused entry for ctct_simple_loss: un-gathered f (N,T,V), g (N,U+1,V).
-// Returns (costs, den, fmax, gmax, grad_f_g, grad_g_g, grad_den); den and the
-// row maxima fmax (N,T), gmax (N,U+1) are defined when normalized, the three
-// compact gradients when requires_grad.
-std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
-           torch::Tensor, torch::Tensor>
+// Returns (costs, den, shifted, grad_f_g, grad_g_g, grad_den).  When normalized,
+// den is defined and shifted = [fmax (N,T), gmax (N,U+1), fexp (N,T,Vp),
+// gexp (N,U+1,Vp)], the row maxima of f and g and the operands shifted by them
+// and exponentiated, which the backward reuses; otherwise shifted is empty.
+// The three compact gradients are defined when requires_grad.
+std::tuple<torch::Tensor, torch::Tensor, std::vector<torch::Tensor>, torch::Tensor, torch::Tensor,
+           torch::Tensor>
 ctct_simple_fwd(const torch::Tensor &f, const torch::Tensor &g, const torch::Tensor &ys,
                 const torch::Tensor &lx, const torch::Tensor &ly, const bool normalized,
                 const bool requires_grad) {
@@ -274,11 +276,16 @@ ctct_simple_fwd(const torch::Tensor &f, const torch::Tensor &g, const torch::Ten
     const DeviceGuard device_guard(device_of(f));
     auto ws = make_bytes(f, warpctct_simple_workspace_bytes(N, T, U));
     auto costs = torch::empty({N}, f.options());
-    torch::Tensor den, fmax, gmax, grad_f, grad_g, grad_den;
+    torch::Tensor den, fmax, gmax, fexp, gexp, grad_f, grad_g, grad_den;
+    std::vector<torch::Tensor> shifted;
     if (normalized) {
+        const int Vp = warpctct_logmm_padded_reduction(V);
         den = torch::empty({N, T, U + 1}, f.options());
         fmax = torch::empty({N, T}, f.options());
         gmax = torch::empty({N, U + 1}, f.options());
+        fexp = torch::empty({N, T, Vp}, f.options());
+        gexp = torch::empty({N, U + 1, Vp}, f.options());
+        shifted = {fmax, gmax, fexp, gexp};
     }
     if (requires_grad) {
         grad_f = torch::empty({N, T, U + 1}, f.options());
@@ -290,20 +297,22 @@ ctct_simple_fwd(const torch::Tensor &f, const torch::Tensor &g, const torch::Ten
                  ly.data_ptr<int>(), N, T, U, V, normalized ? 1 : 0, ws.data_ptr(), ws.numel(),
                  normalized ? den.data_ptr<float>() : nullptr,
                  normalized ? fmax.data_ptr<float>() : nullptr,
-                 normalized ? gmax.data_ptr<float>() : nullptr, costs.data_ptr<float>(),
+                 normalized ? gmax.data_ptr<float>() : nullptr,
+                 normalized ? fexp.data_ptr<float>() : nullptr,
+                 normalized ? gexp.data_ptr<float>() : nullptr, costs.data_ptr<float>(),
                  requires_grad ? grad_f.data_ptr<float>() : nullptr,
                  requires_grad ? grad_g.data_ptr<float>() : nullptr,
                  (requires_grad && normalized) ? grad_den.data_ptr<float>() : nullptr,
                  current_stream()),
              "ctct_simple_fwd");
-    return std::make_tuple(costs, den, fmax, gmax, grad_f, grad_g, grad_den);
+    return std::make_tuple(costs, den, shifted, grad_f, grad_g, grad_den);
 }
 
 // Dense gradients (N,T,V) and (N,U+1,V) of the fused entry, scaled by
 // grad_out[n]; den / grad_den undefined selects the unnormalised variant.
 std::tuple<torch::Tensor, torch::Tensor> ctct_simple_bwd(
     const torch::Tensor &f, const torch::Tensor &g, const c10::optional<torch::Tensor> &den,
-    const c10::optional<torch::Tensor> &fmax, const c10::optional<torch::Tensor> &gmax,
+    const std::vector<torch::Tensor> &shifted,
     const torch::Tensor &grad_f_g, const torch::Tensor &grad_g_g,
     const c10::optional<torch::Tensor> &grad_den, const torch::Tensor &ys, const torch::Tensor &lx,
     const torch::Tensor &ly, const torch::Tensor &grad_out, const bool want_f, const bool want_g) {
@@ -338,16 +347,19 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_simple_bwd(
         CHECK_FLOAT(*grad_den);
         TORCH_CHECK(den->numel() == (int64_t)N * T * (U + 1) && grad_den->numel() == den->numel(),
                     "den and grad_den must be (N,T,U+1)");
-        TORCH_CHECK(fmax.has_value() && fmax->defined() && gmax.has_value() && gmax->defined(),
-                    "fmax and gmax are required with den");
-        CHECK_CONTIGUOUS(*fmax);
-        CHECK_FLOAT(*fmax);
-        CHECK_DEVICE(*fmax);
-        CHECK_CONTIGUOUS(*gmax);
-        CHECK_FLOAT(*gmax);
-        CHECK_DEVICE(*gmax);
-        TORCH_CHECK(fmax->numel() == (int64_t)N * T && gmax->numel() == (int64_t)N * (U + 1),
+        const int Vp = warpctct_logmm_padded_reduction(V);
+        TORCH_CHECK(shifted.size() == 4, "shifted = [fmax, gmax, fexp, gexp] is required with den");
+        for (const auto &t : shifted) {
+            CHECK_CONTIGUOUS(t);
+            CHECK_FLOAT(t);
+            CHECK_DEVICE(t);
+        }
+        TORCH_CHECK(shifted[0].numel() == (int64_t)N * T &&
+                        shifted[1].numel() == (int64_t)N * (U + 1),
                     "fmax must be (N,T), gmax (N,U+1)");
+        TORCH_CHECK(shifted[2].numel() == (int64_t)N * T * Vp &&
+                        shifted[3].numel() == (int64_t)N * (U + 1) * Vp,
+                    "fexp must be (N,T,Vp), gexp (N,U+1,Vp)");
     }
     const DeviceGuard device_guard(device_of(f));
     torch::Tensor dense_f, dense_g;
@@ -357,8 +369,10 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_simple_bwd(
     check_rc(warpctct_simple_backward_f32(
                  f.data_ptr<float>(), g.data_ptr<float>(),
                  normalized ? den->data_ptr<float>() : nullptr,
-                 normalized ? fmax->data_ptr<float>() : nullptr,
-                 normalized ? gmax->data_ptr<float>() : nullptr, grad_f_g.data_ptr<float>(),
+                 normalized ? shifted[0].data_ptr<float>() : nullptr,
+                 normalized ? shifted[1].data_ptr<float>() : nullptr,
+                 normalized ? shifted[2].data_ptr<float>() : nullptr,
+                 normalized ? shifted[3].data_ptr<float>() : nullptr, grad_f_g.data_ptr<float>(),
                  grad_g_g.data_ptr<float>(), normalized ? grad_den->data_ptr<float>() : nullptr,
                  ys.data_ptr<int>(), lx.data_ptr<int>(), ly.data_ptr<int>(),
                  grad_out.data_ptr<float>(), N, T, U, V, ws.data_ptr(), ws.numel(),
@@ -385,7 +399,7 @@ torch::Tensor log_matmul(const torch::Tensor &self, const torch::Tensor &other) 
     const DeviceGuard device_guard(device_of(self));
     const int B = self.size(0), M = self.size(1), K = self.size(2), Nn = other.size(2);
     auto out = torch::empty({B, M, Nn}, self.options());
-    auto ws = make_bytes(self, warpctct_logmm_workspace_bytes(B, M, Nn));
+    auto ws = make_bytes(self, warpctct_logmm_workspace_bytes(B, M, K, Nn));
     check_rc(warpctct_logmm_fwd_f32(self.data_ptr<float>(), self.stride(0), self.stride(1),
                                     self.stride(2), other.data_ptr<float>(),
                                     batch_stride(other, B), other.stride(1), other.stride(2), B, M,
@@ -419,7 +433,7 @@ std::tuple<torch::Tensor, torch::Tensor> log_matmul_backward(
     auto res = result.contiguous();
     if (grad_input_mask[0]) grad_lhs = torch::empty({B, M, K}, lhs.options());
     if (grad_input_mask[1]) grad_rhs = torch::empty({B, K, Nn}, rhs.options());
-    auto ws = make_bytes(lhs, warpctct_logmm_workspace_bytes(B, M, Nn));
+    auto ws = make_bytes(lhs, warpctct_logmm_workspace_bytes(B, M, K, Nn));
     check_rc(warpctct_logmm_bwd_f32(
                  go.data_ptr<float>(), lhs.data_ptr<float>(), lhs.stride(0), lhs.stride(1),
                  lhs.stride(2), rhs.data_ptr<float>(), rhs.stride(0), rhs.stride(1), rhs.stride(2),
@@ -462,7 +476,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           pybind11::arg("f"), pybind11::arg("g"), pybind11::arg("ys"), pybind11::arg("lx"),
           pybind11::arg("ly"), pybind11::arg("normalized"), pybind11::arg("requires_grad"));
     m.def("ctct_simple_bwd", &ctct_simple_bwd, "Dense gradients wrt f and g.", pybind11::arg("f"),
-          pybind11::arg("g"), pybind11::arg("den"), pybind11::arg("fmax"), pybind11::arg("gmax"),
+          pybind11::arg("g"), pybind11::arg("den"), pybind11::arg("shifted"),
           pybind11::arg("grad_f"),
           pybind11::arg("grad_g"), pybind11::arg("grad_den"), pybind11::arg("ys"),
           pybind11::arg("lx"), pybind11::arg("ly"), pybind11::arg("grad_out"),

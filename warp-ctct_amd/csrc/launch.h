@@ -81,15 +81,24 @@ struct LogmmGrad {
     long sb, s1, s2;
 };
 
-// lmax (B,M) / rmax (B,Nn): maxima of every lhs row and rhs column over k; the
-// forward computes them, the backward takes them as inputs (launch_logmm_max
-// recomputes them when they were not kept).
+// The reduction index of the shifted exponentials is padded to a multiple of
+// the GEMM chunk (32) with zeros.
+inline int logmm_padded_reduction(int K) { return (K + 31) / 32 * 32; }
+
+// Shifted exponentials of both operands and the shifts:
+//   lmax (B,M) = max_k lhs, El (B,M,Kp) = exp(lhs - lmax);
+//   rmax (B,Nn) = max_k rhs, Er (B,Nn,Kp) = exp(rhs - rmax) with k contiguous.
+struct LogmmShifted {
+    float *lmax, *rmax, *El, *Er;
+};
+
 // row_len / col_len (may be null): per-batch number of valid rows of lhs and
 // index of the last valid column of rhs; outputs outside are not computed.
-hipError_t launch_logmm_max(const LogmmOperand &lhs, const LogmmOperand &rhs, float *lmax,
-                            float *rmax, int B, int M, int K, int Nn, hipStream_t stream);
-hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs, float *lmax,
-                            float *rmax, float *res, int B, int M, int K, int Nn,
+hipError_t launch_logmm_shift_exp(const LogmmOperand &lhs, const LogmmOperand &rhs,
+                                  const LogmmShifted &sh, int B, int M, int K, int Nn,
+                                  const int *row_len, const int *col_len, hipStream_t stream);
+hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
+                            const LogmmShifted &sh, float *res, int B, int M, int K, int Nn,
                             const int *row_len, const int *col_len, hipStream_t stream);
 // C (B,M,Nn) and flags (B,M): the pair factors go * exp(lmax + rmax - res) that
 // both gradients share, and per row whether a pair was left to the exact pass;
@@ -99,16 +108,14 @@ hipError_t launch_logmm_pair_factor(const float *go, const float *res, const flo
                                     const int *row_len, const int *col_len, float *C, int *flags,
                                     int B, int M, int Nn, hipStream_t stream);
 hipError_t launch_logmm_bwd_lhs(const LogmmOperand &lhs, const LogmmOperand &rhs,
-                                const float *lmax, const float *rmax, const float *go,
-                                const float *res, const float *C, const int *flags,
-                                const LogmmGrad &grad, int B, int M, int K, int Nn,
-                                const int *row_len, const int *col_len, const float *batch_scale,
-                                hipStream_t stream);
+                                const LogmmShifted &sh, const float *go, const float *res,
+                                const float *C, const int *flags, const LogmmGrad &grad, int B,
+                                int M, int K, int Nn, const int *row_len, const int *col_len,
+                                const float *batch_scale, hipStream_t stream);
 hipError_t launch_logmm_bwd_rhs(const LogmmOperand &lhs, const LogmmOperand &rhs,
-                                const float *lmax, const float *rmax, const float *go,
-                                const float *res, const float *C, const int *flags,
-                                const LogmmGrad &grad, int B, int M, int K, int Nn,
-                                const int *row_len, const int *col_len, const float *batch_scale,
-                                hipStream_t stream);
+                                const LogmmShifted &sh, const float *go, const float *res,
+                                const float *C, const int *flags, const LogmmGrad &grad, int B,
+                                int M, int K, int Nn, const int *row_len, const int *col_len,
+                                const float *batch_scale, hipStream_t stream);
 
 }  // namespace wctct

@@ -10,22 +10,24 @@
 //
 // The reference launches one block per output element and evaluates two
 // exponentials per term.  Here every operand row is shifted by its own
-// maximum m and exponentiated ONCE while it is staged in LDS,
-//     E_l[i,k] = exp(lhs[i,k] - ml[i]),   E_r[k,j] = exp(rhs[k,j] - mr[j]),
-// all in [0,1], and the contraction becomes a plain fp32 GEMM on the matrix
-// cores (v_mfma_f32_16x16x4_f32): a workgroup owns a tile of the output, each
-// of its wavefronts RB x CB blocks of 16x16; operands are read from LDS; the
-// next chunk of the reduction is fetched into registers while the current one
-// is multiplied (two LDS buffers, one barrier per chunk).
-//     res[i,j]      = ml[i] + mr[j] + log(sum_k E_l[i,k] E_r[k,j])
-//     grad_lhs[i,k] = E_l[i,k] * sum_j C[i,j] E_r[k,j],
+// maximum m and exponentiated ONCE, by a kernel that reads the operand and
+// writes
+//     E_l[i,k] = exp(lhs[i,k] - ml[i]),   E_r[j,k] = exp(rhs[k,j] - mr[j]),
+// all in [0,1], k contiguous, rows padded with zeros to a multiple of 32.
+// Forward and both gradients are then plain fp32 GEMMs on the matrix cores
+// (v_mfma_f32_16x16x4_f32) whose operands are copied global -> LDS as 16-byte
+// vectors while the previous chunk is multiplied:
+//     res[i,j]      = ml[i] + mr[j] + log(sum_k E_l[i,k] E_r[j,k])
+//     grad_lhs[i,k] = E_l[i,k] * sum_j C[i,j] E_r[j,k],
 //     C[i,j]        = go[i,j] * exp(ml[i] + mr[j] - res[i,j])     (likewise rhs)
 // The shift cannot overflow.  It can underflow when the maxima of a row and a
 // column sit at far-apart k: an output whose shifted sum falls below 2^-60 is
 // recomputed exactly with its own maximum, and in the backward a pair (i,j)
 // whose C would exceed 2^60 is left out of the GEMM and added by an exact
-// per-term pass (taken only by tiles that contain such a pair).  Results never
-// depend on the shift beyond fp32 rounding.
+// per-term pass (taken only by tiles that depend on such a pair).  Results
+// never depend on the shift beyond fp32 rounding.
+#include <algorithm>
+
 #include "device_utils.h"
 #include "launch.h"
 
@@ -38,42 +40,85 @@ constexpr float kLn2F = 0.6931471805599453f;
 constexpr float kTiny = 8.6736174e-19f;   // 2^-60
 constexpr float kMaxShiftLog2 = 60.0f;
 
+typedef float v4f __attribute__((ext_vector_type(4)));
+
 __device__ __forceinline__ float neg_inf_f() { return -__builtin_huge_valf(); }
 __device__ __forceinline__ float finite_or_zero(float m) { return m == neg_inf_f() ? 0.0f : m; }
 
-// ---- maxima over the reduction dimension -----------------------------------
-// out[b, r] = max_k x[b*sb + r*sr + k*sk], one wavefront per (b, r).
-__global__ __launch_bounds__(256) void reduce_max_kernel(const float *__restrict__ x, long sb,
-                                                         long sr, long sk, int R, int K,
-                                                         float *__restrict__ out) {
+// ---- shifted exponentials of an operand --------------------------------------
+// One wavefront per row r of x[b, r, k] (element strides sb, sr, sk):
+//   mx[b,r]  = max_k x[b,r,k]
+//   E[b,r,k] = exp(x[b,r,k] - mx[b,r])  for k < K,  0 for K <= k < Kp
+// (the shift is 0 for an all -inf row).  Rows r >= len[b] + extra are padding:
+// mx = -inf, E = 0.  E is (B, R, Kp) contiguous.  The row is read twice; the
+// second read comes from cache.
+__global__ __launch_bounds__(256) void shift_exp_kernel(const float *__restrict__ x, long sb,
+                                                        long sr, long sk, int R, int K, int Kp,
+                                                        const int *__restrict__ len, int extra,
+                                                        float *__restrict__ mx,
+                                                        float *__restrict__ E) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int r = blockIdx.x * 4 + wave;
     const int b = blockIdx.y;
     if (r >= R) return;
+    const int Rb = len ? min(max(len[b], 0) + extra, R) : R;
+    float *e = E + ((size_t)b * R + r) * Kp;
+    const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (r >= Rb) {
+        for (int k = lane * 4; k < Kp; k += 256) *reinterpret_cast<v4f *>(e + k) = zero;
+        if (lane == 0) mx[(size_t)b * R + r] = neg_inf_f();
+        return;
+    }
     const float *p = x + (size_t)b * sb + (size_t)r * sr;
+    // 16-byte loads when the row is contiguous and aligned
+    const bool vec = sk == 1 && (K & 3) == 0 && (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
     float m = neg_inf_f();
-    for (int k = lane; k < K; k += 64) m = fmaxf(m, p[(size_t)k * sk]);
+    if (vec) {
+        for (int k = lane * 4; k < K; k += 256) {
+            const v4f v = *reinterpret_cast<const v4f *>(p + k);
+            m = fmaxf(fmaxf(m, fmaxf(v.x, v.y)), fmaxf(v.z, v.w));
+        }
+    } else {
+        for (int k = lane; k < K; k += 64) m = fmaxf(m, p[(size_t)k * sk]);
+    }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
-    if (lane == 0) out[(size_t)b * R + r] = m;
+    if (lane == 0) mx[(size_t)b * R + r] = m;
+    const float shift = finite_or_zero(m);
+    if (vec) {
+        for (int k = lane * 4; k < Kp; k += 256) {
+            v4f o = zero;
+            if (k < K) {
+                const v4f v = *reinterpret_cast<const v4f *>(p + k);
+                o.x = exp2_hw((v.x - shift) * kLog2eF);
+                o.y = exp2_hw((v.y - shift) * kLog2eF);
+                o.z = exp2_hw((v.z - shift) * kLog2eF);
+                o.w = exp2_hw((v.w - shift) * kLog2eF);
+            }
+            *reinterpret_cast<v4f *>(e + k) = o;
+        }
+    } else {
+        for (int k = lane; k < Kp; k += 64)
+            e[k] = (k < K) ? exp2_hw((p[(size_t)k * sk] - shift) * kLog2eF) : 0.0f;
+    }
 }
 
-// ---- shared MFMA tile ----------------------------------------------------------
-constexpr int TQ = 32;        // reduction chunk
-constexpr int LDK = TQ + 4;   // LDS row stride (floats) of a [row][q] slab: 16-byte aligned rows
-
-typedef float v4f __attribute__((ext_vector_type(4)));
-
+// ---- MFMA tiles ----------------------------------------------------------------
+// v_mfma_f32_16x16x4_f32: lane l supplies A[l%16][l/16] and B[l/16][l%16] and
+// holds D[4*(l/16) + r][l%16] in register r of the accumulator.
 // A workgroup of WR x WC wavefronts owns a (16*RB*WR) x (16*CB*WC) tile; the
 // wavefront at (wr, wc) owns RB x CB blocks of 16x16 starting at row
-// wr*16*RB, column wc*16*CB.  Both operands lie in LDS as [row or column][q].
-// v_mfma_f32_16x16x4_f32: lane l supplies A[l%16][l/16] and B[l/16][l%16] and
-// holds D[4*(l/16) + r][l%16] in register r of the accumulator.  The order of
-// summation over q is free, so lane group g = l/16 takes q = 8g .. 8g+7 of the
-// chunk, which it reads as two 16-byte vectors per block.
+// wr*16*RB, column wc*16*CB.  The reduction runs in chunks of TQ = 32.
+constexpr int TQ = 32;
+constexpr int kDepth = 4;     // chunks of global loads in flight in the forward (even)
+constexpr int LDK = TQ + 4;   // row stride (floats) of a [row][q] slab: 16-byte aligned rows
+
+// Both operands in LDS as [row or column][q].  The order of summation over q
+// is free, so lane group g = l/16 takes q = 8g .. 8g+7 of the chunk, which it
+// reads as two 16-byte vectors per block.
 template <int RB, int CB>
-__device__ __forceinline__ void tile_mfma(const float (*sa)[LDK], const float (*sb)[LDK], int row0,
-                                          int col0, int lane, v4f (&acc)[RB][CB]) {
+__device__ __forceinline__ void tile_mfma_qq(const float (*sa)[LDK], const float (*sb)[LDK],
+                                             int row0, int col0, int lane, v4f (&acc)[RB][CB]) {
     const int r = lane & 15, g = lane >> 4;
     v4f a[RB][2], b[CB][2];
 #pragma unroll
@@ -97,6 +142,29 @@ __device__ __forceinline__ void tile_mfma(const float (*sa)[LDK], const float (*
                                                                    acc[rb][cb], 0, 0, 0);
 }
 
+// A in LDS as [row][q] (stride LDA), B as [q][column] (stride LDB): lane group
+// g takes q = 4s + g in step s; 4-byte reads, free of bank conflicts for
+// LDA = 36 and LDB = 16 (mod 64).
+template <int RB, int CB, int LDA, int LDB>
+__device__ __forceinline__ void tile_mfma_qc(const float (*sa)[LDA], const float (*sb)[LDB],
+                                             int row0, int col0, int lane, v4f (&acc)[RB][CB]) {
+    const int r = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        float a[RB], b[CB];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) a[rb] = sa[row0 + rb * 16 + r][4 * s + g];
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) b[cb] = sb[4 * s + g][col0 + cb * 16 + r];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+                acc[rb][cb] =
+                    __builtin_amdgcn_mfma_f32_16x16x4f32(a[rb], b[cb], acc[rb][cb], 0, 0, 0);
+    }
+}
+
 // ---- forward ----------------------------------------------------------------
 __device__ float exact_lse(const float *lrow, long lsk, const float *rcol, long rsk, int K) {
     float mx = neg_inf_f();
@@ -108,117 +176,128 @@ __device__ float exact_lse(const float *lrow, long lsk, const float *rcol, long 
     return mx + log2_hw(s) * kLn2F;
 }
 
+struct FwdArgs {
+    const float *El, *Er;     // (B,M,Kp), (B,Nn,Kp): shifted exponentials
+    const float *lmax, *rmax; // (B,M), (B,Nn)
+    const float *lhs, *rhs;   // the operands themselves, for the exact fallback
+    long lsb, lsm, lsk, rsb, rsk, rsn;
+    float *res;               // (B,M,Nn)
+    int M, K, Kp, Nn;
+    const int *row_len, *col_len;
+};
+
 // grid (ceil(M/TM), ceil(Nn/TN), B) with TM = 16*RB*WR rows i and TN = 16*CB*WC
 // columns j per workgroup of 64*WR*WC threads.
 template <int RB, int CB, int WR, int WC>
-__global__ __launch_bounds__(64 * WR * WC) void logmm_fwd_kernel(
-    const float *__restrict__ lhs, long lsb, long lsm, long lsk, const float *__restrict__ rhs,
-    long rsb, long rsk, long rsn, const float *__restrict__ lmax, const float *__restrict__ rmax,
-    float *__restrict__ res, int M, int K, int Nn, const int *__restrict__ row_len,
-    const int *__restrict__ col_len) {
+__global__ __launch_bounds__(64 * WR * WC) void logmm_fwd_kernel(const FwdArgs a) {
     constexpr int TM = 16 * RB * WR, TN = 16 * CB * WC, NT = 64 * WR * WC;
-    constexpr int SA = TM * TQ / NT, SB = TN * TQ / NT;   // staged elements per thread
-    static_assert(TM * TQ % NT == 0 && TN * TQ % NT == 0, "slabs must divide over the threads");
+    constexpr int VA = TM * TQ / 4, VB = TN * TQ / 4;   // 16-byte vectors per slab
+    constexpr int SA = VA / NT, SB = VB / NT;           // ... per thread
+    static_assert(VA % NT == 0 && VB % NT == 0, "slabs must divide over the threads");
     __shared__ __attribute__((aligned(16))) float sa[2][TM][LDK];   // E_l[i][k]
     __shared__ __attribute__((aligned(16))) float sb_[2][TN][LDK];  // E_r[j][k]
     const int b = blockIdx.z;
     const int i0 = blockIdx.x * TM, j0 = blockIdx.y * TN;
+    const int M = a.M, Nn = a.Nn, Kp = a.Kp;
     // lengths-aware: rows >= row_len[b] and cols > col_len[b] are padding
-    const int Mb = row_len ? min(max(row_len[b], 0), M) : M;
-    const int Nb = col_len ? min(max(col_len[b], 0) + 1, Nn) : Nn;
+    const int Mb = a.row_len ? min(max(a.row_len[b], 0), M) : M;
+    const int Nb = a.col_len ? min(max(a.col_len[b], 0) + 1, Nn) : Nn;
     if (i0 >= Mb || j0 >= Nb) return;
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int row0 = (wave % WR) * 16 * RB, col0 = (wave / WR) * 16 * CB;
-    const float *lb = lhs + (size_t)b * lsb;
-    const float *rb = rhs + (size_t)b * rsb;
-    const float *lm = lmax + (size_t)b * M;
-    const float *rm = rmax + (size_t)b * Nn;
 
-    // staging: thread tid takes q = tid % 32 of rows tid/32 + (NT/32)*s: the 32
-    // lanes of a row read 128 contiguous bytes (k is contiguous for a row-major
-    // lhs and for the transposed view that is the rhs of the joiner)
-    const int sq = tid & (TQ - 1), sr0 = tid / TQ;
-    float shl[SA], shr[SB];              // per staged row: its shift (0 if the row is all -inf)
-    bool okl[SA], okr[SB];
-    const float *pl[SA], *pr[SB];
+    // staging: vector e = tid + NT*s of a slab is (row, 4 k's) = (e / 8, e % 8);
+    // rows beyond the operand are clamped (their outputs are not stored)
+    const float *pa[SA], *pb[SB];
 #pragma unroll
-    for (int s2 = 0; s2 < SA; ++s2) {
-        const int i = i0 + sr0 + (NT / TQ) * s2;
-        okl[s2] = i < Mb;
-        shl[s2] = okl[s2] ? finite_or_zero(lm[i]) : 0.0f;
-        pl[s2] = lb + (size_t)min(i, M - 1) * lsm;
+    for (int s = 0; s < SA; ++s) {
+        const int e = tid + NT * s;
+        pa[s] = a.El + ((size_t)b * M + min(i0 + e / 8, M - 1)) * Kp + (e % 8) * 4;
     }
 #pragma unroll
-    for (int s2 = 0; s2 < SB; ++s2) {
-        const int j = j0 + sr0 + (NT / TQ) * s2;
-        okr[s2] = j < Nb;
-        shr[s2] = okr[s2] ? finite_or_zero(rm[j]) : 0.0f;
-        pr[s2] = rb + (size_t)min(j, Nn - 1) * rsn;
+    for (int s = 0; s < SB; ++s) {
+        const int e = tid + NT * s;
+        pb[s] = a.Er + ((size_t)b * Nn + min(j0 + e / 8, Nn - 1)) * Kp + (e % 8) * 4;
     }
-    float rl[SA], rr[SB];
-    auto fetch = [&](int k0) {
-        // loads are unconditional from clamped (always valid) addresses and the
-        // padding is selected afterwards: no branch separates the loads from
-        // the matrix instructions that are meant to hide their latency
-        const int k = k0 + sq;
-        const bool kin = k < K;
-        const size_t kc = (size_t)min(k, K - 1);
+    // The reduction is pipelined kDepth chunks deep: a chunk's global loads are
+    // issued kDepth - 1 iterations before they are copied to LDS (a round trip
+    // to memory takes several times the ~770 cycles of one chunk's MFMAs).
+    // No load or LDS store sits behind a branch or a lane mask, so that the
+    // compiler can wait for exactly the oldest chunk (a masked load makes it
+    // wait for all of them); chunks past the end are clamped duplicates.
+    v4f ra[kDepth][SA], rb[kDepth][SB];
+    auto fetch = [&](int set, int k0) {
 #pragma unroll
-        for (int s2 = 0; s2 < SA; ++s2) {
-            const float v = pl[s2][kc * lsk];
-            rl[s2] = (okl[s2] && kin) ? v : neg_inf_f();
-        }
+        for (int s = 0; s < SA; ++s)
+            ra[set][s] = *reinterpret_cast<const v4f *>(pa[s] + k0);
 #pragma unroll
-        for (int s2 = 0; s2 < SB; ++s2) {
-            const float v = pr[s2][kc * rsk];
-            rr[s2] = (okr[s2] && kin) ? v : neg_inf_f();
-        }
+        for (int s = 0; s < SB; ++s)
+            rb[set][s] = *reinterpret_cast<const v4f *>(pb[s] + k0);
     };
-    auto stash = [&](int buf) {
+    auto stash = [&](int set, int buf) {
 #pragma unroll
-        for (int s2 = 0; s2 < SA; ++s2)
-            sa[buf][sr0 + (NT / TQ) * s2][sq] = exp2_hw((rl[s2] - shl[s2]) * kLog2eF);
+        for (int s = 0; s < SA; ++s) {
+            const int e = tid + NT * s;
+            *reinterpret_cast<v4f *>(&sa[buf][e / 8][(e % 8) * 4]) = ra[set][s];
+        }
 #pragma unroll
-        for (int s2 = 0; s2 < SB; ++s2)
-            sb_[buf][sr0 + (NT / TQ) * s2][sq] = exp2_hw((rr[s2] - shr[s2]) * kLog2eF);
+        for (int s = 0; s < SB; ++s) {
+            const int e = tid + NT * s;
+            *reinterpret_cast<v4f *>(&sb_[buf][e / 8][(e % 8) * 4]) = rb[set][s];
+        }
     };
 
     v4f acc[RB][CB];
 #pragma unroll
-    for (int a = 0; a < RB; ++a)
+    for (int r = 0; r < RB; ++r)
 #pragma unroll
-        for (int c = 0; c < CB; ++c) acc[a][c] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int c = 0; c < CB; ++c) acc[r][c] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
-    fetch(0);
-    stash(0);
-    __syncthreads();
-    int buf = 0;
-    for (int k0 = 0; k0 < K; k0 += TQ) {
-        const bool more = (k0 + TQ) < K;
-        if (more) fetch(k0 + TQ);              // global loads in flight during the MFMAs
-        tile_mfma<RB, CB>(sa[buf], sb_[buf], row0, col0, lane, acc);
-        if (more) stash(buf ^ 1);
-        __syncthreads();
-        buf ^= 1;
-    }
+    // chunk j lives in register set j % kDepth and in LDS buffer j % 2; an empty
+    // reduction leaves the sums at 0: log 0 below
+    const int n = Kp / TQ;
+    const int k_last = max(Kp - TQ, 0);
+    if (n > 0) {
 #pragma unroll
-    for (int a = 0; a < RB; ++a) {
+        for (int d = 0; d < kDepth; ++d) fetch(d, min(d * TQ, k_last));
+        stash(0, 0);
+        fetch(0, min(kDepth * TQ, k_last));
+        __syncthreads();
+    }
+    for (int j0 = 0; j0 < n; j0 += kDepth) {
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d) {
+            const int j = j0 + d;
+            if (j < n) {   // uniform over the workgroup
+                tile_mfma_qq<RB, CB>(sa[d & 1], sb_[d & 1], row0, col0, lane, acc);
+                stash((d + 1) % kDepth, (d + 1) & 1);
+                // set (d+1) % kDepth is free again: refill it kDepth chunks ahead
+                fetch((d + 1) % kDepth, min((j + 1 + kDepth) * TQ, k_last));
+                __syncthreads();
+            }
+        }
+    }
+    const float *lm = a.lmax + (size_t)b * M;
+    const float *rm = a.rmax + (size_t)b * Nn;
+#pragma unroll
+    for (int r4 = 0; r4 < RB; ++r4) {
 #pragma unroll
         for (int c = 0; c < CB; ++c) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int i = i0 + row0 + a * 16 + 4 * (lane >> 4) + r;
+                const int i = i0 + row0 + r4 * 16 + 4 * (lane >> 4) + r;
                 const int j = j0 + col0 + c * 16 + (lane & 15);
                 if (i >= Mb || j >= Nb) continue;
-                const float s = acc[a][c][r];
+                const float s = acc[r4][c][r];
                 float out;
                 if (s >= kTiny && s < __builtin_huge_valf()) {
                     out = lm[i] + rm[j] + log2_hw(s) * kLn2F;
                 } else {
-                    out = exact_lse(lb + (size_t)i * lsm, lsk, rb + (size_t)j * rsn, rsk, K);
+                    out = exact_lse(a.lhs + (size_t)b * a.lsb + (size_t)i * a.lsm, a.lsk,
+                                    a.rhs + (size_t)b * a.rsb + (size_t)j * a.rsn, a.rsk, a.K);
                 }
-                res[((size_t)b * M + i) * Nn + j] = out;
+                a.res[((size_t)b * M + i) * Nn + j] = out;
             }
         }
     }
@@ -272,38 +351,66 @@ __global__ __launch_bounds__(256) void logmm_pair_factor_kernel(
 // columns k per workgroup of 64*WR*WC threads.  Offsets inside one batch are
 // 32-bit (the launcher checks the extents).
 struct BwdArgs {
-    const float *own, *oth, *own_max, *oth_max, *C, *go, *res, *batch_scale;
-    const int *flags;       // (B, rows i): 1 = the row holds a pair left out of C
+    const float *Eown, *Eoth;  // (B,P,Kp), (B,Q,Kp): shifted exponentials
+    const float *C;            // pair factors
+    const int *flags;          // (B, rows i): 1 = the row holds a pair left out of C
+    // for the exact pass only: the operands, their maxima, grad_out and res
+    const float *own, *oth, *own_max, *oth_max, *go, *res, *batch_scale;
     float *grad;
     long osb, tsb, gsb, dsb;   // batch strides
     int osp, osk, tsq, tsk, gp, gq, dsp, dsk;
-    int P, Q, K;
+    int P, Q, K, Kp;
     const int *p_len, *q_len;
     int p_extra, q_extra;
-    int flags_follow_p;     // rows i are p (lhs gradient) or q (rhs gradient)
+    int flags_follow_p;        // rows i are p (lhs gradient) or q (rhs gradient)
 };
 
-template <int RB, int CB, int WR, int WC>
+// E_own * sum; the sum is 0 where nothing was added: avoid 0 * inf or 0 * nan
+__device__ __forceinline__ float scaled_sum(float s, float e_own) {
+    return (s != 0.0f) ? e_own * s : 0.0f;
+}
+
+// Exact per-term pass over the pairs (p, q) that C left out (exponent > 2^60).
+__device__ float exact_pairs(const BwdArgs &a, int b, int p, int k, int Qb) {
+    const float *ob = a.own + (size_t)b * a.osb;
+    const float *tb = a.oth + (size_t)b * a.tsb;
+    const float *om = a.own_max + (size_t)b * a.P;
+    const float *tm = a.oth_max + (size_t)b * a.Q;
+    const float *gb = a.go + (size_t)b * a.gsb;
+    const float *rb = a.res + (size_t)b * a.gsb;
+    const float scale = a.batch_scale ? a.batch_scale[b] : 1.0f;
+    const float x_own = ob[p * a.osp + k * a.osk];
+    float v = 0.0f;
+    for (int qq = 0; qq < Qb; ++qq) {
+        const float rr = rb[p * a.gp + qq * a.gq];
+        const float gv = gb[p * a.gp + qq * a.gq] * scale;
+        if (gv == 0.0f || rr == neg_inf_f()) continue;
+        if ((om[p] + tm[qq] - rr) * kLog2eF <= kMaxShiftLog2) continue;
+        const float x = x_own + tb[qq * a.tsq + k * a.tsk] - rr;
+        v += gv * exp2_hw(x * kLog2eF);
+    }
+    return v;
+}
+
+template <int RB, int CB, int WR, int WC, int DEPTH, bool REFILL>
 __global__ __launch_bounds__(64 * WR * WC) void logmm_bwd_kernel(const BwdArgs a) {
     constexpr int TP = 16 * RB * WR, TK = 16 * CB * WC, NT = 64 * WR * WC;
-    constexpr int SC = TP * TQ / NT, SE = TK * TQ / NT;   // staged elements per thread
-    static_assert(TP * TQ % NT == 0 && TK * TQ % NT == 0, "slabs must divide over the threads");
-    static_assert(NT % TK == 0, "a thread stages one column k of the E slab");
+    constexpr int LDE = TK + 16;                        // 16 (mod 64): see tile_mfma_qc
+    constexpr int SC = TP * TQ / NT;                    // C elements per thread and chunk
+    constexpr int VE = TQ * TK / 4, SE = VE / NT;       // E vectors per chunk / thread
+    static_assert(TP * TQ % NT == 0 && VE % NT == 0, "slabs must divide over the threads");
     __shared__ __attribute__((aligned(16))) float s_c[2][TP][LDK];   // C[p][q]
-    __shared__ __attribute__((aligned(16))) float s_e[2][TK][LDK];   // E_oth[k][q]
+    __shared__ __attribute__((aligned(16))) float s_e[2][TQ][LDE];   // E_oth[q][k]
     const int b = blockIdx.z;
     const int p0 = blockIdx.x * TP, k0 = blockIdx.y * TK;
-    const int P = a.P, Q = a.Q, K = a.K;
+    const int P = a.P, Q = a.Q, K = a.K, Kp = a.Kp;
     const int Pb = a.p_len ? min(max(a.p_len[b], 0) + a.p_extra, P) : P;
     const int Qb = a.q_len ? min(max(a.q_len[b], 0) + a.q_extra, Q) : Q;
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int row0 = (wave % WR) * 16 * RB, col0 = (wave / WR) * 16 * CB;
-    const float *ob = a.own + (size_t)b * a.osb;
-    const float *tb = a.oth + (size_t)b * a.tsb;
-    const float *om = a.own_max + (size_t)b * P;
-    const float *tm = a.oth_max + (size_t)b * Q;
     const float *cb = a.C + (size_t)b * a.gsb;
+    const float *eo = a.Eoth + (size_t)b * Q * Kp;
     float *db = a.grad + (size_t)b * a.dsb;
 
     v4f acc[RB][CB];
@@ -321,66 +428,87 @@ __global__ __launch_bounds__(64 * WR * WC) void logmm_bwd_kernel(const BwdArgs a
         } else {
             for (int r = tid; r < Qb; r += NT) unsafe |= fl[r];
         }
-        // E_oth slab (TQ x TK): thread takes column k0 + tid % TK (contiguous in
-        // memory over the lanes) of rows q = tid / TK + (NT/TK)*s.
-        // C slab (TP x TQ): element e = tid + NT*s is (p, q) = (e / TQ, e % TQ)
-        // when q is the contiguous index of C (gq == 1), else (e % TP, e / TP):
+        // E_oth slab (TQ x TK): vector e = tid + NT*s is (q, 4 k's) = (e / (TK/4),
+        // e % (TK/4)).  Columns beyond Kp and rows beyond Q are clamped to valid
+        // memory: such columns are never stored, and such rows meet C = 0.
+        // C slab (TP x TQ): element e is (p, q) = (e / TQ, e % TQ) when q is
+        // the contiguous index of C (gq == 1), else (e % TP, e / TP):
         // consecutive lanes read consecutive addresses.
-        // fetch() only loads (clamped, always valid addresses; nothing is
-        // computed from the values, so no wait separates the loads from the
-        // matrix instructions); stash() selects the padding and does the math.
-        const int ek = tid % TK, eq0 = tid / TK;
-        const bool ek_ok = (k0 + ek) < K;
-        const float *pe = tb + min(k0 + ek, K - 1) * a.tsk;
-        const int q_last = (Q - 1) * a.tsq, c_last = (Q - 1) * a.gq;
+        const float *pe[SE];
+        int eq[SE], ek[SE];
+#pragma unroll
+        for (int s = 0; s < SE; ++s) {
+            const int e = tid + NT * s;
+            eq[s] = e / (TK / 4);
+            ek[s] = (e % (TK / 4)) * 4;
+            pe[s] = eo + min(k0 + ek[s], Kp - 4);
+        }
+        const int c_last = (Q - 1) * a.gq;
         int cp[SC], cq[SC];
         bool cp_ok[SC];
         const float *c_row[SC];
 #pragma unroll
-        for (int s2 = 0; s2 < SC; ++s2) {
-            const int e = tid + NT * s2;
-            cp[s2] = (a.gq == 1) ? e / TQ : e % TP;
-            cq[s2] = (a.gq == 1) ? e % TQ : e / TP;
-            cp_ok[s2] = (p0 + cp[s2]) < Pb;
-            c_row[s2] = cb + min(p0 + cp[s2], P - 1) * a.gp;
+        for (int s = 0; s < SC; ++s) {
+            const int e = tid + NT * s;
+            cp[s] = (a.gq == 1) ? e / TQ : e % TP;
+            cq[s] = (a.gq == 1) ? e % TQ : e / TP;
+            cp_ok[s] = (p0 + cp[s]) < Pb;
+            c_row[s] = cb + min(p0 + cp[s], P - 1) * a.gp;
         }
-        float re[SE], rtm[SE], rc[SC];
-        auto fetch = [&](int q0) {
+        v4f re[DEPTH][SE];
+        float rc[DEPTH][SC];
+        auto fetch = [&](int set, int q0) {
 #pragma unroll
-            for (int s2 = 0; s2 < SE; ++s2) {
-                const int q = q0 + eq0 + (NT / TK) * s2;
-                re[s2] = pe[min(q * a.tsq, q_last)];
-                rtm[s2] = tm[min(q, Q - 1)];
-            }
+            for (int s = 0; s < SE; ++s)
+                re[set][s] = *reinterpret_cast<const v4f *>(
+                    pe[s] + (size_t)min(q0 + eq[s], Q - 1) * Kp);
 #pragma unroll
-            for (int s2 = 0; s2 < SC; ++s2) rc[s2] = c_row[s2][min((q0 + cq[s2]) * a.gq, c_last)];
+            for (int s = 0; s < SC; ++s)
+                rc[set][s] = c_row[s][min((q0 + cq[s]) * a.gq, c_last)];
         };
-        auto stash = [&](int buf, int q0) {
+        auto stash = [&](int set, int buf, int q0) {
 #pragma unroll
-            for (int s2 = 0; s2 < SE; ++s2) {
-                const int qq = q0 + eq0 + (NT / TK) * s2;
-                const float x = (qq < Qb && ek_ok) ? re[s2] - finite_or_zero(rtm[s2]) : neg_inf_f();
-                s_e[buf][ek][eq0 + (NT / TK) * s2] = exp2_hw(x * kLog2eF);
-            }
+            for (int s = 0; s < SE; ++s)
+                *reinterpret_cast<v4f *>(&s_e[buf][eq[s]][ek[s]]) = re[set][s];
 #pragma unroll
-            for (int s2 = 0; s2 < SC; ++s2)
-                s_c[buf][cp[s2]][cq[s2]] = (cp_ok[s2] && (q0 + cq[s2]) < Qb) ? rc[s2] : 0.0f;
+            for (int s = 0; s < SC; ++s)
+                s_c[buf][cp[s]][cq[s]] = (cp_ok[s] && (q0 + cq[s]) < Qb) ? rc[set][s] : 0.0f;
         };
-        fetch(0);
-        stash(0, 0);
-        __syncthreads();
-        int buf = 0;
-        for (int q0 = 0; q0 < Qb; q0 += TQ) {
-            const bool more = (q0 + TQ) < Qb;
-            if (more) fetch(q0 + TQ);
-            tile_mfma<RB, CB>(s_c[buf], s_e[buf], row0, col0, lane, acc);
-            if (more) stash(buf ^ 1, q0 + TQ);
+        // Pipelined like the forward: chunk j in register set j % DEPTH and in
+        // LDS buffer j % 2.  REFILL = false is for reductions of at most DEPTH
+        // chunks: everything is fetched up front, each chunk once.  With
+        // REFILL a set is loaded again as soon as it has been copied to LDS,
+        // unconditionally (chunks past the end read clamped addresses and are
+        // never multiplied), so that the compiler can wait for exactly the
+        // oldest chunk.
+        const int n = (Qb + TQ - 1) / TQ;
+        if (n > 0) {
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d)
+                if (REFILL || d < n) fetch(d, d * TQ);
+            stash(0, 0, 0);
+            if (REFILL) fetch(0, DEPTH * TQ);
             __syncthreads();
-            buf ^= 1;
+        }
+        for (int j0 = 0; j0 < n; j0 += DEPTH) {
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) {
+                const int j = j0 + d;
+                if (j < n) {   // uniform over the workgroup
+                    tile_mfma_qc<RB, CB, LDK, LDE>(s_c[j & 1], s_e[j & 1], row0, col0, lane, acc);
+                    if (REFILL) {
+                        stash((d + 1) % DEPTH, (j + 1) & 1, (j + 1) * TQ);
+                        fetch((d + 1) % DEPTH, (j + 1 + DEPTH) * TQ);
+                    } else if (j + 1 < n) {
+                        stash((d + 1) % DEPTH, (j + 1) & 1, (j + 1) * TQ);
+                    }
+                    __syncthreads();
+                }
+            }
         }
     }
     const bool slow = __syncthreads_or(unsafe) != 0;
-    const float scale = a.batch_scale ? a.batch_scale[b] : 1.0f;
+    const float *eown = a.Eown + (size_t)b * P * Kp;
 #pragma unroll
     for (int r4 = 0; r4 < RB; ++r4)
 #pragma unroll
@@ -392,75 +520,148 @@ __global__ __launch_bounds__(64 * WR * WC) void logmm_bwd_kernel(const BwdArgs a
                 if (p >= P || k >= K) continue;
                 float v = 0.0f;
                 if (p < Pb) {
-                    const float x_own = ob[p * a.osp + k * a.osk];
-                    const float e_own = exp2_hw((x_own - finite_or_zero(om[p])) * kLog2eF);
-                    const float s = acc[r4][c][r];
-                    // s is 0 where nothing was added: avoid 0 * inf for a +inf operand
-                    v = (s != 0.0f) ? e_own * s : 0.0f;
-                    if (slow) {
-                        // exact per-term pass over the pairs that C left out
-                        const float *gb = a.go + (size_t)b * a.gsb, *rb = a.res + (size_t)b * a.gsb;
-                        for (int qq = 0; qq < Qb; ++qq) {
-                            const float rr = rb[p * a.gp + qq * a.gq];
-                            const float gv = gb[p * a.gp + qq * a.gq] * scale;
-                            if (gv == 0.0f || rr == neg_inf_f()) continue;
-                            if ((om[p] + tm[qq] - rr) * kLog2eF <= kMaxShiftLog2) continue;
-                            const float x = x_own + tb[qq * a.tsq + k * a.tsk] - rr;
-                            v += gv * exp2_hw(x * kLog2eF);
-                        }
-                    }
+                    v = scaled_sum(acc[r4][c][r], eown[(size_t)p * Kp + k]);
+                    if (slow) v += exact_pairs(a, b, p, k, Qb);
                 }
                 db[p * a.dsp + k * a.dsk] = v;
             }
 }
 
-// Tiles: 64 x 64 or 96 x 64 outputs, whichever pads the tiled extent less.
+// The same for short reductions (Q <= 96, e.g. the gradient wrt f of the
+// joiner, where q runs over the U+1 contexts): the C slab of a 64-row tile is
+// loaded into LDS once and the workgroup then walks over `tiles_per_wg`
+// 64-column tiles of k, fetching the next tile's E_oth rows and this tile's
+// E_own values while the current tile is multiplied.  Set-up, the C slab and
+// the load latency are paid once per workgroup instead of once per tile.
+// grid (ceil(P/64), ceil(ceil(K/64) / tiles_per_wg), B), 256 threads.
+constexpr int QR = 96;        // longest resident reduction
+constexpr int LDC = QR + 4;   // 36 (mod 64), like LDK
+
+__global__ __launch_bounds__(256) void logmm_bwd_resident_kernel(const BwdArgs a,
+                                                                 int tiles_per_wg) {
+    constexpr int TP = 64, TK = 64, NT = 256, LDE = TK + 16, CB = 4;
+    constexpr int SC = TP * QR / NT;           // C elements per thread
+    constexpr int SE = QR * TK / 4 / NT;       // E vectors per thread and tile
+    __shared__ __attribute__((aligned(16))) float s_c[TP][LDC];   // C[p][q]
+    __shared__ __attribute__((aligned(16))) float s_e[QR][LDE];   // E_oth[q][k]
+    const int b = blockIdx.z;
+    const int p0 = blockIdx.x * TP;
+    const int P = a.P, Q = a.Q, K = a.K, Kp = a.Kp;
+    const int ktiles = (K + TK - 1) / TK;
+    const int kt_begin = blockIdx.y * tiles_per_wg;
+    const int kt_end = min(kt_begin + tiles_per_wg, ktiles);
+    const int Pb = a.p_len ? min(max(a.p_len[b], 0) + a.p_extra, P) : P;
+    const int Qb = a.q_len ? min(max(a.q_len[b], 0) + a.q_extra, Q) : Q;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int row0 = wave * 16;
+    float *db = a.grad + (size_t)b * a.dsb;
+    const int my_p = p0 + row0 + 4 * (lane >> 4);   // first of this lane's 4 rows
+
+    if (p0 >= Pb) {   // a tile of padding rows: zeros
+        for (int kt = kt_begin; kt < kt_end; ++kt)
+#pragma unroll
+            for (int c = 0; c < CB; ++c)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int p = my_p + r, k = kt * TK + c * 16 + (lane & 15);
+                    if (p < P && k < K) db[p * a.dsp + k * a.dsk] = 0.0f;
+                }
+        return;
+    }
+
+    int unsafe = 0;
+    {
+        const int *fl = a.flags + (size_t)b * (a.flags_follow_p ? P : Q);
+        if (a.flags_follow_p) {
+            for (int r = tid; r < TP; r += NT) unsafe |= (p0 + r < Pb) ? fl[p0 + r] : 0;
+        } else {
+            for (int r = tid; r < Qb; r += NT) unsafe |= fl[r];
+        }
+    }
+    // C slab, whole reduction: element e = tid + NT*s is (p, q) = (e / QR, e % QR)
+    // when q is the contiguous index of C, else (e % TP, e / TP)
+    {
+        const float *cb = a.C + (size_t)b * a.gsb;
+        const int c_last = (Q - 1) * a.gq;
+        float rc[SC];
+#pragma unroll
+        for (int s = 0; s < SC; ++s) {
+            const int e = tid + NT * s;
+            const int cp = (a.gq == 1) ? e / QR : e % TP, cq = (a.gq == 1) ? e % QR : e / TP;
+            rc[s] = cb[min(p0 + cp, P - 1) * a.gp + min(cq * a.gq, c_last)];
+        }
+#pragma unroll
+        for (int s = 0; s < SC; ++s) {
+            const int e = tid + NT * s;
+            const int cp = (a.gq == 1) ? e / QR : e % TP, cq = (a.gq == 1) ? e % QR : e / TP;
+            s_c[cp][cq] = ((p0 + cp) < Pb && cq < Qb) ? rc[s] : 0.0f;
+        }
+    }
+    // E_oth rows of one tile: vector e = tid + NT*s is (q, 4 k's) = (e / 16, e % 16);
+    // rows beyond Q and columns beyond Kp are clamped to valid memory (they
+    // meet C = 0, or are never stored)
+    const float *eo = a.Eoth + (size_t)b * Q * Kp;
+    const float *eown = a.Eown + (size_t)b * P * Kp;
+    v4f re[SE];
+    auto fetch = [&](int kt) {
+#pragma unroll
+        for (int s = 0; s < SE; ++s) {
+            const int e = tid + NT * s;
+            re[s] = *reinterpret_cast<const v4f *>(eo + (size_t)min(e / 16, Q - 1) * Kp +
+                                                   min(kt * TK + (e % 16) * 4, Kp - 4));
+        }
+    };
+    fetch(kt_begin);
+    const bool slow = __syncthreads_or(unsafe) != 0;   // also: the C slab is in LDS
+    const int nq = (Qb + TQ - 1) / TQ;
+    for (int kt = kt_begin; kt < kt_end; ++kt) {
+        const int k0 = kt * TK;
+#pragma unroll
+        for (int s = 0; s < SE; ++s) {
+            const int e = tid + NT * s;
+            *reinterpret_cast<v4f *>(&s_e[e / 16][(e % 16) * 4]) = re[s];
+        }
+        __syncthreads();
+        if (kt + 1 < kt_end) fetch(kt + 1);
+        float ev[CB][4];   // E_own of this lane's outputs, in flight during the MFMAs
+#pragma unroll
+        for (int c = 0; c < CB; ++c)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                ev[c][r] = eown[(size_t)min(my_p + r, P - 1) * Kp +
+                                min(k0 + c * 16 + (lane & 15), Kp - 1)];
+        v4f acc[1][CB];
+#pragma unroll
+        for (int c = 0; c < CB; ++c) acc[0][c] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int c3 = 0; c3 < nq; ++c3)
+            tile_mfma_qc<1, CB, LDC, LDE>(
+                reinterpret_cast<const float (*)[LDC]>(&s_c[0][c3 * TQ]), &s_e[c3 * TQ], row0, 0,
+                lane, acc);
+#pragma unroll
+        for (int c = 0; c < CB; ++c)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int p = my_p + r, k = k0 + c * 16 + (lane & 15);
+                if (p >= P || k >= K) continue;
+                float v = 0.0f;
+                if (p < Pb) {
+                    v = scaled_sum(acc[0][c][r], ev[c][r]);
+                    if (slow) v += exact_pairs(a, b, p, k, Qb);
+                }
+                db[p * a.dsp + k * a.dsk] = v;
+            }
+        __syncthreads();   // everyone is done with s_e
+    }
+}
+
+// Tiles of 64 or 96 along an extent, whichever pads the tiled extent less.
 inline bool prefer_96(int extent) {
     return (extent + 95) / 96 * 96 < (extent + 63) / 64 * 64;
 }
 
-}  // namespace
-
-hipError_t launch_reduce_max(const float *x, long sb, long sr, long sk, int B, int R, int K,
-                             float *out, hipStream_t stream) {
-    if (B == 0 || R == 0) return hipSuccess;
-    hipLaunchKernelGGL(reduce_max_kernel, dim3((R + 3) / 4, B), dim3(256), 0, stream, x, sb, sr,
-                       sk, R, K, out);
-    return hipGetLastError();
-}
-
-hipError_t launch_logmm_max(const LogmmOperand &lhs, const LogmmOperand &rhs, float *lmax,
-                            float *rmax, int B, int M, int K, int Nn, hipStream_t stream) {
-    hipError_t e = launch_reduce_max(lhs.p, lhs.sb, lhs.s1, lhs.s2, B, M, K, lmax, stream);
-    if (e != hipSuccess) return e;
-    // rhs[b,k,j]: the rows to reduce are j (stride s2), k has stride s1
-    return launch_reduce_max(rhs.p, rhs.sb, rhs.s2, rhs.s1, B, Nn, K, rmax, stream);
-}
-
-hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs, float *lmax,
-                            float *rmax, float *res, int B, int M, int K, int Nn,
-                            const int *row_len, const int *col_len, hipStream_t stream) {
-    if (B == 0 || M == 0 || Nn == 0) return hipSuccess;
-    hipError_t e = launch_logmm_max(lhs, rhs, lmax, rmax, B, M, K, Nn, stream);
-    if (e != hipSuccess) return e;
-    // 8 wavefronts per workgroup: 64 rows i by 96 or 64 columns j
-    if (prefer_96(Nn)) {
-        dim3 grid((M + 63) / 64, (Nn + 95) / 96, B);
-        hipLaunchKernelGGL((logmm_fwd_kernel<1, 3, 4, 2>), grid, dim3(512), 0, stream, lhs.p,
-                           lhs.sb, lhs.s1, lhs.s2, rhs.p, rhs.sb, rhs.s1, rhs.s2, lmax, rmax, res,
-                           M, K, Nn, row_len, col_len);
-    } else {
-        dim3 grid((M + 63) / 64, (Nn + 63) / 64, B);
-        hipLaunchKernelGGL((logmm_fwd_kernel<1, 2, 4, 2>), grid, dim3(512), 0, stream, lhs.p,
-                           lhs.sb, lhs.s1, lhs.s2, rhs.p, rhs.sb, rhs.s1, rhs.s2, lmax, rmax, res,
-                           M, K, Nn, row_len, col_len);
-    }
-    return hipGetLastError();
-}
-
-namespace {
-
 bool fits_int(long extent) { return extent >= 0 && extent < 0x7fffffffL; }
+bool stride_ok(long s) { return s >= 0 && s < 0x7fffffffL; }
 
 // 4 wavefronts per workgroup: 64 rows p (one 16-row block per wavefront, all 64
 // columns) or 96 rows p (all rows, 16 columns per wavefront) by 64 columns k
@@ -471,19 +672,79 @@ hipError_t launch_bwd(const BwdArgs &a, int B, hipStream_t stream) {
         !fits_int((long)(a.P - 1) * a.dsp + (long)(a.K - 1) * a.dsk + 1) ||
         !fits_int((long)a.P * a.Q))
         return hipErrorInvalidValue;
+    if (a.Q <= QR && !prefer_96(a.P)) {
+        // short reduction, many rows: C slab resident, a few k tiles per workgroup
+        const int ptiles = (a.P + 63) / 64, ktiles = (a.K + 63) / 64;
+        const long wgs = (long)ptiles * ktiles * B;
+        const int per = (int)std::min<long>(8, std::max<long>(1, wgs / 2048));
+        dim3 grid(ptiles, (ktiles + per - 1) / per, B);
+        hipLaunchKernelGGL(logmm_bwd_resident_kernel, grid, dim3(256), 0, stream, a, per);
+        return hipGetLastError();
+    }
+    // a reduction of up to 4 chunks (Q <= 128) is fetched whole, up front;
+    // longer ones run a pipeline 3 chunks deep
+    const bool short_q = a.Q <= 4 * TQ;
     if (prefer_96(a.P)) {
         dim3 grid((a.P + 95) / 96, (a.K + 63) / 64, B);
-        hipLaunchKernelGGL((logmm_bwd_kernel<6, 1, 1, 4>), grid, dim3(256), 0, stream, a);
+        if (short_q)
+            hipLaunchKernelGGL((logmm_bwd_kernel<6, 1, 1, 4, 4, false>), grid, dim3(256), 0,
+                               stream, a);
+        else
+            hipLaunchKernelGGL((logmm_bwd_kernel<6, 1, 1, 4, 3, true>), grid, dim3(256), 0, stream,
+                               a);
     } else {
         dim3 grid((a.P + 63) / 64, (a.K + 63) / 64, B);
-        hipLaunchKernelGGL((logmm_bwd_kernel<1, 4, 4, 1>), grid, dim3(256), 0, stream, a);
+        if (short_q)
+            hipLaunchKernelGGL((logmm_bwd_kernel<1, 4, 4, 1, 4, false>), grid, dim3(256), 0,
+                               stream, a);
+        else
+            hipLaunchKernelGGL((logmm_bwd_kernel<1, 4, 4, 1, 3, true>), grid, dim3(256), 0, stream,
+                               a);
     }
     return hipGetLastError();
 }
 
-bool stride_ok(long s) { return s >= 0 && s < 0x7fffffffL; }
-
 }  // namespace
+
+hipError_t launch_logmm_shift_exp(const LogmmOperand &lhs, const LogmmOperand &rhs,
+                                  const LogmmShifted &sh, int B, int M, int K, int Nn,
+                                  const int *row_len, const int *col_len, hipStream_t stream) {
+    const int Kp = logmm_padded_reduction(K);
+    if (B == 0 || Kp == 0) return hipSuccess;
+    if (M > 0) {
+        hipLaunchKernelGGL(shift_exp_kernel, dim3((M + 3) / 4, B), dim3(256), 0, stream, lhs.p,
+                           lhs.sb, lhs.s1, lhs.s2, M, K, Kp, row_len, 0, sh.lmax, sh.El);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    if (Nn > 0) {
+        // rhs[b,k,j]: the rows are j (stride s2), k has stride s1
+        hipLaunchKernelGGL(shift_exp_kernel, dim3((Nn + 3) / 4, B), dim3(256), 0, stream, rhs.p,
+                           rhs.sb, rhs.s2, rhs.s1, Nn, K, Kp, col_len, 1, sh.rmax, sh.Er);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
+                            const LogmmShifted &sh, float *res, int B, int M, int K, int Nn,
+                            const int *row_len, const int *col_len, hipStream_t stream) {
+    if (B == 0 || M == 0 || Nn == 0) return hipSuccess;
+    FwdArgs a;
+    a.El = sh.El, a.Er = sh.Er, a.lmax = sh.lmax, a.rmax = sh.rmax;
+    a.lhs = lhs.p, a.lsb = lhs.sb, a.lsm = lhs.s1, a.lsk = lhs.s2;
+    a.rhs = rhs.p, a.rsb = rhs.sb, a.rsk = rhs.s1, a.rsn = rhs.s2;
+    a.res = res, a.M = M, a.K = K, a.Kp = logmm_padded_reduction(K), a.Nn = Nn;
+    a.row_len = row_len, a.col_len = col_len;
+    // 4 wavefronts per workgroup: 32 rows i by 96 or 64 columns j
+    if (prefer_96(Nn)) {
+        dim3 grid((M + 31) / 32, (Nn + 95) / 96, B);
+        hipLaunchKernelGGL((logmm_fwd_kernel<1, 3, 2, 2>), grid, dim3(256), 0, stream, a);
+    } else {
+        dim3 grid((M + 31) / 32, (Nn + 63) / 64, B);
+        hipLaunchKernelGGL((logmm_fwd_kernel<1, 2, 2, 2>), grid, dim3(256), 0, stream, a);
+    }
+    return hipGetLastError();
+}
 
 hipError_t launch_logmm_pair_factor(const float *go, const float *res, const float *lmax,
                                     const float *rmax, const float *batch_scale,
@@ -496,35 +757,34 @@ hipError_t launch_logmm_pair_factor(const float *go, const float *res, const flo
 }
 
 hipError_t launch_logmm_bwd_lhs(const LogmmOperand &lhs, const LogmmOperand &rhs,
-                                const float *lmax, const float *rmax, const float *go,
-                                const float *res, const float *C, const int *flags,
-                                const LogmmGrad &grad, int B, int M, int K, int Nn,
-                                const int *row_len, const int *col_len, const float *batch_scale,
-                                hipStream_t stream) {
+                                const LogmmShifted &sh, const float *go, const float *res,
+                                const float *C, const int *flags, const LogmmGrad &grad, int B,
+                                int M, int K, int Nn, const int *row_len, const int *col_len,
+                                const float *batch_scale, hipStream_t stream) {
     if (B == 0 || M == 0 || K == 0) return hipSuccess;
     if (!stride_ok(lhs.s1) || !stride_ok(lhs.s2) || !stride_ok(rhs.s1) || !stride_ok(rhs.s2) ||
         !stride_ok(grad.s1) || !stride_ok(grad.s2))
         return hipErrorInvalidValue;
     // own = lhs[b,i,k]; oth[q=j][k] = rhs[b,k,j]; C/go/res[i,j]: p stride Nn, q stride 1
     BwdArgs a;
+    a.Eown = sh.El, a.Eoth = sh.Er;
     a.own = lhs.p, a.osb = lhs.sb, a.osp = (int)lhs.s1, a.osk = (int)lhs.s2;
     a.oth = rhs.p, a.tsb = rhs.sb, a.tsq = (int)rhs.s2, a.tsk = (int)rhs.s1;
-    a.own_max = lmax, a.oth_max = rmax;
+    a.own_max = sh.lmax, a.oth_max = sh.rmax;
     a.C = C, a.go = go, a.res = res, a.gsb = (long)M * Nn, a.gp = Nn, a.gq = 1;
     a.flags = flags, a.flags_follow_p = 1;
     a.grad = grad.p, a.dsb = grad.sb, a.dsp = (int)grad.s1, a.dsk = (int)grad.s2;
-    a.P = M, a.Q = Nn, a.K = K;
+    a.P = M, a.Q = Nn, a.K = K, a.Kp = logmm_padded_reduction(K);
     a.p_len = row_len, a.p_extra = 0, a.q_len = col_len, a.q_extra = 1;
     a.batch_scale = batch_scale;
     return launch_bwd(a, B, stream);
 }
 
 hipError_t launch_logmm_bwd_rhs(const LogmmOperand &lhs, const LogmmOperand &rhs,
-                                const float *lmax, const float *rmax, const float *go,
-                                const float *res, const float *C, const int *flags,
-                                const LogmmGrad &grad, int B, int M, int K, int Nn,
-                                const int *row_len, const int *col_len, const float *batch_scale,
-                                hipStream_t stream) {
+                                const LogmmShifted &sh, const float *go, const float *res,
+                                const float *C, const int *flags, const LogmmGrad &grad, int B,
+                                int M, int K, int Nn, const int *row_len, const int *col_len,
+                                const float *batch_scale, hipStream_t stream) {
     if (B == 0 || Nn == 0 || K == 0) return hipSuccess;
     if (!stride_ok(lhs.s1) || !stride_ok(lhs.s2) || !stride_ok(rhs.s1) || !stride_ok(rhs.s2) ||
         !stride_ok(grad.s1) || !stride_ok(grad.s2))
@@ -532,13 +792,14 @@ hipError_t launch_logmm_bwd_rhs(const LogmmOperand &lhs, const LogmmOperand &rhs
     // own[p=j][k] = rhs[b,k,j]; oth[q=i][k] = lhs[b,i,k]; C/go/res[i,j]: p stride 1, q stride Nn.
     // grad is addressed [b, j, k] through (s2, s1) of the (B,K,Nn) gradient layout.
     BwdArgs a;
+    a.Eown = sh.Er, a.Eoth = sh.El;
     a.own = rhs.p, a.osb = rhs.sb, a.osp = (int)rhs.s2, a.osk = (int)rhs.s1;
     a.oth = lhs.p, a.tsb = lhs.sb, a.tsq = (int)lhs.s1, a.tsk = (int)lhs.s2;
-    a.own_max = rmax, a.oth_max = lmax;
+    a.own_max = sh.rmax, a.oth_max = sh.lmax;
     a.C = C, a.go = go, a.res = res, a.gsb = (long)M * Nn, a.gp = 1, a.gq = Nn;
     a.flags = flags, a.flags_follow_p = 0;
     a.grad = grad.p, a.dsb = grad.sb, a.dsp = (int)grad.s2, a.dsk = (int)grad.s1;
-    a.P = Nn, a.Q = M, a.K = K;
+    a.P = Nn, a.Q = M, a.K = K, a.Kp = logmm_padded_reduction(K);
     a.p_len = col_len, a.p_extra = 1, a.q_len = row_len, a.q_extra = 0;
     a.batch_scale = batch_scale;
     return launch_bwd(a, B, stream);

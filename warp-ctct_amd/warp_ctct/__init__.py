@@ -107,25 +107,26 @@ class _SimpleCTCTLoss(torch.autograd.Function):
     two gathers (:204-215) and SimpleCTCTLoss (:55-85).  Forward computes den
     (if normalized), the lattice and the compact gradients wrt the gathered f,
     g and den; backward expands them to dense gradients wrt f and g, including
-    the path through den, scaled by grad_output[n]."""
+    the path through den, scaled by grad_output[n].  The forward's exp(f - max f)
+    and exp(g - max g) are kept for the backward (one more tensor of f's size)."""
 
     @staticmethod
     def forward(ctx, f, g, labels, lx, ly, normalized, track_f, track_g):
         need_grad = track_f or track_g
-        costs, den, fmax, gmax, grad_f, grad_g, grad_den = _run(
+        costs, den, shifted, grad_f, grad_g, grad_den = _run(
             "simple_forward", lambda: core.ctct_simple_fwd(f, g, labels, lx, ly, normalized,
                                                            need_grad))
         if need_grad:
-            ctx.save_for_backward(f, g, den, fmax, gmax, grad_f, grad_g, grad_den, labels, lx, ly)
+            ctx.save_for_backward(f, g, den, grad_f, grad_g, grad_den, labels, lx, ly, *shifted)
             ctx.track = (track_f, track_g)
         return costs
 
     @staticmethod
     def backward(ctx, grad_outputs):
-        f, g, den, fmax, gmax, grad_f, grad_g, grad_den, labels, lx, ly = ctx.saved_tensors
+        f, g, den, grad_f, grad_g, grad_den, labels, lx, ly, *shifted = ctx.saved_tensors
         grad_outputs = grad_outputs.reshape(-1).float().contiguous()
         dense_f, dense_g = _run("simple_backward", lambda: core.ctct_simple_bwd(
-            f, g, den, fmax, gmax, grad_f, grad_g, grad_den, labels, lx, ly, grad_outputs,
+            f, g, den, list(shifted), grad_f, grad_g, grad_den, labels, lx, ly, grad_outputs,
             ctx.track[0], ctx.track[1]))
         return dense_f, dense_g, None, None, None, None, None, None
 
