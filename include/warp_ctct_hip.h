@@ -123,6 +123,41 @@ int warpctct_loss_forward_f32(const float *joint, const int *ys, const int *lx, 
                               size_t workspace_bytes, float *costs, float *unit_grads,
                               void *stream);
 
+/* Element types of the joint tensor and of its dense gradient. */
+#define WARPCTCT_F32 0
+#define WARPCTCT_F16 1
+#define WARPCTCT_BF16 2
+
+/* ctct_loss forward as the Python function uses it: gather + lattices on a
+ * joint of type `dtype` (the reference converts to float after its gather,
+ * warp_ctct/__init__.py:124-136; here the conversion happens in the gather's
+ * loads), with the reduction of warp_ctct/__init__.py:138-147 folded in:
+ * costs[n] is divided by lx[n] if average_frames, and for reduction 1 (sum)
+ * or 2 (mean) *reduced receives the sum or mean over the batch, added in a
+ * fixed order (reduction 0: reduced is ignored).  The workspace holds what
+ * warpctct_dense_grad_lattice needs and must be kept until it has run.
+ * want_alpha == 0 is the no-grad mode (beta only). */
+int warpctct_loss_lattice(const void *joint, int dtype, const int *ys, const int *lx,
+                          const int *ly, int N, int T, int U, int V, void *workspace,
+                          size_t workspace_bytes, float *costs, int want_alpha, int reduction,
+                          int average_frames, float *reduced, void *stream);
+
+/* Dense gradient of type `dtype` from that workspace (see
+ * warpctct_dense_grad_lattice_f32 below for the weights); values are summed in
+ * fp32 and rounded once to nearest even. */
+int warpctct_dense_grad_lattice(const void *workspace, size_t workspace_bytes, const int *ys,
+                                const int *lx, const int *ly, const float *grad_out,
+                                int grad_out_stride, float scale, int average_frames, void *dense,
+                                int dtype, int N, int T, int U, int V, void *stream);
+int warpctct_dense_patch_lattice(const void *workspace, size_t workspace_bytes, const int *ys,
+                                 const int *lx, const int *ly, const float *grad_out,
+                                 int grad_out_stride, float scale, int average_frames, void *dense,
+                                 int dtype, int N, int T, int U, int V, void *stream);
+
+/* p[0..bytes) = 0 with a kernel (one 16-byte store per thread; safe to capture
+ * in a HIP graph). */
+int warpctct_zero_fill(void *p, size_t bytes, void *stream);
+
 /* The same without unit gradients: gather + lattices only.  The workspace then
  * holds everything the dense gradient needs (units, alpha, beta) and must be
  * kept until warpctct_dense_grad_lattice_f32 has run.  want_alpha == 0 is the

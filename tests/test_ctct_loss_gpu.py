@@ -26,11 +26,12 @@ LN2 = math.log(2.0)
 LOG2E = np.float64(1.4426950408889634074)
 
 
-def assert_support(got, ref, what):
+def assert_support(got, ref, what, underflow=1e-30):
     """Structural zeros of the oracle are exact zeros here; an exact zero here
-    is either structural or an fp32 underflow of a negligible value."""
+    is either structural or an underflow of a negligible value (below
+    `underflow`: fp32's range by default)."""
     assert np.all(got[ref == 0] == 0), what + ": non-zero where the oracle has a structural zero"
-    assert np.all(np.abs(ref[got == 0]) < 1e-30), what + ": zero where the oracle has mass"
+    assert np.all(np.abs(ref[got == 0]) < underflow), what + ": zero where the oracle has mass"
 
 
 def dev(a, dtype=None):
@@ -217,6 +218,81 @@ def test_no_grad_and_int64_lengths_and_half_input():
     np.testing.assert_allclose(ch.detach().cpu().numpy(), ref_h, rtol=LOSS_RTOL)
     ch.sum().backward()
     assert xh.grad.dtype == torch.float16 and xh.grad.shape == xh.shape
+
+
+HALF_TYPES = [
+    # torch dtype, relative spacing of the type (one unit in the last place)
+    (torch.float16, 2.0 ** -10),
+    (torch.bfloat16, 2.0 ** -7),
+]
+
+
+@pytest.mark.parametrize("dtype,ulp", HALF_TYPES, ids=["float16", "bfloat16"])
+@pytest.mark.parametrize("reduction", ["none", "mean"])
+def test_half_precision_joint_is_read_and_written_natively(dtype, ulp, reduction):
+    """A float16 / bfloat16 joint: the loss is that of the rounded inputs,
+    computed in float32 (the reference casts after its gather,
+    warp_ctct/__init__.py:135), and the gradient comes back in the input's
+    type.  Every gradient element must be the float64 oracle's value rounded
+    to the type: within one unit in the last place (half an ulp of rounding
+    plus the fp32 error of the value), structural zeros exact.  Odd V makes
+    rows start at 2-byte, not 4-byte, aligned addresses."""
+    import warp_ctct
+    joint, ys, lx, ly = make_joint_case(31, 4, 26, 9, 33, lx=range(14, 27), ly=range(3, 10))
+    xh = dev(joint).to(dtype).requires_grad_(True)
+    rounded = xh.detach().double().cpu().numpy()
+    w = np.linspace(0.5, 2.0, 4)
+    ref_loss, ref_dense, _ = O.ctct_loss(rounded, ys, lx, ly, reduction=reduction,
+                                         grad_output=w if reduction == "none" else None)
+    loss = warp_ctct.ctct_loss(xh, dev(ys), dev(lx), dev(ly), reduction=reduction)
+    assert loss.dtype == torch.float32
+    np.testing.assert_allclose(loss.detach().cpu().numpy(), ref_loss, rtol=LOSS_RTOL)
+    if reduction == "none":
+        loss.backward(dev(w, torch.float32))
+    else:
+        loss.backward()
+    assert xh.grad.dtype == dtype and xh.grad.shape == xh.shape
+    got = xh.grad.double().cpu().numpy()
+    tiny = 1e-7 if dtype == torch.float16 else 1e-30   # float16 subnormals end at 6e-8
+    assert_support(got, ref_dense, "half dense gradient", underflow=tiny)
+    assert np.all(np.abs(got - ref_dense) <= ulp * np.abs(ref_dense) + tiny)
+    # and it is the float32 path's gradient, rounded once
+    x32 = xh.detach().float().requires_grad_(True)
+    loss32 = warp_ctct.ctct_loss(x32, dev(ys), dev(lx), dev(ly), reduction=reduction)
+    if reduction == "none":
+        loss32.backward(dev(w, torch.float32))
+    else:
+        loss32.backward()
+    assert torch.equal(xh.grad, x32.grad.to(dtype))
+    assert torch.equal(loss, loss32)
+
+
+def test_double_joint_is_converted_like_the_reference():
+    import warp_ctct
+    joint, ys, lx, ly = make_joint_case(32, 2, 12, 4, 7)
+    xd = dev(joint).double().requires_grad_(True)
+    _, ref_dense, ref_costs = O.ctct_loss(joint, ys, lx, ly, reduction="sum")
+    loss = warp_ctct.ctct_loss(xd, dev(ys), dev(lx), dev(ly), reduction="sum")
+    np.testing.assert_allclose(loss.item(), ref_costs.sum(), rtol=LOSS_RTOL)
+    loss.backward()
+    assert xd.grad.dtype == torch.float64
+    np.testing.assert_allclose(xd.grad.cpu().numpy(), ref_dense, atol=GRAD_ATOL, rtol=0)
+
+
+def test_batch_reduction_is_deterministic_and_handles_large_batches():
+    """The in-kernel sum over the batch adds in a fixed order: two calls give
+    the same bits, for a batch larger than one wavefront too."""
+    import warp_ctct
+    joint, ys, lx, ly = make_joint_case(33, 150, 9, 3, 6, lx=range(4, 10), ly=range(1, 4))
+    _, _, ref_costs = O.ctct_loss(joint, ys, lx, ly, reduction="none")
+    x = dev(joint)
+    for reduction, ref in (("sum", ref_costs.sum()), ("mean", ref_costs.mean())):
+        a = warp_ctct.ctct_loss(x, dev(ys), dev(lx), dev(ly), reduction=reduction)
+        b = warp_ctct.ctct_loss(x, dev(ys), dev(lx), dev(ly), reduction=reduction)
+        assert a.dim() == 0 and torch.equal(a, b)
+        np.testing.assert_allclose(a.item(), ref, rtol=LOSS_RTOL)
+    af = warp_ctct.ctct_loss(x, dev(ys), dev(lx), dev(ly), reduction="mean", average_frames=True)
+    np.testing.assert_allclose(af.item(), (ref_costs / lx).mean(), rtol=LOSS_RTOL)
 
 
 def test_operator_surface_on_gathered_units():

@@ -31,6 +31,7 @@ struct Workspace {
     double *units;    // (N,T,P,3),   P = padded_contexts(U)
     double *alphas;   // (N,T+1,P,2)
     double *betas;    // (N,T+1,P,2)
+    unsigned *counter;   // arrivals of the batch reduction (see CostReduce)
     size_t bytes;
 };
 
@@ -43,13 +44,14 @@ Workspace carve(void *base, int N, int T, int U) {
     w.units = reinterpret_cast<double *>(p);
     w.alphas = reinterpret_cast<double *>(p + units_b);
     w.betas = reinterpret_cast<double *>(p + units_b + lat_b);
-    w.bytes = units_b + 2 * lat_b;
+    w.counter = reinterpret_cast<unsigned *>(p + units_b + 2 * lat_b);
+    w.bytes = units_b + 2 * lat_b + 256;
     return w;
 }
 
 int forward_from_units(const Workspace &w, const int *ys, const int *lx, const int *ly, int N,
                        int T, int U, float *costs, float *unit_grads, hipStream_t stream) {
-    LatticeArgs a;
+    LatticeArgs a = {};
     a.units = w.units;
     a.ys = ys;
     a.lx = lx;
@@ -165,8 +167,8 @@ int warpctct_gather_units_f32(const float *joint, const int *ys, const int *lx, 
     if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
     if (N == 0 || T == 0) return WARPCTCT_OK;
     if (!joint || !lx || !ly || !units_out || (U > 0 && !ys)) return WARPCTCT_EINVAL;
-    return done(launch_gather_units(joint, ys, lx, ly, units_out, N, T, U, V, false,
-                                    as_stream(stream)));
+    return done(launch_gather_units(joint, kIoF32, ys, lx, ly, units_out, N, T, U, V, false,
+                                    nullptr, as_stream(stream)));
 }
 
 int warpctct_scale_units_f32(const float *units_nat, const int *lx, const int *ly,
@@ -194,7 +196,7 @@ int warpctct_lattice_f32(const double *units, const int *ys, const int *lx, cons
     if (!lx || !ly || !betas || !costs || (T > 0 && !units) || (U > 0 && !ys))
         return WARPCTCT_EINVAL;
     if (!beta_only && !alphas) return WARPCTCT_EINVAL;
-    LatticeArgs a;
+    LatticeArgs a = {};
     a.units = units;
     a.ys = ys;
     a.lx = lx;
@@ -240,21 +242,29 @@ int warpctct_dense_patch_f32(const float *unit_grads, const int *ys, const int *
                                    as_stream(stream)));
 }
 
-int warpctct_loss_lattice_f32(const float *joint, const int *ys, const int *lx, const int *ly,
-                              int N, int T, int U, int V, void *workspace, size_t workspace_bytes,
-                              float *costs, int want_alpha, void *stream) {
-    if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
+int warpctct_loss_lattice(const void *joint, int dtype, const int *ys, const int *lx,
+                          const int *ly, int N, int T, int U, int V, void *workspace,
+                          size_t workspace_bytes, float *costs, int want_alpha, int reduction,
+                          int average_frames, float *reduced, void *stream) {
+    if (!dims_ok(N, T, U) || V < 1 || !io_valid(dtype) || reduction < 0 || reduction > 2)
+        return WARPCTCT_EINVAL;
     if (N == 0) return WARPCTCT_OK;
     if (!lx || !ly || !costs || !workspace || (T > 0 && !joint) || (U > 0 && !ys))
         return WARPCTCT_EINVAL;
+    if (reduction != 0 && !reduced) return WARPCTCT_EINVAL;
     const Workspace w = carve(workspace, N, T, U);
     if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
+    hipStream_t st = as_stream(stream);
+    unsigned *counter = reduction != 0 ? w.counter : nullptr;
     if (T > 0) {
-        int rc = done(launch_gather_units(joint, ys, lx, ly, w.units, N, T, U, V, true,
-                                          as_stream(stream)));
+        int rc = done(launch_gather_units(joint, dtype, ys, lx, ly, w.units, N, T, U, V, true,
+                                          counter, st));
+        if (rc != WARPCTCT_OK) return rc;
+    } else if (counter) {
+        int rc = done(launch_clear_counter(counter, st));
         if (rc != WARPCTCT_OK) return rc;
     }
-    LatticeArgs a;
+    LatticeArgs a = {};
     a.units = w.units;
     a.ys = ys;
     a.lx = lx;
@@ -266,35 +276,72 @@ int warpctct_loss_lattice_f32(const float *joint, const int *ys, const int *lx, 
     a.T = T;
     a.U = U;
     a.beta_only = (want_alpha == 0);
-    return done(launch_lattice(a, as_stream(stream)));
+    a.reduce.reduced = reduction != 0 ? reduced : nullptr;
+    a.reduce.counter = counter;
+    a.reduce.mode = reduction;
+    a.reduce.average_frames = average_frames != 0;
+    return done(launch_lattice(a, st));
+}
+
+int warpctct_loss_lattice_f32(const float *joint, const int *ys, const int *lx, const int *ly,
+                              int N, int T, int U, int V, void *workspace, size_t workspace_bytes,
+                              float *costs, int want_alpha, void *stream) {
+    return warpctct_loss_lattice(joint, WARPCTCT_F32, ys, lx, ly, N, T, U, V, workspace,
+                                 workspace_bytes, costs, want_alpha, 0, 0, nullptr, stream);
+}
+
+int warpctct_dense_patch_lattice(const void *workspace, size_t workspace_bytes, const int *ys,
+                                 const int *lx, const int *ly, const float *grad_out,
+                                 int grad_out_stride, float scale, int average_frames, void *dense,
+                                 int dtype, int N, int T, int U, int V, void *stream) {
+    if (!dims_ok(N, T, U) || V < 1 || grad_out_stride < 0 || !io_valid(dtype))
+        return WARPCTCT_EINVAL;
+    if (N == 0 || T == 0) return WARPCTCT_OK;
+    if (!workspace || !lx || !ly || !dense || (U > 0 && !ys)) return WARPCTCT_EINVAL;
+    const Workspace w = carve(const_cast<void *>(workspace), N, T, U);
+    if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
+    return done(launch_dense_patch_lattice(w.units, w.alphas, w.betas, ys, lx, ly, grad_out,
+                                           grad_out_stride, scale, average_frames, dense, dtype, N,
+                                           T, U, V, as_stream(stream)));
+}
+
+int warpctct_dense_grad_lattice(const void *workspace, size_t workspace_bytes, const int *ys,
+                                const int *lx, const int *ly, const float *grad_out,
+                                int grad_out_stride, float scale, int average_frames, void *dense,
+                                int dtype, int N, int T, int U, int V, void *stream) {
+    if (!dims_ok(N, T, U) || V < 1 || !io_valid(dtype)) return WARPCTCT_EINVAL;
+    if (N == 0 || T == 0) return WARPCTCT_OK;
+    if (!dense) return WARPCTCT_EINVAL;
+    int rc = done(launch_zero_fill_bytes(dense, (size_t)N * T * (U + 1) * V * io_size(dtype),
+                                         as_stream(stream)));
+    if (rc != WARPCTCT_OK) return rc;
+    return warpctct_dense_patch_lattice(workspace, workspace_bytes, ys, lx, ly, grad_out,
+                                        grad_out_stride, scale, average_frames, dense, dtype, N, T,
+                                        U, V, stream);
 }
 
 int warpctct_dense_patch_lattice_f32(const void *workspace, size_t workspace_bytes, const int *ys,
                                      const int *lx, const int *ly, const float *grad_out,
                                      int grad_out_stride, float scale, int average_frames,
                                      float *dense, int N, int T, int U, int V, void *stream) {
-    if (!dims_ok(N, T, U) || V < 1 || grad_out_stride < 0) return WARPCTCT_EINVAL;
-    if (N == 0 || T == 0) return WARPCTCT_OK;
-    if (!workspace || !lx || !ly || !dense || (U > 0 && !ys)) return WARPCTCT_EINVAL;
-    const Workspace w = carve(const_cast<void *>(workspace), N, T, U);
-    if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
-    return done(launch_dense_patch_lattice(w.units, w.alphas, w.betas, ys, lx, ly, grad_out,
-                                           grad_out_stride, scale, average_frames, dense, N, T, U,
-                                           V, as_stream(stream)));
+    return warpctct_dense_patch_lattice(workspace, workspace_bytes, ys, lx, ly, grad_out,
+                                        grad_out_stride, scale, average_frames, dense,
+                                        WARPCTCT_F32, N, T, U, V, stream);
 }
 
 int warpctct_dense_grad_lattice_f32(const void *workspace, size_t workspace_bytes, const int *ys,
                                     const int *lx, const int *ly, const float *grad_out,
                                     int grad_out_stride, float scale, int average_frames,
                                     float *dense, int N, int T, int U, int V, void *stream) {
-    if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
-    if (N == 0 || T == 0) return WARPCTCT_OK;
-    if (!dense) return WARPCTCT_EINVAL;
-    int rc = done(launch_zero_fill(dense, (size_t)N * T * (U + 1) * V, as_stream(stream)));
-    if (rc != WARPCTCT_OK) return rc;
-    return warpctct_dense_patch_lattice_f32(workspace, workspace_bytes, ys, lx, ly, grad_out,
-                                            grad_out_stride, scale, average_frames, dense, N, T, U,
-                                            V, stream);
+    return warpctct_dense_grad_lattice(workspace, workspace_bytes, ys, lx, ly, grad_out,
+                                       grad_out_stride, scale, average_frames, dense, WARPCTCT_F32,
+                                       N, T, U, V, stream);
+}
+
+int warpctct_zero_fill(void *p, size_t bytes, void *stream) {
+    if (bytes == 0) return WARPCTCT_OK;
+    if (!p) return WARPCTCT_EINVAL;
+    return done(launch_zero_fill_bytes(p, bytes, as_stream(stream)));
 }
 
 int warpctct_loss_forward_f32(const float *joint, const int *ys, const int *lx, const int *ly,
@@ -307,8 +354,8 @@ int warpctct_loss_forward_f32(const float *joint, const int *ys, const int *lx, 
     const Workspace w = carve(workspace, N, T, U);
     if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
     if (T > 0) {
-        int rc = done(launch_gather_units(joint, ys, lx, ly, w.units, N, T, U, V, true,
-                                          as_stream(stream)));
+        int rc = done(launch_gather_units(joint, kIoF32, ys, lx, ly, w.units, N, T, U, V, true,
+                                          nullptr, as_stream(stream)));
         if (rc != WARPCTCT_OK) return rc;
     }
     return forward_from_units(w, ys, lx, ly, N, T, U, costs, T > 0 ? unit_grads : nullptr,

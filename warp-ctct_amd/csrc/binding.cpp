@@ -93,46 +93,73 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_loss_fwd(const torch::Tensor &log_
     return std::make_tuple(costs, costs);   // as the reference, binding.cpp:98
 }
 
-// Fused entry for ctct_loss: takes the un-gathered joint (N,T,U+1,V), so the
-// index build + torch.gather of warp_ctct/__init__.py:124-131 happens inside.
-// Returns (costs, workspace): the workspace (units, alpha, beta) is what
+// Element type of a joint tensor for the C ABI; anything but float, half and
+// bfloat16 is refused (the Python wrapper converts other types to float).
+int io_type_of(const torch::Tensor &t) {
+    switch (t.scalar_type()) {
+        case at::ScalarType::Float: return WARPCTCT_F32;
+        case at::ScalarType::Half: return WARPCTCT_F16;
+        case at::ScalarType::BFloat16: return WARPCTCT_BF16;
+        default: TORCH_CHECK(false, "joint must be float32, float16 or bfloat16");
+    }
+    return -1;
+}
+
+// Fused entry for ctct_loss: takes the un-gathered joint (N,T,U+1,V) of type
+// float, half or bfloat16, so the index build + torch.gather + .float() of
+// warp_ctct/__init__.py:124-136 happen inside, and the reduction of :138-147
+// too: reduction 0 = none, 1 = sum, 2 = mean.  Returns (loss, workspace): loss
+// is the (N,) costs (divided by lx if average_frames) or the reduced scalar,
+// always float32; the workspace (units, alpha, beta) is what
 // dense_patch_lattice needs in backward; without requires_grad only beta runs
-// and costs is returned twice (as the reference does, binding.cpp:98).
+// and loss is returned twice (as the reference does, binding.cpp:98).
 std::tuple<torch::Tensor, torch::Tensor> ctct_loss_joint_fwd(const torch::Tensor &joint,
                                                              const torch::Tensor &ys,
                                                              const torch::Tensor &lx,
                                                              const torch::Tensor &ly,
-                                                             const bool requires_grad) {
+                                                             const bool requires_grad,
+                                                             const int64_t reduction,
+                                                             const bool average_frames) {
     CHECK_CONTIGUOUS(joint);
-    CHECK_FLOAT(joint);
     CHECK_DEVICE(joint);
+    const int dtype = io_type_of(joint);
     TORCH_CHECK(joint.dim() == 4, "log probs must have 4 dims.");
+    TORCH_CHECK(reduction >= 0 && reduction <= 2, "reduction must be 0 (none), 1 (sum), 2 (mean)");
     const int N = joint.size(0), T = joint.size(1), U = joint.size(2) - 1, V = joint.size(3);
     check_lengths(ys, lx, ly, N, U);
     const DeviceGuard device_guard(device_of(joint));
 
     auto ws = make_workspace(joint, N, T, U);
-    auto costs = torch::empty({N}, joint.options());
-    check_rc(warpctct_loss_lattice_f32(joint.data_ptr<float>(), ys.data_ptr<int>(),
-                                       lx.data_ptr<int>(), ly.data_ptr<int>(), N, T, U, V,
-                                       ws.data_ptr(), ws.numel(), costs.data_ptr<float>(),
-                                       requires_grad ? 1 : 0, current_stream()),
+    const auto f32 = joint.options().dtype(at::ScalarType::Float);
+    auto costs = torch::empty({N}, f32);
+    torch::Tensor reduced;
+    if (reduction != 0) reduced = N > 0 ? torch::empty({}, f32) : torch::zeros({}, f32);
+    check_rc(warpctct_loss_lattice(joint.data_ptr(), dtype, ys.data_ptr<int>(),
+                                   lx.data_ptr<int>(), ly.data_ptr<int>(), N, T, U, V,
+                                   ws.data_ptr(), ws.numel(), costs.data_ptr<float>(),
+                                   requires_grad ? 1 : 0, static_cast<int>(reduction),
+                                   average_frames ? 1 : 0,
+                                   reduction != 0 ? reduced.data_ptr<float>() : nullptr,
+                                   current_stream()),
              "ctct_loss_joint_fwd");
-    if (requires_grad) return std::make_tuple(costs, ws);
-    return std::make_tuple(costs, costs);
+    const torch::Tensor &loss = reduction != 0 ? reduced : costs;
+    if (requires_grad) return std::make_tuple(loss, ws);
+    return std::make_tuple(loss, loss);
 }
 
 // The two halves of the dense gradient as separate operators, so that a caller
-// can bracket the zero-fill kernel alone with HIP events.
+// can bracket the zero-fill kernel alone with HIP events.  `like` gives the
+// device and the element type (float, half or bfloat16).
 torch::Tensor dense_zero_fill(const torch::Tensor &like, const int64_t N, const int64_t T,
                               const int64_t U1, const int64_t V) {
     CHECK_DEVICE(like);
-    CHECK_FLOAT(like);
+    io_type_of(like);
     TORCH_CHECK(N >= 0 && T >= 0 && U1 >= 1 && V >= 1, "invalid sizes");
     const DeviceGuard device_guard(device_of(like));
     auto dense = torch::empty({N, T, U1, V}, like.options());
-    check_rc(warpctct_zero_fill_f32(dense.data_ptr<float>(), static_cast<size_t>(dense.numel()),
-                                    current_stream()),
+    check_rc(warpctct_zero_fill(dense.data_ptr(),
+                                static_cast<size_t>(dense.numel()) * dense.element_size(),
+                                current_stream()),
              "dense_zero_fill");
     return dense;
 }
@@ -151,18 +178,18 @@ void dense_patch_lattice(const torch::Tensor &workspace, const torch::Tensor &ys
     CHECK_FLOAT(grad_out);
     CHECK_DEVICE(grad_out);
     CHECK_CONTIGUOUS(dense);
-    CHECK_FLOAT(dense);
     CHECK_DEVICE(dense);
+    const int dtype = io_type_of(dense);
     TORCH_CHECK(dense.dim() == 4, "dense must be (N,T,U+1,V)");
     const int N = dense.size(0), T = dense.size(1), U = dense.size(2) - 1, V = dense.size(3);
     TORCH_CHECK(grad_out.numel() == N || grad_out.numel() == 1, "grad_out must have N or 1 elements");
     check_lengths(ys, lx, ly, N, U);
     const DeviceGuard device_guard(device_of(dense));
     const int stride = (grad_out.numel() == 1 && N > 1) ? 0 : 1;
-    check_rc(warpctct_dense_patch_lattice_f32(
+    check_rc(warpctct_dense_patch_lattice(
                  workspace.data_ptr(), workspace.numel(), ys.data_ptr<int>(), lx.data_ptr<int>(),
                  ly.data_ptr<int>(), grad_out.data_ptr<float>(), stride, static_cast<float>(scale),
-                 average_frames ? 1 : 0, dense.data_ptr<float>(), N, T, U, V, current_stream()),
+                 average_frames ? 1 : 0, dense.data_ptr(), dtype, N, T, U, V, current_stream()),
              "dense_patch_lattice");
 }
 
@@ -454,7 +481,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("ctct_loss_joint_fwd", &ctct_loss_joint_fwd,
           "CTC-Transducer loss on the un-gathered joint (forward).", pybind11::arg("log_probs"),
           pybind11::arg("ys"), pybind11::arg("lx"), pybind11::arg("ly"),
-          pybind11::arg("requires_grad"));
+          pybind11::arg("requires_grad"), pybind11::arg("reduction") = 0,
+          pybind11::arg("average_frames") = false);
     m.def("ctct_loss_joint_bwd", &ctct_loss_joint_bwd,
           "Dense gradient wrt the joint from unit gradients.", pybind11::arg("unit_grads"),
           pybind11::arg("ys"), pybind11::arg("lx"), pybind11::arg("ly"),

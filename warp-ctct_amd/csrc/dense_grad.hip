@@ -36,17 +36,19 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kBlock = 256;
 
+// p[i] = 0 for i < n bytes, for the few bytes before and after the 16-byte
+// aligned body of a buffer.
+__global__ __launch_bounds__(kBlock) void zero_fill_byte_kernel(unsigned char *__restrict__ p,
+                                                                size_t n) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
 // p4[i] = 0 for i < n4: one store per thread, no loop.
 __global__ __launch_bounds__(kBlock) void zero_fill_vec_kernel(v4f *__restrict__ p4, size_t n4) {
     const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
     const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};
     if (i < n4) p4[i] = z;
-}
-
-__global__ __launch_bounds__(kBlock) void zero_fill_scalar_kernel(float *__restrict__ p,
-                                                                  size_t n) {
-    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i < n) p[i] = 0.0f;
 }
 
 // Per-sample weight of the upstream gradient: grad_out[n * stride] (stride 0
@@ -70,7 +72,8 @@ __device__ __forceinline__ float sample_weight(const Weight &w, int n, int lxn) 
 // Writes (not adds) the non-zero entries of row (n,t,u) of the dense gradient:
 // columns 0, y[u-1], y[u]; columns that coincide are summed first so that
 // every element is written by exactly one store.
-__device__ __forceinline__ void patch_row(float *out, const int *y, int u, int Un, int V, float v0,
+template <typename IO>
+__device__ __forceinline__ void patch_row(IO *out, const int *y, int u, int Un, int V, float v0,
                                           float v1, float v2) {
     const bool has1 = (u >= 1), has2 = (u < Un);
     const int c1 = has1 ? min(max(y[u - 1], 0), V - 1) : -1;
@@ -83,20 +86,20 @@ __device__ __forceinline__ void patch_row(float *out, const int *y, int u, int U
     }
     if (c1 == 0) v0 += v1;   // a label equal to the blank index
     if (c2 == 0) v0 += v2;
-    out[0] = v0;
-    if (c1 > 0) out[c1] = v1;
-    if (c2 > 0 && c2 != c1) out[c2] = v2;
+    store_from_float(out, v0);
+    if (c1 > 0) store_from_float(out + c1, v1);
+    if (c2 > 0 && c2 != c1) store_from_float(out + c2, v2);
 }
 
 // One thread per cell (t,u) of sample blockIdx.y; FROM_LATTICE computes the
 // unit gradients on the fly from units / alpha / beta (work-buffer layout, P
 // contexts per frame), otherwise they are read from the (N,T,U+1,3) tensor.
-template <bool FROM_LATTICE>
+template <bool FROM_LATTICE, typename IO>
 __global__ __launch_bounds__(kBlock) void patch_kernel(
     const float *__restrict__ unit_grads, const double *__restrict__ units,
     const double *__restrict__ alphas, const double *__restrict__ betas,
     const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
-    Weight weight, float *__restrict__ dense, int T, int U, int V, int P) {
+    Weight weight, IO *__restrict__ dense, int T, int U, int V, int P) {
     const int U1 = U + 1;
     const int n = blockIdx.y;
     const int cell = blockIdx.x * kBlock + threadIdx.x;
@@ -127,18 +130,16 @@ __global__ __launch_bounds__(kBlock) void patch_kernel(
 
 }  // namespace
 
-hipError_t launch_zero_fill(float *p, size_t n, hipStream_t stream) {
-    if (n == 0) return hipSuccess;
-    // leading floats up to the first 16-byte boundary, then vectors, then the tail
-    const uintptr_t addr = reinterpret_cast<uintptr_t>(p);
-    size_t head = ((16 - (addr & 15u)) & 15u) / sizeof(float);
-    if ((addr & 3u) != 0) head = n;   // not even float-aligned: all scalar
-    if (head > n) head = n;
-    const size_t n4 = (n - head) / 4;
-    const size_t tail = n - head - n4 * 4;
+hipError_t launch_zero_fill_bytes(void *ptr, size_t bytes, hipStream_t stream) {
+    if (bytes == 0) return hipSuccess;
+    // leading bytes up to the first 16-byte boundary, then vectors, then the tail
+    unsigned char *p = static_cast<unsigned char *>(ptr);
+    size_t head = (16 - (reinterpret_cast<uintptr_t>(p) & 15u)) & 15u;
+    if (head > bytes) head = bytes;
+    const size_t n4 = (bytes - head) / 16;
+    const size_t tail = bytes - head - n4 * 16;
     if (head) {
-        hipLaunchKernelGGL(zero_fill_scalar_kernel, dim3((unsigned)((head + kBlock - 1) / kBlock)),
-                           dim3(kBlock), 0, stream, p, head);
+        hipLaunchKernelGGL(zero_fill_byte_kernel, dim3(1), dim3(kBlock), 0, stream, p, head);
     }
     if (n4) {
         const size_t blocks = (n4 + kBlock - 1) / kBlock;
@@ -147,10 +148,14 @@ hipError_t launch_zero_fill(float *p, size_t n, hipStream_t stream) {
                            reinterpret_cast<v4f *>(p + head), n4);
     }
     if (tail) {
-        hipLaunchKernelGGL(zero_fill_scalar_kernel, dim3(1), dim3(kBlock), 0, stream,
-                           p + head + n4 * 4, tail);
+        hipLaunchKernelGGL(zero_fill_byte_kernel, dim3(1), dim3(kBlock), 0, stream,
+                           p + head + n4 * 16, tail);
     }
     return hipGetLastError();
+}
+
+hipError_t launch_zero_fill(float *p, size_t n, hipStream_t stream) {
+    return launch_zero_fill_bytes(p, n * sizeof(float), stream);
 }
 
 hipError_t launch_dense_patch(const float *unit_grads, const int *ys, const int *lx,
@@ -160,22 +165,40 @@ hipError_t launch_dense_patch(const float *unit_grads, const int *ys, const int 
     if (cells == 0 || N == 0) return hipSuccess;
     dim3 grid((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N);
     const Weight w = {grad_out, 1, 1.0f, 0};
-    hipLaunchKernelGGL(patch_kernel<false>, grid, dim3(kBlock), 0, stream, unit_grads, nullptr,
-                       nullptr, nullptr, ys, lx, ly, w, dense, T, U, V, 0);
+    hipLaunchKernelGGL((patch_kernel<false, float>), grid, dim3(kBlock), 0, stream, unit_grads,
+                       nullptr, nullptr, nullptr, ys, lx, ly, w, dense, T, U, V, 0);
     return hipGetLastError();
 }
 
 hipError_t launch_dense_patch_lattice(const double *units, const double *alphas,
                                       const double *betas, const int *ys, const int *lx,
                                       const int *ly, const float *grad_out, int grad_out_stride,
-                                      float scale, int average_frames, float *dense, int N, int T,
-                                      int U, int V, hipStream_t stream) {
+                                      float scale, int average_frames, void *dense, int io_type,
+                                      int N, int T, int U, int V, hipStream_t stream) {
     const long cells = (long)T * (U + 1);
     if (cells == 0 || N == 0) return hipSuccess;
     dim3 grid((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N);
     const Weight w = {grad_out, grad_out_stride, scale, average_frames};
-    hipLaunchKernelGGL(patch_kernel<true>, grid, dim3(kBlock), 0, stream, nullptr, units, alphas,
-                       betas, ys, lx, ly, w, dense, T, U, V, padded_contexts(U));
+    const int P = padded_contexts(U);
+    switch (io_type) {
+        case kIoF32:
+            hipLaunchKernelGGL((patch_kernel<true, float>), grid, dim3(kBlock), 0, stream, nullptr,
+                               units, alphas, betas, ys, lx, ly, w, static_cast<float *>(dense), T,
+                               U, V, P);
+            break;
+        case kIoF16:
+            hipLaunchKernelGGL((patch_kernel<true, __half>), grid, dim3(kBlock), 0, stream,
+                               nullptr, units, alphas, betas, ys, lx, ly, w,
+                               static_cast<__half *>(dense), T, U, V, P);
+            break;
+        case kIoBF16:
+            hipLaunchKernelGGL((patch_kernel<true, __hip_bfloat16>), grid, dim3(kBlock), 0, stream,
+                               nullptr, units, alphas, betas, ys, lx, ly, w,
+                               static_cast<__hip_bfloat16 *>(dense), T, U, V, P);
+            break;
+        default:
+            return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

@@ -3,9 +3,25 @@
 // wavefront data movement through DPP.
 #pragma once
 
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
 namespace wctct {
+
+// Element types of the joint tensor and of its dense gradient: the lattice
+// always computes in fp32 / fp64, only the loads and stores at the two ends
+// differ.  Stores round to nearest even.
+__device__ __forceinline__ float load_as_float(const float *p) { return *p; }
+__device__ __forceinline__ float load_as_float(const __half *p) { return __half2float(*p); }
+__device__ __forceinline__ float load_as_float(const __hip_bfloat16 *p) {
+    return __bfloat162float(*p);
+}
+__device__ __forceinline__ void store_from_float(float *p, float v) { *p = v; }
+__device__ __forceinline__ void store_from_float(__half *p, float v) { *p = __float2half(v); }
+__device__ __forceinline__ void store_from_float(__hip_bfloat16 *p, float v) {
+    *p = __float2bfloat16(v);
+}
 
 constexpr int kWave = 64;
 constexpr double kLog2e = 1.4426950408889634074;

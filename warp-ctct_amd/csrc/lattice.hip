@@ -243,7 +243,8 @@ __global__ __launch_bounds__(64 * W) void lattice_kernel(const double *__restric
                                                          const int *__restrict__ ly,
                                                          double *__restrict__ alphas,
                                                          double *__restrict__ betas,
-                                                         float *__restrict__ costs, int T, int U) {
+                                                         float *__restrict__ costs, int T, int U,
+                                                         const CostReduce red) {
     __shared__ Relay<W> relay;
     const int n = blockIdx.x;
     constexpr int P = 64 * W;
@@ -261,17 +262,42 @@ __global__ __launch_bounds__(64 * W) void lattice_kernel(const double *__restric
     const double *units_n = units + (size_t)n * T * P * 3;
     const int *y = ys + (size_t)n * U;
     const size_t lat = (size_t)(T + 1) * P * 2;
-    if (blockIdx.y == 0)
-        sweep<W, true>(units_n, y, Tn, Un, betas + (size_t)n * lat, costs + n, relay);
-    else
+    if (blockIdx.y != 0) {
         sweep<W, false>(units_n, y, Tn, Un, alphas + (size_t)n * lat, nullptr, relay);
+        return;
+    }
+    sweep<W, true>(units_n, y, Tn, Un, betas + (size_t)n * lat, costs + n, relay);
+    if (threadIdx.x >= 64) return;
+    // thread 0 (context 0) has just written costs[n]
+    if (red.average_frames && threadIdx.x == 0) costs[n] /= (float)lx[n];
+    if (red.reduced == nullptr) return;
+    // Reduction over the batch (warp_ctct/__init__.py:142-147 of the reference)
+    // by the workgroup that finishes last: every workgroup publishes its cost
+    // (release fence), then counts itself; the one that sees N-1 earlier
+    // arrivals reads all N costs (acquire fence) and adds them in a fixed
+    // order, so the result does not depend on the order of arrival.
+    const int N = gridDim.x;
+    int last = 0;
+    if (threadIdx.x == 0) {
+        __threadfence();
+        last = (atomicAdd(red.counter, 1u) == (unsigned)(N - 1)) ? 1 : 0;
+    }
+    last = __shfl(last, 0, 64);
+    if (!last) return;
+    __threadfence();
+    float s = 0.0f;
+    for (int i = threadIdx.x; i < N; i += 64)
+        s += __hip_atomic_load(costs + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) s += __shfl_xor(s, off, 64);
+    if (threadIdx.x == 0) *red.reduced = (red.mode == 2) ? s / (float)N : s;
 }
 
 template <int W>
 hipError_t launch_lattice_w(const LatticeArgs &a, hipStream_t stream) {
     dim3 grid(a.N, a.beta_only ? 1 : 2);
     hipLaunchKernelGGL((lattice_kernel<W>), grid, dim3(64 * W), 0, stream, a.units, a.ys, a.lx,
-                       a.ly, a.alphas, a.betas, a.costs, a.T, a.U);
+                       a.ly, a.alphas, a.betas, a.costs, a.T, a.U, a.reduce);
     return hipGetLastError();
 }
 

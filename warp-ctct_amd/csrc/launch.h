@@ -12,6 +12,21 @@ namespace wctct {
 // stores without lane masks.
 inline int padded_contexts(int U) { return ((U + 1 + 63) / 64) * 64; }
 
+// Element type of the joint tensor / its dense gradient (values of the C ABI).
+enum IoType { kIoF32 = 0, kIoF16 = 1, kIoBF16 = 2 };
+inline size_t io_size(int t) { return t == kIoF32 ? 4 : 2; }
+inline bool io_valid(int t) { return t == kIoF32 || t == kIoF16 || t == kIoBF16; }
+
+// Reduction over the batch folded into the lattice kernel: the workgroup that
+// finishes last (counted in *counter, which must be 0 at launch) adds up the N
+// costs in a fixed order.  mode 0 = none, 1 = sum, 2 = mean.
+struct CostReduce {
+    float *reduced;       // 1 float, or null
+    unsigned *counter;
+    int mode;
+    int average_frames;   // costs[n] /= lx[n] before anything else
+};
+
 struct LatticeArgs {
     const double *units;  // (N,T,P,3) log2 units, neutral values in the padding
     const int *ys;        // (N,U)
@@ -22,6 +37,7 @@ struct LatticeArgs {
     float *costs;         // (N)
     int N, T, U;
     bool beta_only;
+    CostReduce reduce;    // zero-initialise for plain per-sample costs
 };
 
 int lattice_max_contexts();
@@ -29,9 +45,11 @@ hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream);
 
 // band_only: cells outside the band of complete alignments get neutral units
 // (same costs and gradients; alpha / beta of dead cells are not the oracle's)
-hipError_t launch_gather_units(const float *joint, const int *ys, const int *lx, const int *ly,
-                               double *units, int N, int T, int U, int V, bool band_only,
-                               hipStream_t stream);
+// counter (may be null): set to 0 by the kernel, for a CostReduce that follows
+hipError_t launch_gather_units(const void *joint, int io_type, const int *ys, const int *lx,
+                               const int *ly, double *units, int N, int T, int U, int V,
+                               bool band_only, unsigned *counter, hipStream_t stream);
+hipError_t launch_clear_counter(unsigned *counter, hipStream_t stream);
 hipError_t launch_scale_units(const float *units_nat, const int *lx, const int *ly, double *units,
                               int N, int T, int U, hipStream_t stream);
 hipError_t launch_simple_units(const float *f_g, const float *g_g, const float *den,
@@ -54,8 +72,8 @@ hipError_t launch_dense_patch(const float *unit_grads, const int *ys, const int 
 hipError_t launch_dense_patch_lattice(const double *units, const double *alphas,
                                       const double *betas, const int *ys, const int *lx,
                                       const int *ly, const float *grad_out, int grad_out_stride,
-                                      float scale, int average_frames, float *dense, int N, int T,
-                                      int U, int V, hipStream_t stream);
+                                      float scale, int average_frames, void *dense, int io_type,
+                                      int N, int T, int U, int V, hipStream_t stream);
 
 // ---- log-add joiner path -------------------------------------------------
 hipError_t launch_simple_gather_units(const float *f, const float *g, const float *den,
@@ -68,6 +86,7 @@ hipError_t launch_simple_scatter(const float *grad_f, const float *grad_g, const
                                  float *dense_f, float *dense_g, int N, int T, int U, int V,
                                  hipStream_t stream);
 hipError_t launch_zero_fill(float *p, size_t n, hipStream_t stream);
+hipError_t launch_zero_fill_bytes(void *p, size_t bytes, hipStream_t stream);
 
 // ---- log-semiring matmul -------------------------------------------------
 // A strided 3-d operand: element [b, i1, i2] lives at p[b*sb + i1*s1 + i2*s2].

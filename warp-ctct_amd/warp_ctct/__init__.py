@@ -66,38 +66,44 @@ def _reduce(costs, frames_lengths, reduction, average_frames):
     return costs
 
 
+_REDUCTION_CODE = {None: 0, "none": 0, "sum": 1, "mean": 2}
+_NATIVE_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
+
+
 class _CTCTLoss(torch.autograd.Function):
     """ctct_loss on the un-gathered joint, reduction included.
 
-    Counterpart of the reference's gather (warp_ctct/__init__.py:124-131),
-    CTCTLoss (:20-33) and the reduction (:138-147).  Forward runs gather and
-    both lattices on the GPU and keeps their workspace; backward zero-fills
-    the dense gradient at full HBM write bandwidth and then writes the <= 3
-    non-zero entries per live row, already weighted by the upstream gradient
-    and by the reduction's own factor (1/N, 1/lx[n]), so autograd launches
-    nothing else."""
+    Counterpart of the reference's gather (warp_ctct/__init__.py:124-131), the
+    cast to float (:135), CTCTLoss (:20-33) and the reduction (:138-147).
+    Forward runs gather, both lattices and the batch reduction on the GPU and
+    keeps their workspace; backward zero-fills the dense gradient at full HBM
+    write bandwidth and then writes the <= 3 non-zero entries per live row,
+    already weighted by the upstream gradient and by the reduction's own
+    factor (1/N, 1/lx[n]), so autograd launches nothing else.  A float16 or
+    bfloat16 joint is read as it is and its gradient is written in the same
+    type (the lattice itself always runs in float32 / float64)."""
 
     @staticmethod
-    def forward(ctx, joint, labels, lx, ly, frames_lengths, requires_grad, reduction,
-                average_frames):
-        costs, workspace = _run("loss_forward", lambda: core.ctct_loss_joint_fwd(
-            joint, labels, lx, ly, requires_grad))
+    def forward(ctx, joint, labels, lx, ly, requires_grad, reduction, average_frames):
+        loss, workspace = _run("loss_forward", lambda: core.ctct_loss_joint_fwd(
+            joint, labels, lx, ly, requires_grad, _REDUCTION_CODE[reduction], average_frames))
         if requires_grad:
             ctx.save_for_backward(workspace, labels, lx, ly)
             ctx.shape = tuple(joint.shape)
+            ctx.like = joint.new_empty(0)
             ctx.scale = 1.0 / joint.size(0) if reduction == "mean" else 1.0
             ctx.average_frames = bool(average_frames)
-        return _reduce(costs, frames_lengths, reduction, average_frames)
+        return loss
 
     @staticmethod
     def backward(ctx, grad_outputs):
         workspace, labels, lx, ly = ctx.saved_tensors
         n, t, u1, v = ctx.shape
         grad_outputs = grad_outputs.reshape(-1).float().contiguous()
-        dense = _run("dense_zero_fill", lambda: core.dense_zero_fill(grad_outputs, n, t, u1, v))
+        dense = _run("dense_zero_fill", lambda: core.dense_zero_fill(ctx.like, n, t, u1, v))
         _run("dense_patch", lambda: core.dense_patch_lattice(
             workspace, labels, lx, ly, grad_outputs, ctx.scale, ctx.average_frames, dense))
-        return dense, None, None, None, None, None, None, None
+        return dense, None, None, None, None, None, None
 
 
 class _SimpleCTCTLoss(torch.autograd.Function):
@@ -157,10 +163,12 @@ def ctct_loss(log_probs: torch.Tensor,
     assert log_probs.size(0) == labels.size(0) == frames_lengths.size(0) == labels_lengths.size(0)
 
     enable_grad = log_probs.requires_grad and torch.is_grad_enabled()
+    if log_probs.dtype not in _NATIVE_DTYPES:
+        log_probs = log_probs.float()      # as the reference does for every dtype (:135)
     with _no_autocast():
-        return _CTCTLoss.apply(log_probs.float().contiguous(), _as_int(labels),
-                               _as_int(frames_lengths), _as_int(labels_lengths), frames_lengths,
-                               enable_grad, reduction, bool(average_frames))
+        return _CTCTLoss.apply(log_probs.contiguous(), _as_int(labels), _as_int(frames_lengths),
+                               _as_int(labels_lengths), enable_grad, reduction,
+                               bool(average_frames))
 
 
 def ctct_simple_loss(f: torch.Tensor,
