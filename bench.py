@@ -85,7 +85,11 @@ OTHER = {
     "c3": ("full", 8, 500, 120, 4096, 2.0),
     "c4": ("simple_norm", 32, 400, 80, 2048, 1.0),
     "c5": ("simple_unnorm", 4, 1500, 300, 8192, 1.0),
+    # the typical batch with a half-precision joint (half the bytes at both ends)
+    "c2_bf16": ("full", 32, 250, 60, 1024, 1.0),
+    "c2_f16": ("full", 32, 250, 60, 1024, 1.0),
 }
+IO_DTYPE = {"c2_bf16": "bfloat16", "c2_f16": "float16"}
 
 
 def other_config(args, torch, warp_ctct):
@@ -99,8 +103,8 @@ def other_config(args, torch, warp_ctct):
         lx = np.full(N, T, np.int32)
         ly = np.full(N, U, np.int32)
     else:
-        lo_t = {"c3": 400, "c4": 300, "c5": 1200}[args.config]
-        lo_u = {"c3": 80, "c4": 50, "c5": 250}[args.config]
+        lo_t = {"c3": 400, "c4": 300, "c5": 1200}.get(args.config, 150)
+        lo_u = {"c3": 80, "c4": 50, "c5": 250}.get(args.config, 30)
         lx = rng.integers(lo_t, T + 1, N).astype(np.int32)
         ly = rng.integers(lo_u, U + 1, N).astype(np.int32)
         lx[0], ly[1] = T, U
@@ -113,9 +117,10 @@ def other_config(args, torch, warp_ctct):
         t_idx = torch.arange(T, device="cuda")[None, :, None, None]
         u_idx = torch.arange(U + 1, device="cuda")[None, None, :, None]
         joint.masked_fill_((t_idx >= d_lx[:, None, None, None]) | (u_idx > d_ly[:, None, None, None]), 0.0)
-        joint.requires_grad_(True)
+        io = getattr(torch, IO_DTYPE.get(args.config, "float32"))
+        joint = joint.to(io).requires_grad_(True)
         leaves = (joint,)
-        alg_bytes = 4 * N * T * (U + 1) * V + 12 * live + 4 * N * (U + 3)
+        alg_bytes = joint.element_size() * (N * T * (U + 1) * V + 3 * live) + 4 * N * (U + 3)
 
         def loss_fn():
             return warp_ctct.ctct_loss(joint, d_ys, d_lx, d_ly)
@@ -164,6 +169,7 @@ def other_config(args, torch, warp_ctct):
         "metric": "lattices/sec (loss+grad)", "value": N * args.steps / elapsed,
         "unit": "lattices/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "dtype": "f32", "data": "synthetic",
+        "io_dtype": IO_DTYPE.get(args.config, "float32"),
         "config": {"workload": args.config, "kind": kind, "N": N, "T": T, "U": U, "V": V,
                    "algorithmic_bytes_per_step": alg_bytes,
                    "step_frac_of_hbm_roofline": alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
@@ -177,7 +183,7 @@ def main():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"],
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "c2_bf16", "c2_f16"],
                     help="workload: c2 (default) is the configuration the headline metric is "
                          "quoted on; the others are the remaining BASELINE.json configurations "
                          "and print a reduced line (no cpu_baseline)")
