@@ -158,6 +158,27 @@ int warpctct_dense_patch_lattice(const void *workspace, size_t workspace_bytes, 
  * in a HIP graph). */
 int warpctct_zero_fill(void *p, size_t bytes, void *stream);
 
+/* ---- ctct_loss on logits --------------------------------------------------
+ * The step before the reference's path fused into it: a caller of the
+ * reference computes log_probs = logits.log_softmax(-1) and passes it to
+ * warp_ctct.ctct_loss (warp_ctct/__init__.py:88-147); here the row-wise
+ * logsumexp is taken inside the gather and the backward of log_softmax inside
+ * the kernel that writes the dense gradient, so the log-probability tensor and
+ * its gradient never exist.  Same arguments and results as
+ * warpctct_loss_lattice / warpctct_dense_grad_lattice, with logits (N,T,U+1,V)
+ * in place of the joint and d(loss)/d(logits) in place of the dense gradient;
+ * the workspace is larger (it also holds the logsumexp of every live row). */
+size_t warpctct_logits_workspace_bytes(int N, int T, int U);
+int warpctct_logits_loss_lattice(const void *logits, int dtype, const int *ys, const int *lx,
+                                 const int *ly, int N, int T, int U, int V, void *workspace,
+                                 size_t workspace_bytes, float *costs, int want_alpha,
+                                 int reduction, int average_frames, float *reduced, void *stream);
+int warpctct_logits_grad_lattice(const void *workspace, size_t workspace_bytes,
+                                 const void *logits, int dtype, const int *ys, const int *lx,
+                                 const int *ly, const float *grad_out, int grad_out_stride,
+                                 float scale, int average_frames, void *grad_logits, int N, int T,
+                                 int U, int V, void *stream);
+
 /* The same without unit gradients: gather + lattices only.  The workspace then
  * holds everything the dense gradient needs (units, alpha, beta) and must be
  * kept until warpctct_dense_grad_lattice_f32 has run.  want_alpha == 0 is the

@@ -321,6 +321,25 @@ def ctct_loss(joint, ys, lx, ly, reduction="mean", average_frames=False, grad_ou
 # --------------------------------------------------------------------------
 # simple (log-add joiner) path
 # --------------------------------------------------------------------------
+def ctct_loss_with_logits(logits, ys, lx, ly, reduction="mean", average_frames=False,
+                          grad_output=None):
+    """ctct_loss on log_softmax(logits) and its gradient wrt the logits.
+
+    What a caller of the reference computes as
+    warp_ctct.ctct_loss(logits.log_softmax(-1), ...) (warp_ctct/__init__.py:88-147)
+    plus autograd through log_softmax: with G = d(loss)/d(log_probs),
+    d(loss)/d(logits) = G - softmax(logits) * sum_v G.
+    Returns (loss, grad_logits, costs).
+    """
+    logits = np.asarray(logits, dtype=np.float64)
+    m = logits.max(axis=-1, keepdims=True)
+    lse = m + np.log(np.exp(logits - m).sum(axis=-1, keepdims=True))
+    log_probs = logits - lse
+    loss, G, costs = ctct_loss(log_probs, ys, lx, ly, reduction, average_frames, grad_output)
+    grad = G - np.exp(log_probs) * G.sum(axis=-1, keepdims=True)
+    return loss, grad, costs
+
+
 def simple_unit_grad_reduce(g, normalized):
     """Unit grads (N,T,U+1,3) -> (grad_f_g (N,T,U+1), grad_g_g (N,U+1,3),
     grad_den (N,T,U+1) or None).  Follows csrc/binding.cpp:198-219."""

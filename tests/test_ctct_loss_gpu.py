@@ -295,6 +295,67 @@ def test_batch_reduction_is_deterministic_and_handles_large_batches():
     np.testing.assert_allclose(af.item(), (ref_costs / lx).mean(), rtol=LOSS_RTOL)
 
 
+LOGITS_CASES = [
+    # name, seed, N, T, U, V, lx, ly, sigma, dtype
+    ("small_f32", 41, 3, 17, 5, 37, range(8, 18), range(2, 6), 2.0, torch.float32),
+    ("vector_rows_f32", 42, 2, 30, 12, 1024, [30, 21], [12, 7], 3.0, torch.float32),
+    ("two_wavefronts_f32", 43, 2, 90, 70, 24, [90, 80], [70, 66], 1.0, torch.float32),
+    ("bf16", 44, 3, 20, 6, 64, range(10, 21), range(2, 7), 2.0, torch.bfloat16),
+    ("f16_odd_vocab", 45, 2, 14, 4, 33, [14, 9], [4, 3], 2.0, torch.float16),
+]
+
+
+@pytest.mark.parametrize("case", LOGITS_CASES, ids=[c[0] for c in LOGITS_CASES])
+@pytest.mark.parametrize("reduction", ["none", "mean"])
+def test_loss_with_logits(case, reduction):
+    """ctct_loss_with_logits(x) == ctct_loss(log_softmax(x)): loss and
+    d(loss)/d(logits) against the float64 oracle on the same (rounded)
+    logits; rows of padding and rows outside the band get exact zeros."""
+    import warp_ctct
+    _, seed, N, T, U, V, lxs, lys, sigma, dtype = case
+    _, ys, lx, ly = make_joint_case(seed, N, T, U, V, lx=lxs, ly=lys)
+    rng = np.random.default_rng(seed)
+    logits = (rng.standard_normal((N, T, U + 1, V)) * sigma + rng.standard_normal((N, T, U + 1, 1)) * 5)
+    x = dev(logits.astype(np.float32)).to(dtype).requires_grad_(True)
+    rounded = x.detach().double().cpu().numpy()
+    w = np.linspace(0.5, 2.0, N)
+    ref_loss, ref_grad, _ = O.ctct_loss_with_logits(
+        rounded, ys, lx, ly, reduction, False, grad_output=w if reduction == "none" else None)
+    loss = warp_ctct.ctct_loss_with_logits(x, dev(ys), dev(lx), dev(ly), reduction=reduction)
+    assert loss.dtype == torch.float32
+    np.testing.assert_allclose(loss.detach().cpu().numpy(), ref_loss, rtol=LOSS_RTOL)
+    if reduction == "none":
+        loss.backward(dev(w, torch.float32))
+    else:
+        loss.backward()
+    assert x.grad.dtype == dtype and x.grad.shape == x.shape
+    got = x.grad.double().cpu().numpy()
+    ulp = {torch.float32: 0.0, torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+    assert np.all(np.abs(got - ref_grad) <= GRAD_ATOL + ulp * np.abs(ref_grad))
+    dead = np.abs(ref_grad).sum(-1) == 0
+    assert np.all(got[dead] == 0), "rows without gradient must be exact zeros"
+    # the unfused route through torch.log_softmax gives the same loss
+    with torch.no_grad():
+        unfused = warp_ctct.ctct_loss(x.float().log_softmax(-1), dev(ys), dev(lx), dev(ly),
+                                      reduction=reduction)
+        fused = warp_ctct.ctct_loss_with_logits(x, dev(ys), dev(lx), dev(ly), reduction=reduction)
+    assert not fused.requires_grad
+    np.testing.assert_allclose(fused.cpu().numpy(), unfused.cpu().numpy(), rtol=LOSS_RTOL)
+
+
+def test_loss_with_logits_average_frames_and_sum():
+    import warp_ctct
+    _, ys, lx, ly = make_joint_case(46, 4, 15, 4, 19, lx=range(7, 16), ly=range(1, 5))
+    logits = np.random.default_rng(46).standard_normal((4, 15, 5, 19)).astype(np.float32) * 2
+    x = dev(logits).requires_grad_(True)
+    ref_loss, ref_grad, _ = O.ctct_loss_with_logits(logits, ys, lx, ly, "sum", True)
+    loss = warp_ctct.ctct_loss_with_logits(x, dev(ys), dev(lx), dev(ly), reduction="sum",
+                                           average_frames=True)
+    np.testing.assert_allclose(loss.item(), ref_loss, rtol=LOSS_RTOL)
+    loss.backward()
+    np.testing.assert_allclose(x.grad.cpu().numpy(), ref_grad, atol=GRAD_ATOL, rtol=0)
+
+
 def test_operator_surface_on_gathered_units():
     """_C.ctct_loss_fwd keeps the reference's contract: gathered (N,T,U+1,3)
     input, (costs, grads) output, grads zero in padding, costs twice when

@@ -146,6 +146,39 @@ def test_unit_grads_match_finite_differences():
                 assert abs(fd - g[0, t, u, k]) < 1e-8
 
 
+def test_logits_variant_against_library_log_softmax_and_finite_differences():
+    """ctct_loss_with_logits: the loss is ctct_loss of torch.log_softmax's
+    output; the gradient is what torch's own log_softmax backward makes of the
+    (already pinned) gradient wrt the log-probabilities, and it matches central
+    differences of the loss wrt single logits (a dropped softmax term or a
+    wrong sign of the row sum fails both)."""
+    rng = np.random.default_rng(77)
+    N, T, U, V = 2, 6, 3, 5
+    logits = rng.standard_normal((N, T, U + 1, V)) * 2.0
+    ys = np.array([[1, 1, 3], [4, 2, 2]])
+    lx, ly = np.array([6, 5]), np.array([3, 2])
+    w = np.array([0.7, 1.9])
+    loss, grad, costs = O.ctct_loss_with_logits(logits, ys, lx, ly, "none", False, grad_output=w)
+    x = torch.tensor(logits, requires_grad=True)
+    lp = torch.log_softmax(x, dim=-1)
+    ref_loss, G, ref_costs = O.ctct_loss(lp.detach().numpy(), ys, lx, ly, "none", False,
+                                         grad_output=w)
+    np.testing.assert_allclose(costs, ref_costs, rtol=1e-12)
+    lp.backward(torch.tensor(G))
+    np.testing.assert_allclose(grad, x.grad.numpy(), rtol=1e-10, atol=1e-13)
+    assert np.all(grad[0, :, :, :][np.abs(G[0]).sum(-1) == 0] == 0)   # untouched rows stay zero
+    eps = 1e-6
+    for idx in [(0, 0, 0, 0), (0, 2, 1, 1), (0, 4, 2, 3), (1, 3, 1, 2), (1, 1, 0, 4)]:
+        p, m = logits.copy(), logits.copy()
+        p[idx] += eps
+        m[idx] -= eps
+        fd = (O.ctct_loss_with_logits(p, ys, lx, ly, "none")[2] @ w
+              - O.ctct_loss_with_logits(m, ys, lx, ly, "none")[2] @ w) / (2 * eps)
+        assert abs(fd - grad[idx]) < 1e-7
+    # rows sum to zero: log_softmax removes the direction of constant shifts
+    assert np.max(np.abs(grad.sum(-1))) < 1e-12
+
+
 def test_gather_closed_form():
     joint, ys, _, _ = make_joint_case(4, 2, 5, 3, 7, dtype=np.float64, zero_pad=False)
     lp3 = O.gather_units(joint, ys)

@@ -338,6 +338,88 @@ int warpctct_dense_grad_lattice_f32(const void *workspace, size_t workspace_byte
                                        N, T, U, V, stream);
 }
 
+namespace {
+
+// Lattice workspace followed by the row-wise logsumexp (N,T,U+1) of the logits.
+struct LogitsWorkspace {
+    Workspace lattice;
+    float *lse;
+    size_t bytes;
+};
+
+LogitsWorkspace carve_logits(void *base, int N, int T, int U) {
+    LogitsWorkspace w;
+    w.lattice = carve(base, N, T, U);
+    w.lse = reinterpret_cast<float *>(reinterpret_cast<uintptr_t>(base) + w.lattice.bytes);
+    w.bytes = w.lattice.bytes + align256((size_t)N * T * (U + 1) * sizeof(float));
+    return w;
+}
+
+}  // namespace
+
+size_t warpctct_logits_workspace_bytes(int N, int T, int U) {
+    if (N < 0 || T < 0 || U < 0) return 0;
+    return carve_logits(nullptr, N, T, U).bytes;
+}
+
+int warpctct_logits_loss_lattice(const void *logits, int dtype, const int *ys, const int *lx,
+                                 const int *ly, int N, int T, int U, int V, void *workspace,
+                                 size_t workspace_bytes, float *costs, int want_alpha,
+                                 int reduction, int average_frames, float *reduced, void *stream) {
+    if (!dims_ok(N, T, U) || V < 1 || !io_valid(dtype) || reduction < 0 || reduction > 2)
+        return WARPCTCT_EINVAL;
+    if (N == 0) return WARPCTCT_OK;
+    if (!lx || !ly || !costs || !workspace || (T > 0 && !logits) || (U > 0 && !ys))
+        return WARPCTCT_EINVAL;
+    if (reduction != 0 && !reduced) return WARPCTCT_EINVAL;
+    const LogitsWorkspace w = carve_logits(workspace, N, T, U);
+    if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
+    hipStream_t st = as_stream(stream);
+    unsigned *counter = reduction != 0 ? w.lattice.counter : nullptr;
+    if (T > 0) {
+        int rc = done(launch_logits_units(logits, dtype, ys, lx, ly, w.lattice.units, w.lse, N, T,
+                                          U, V, counter, st));
+        if (rc != WARPCTCT_OK) return rc;
+    } else if (counter) {
+        int rc = done(launch_clear_counter(counter, st));
+        if (rc != WARPCTCT_OK) return rc;
+    }
+    LatticeArgs a = {};
+    a.units = w.lattice.units;
+    a.ys = ys;
+    a.lx = lx;
+    a.ly = ly;
+    a.alphas = w.lattice.alphas;
+    a.betas = w.lattice.betas;
+    a.costs = costs;
+    a.N = N;
+    a.T = T;
+    a.U = U;
+    a.beta_only = (want_alpha == 0);
+    a.reduce.reduced = reduction != 0 ? reduced : nullptr;
+    a.reduce.counter = counter;
+    a.reduce.mode = reduction;
+    a.reduce.average_frames = average_frames != 0;
+    return done(launch_lattice(a, st));
+}
+
+int warpctct_logits_grad_lattice(const void *workspace, size_t workspace_bytes,
+                                 const void *logits, int dtype, const int *ys, const int *lx,
+                                 const int *ly, const float *grad_out, int grad_out_stride,
+                                 float scale, int average_frames, void *grad_logits, int N, int T,
+                                 int U, int V, void *stream) {
+    if (!dims_ok(N, T, U) || V < 1 || grad_out_stride < 0 || !io_valid(dtype))
+        return WARPCTCT_EINVAL;
+    if (N == 0 || T == 0) return WARPCTCT_OK;
+    if (!workspace || !logits || !lx || !ly || !grad_logits || (U > 0 && !ys))
+        return WARPCTCT_EINVAL;
+    const LogitsWorkspace w = carve_logits(const_cast<void *>(workspace), N, T, U);
+    if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
+    return done(launch_logits_grad(logits, dtype, w.lse, w.lattice.units, w.lattice.alphas,
+                                   w.lattice.betas, ys, lx, ly, grad_out, grad_out_stride, scale,
+                                   average_frames, grad_logits, N, T, U, V, as_stream(stream)));
+}
+
 int warpctct_zero_fill(void *p, size_t bytes, void *stream) {
     if (bytes == 0) return WARPCTCT_OK;
     if (!p) return WARPCTCT_EINVAL;

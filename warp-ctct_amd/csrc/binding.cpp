@@ -63,6 +63,10 @@ torch::Tensor make_workspace(const torch::Tensor &like, int N, int T, int U) {
                         like.options().dtype(at::ScalarType::Byte));
 }
 
+torch::Tensor make_bytes(const torch::Tensor &like, size_t bytes) {
+    return torch::empty({static_cast<int64_t>(bytes)}, like.options().dtype(at::ScalarType::Byte));
+}
+
 // Reference surface: _C.ctct_loss_fwd (csrc/binding.cpp:31-100).
 // log_probs is already gathered to (N,T,U+1,3).
 std::tuple<torch::Tensor, torch::Tensor> ctct_loss_fwd(const torch::Tensor &log_probs,
@@ -193,6 +197,74 @@ void dense_patch_lattice(const torch::Tensor &workspace, const torch::Tensor &ys
              "dense_patch_lattice");
 }
 
+// ctct_loss on logits: log_softmax over the vocabulary happens inside (the
+// caller of the reference applies it before warp_ctct.ctct_loss).  Same
+// contract as ctct_loss_joint_fwd; the workspace also holds the row-wise
+// logsumexp that logits_grad needs.
+std::tuple<torch::Tensor, torch::Tensor> ctct_loss_logits_fwd(const torch::Tensor &logits,
+                                                              const torch::Tensor &ys,
+                                                              const torch::Tensor &lx,
+                                                              const torch::Tensor &ly,
+                                                              const bool requires_grad,
+                                                              const int64_t reduction,
+                                                              const bool average_frames) {
+    CHECK_CONTIGUOUS(logits);
+    CHECK_DEVICE(logits);
+    const int dtype = io_type_of(logits);
+    TORCH_CHECK(logits.dim() == 4, "logits must have 4 dims.");
+    TORCH_CHECK(reduction >= 0 && reduction <= 2, "reduction must be 0 (none), 1 (sum), 2 (mean)");
+    const int N = logits.size(0), T = logits.size(1), U = logits.size(2) - 1, V = logits.size(3);
+    check_lengths(ys, lx, ly, N, U);
+    const DeviceGuard device_guard(device_of(logits));
+    auto ws = make_bytes(logits, warpctct_logits_workspace_bytes(N, T, U));
+    const auto f32 = logits.options().dtype(at::ScalarType::Float);
+    auto costs = torch::empty({N}, f32);
+    torch::Tensor reduced;
+    if (reduction != 0) reduced = N > 0 ? torch::empty({}, f32) : torch::zeros({}, f32);
+    check_rc(warpctct_logits_loss_lattice(logits.data_ptr(), dtype, ys.data_ptr<int>(),
+                                          lx.data_ptr<int>(), ly.data_ptr<int>(), N, T, U, V,
+                                          ws.data_ptr(), ws.numel(), costs.data_ptr<float>(),
+                                          requires_grad ? 1 : 0, static_cast<int>(reduction),
+                                          average_frames ? 1 : 0,
+                                          reduction != 0 ? reduced.data_ptr<float>() : nullptr,
+                                          current_stream()),
+             "ctct_loss_logits_fwd");
+    const torch::Tensor &loss = reduction != 0 ? reduced : costs;
+    if (requires_grad) return std::make_tuple(loss, ws);
+    return std::make_tuple(loss, loss);
+}
+
+// d(loss)/d(logits), every element written; grad_out, scale, average_frames as
+// in dense_patch_lattice.
+torch::Tensor ctct_loss_logits_bwd(const torch::Tensor &workspace, const torch::Tensor &logits,
+                                   const torch::Tensor &ys, const torch::Tensor &lx,
+                                   const torch::Tensor &ly, const torch::Tensor &grad_out,
+                                   const double scale, const bool average_frames) {
+    CHECK_CONTIGUOUS(workspace);
+    CHECK_DEVICE(workspace);
+    TORCH_CHECK(workspace.scalar_type() == at::ScalarType::Byte, "workspace must be a byte tensor");
+    CHECK_CONTIGUOUS(grad_out);
+    CHECK_FLOAT(grad_out);
+    CHECK_DEVICE(grad_out);
+    CHECK_CONTIGUOUS(logits);
+    CHECK_DEVICE(logits);
+    const int dtype = io_type_of(logits);
+    TORCH_CHECK(logits.dim() == 4, "logits must be (N,T,U+1,V)");
+    const int N = logits.size(0), T = logits.size(1), U = logits.size(2) - 1, V = logits.size(3);
+    TORCH_CHECK(grad_out.numel() == N || grad_out.numel() == 1, "grad_out must have N or 1 elements");
+    check_lengths(ys, lx, ly, N, U);
+    const DeviceGuard device_guard(device_of(logits));
+    auto grad = torch::empty_like(logits);
+    const int stride = (grad_out.numel() == 1 && N > 1) ? 0 : 1;
+    check_rc(warpctct_logits_grad_lattice(
+                 workspace.data_ptr(), workspace.numel(), logits.data_ptr(), dtype,
+                 ys.data_ptr<int>(), lx.data_ptr<int>(), ly.data_ptr<int>(),
+                 grad_out.data_ptr<float>(), stride, static_cast<float>(scale),
+                 average_frames ? 1 : 0, grad.data_ptr(), N, T, U, V, current_stream()),
+             "ctct_loss_logits_bwd");
+    return grad;
+}
+
 // Backward of the fused entry: CTCTLoss.backward (warp_ctct/__init__.py:30-33)
 // and the gather backward.  grad_out (N) scales sample n.
 torch::Tensor ctct_loss_joint_bwd(const torch::Tensor &unit_grads, const torch::Tensor &ys,
@@ -218,10 +290,6 @@ torch::Tensor ctct_loss_joint_bwd(const torch::Tensor &unit_grads, const torch::
                                      static_cast<int>(V), current_stream()),
              "ctct_loss_joint_bwd");
     return dense;
-}
-
-torch::Tensor make_bytes(const torch::Tensor &like, size_t bytes) {
-    return torch::empty({static_cast<int64_t>(bytes)}, like.options().dtype(at::ScalarType::Byte));
 }
 
 // Reference surface: _C.ctct_loss_simple_fwd (csrc/binding.cpp:103-222).
@@ -483,6 +551,15 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           pybind11::arg("ys"), pybind11::arg("lx"), pybind11::arg("ly"),
           pybind11::arg("requires_grad"), pybind11::arg("reduction") = 0,
           pybind11::arg("average_frames") = false);
+    m.def("ctct_loss_logits_fwd", &ctct_loss_logits_fwd,
+          "CTC-Transducer loss on logits, log_softmax inside (forward).", pybind11::arg("logits"),
+          pybind11::arg("ys"), pybind11::arg("lx"), pybind11::arg("ly"),
+          pybind11::arg("requires_grad"), pybind11::arg("reduction") = 0,
+          pybind11::arg("average_frames") = false);
+    m.def("ctct_loss_logits_bwd", &ctct_loss_logits_bwd, "Gradient wrt the logits.",
+          pybind11::arg("workspace"), pybind11::arg("logits"), pybind11::arg("ys"),
+          pybind11::arg("lx"), pybind11::arg("ly"), pybind11::arg("grad_out"),
+          pybind11::arg("scale"), pybind11::arg("average_frames"));
     m.def("ctct_loss_joint_bwd", &ctct_loss_joint_bwd,
           "Dense gradient wrt the joint from unit gradients.", pybind11::arg("unit_grads"),
           pybind11::arg("ys"), pybind11::arg("lx"), pybind11::arg("ly"),

@@ -51,24 +51,6 @@ __global__ __launch_bounds__(kBlock) void zero_fill_vec_kernel(v4f *__restrict__
     if (i < n4) p4[i] = z;
 }
 
-// Per-sample weight of the upstream gradient: grad_out[n * stride] (stride 0
-// broadcasts a scalar), times `scale` (1/N for reduction='mean'), divided by
-// lx[n] when the loss was averaged over frames (warp_ctct/__init__.py:138-147
-// of the reference, differentiated).
-struct Weight {
-    const float *grad_out;   // null = ones
-    int stride;
-    float scale;
-    int average_frames;
-};
-
-__device__ __forceinline__ float sample_weight(const Weight &w, int n, int lxn) {
-    float v = w.grad_out ? w.grad_out[(size_t)n * w.stride] : 1.0f;
-    v *= w.scale;
-    if (w.average_frames) v /= (float)lxn;
-    return v;
-}
-
 // Writes (not adds) the non-zero entries of row (n,t,u) of the dense gradient:
 // columns 0, y[u-1], y[u]; columns that coincide are summed first so that
 // every element is written by exactly one store.

@@ -75,6 +75,18 @@ hipError_t launch_dense_patch_lattice(const double *units, const double *alphas,
                                       float scale, int average_frames, void *dense, int io_type,
                                       int N, int T, int U, int V, hipStream_t stream);
 
+// ---- ctct_loss on logits (log_softmax inside) --------------------------------
+// units + lse (N,T,U+1) from the logits; counter as in launch_gather_units
+hipError_t launch_logits_units(const void *logits, int io_type, const int *ys, const int *lx,
+                               const int *ly, double *units, float *lse, int N, int T, int U,
+                               int V, unsigned *counter, hipStream_t stream);
+// dense gradient wrt the logits, every element written
+hipError_t launch_logits_grad(const void *logits, int io_type, const float *lse,
+                              const double *units, const double *alphas, const double *betas,
+                              const int *ys, const int *lx, const int *ly, const float *grad_out,
+                              int grad_out_stride, float scale, int average_frames, void *grad,
+                              int N, int T, int U, int V, hipStream_t stream);
+
 // ---- log-add joiner path -------------------------------------------------
 hipError_t launch_simple_gather_units(const float *f, const float *g, const float *den,
                                       const int *ys, const int *lx, const int *ly, double *units,

@@ -1,0 +1,294 @@
+// ctct_loss on un-normalised joiner outputs ("logits"): log_softmax over the
+// vocabulary is taken inside the gather, and its backward inside the kernel
+// that writes the dense gradient, so the (N,T,U+1,V) log-probability tensor
+// that a caller of the reference has to materialise before
+// warp_ctct.ctct_loss (and whose gradient autograd has to push back through
+// log_softmax) never exists:
+//   forward   lse[n,t,u] = logsumexp_v logits[n,t,u,v]          (live rows only)
+//             units      = logits[n,t,u,{0, y[u-1], y[u]}] - lse
+//   backward  d/dlogits[v] = w_n * (G[v] - softmax[v] * (g0 + g1 + g2))
+// where G is the gather backward of the unit gradients g (non-zero in at most
+// three columns, csrc/gather.cu:311-374 of the reference) and w_n the upstream
+// weight of sample n.  Rows of padding and rows outside the band of complete
+// alignments are not read at all; their gradient is zero.
+// One wavefront per row; a row is read once in each direction.
+#include "device_utils.h"
+#include "launch.h"
+#include "unit_grad.h"
+
+namespace wctct {
+
+namespace {
+
+constexpr int kRowsPerBlock = 4;
+constexpr float kLog2eF = 1.4426950408889634f;
+constexpr float kLn2F = 0.6931471805599453f;
+
+template <typename IO> struct Vec4;   // 4 elements of the joint, loaded as one vector
+template <> struct Vec4<float> {
+    typedef float type __attribute__((ext_vector_type(4)));
+};
+template <> struct Vec4<__half> {
+    typedef _Float16 type __attribute__((ext_vector_type(4)));
+};
+template <> struct Vec4<__hip_bfloat16> {
+    typedef unsigned short type __attribute__((ext_vector_type(4)));
+};
+
+__device__ __forceinline__ float elem_to_float(float v) { return v; }
+__device__ __forceinline__ float elem_to_float(_Float16 v) { return (float)v; }
+__device__ __forceinline__ float elem_to_float(unsigned short v) {   // bfloat16 bits
+    return __uint_as_float((unsigned)v << 16);
+}
+
+template <typename IO>
+__device__ __forceinline__ void load4(const IO *p, float (&x)[4]) {
+    const typename Vec4<IO>::type v = *reinterpret_cast<const typename Vec4<IO>::type *>(p);
+    x[0] = elem_to_float(v.x);
+    x[1] = elem_to_float(v.y);
+    x[2] = elem_to_float(v.z);
+    x[3] = elem_to_float(v.w);
+}
+
+__device__ __forceinline__ void store4(float *p, const float (&x)[4]) {
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    *reinterpret_cast<v4f *>(p) = v4f{x[0], x[1], x[2], x[3]};
+}
+__device__ __forceinline__ void store4(__half *p, const float (&x)[4]) {
+    __half h[4] = {__float2half(x[0]), __float2half(x[1]), __float2half(x[2]), __float2half(x[3])};
+    *reinterpret_cast<uint2 *>(p) = *reinterpret_cast<const uint2 *>(h);
+}
+__device__ __forceinline__ void store4(__hip_bfloat16 *p, const float (&x)[4]) {
+    __hip_bfloat16 h[4] = {__float2bfloat16(x[0]), __float2bfloat16(x[1]), __float2bfloat16(x[2]),
+                           __float2bfloat16(x[3])};
+    *reinterpret_cast<uint2 *>(p) = *reinterpret_cast<const uint2 *>(h);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// Rows are 4-element-vector addressable when every row starts on a vector
+// boundary.
+template <typename IO>
+__device__ __forceinline__ bool rows_vectorised(const IO *base, int V) {
+    return (V & 3) == 0 && (reinterpret_cast<uintptr_t>(base) & (4 * sizeof(IO) - 1)) == 0;
+}
+
+// One wavefront per cell (t,u) of the work buffer (P contexts per frame) of
+// sample blockIdx.y.  Live cells inside the band: logsumexp of the row in one
+// pass (running maximum and rescaled sum per lane, combined over the
+// wavefront), then the three units.  Other cells of live frames: neutral
+// units, as gather_units_kernel.
+template <typename IO>
+__global__ __launch_bounds__(64 * kRowsPerBlock) void logits_units_kernel(
+    const IO *__restrict__ logits, const int *__restrict__ ys, const int *__restrict__ lx,
+    const int *__restrict__ ly, double *__restrict__ units, float *__restrict__ lse, int T, int U,
+    int V, int P, unsigned *__restrict__ counter) {
+    if (counter && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *counter = 0u;
+    const int n = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const int cell = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+    if (cell >= T * P) return;
+    const int t = cell / P, u = cell - t * P;
+    const int Tn = min(max(lx[n], 0), T), Un = min(max(ly[n], 0), U);
+    if (t >= Tn) return;
+    double *o = units + (((size_t)n * T + t) * P + u) * 3;
+    if (u > Un || outside_band(t, u, Tn, Un)) {
+        if (lane == 0) {
+            o[0] = 0.0;
+            o[1] = 0.0;
+            o[2] = neg_inf();
+        }
+        return;
+    }
+    const size_t r = ((size_t)n * T + t) * (U + 1) + u;
+    const IO *row = logits + r * (size_t)V;
+    // running maximum m and sum s of 2^(x*log2e - m) over this lane's elements
+    float m = -__builtin_huge_valf(), s = 0.0f;
+    if (rows_vectorised(logits, V)) {
+        for (int k = lane * 4; k < V; k += 256) {
+            float x[4];
+            load4(row + k, x);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) x[i] *= kLog2eF;
+            const float mn = fmaxf(fmaxf(m, fmaxf(x[0], x[1])), fmaxf(x[2], x[3]));
+            // mn = -inf only while everything seen is -inf: keep s = 0
+            const float mf = fmaxf(mn, -3.0e38f);
+            s = s * exp2_hw(m - mf) + exp2_hw(x[0] - mf) + exp2_hw(x[1] - mf) +
+                exp2_hw(x[2] - mf) + exp2_hw(x[3] - mf);
+            m = mn;
+        }
+    } else {
+        for (int k = lane; k < V; k += 64) {
+            const float x = load_as_float(row + k) * kLog2eF;
+            const float mn = fmaxf(m, x);
+            const float mf = fmaxf(mn, -3.0e38f);
+            s = s * exp2_hw(m - mf) + exp2_hw(x - mf);
+            m = mn;
+        }
+    }
+    const float M = wave_max(m);
+    const float Mf = fmaxf(M, -3.0e38f);
+    const float S = wave_sum(s * exp2_hw(m - Mf));
+    if (lane == 0) {
+        const float l = (M + log2_hw(S)) * kLn2F;   // natural-log logsumexp of the row
+        lse[r] = l;
+        const int *y = ys + (size_t)n * U;
+        const double b = (double)load_as_float(row) - (double)l;
+        double cur = b, nxt = neg_inf();
+        if (u >= 1) cur = (double)load_as_float(row + min(max(y[u - 1], 0), V - 1)) - (double)l;
+        if (u < Un)
+            nxt = ((double)load_as_float(row + min(max(y[u], 0), V - 1)) - (double)l) * kLog2e;
+        o[0] = b * kLog2e;
+        o[1] = cur * kLog2e;
+        o[2] = nxt;
+    }
+}
+
+// One wavefront per row (n,t,u) of the gradient, blockIdx.y = n.
+template <typename IO>
+__global__ __launch_bounds__(64 * kRowsPerBlock) void logits_grad_kernel(
+    const IO *__restrict__ logits, const float *__restrict__ lse, const double *__restrict__ units,
+    const double *__restrict__ alphas, const double *__restrict__ betas,
+    const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
+    Weight weight, IO *__restrict__ grad, int T, int U, int V, int P) {
+    const int U1 = U + 1;
+    const int n = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const int cell = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+    if (cell >= T * U1) return;
+    const int t = cell / U1, u = cell - t * U1;
+    const int lxn = lx[n];
+    const int Tn = min(max(lxn, 0), T), Un = min(max(ly[n], 0), U);
+    const size_t r = ((size_t)n * T + t) * U1 + u;
+    IO *out = grad + r * (size_t)V;
+    const bool vec = rows_vectorised(logits, V) && rows_vectorised(grad, V);
+    if (t >= Tn || u > Un || outside_band(t, u, Tn, Un)) {
+        const float z[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (vec) {
+            for (int k = lane * 4; k < V; k += 256) store4(out + k, z);
+        } else {
+            for (int k = lane; k < V; k += 64) store_from_float(out + k, 0.0f);
+        }
+        return;
+    }
+    const int *y = ys + (size_t)n * U;
+    const size_t lat = (size_t)(T + 1) * P * 2;
+    const UnitGrad g = unit_grad_cell(units + (size_t)n * T * P * 3, alphas + (size_t)n * lat,
+                                      betas + (size_t)n * lat, y, t, u, Un, P);
+    const float w = sample_weight(weight, n, lxn);
+    const float g0 = g.g0 * w, g1 = g.g1 * w, g2 = g.g2 * w;   // g1 = 0 at u = 0, g2 = 0 at u = Un
+    const float total = g0 + g1 + g2;
+    const int c1 = (u >= 1) ? min(max(y[u - 1], 0), V - 1) : -1;
+    const int c2 = (u < Un) ? min(max(y[u], 0), V - 1) : -1;
+    const float shift = lse[r] * kLog2eF;
+    const IO *row = logits + r * (size_t)V;
+    if (vec) {
+        for (int k = lane * 4; k < V; k += 256) {
+            float x[4];
+            load4(row + k, x);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float v = -total * exp2_hw(x[i] * kLog2eF - shift);
+                const int col = k + i;
+                if (col == 0) v += g0;
+                if (col == c1) v += g1;
+                if (col == c2) v += g2;
+                x[i] = v;
+            }
+            store4(out + k, x);
+        }
+    } else {
+        for (int k = lane; k < V; k += 64) {
+            float v = -total * exp2_hw(load_as_float(row + k) * kLog2eF - shift);
+            if (k == 0) v += g0;
+            if (k == c1) v += g1;
+            if (k == c2) v += g2;
+            store_from_float(out + k, v);
+        }
+    }
+}
+
+template <typename IO>
+void launch_units_typed(const void *logits, const int *ys, const int *lx, const int *ly,
+                        double *units, float *lse, int N, int T, int U, int V, unsigned *counter,
+                        hipStream_t stream) {
+    const int P = padded_contexts(U);
+    const long cells = (long)T * P;
+    dim3 grid((unsigned)((cells + kRowsPerBlock - 1) / kRowsPerBlock), (unsigned)N);
+    hipLaunchKernelGGL((logits_units_kernel<IO>), grid, dim3(64 * kRowsPerBlock), 0, stream,
+                       static_cast<const IO *>(logits), ys, lx, ly, units, lse, T, U, V, P,
+                       counter);
+}
+
+template <typename IO>
+void launch_grad_typed(const void *logits, const float *lse, const double *units,
+                       const double *alphas, const double *betas, const int *ys, const int *lx,
+                       const int *ly, const Weight &w, void *grad, int N, int T, int U, int V,
+                       hipStream_t stream) {
+    const long cells = (long)T * (U + 1);
+    dim3 grid((unsigned)((cells + kRowsPerBlock - 1) / kRowsPerBlock), (unsigned)N);
+    hipLaunchKernelGGL((logits_grad_kernel<IO>), grid, dim3(64 * kRowsPerBlock), 0, stream,
+                       static_cast<const IO *>(logits), lse, units, alphas, betas, ys, lx, ly, w,
+                       static_cast<IO *>(grad), T, U, V, padded_contexts(U));
+}
+
+}  // namespace
+
+hipError_t launch_logits_units(const void *logits, int io_type, const int *ys, const int *lx,
+                               const int *ly, double *units, float *lse, int N, int T, int U,
+                               int V, unsigned *counter, hipStream_t stream) {
+    if (N == 0 || T == 0) return hipSuccess;
+    switch (io_type) {
+        case kIoF32:
+            launch_units_typed<float>(logits, ys, lx, ly, units, lse, N, T, U, V, counter, stream);
+            break;
+        case kIoF16:
+            launch_units_typed<__half>(logits, ys, lx, ly, units, lse, N, T, U, V, counter,
+                                       stream);
+            break;
+        case kIoBF16:
+            launch_units_typed<__hip_bfloat16>(logits, ys, lx, ly, units, lse, N, T, U, V, counter,
+                                               stream);
+            break;
+        default:
+            return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_logits_grad(const void *logits, int io_type, const float *lse,
+                              const double *units, const double *alphas, const double *betas,
+                              const int *ys, const int *lx, const int *ly, const float *grad_out,
+                              int grad_out_stride, float scale, int average_frames, void *grad,
+                              int N, int T, int U, int V, hipStream_t stream) {
+    if (N == 0 || T == 0) return hipSuccess;
+    const Weight w = {grad_out, grad_out_stride, scale, average_frames};
+    switch (io_type) {
+        case kIoF32:
+            launch_grad_typed<float>(logits, lse, units, alphas, betas, ys, lx, ly, w, grad, N, T,
+                                     U, V, stream);
+            break;
+        case kIoF16:
+            launch_grad_typed<__half>(logits, lse, units, alphas, betas, ys, lx, ly, w, grad, N, T,
+                                      U, V, stream);
+            break;
+        case kIoBF16:
+            launch_grad_typed<__hip_bfloat16>(logits, lse, units, alphas, betas, ys, lx, ly, w,
+                                              grad, N, T, U, V, stream);
+            break;
+        default:
+            return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace wctct

@@ -22,7 +22,7 @@ except ImportError as exc:  # pragma: no cover - exercised only on a broken inst
         "(needs hipcc, --offload-arch=gfx950)"
     ) from exc
 
-__all__ = ["ctct_loss", "ctct_simple_loss"]
+__all__ = ["ctct_loss", "ctct_loss_with_logits", "ctct_simple_loss"]
 __version__ = core.library_version()
 
 
@@ -106,6 +106,33 @@ class _CTCTLoss(torch.autograd.Function):
         return dense, None, None, None, None, None, None
 
 
+class _CTCTLossLogits(torch.autograd.Function):
+    """ctct_loss(logits.log_softmax(-1), ...) without the log-probability tensor.
+
+    Forward takes the row-wise logsumexp inside the gather and keeps it next
+    to the lattices; backward writes d(loss)/d(logits) = w * (G - softmax *
+    sum(G)) in one pass, G being the <= 3 non-zero gather-backward entries of
+    the row.  Rows of padding are never read."""
+
+    @staticmethod
+    def forward(ctx, logits, labels, lx, ly, requires_grad, reduction, average_frames):
+        loss, workspace = _run("logits_forward", lambda: core.ctct_loss_logits_fwd(
+            logits, labels, lx, ly, requires_grad, _REDUCTION_CODE[reduction], average_frames))
+        if requires_grad:
+            ctx.save_for_backward(workspace, logits, labels, lx, ly)
+            ctx.scale = 1.0 / logits.size(0) if reduction == "mean" else 1.0
+            ctx.average_frames = bool(average_frames)
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_outputs):
+        workspace, logits, labels, lx, ly = ctx.saved_tensors
+        grad_outputs = grad_outputs.reshape(-1).float().contiguous()
+        grad = _run("logits_backward", lambda: core.ctct_loss_logits_bwd(
+            workspace, logits, labels, lx, ly, grad_outputs, ctx.scale, ctx.average_frames))
+        return grad, None, None, None, None, None, None
+
+
 class _SimpleCTCTLoss(torch.autograd.Function):
     """ctct_simple_loss on the un-gathered f (N,T,V) and g (N,U+1,V).
 
@@ -169,6 +196,38 @@ def ctct_loss(log_probs: torch.Tensor,
         return _CTCTLoss.apply(log_probs.contiguous(), _as_int(labels), _as_int(frames_lengths),
                                _as_int(labels_lengths), enable_grad, reduction,
                                bool(average_frames))
+
+
+def ctct_loss_with_logits(logits: torch.Tensor,
+                          labels: torch.Tensor,
+                          frames_lengths: torch.Tensor,
+                          labels_lengths: torch.Tensor,
+                          reduction: Optional[str] = "mean",
+                          average_frames: bool = False) -> torch.Tensor:
+    """``ctct_loss(logits.log_softmax(-1), ...)`` in one pass over the logits.
+
+    The reference expects normalised log-probabilities, so its callers run
+    ``log_softmax`` over the (N, T, U, V) joiner output first and autograd
+    pushes the dense gradient back through it.  This function takes the
+    joiner output itself: the normalisation happens inside the gather, its
+    backward inside the kernel that writes the gradient, and the
+    log-probability tensor is never materialised.  Arguments and result are
+    those of :func:`ctct_loss`; ``logits`` may be float32, float16 or
+    bfloat16 (other types are converted to float32)."""
+    assert average_frames is None or isinstance(average_frames, bool)
+    assert reduction is None or reduction in ("none", "mean", "sum")
+    assert logits.dim() == 4
+    assert labels.dim() == 2
+    assert logits.size(2) == labels.size(1) + 1
+    assert logits.size(0) == labels.size(0) == frames_lengths.size(0) == labels_lengths.size(0)
+
+    enable_grad = logits.requires_grad and torch.is_grad_enabled()
+    if logits.dtype not in _NATIVE_DTYPES:
+        logits = logits.float()
+    with _no_autocast():
+        return _CTCTLossLogits.apply(logits.contiguous(), _as_int(labels),
+                                     _as_int(frames_lengths), _as_int(labels_lengths),
+                                     enable_grad, reduction, bool(average_frames))
 
 
 def ctct_simple_loss(f: torch.Tensor,
