@@ -88,8 +88,13 @@ OTHER = {
     # the typical batch with a half-precision joint (half the bytes at both ends)
     "c2_bf16": ("full", 32, 250, 60, 1024, 1.0),
     "c2_f16": ("full", 32, 250, 60, 1024, 1.0),
+    # the typical batch from logits: log_softmax inside the loss (fused), and
+    # torch.log_softmax followed by ctct_loss (what a caller of the reference does)
+    "c2_logits": ("logits", 32, 250, 60, 1024, 1.0),
+    "c2_logits_bf16": ("logits", 32, 250, 60, 1024, 1.0),
+    "c2_logits_unfused": ("logits_unfused", 32, 250, 60, 1024, 1.0),
 }
-IO_DTYPE = {"c2_bf16": "bfloat16", "c2_f16": "float16"}
+IO_DTYPE = {"c2_bf16": "bfloat16", "c2_f16": "float16", "c2_logits_bf16": "bfloat16"}
 
 
 def other_config(args, torch, warp_ctct):
@@ -124,6 +129,20 @@ def other_config(args, torch, warp_ctct):
 
         def loss_fn():
             return warp_ctct.ctct_loss(joint, d_ys, d_lx, d_ly)
+    elif kind in ("logits", "logits_unfused"):
+        io = getattr(torch, IO_DTYPE.get(args.config, "float32"))
+        logits = torch.randn(N, T, U + 1, V, device="cuda", generator=gen).mul_(3.0).to(io)
+        logits.requires_grad_(True)
+        leaves = (logits,)
+        # algorithmic bytes: live rows read twice (forward, backward), gradient written once
+        alg_bytes = logits.element_size() * V * (2 * live + N * T * (U + 1))
+
+        if kind == "logits":
+            def loss_fn():
+                return warp_ctct.ctct_loss_with_logits(logits, d_ys, d_lx, d_ly)
+        else:
+            def loss_fn():
+                return warp_ctct.ctct_loss(logits.log_softmax(-1), d_ys, d_lx, d_ly)
     else:
         f = torch.randn(N, T, V, device="cuda", generator=gen)
         g = torch.randn(N, U + 1, V, device="cuda", generator=gen)
@@ -183,7 +202,8 @@ def main():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "c2_bf16", "c2_f16"],
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "c2_bf16", "c2_f16", "c2_logits",
+                             "c2_logits_bf16", "c2_logits_unfused"],
                     help="workload: c2 (default) is the configuration the headline metric is "
                          "quoted on; the others are the remaining BASELINE.json configurations "
                          "and print a reduced line (no cpu_baseline)")

@@ -21,6 +21,7 @@ namespace wctct {
 namespace {
 
 constexpr int kRowsPerBlock = 4;
+constexpr int kVecStride = 256;   // elements covered by one 4-element vector load of a wavefront
 constexpr float kLog2eF = 1.4426950408889634f;
 constexpr float kLn2F = 0.6931471805599453f;
 
@@ -111,19 +112,42 @@ __global__ __launch_bounds__(64 * kRowsPerBlock) void logits_units_kernel(
     }
     const size_t r = ((size_t)n * T + t) * (U + 1) + u;
     const IO *row = logits + r * (size_t)V;
+    // the three logits that become units are requested now (every lane the
+    // same address), so that their latency runs in parallel with the row's
+    // instead of after the reduction
+    const int *y = ys + (size_t)n * U;
+    const int c1 = (u >= 1) ? min(max(y[u - 1], 0), V - 1) : 0;
+    const int c2 = (u < Un) ? min(max(y[u], 0), V - 1) : 0;
+    const float xb = load_as_float(row), x1 = load_as_float(row + c1), x2 = load_as_float(row + c2);
     // running maximum m and sum s of 2^(x*log2e - m) over this lane's elements
     float m = -__builtin_huge_valf(), s = 0.0f;
     if (rows_vectorised(logits, V)) {
-        for (int k = lane * 4; k < V; k += 256) {
-            float x[4];
-            load4(row + k, x);
+        // 1024 elements per round: four 4-element vectors per lane, all four
+        // loads issued before anything is computed (addresses past the row are
+        // clamped into it and the values dropped)
+        for (int k0 = 0; k0 < V; k0 += 4 * kVecStride) {
+            float x[4][4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) x[i] *= kLog2eF;
-            const float mn = fmaxf(fmaxf(m, fmaxf(x[0], x[1])), fmaxf(x[2], x[3]));
+            for (int j = 0; j < 4; ++j)
+                load4(row + min(k0 + j * kVecStride + lane * 4, V - 4), x[j]);
+            float mn = m;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool in = (k0 + j * kVecStride + lane * 4) < V;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    x[j][i] = in ? x[j][i] * kLog2eF : -__builtin_huge_valf();
+                    mn = fmaxf(mn, x[j][i]);
+                }
+            }
             // mn = -inf only while everything seen is -inf: keep s = 0
             const float mf = fmaxf(mn, -3.0e38f);
-            s = s * exp2_hw(m - mf) + exp2_hw(x[0] - mf) + exp2_hw(x[1] - mf) +
-                exp2_hw(x[2] - mf) + exp2_hw(x[3] - mf);
+            float acc = s * exp2_hw(m - mf);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc += exp2_hw(x[j][i] - mf);
+            s = acc;
             m = mn;
         }
     } else {
@@ -141,12 +165,10 @@ __global__ __launch_bounds__(64 * kRowsPerBlock) void logits_units_kernel(
     if (lane == 0) {
         const float l = (M + log2_hw(S)) * kLn2F;   // natural-log logsumexp of the row
         lse[r] = l;
-        const int *y = ys + (size_t)n * U;
-        const double b = (double)load_as_float(row) - (double)l;
+        const double b = (double)xb - (double)l;
         double cur = b, nxt = neg_inf();
-        if (u >= 1) cur = (double)load_as_float(row + min(max(y[u - 1], 0), V - 1)) - (double)l;
-        if (u < Un)
-            nxt = ((double)load_as_float(row + min(max(y[u], 0), V - 1)) - (double)l) * kLog2e;
+        if (u >= 1) cur = (double)x1 - (double)l;
+        if (u < Un) nxt = ((double)x2 - (double)l) * kLog2e;
         o[0] = b * kLog2e;
         o[1] = cur * kLog2e;
         o[2] = nxt;
@@ -180,6 +202,14 @@ __global__ __launch_bounds__(64 * kRowsPerBlock) void logits_grad_kernel(
         }
         return;
     }
+    // the first 1024 elements of the row are requested before the (dependent)
+    // loads of the unit gradients, not after them
+    const IO *row = logits + r * (size_t)V;
+    float x[4][4];
+    if (vec) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) load4(row + min(j * kVecStride + lane * 4, V - 4), x[j]);
+    }
     const int *y = ys + (size_t)n * U;
     const size_t lat = (size_t)(T + 1) * P * 2;
     const UnitGrad g = unit_grad_cell(units + (size_t)n * T * P * 3, alphas + (size_t)n * lat,
@@ -190,21 +220,28 @@ __global__ __launch_bounds__(64 * kRowsPerBlock) void logits_grad_kernel(
     const int c1 = (u >= 1) ? min(max(y[u - 1], 0), V - 1) : -1;
     const int c2 = (u < Un) ? min(max(y[u], 0), V - 1) : -1;
     const float shift = lse[r] * kLog2eF;
-    const IO *row = logits + r * (size_t)V;
     if (vec) {
-        for (int k = lane * 4; k < V; k += 256) {
-            float x[4];
-            load4(row + k, x);
+        for (int k0 = 0; k0 < V; k0 += 4 * kVecStride) {
+            if (k0 > 0) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float v = -total * exp2_hw(x[i] * kLog2eF - shift);
-                const int col = k + i;
-                if (col == 0) v += g0;
-                if (col == c1) v += g1;
-                if (col == c2) v += g2;
-                x[i] = v;
+                for (int j = 0; j < 4; ++j)
+                    load4(row + min(k0 + j * kVecStride + lane * 4, V - 4), x[j]);
             }
-            store4(out + k, x);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int k = k0 + j * kVecStride + lane * 4;
+                if (k >= V) continue;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float v = -total * exp2_hw(x[j][i] * kLog2eF - shift);
+                    const int col = k + i;
+                    if (col == 0) v += g0;
+                    if (col == c1) v += g1;
+                    if (col == c2) v += g2;
+                    x[j][i] = v;
+                }
+                store4(out + k, x[j]);
+            }
         }
     } else {
         for (int k = lane; k < V; k += 64) {
