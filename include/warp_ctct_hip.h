@@ -158,6 +158,15 @@ int warpctct_dense_patch_lattice(const void *workspace, size_t workspace_bytes, 
  * in a HIP graph). */
 int warpctct_zero_fill(void *p, size_t bytes, void *stream);
 
+/* warpctct_loss_forward_f32 (below) for a joint of type `dtype`: costs and the
+ * compact unit gradients (N,T,U+1,3) fp32, i.e. what _C.ctct_loss_fwd of the
+ * reference returns (csrc/binding.cpp:31-100), computed from the un-gathered
+ * joint.  For callers that own the joiner and apply the gradient themselves
+ * instead of receiving the dense (N,T,U+1,V) tensor. */
+int warpctct_loss_forward(const void *joint, int dtype, const int *ys, const int *lx,
+                          const int *ly, int N, int T, int U, int V, void *workspace,
+                          size_t workspace_bytes, float *costs, float *unit_grads, void *stream);
+
 /* ---- ctct_loss on logits --------------------------------------------------
  * The step before the reference's path fused into it: a caller of the
  * reference computes log_probs = logits.log_softmax(-1) and passes it to

@@ -51,3 +51,44 @@ def test_invalid_arguments_are_rejected_on_the_host():
     # empty batch is a no-op
     assert lib.warpctct_loss_forward_f32(null, null, null, null, 0, 4, 2, 8, null,
                                          ctypes.c_size_t(0), null, null, null) == 0
+
+
+def test_generic_dtype_and_logits_entry_points_check_their_arguments():
+    lib = hip_lib.lib()
+    lib.warpctct_logits_workspace_bytes.restype = ctypes.c_size_t
+    lib.warpctct_logmm_workspace_bytes.restype = ctypes.c_size_t
+    lib.warpctct_simple_backward_workspace_bytes.restype = ctypes.c_size_t
+    null = ctypes.c_void_p(0)
+    EINVAL, EWORKSPACE = 1, 3
+    buf = (ctypes.c_float * 16)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    small = ctypes.c_size_t(16)
+    f = ctypes.c_float
+    # unknown element type, unknown reduction, reduction without a place for the result
+    assert lib.warpctct_loss_lattice(p, 7, p, p, p, 1, 1, 1, 8, p, small, p, 1, 0, 0, null, null) == EINVAL
+    assert lib.warpctct_loss_lattice(p, 0, p, p, p, 1, 1, 1, 8, p, small, p, 1, 3, 0, p, null) == EINVAL
+    assert lib.warpctct_loss_lattice(p, 2, p, p, p, 1, 1, 1, 8, p, small, p, 1, 2, 0, null, null) == EINVAL
+    # valid arguments, workspace too small (checked before any launch)
+    assert lib.warpctct_loss_lattice(p, 2, p, p, p, 1, 1, 1, 8, p, small, p, 1, 2, 0, p, null) == EWORKSPACE
+    assert lib.warpctct_logits_loss_lattice(p, 1, p, p, p, 1, 1, 1, 8, p, small, p, 1, 0, 0, null,
+                                            null) == EWORKSPACE
+    assert lib.warpctct_logits_grad_lattice(p, small, p, 0, p, p, p, p, 1, f(1.0), 0, p, 1, 1, 1, 8,
+                                            null) == EWORKSPACE
+    assert lib.warpctct_logits_grad_lattice(p, small, p, 5, p, p, p, p, 1, f(1.0), 0, p, 1, 1, 1, 8,
+                                            null) == EINVAL
+    assert lib.warpctct_dense_grad_lattice(p, small, p, p, p, p, 1, f(1.0), 0, null, 0, 1, 1, 1, 8,
+                                           null) == EINVAL
+    assert lib.warpctct_loss_forward(p, 9, p, p, p, 1, 1, 1, 8, p, small, p, p, null) == EINVAL
+    assert lib.warpctct_zero_fill(null, ctypes.c_size_t(64), null) == EINVAL
+    assert lib.warpctct_zero_fill(null, ctypes.c_size_t(0), null) == 0
+    # workspace sizes: logits = lattice + one float per row; log-matmul grows with K
+    N, T, U = 4, 50, 20
+    lat = lib.warpctct_workspace_bytes(N, T, U)
+    lg = lib.warpctct_logits_workspace_bytes(N, T, U)
+    assert lat + 4 * N * T * (U + 1) <= lg < lat + 4 * N * T * (U + 1) + 256
+    assert lib.warpctct_logmm_padded_reduction(1) == 32 and lib.warpctct_logmm_padded_reduction(2048) == 2048
+    assert lib.warpctct_logmm_padded_reduction(2049) == 2080
+    w1 = lib.warpctct_logmm_workspace_bytes(2, 10, 64, 5)
+    w2 = lib.warpctct_logmm_workspace_bytes(2, 10, 65, 5)
+    assert w2 - w1 == 4 * 32 * 2 * (10 + 5)
+    assert lib.warpctct_simple_backward_workspace_bytes(N, T, U) >= 4 * N * T * (U + 1) + 4 * N * T

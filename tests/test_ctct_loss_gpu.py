@@ -356,6 +356,27 @@ def test_loss_with_logits_average_frames_and_sum():
     np.testing.assert_allclose(x.grad.cpu().numpy(), ref_grad, atol=GRAD_ATOL, rtol=0)
 
 
+def test_compact_hand_off_rebuilds_the_dense_gradient():
+    """ctct_loss_compact: costs, unit gradients and the gather index; a
+    scatter_add of the compact gradient is the dense gradient of the sum."""
+    import warp_ctct
+    joint, ys, lx, ly = make_joint_case(51, 3, 19, 6, 23, lx=range(9, 20), ly=range(2, 7))
+    _, ref_dense, ref_costs = O.ctct_loss(joint, ys, lx, ly, reduction="sum")
+    for dtype in (torch.float32, torch.bfloat16):
+        x = dev(joint).to(dtype)
+        if dtype != torch.float32:
+            _, ref_dense, ref_costs = O.ctct_loss(x.double().cpu().numpy(), ys, lx, ly,
+                                                  reduction="sum")
+        costs, ug, index = warp_ctct.ctct_loss_compact(x, dev(ys), dev(lx), dev(ly))
+        assert costs.dtype == ug.dtype == torch.float32 and index.dtype == torch.long
+        assert tuple(ug.shape) == (3, 19, 7, 3) and tuple(index.shape) == (3, 7, 3)
+        np.testing.assert_allclose(costs.cpu().numpy(), ref_costs, rtol=LOSS_RTOL)
+        np.testing.assert_array_equal(index.cpu().numpy(), O.gather_index(ys, 7))
+        dense = torch.zeros(3, 19, 7, 23, device="cuda")
+        dense.scatter_add_(3, index[:, None].expand_as(ug), ug)
+        np.testing.assert_allclose(dense.cpu().numpy(), ref_dense, atol=GRAD_ATOL, rtol=0)
+
+
 def test_operator_surface_on_gathered_units():
     """_C.ctct_loss_fwd keeps the reference's contract: gathered (N,T,U+1,3)
     input, (costs, grads) output, grads zero in padding, costs twice when

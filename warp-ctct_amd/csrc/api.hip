@@ -426,22 +426,29 @@ int warpctct_zero_fill(void *p, size_t bytes, void *stream) {
     return done(launch_zero_fill_bytes(p, bytes, as_stream(stream)));
 }
 
-int warpctct_loss_forward_f32(const float *joint, const int *ys, const int *lx, const int *ly,
-                              int N, int T, int U, int V, void *workspace, size_t workspace_bytes,
-                              float *costs, float *unit_grads, void *stream) {
-    if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
+int warpctct_loss_forward(const void *joint, int dtype, const int *ys, const int *lx,
+                          const int *ly, int N, int T, int U, int V, void *workspace,
+                          size_t workspace_bytes, float *costs, float *unit_grads, void *stream) {
+    if (!dims_ok(N, T, U) || V < 1 || !io_valid(dtype)) return WARPCTCT_EINVAL;
     if (N == 0) return WARPCTCT_OK;
     if (!lx || !ly || !costs || !workspace || (T > 0 && !joint) || (U > 0 && !ys))
         return WARPCTCT_EINVAL;
     const Workspace w = carve(workspace, N, T, U);
     if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
     if (T > 0) {
-        int rc = done(launch_gather_units(joint, kIoF32, ys, lx, ly, w.units, N, T, U, V, true,
+        int rc = done(launch_gather_units(joint, dtype, ys, lx, ly, w.units, N, T, U, V, true,
                                           nullptr, as_stream(stream)));
         if (rc != WARPCTCT_OK) return rc;
     }
     return forward_from_units(w, ys, lx, ly, N, T, U, costs, T > 0 ? unit_grads : nullptr,
                               as_stream(stream));
+}
+
+int warpctct_loss_forward_f32(const float *joint, const int *ys, const int *lx, const int *ly,
+                              int N, int T, int U, int V, void *workspace, size_t workspace_bytes,
+                              float *costs, float *unit_grads, void *stream) {
+    return warpctct_loss_forward(joint, WARPCTCT_F32, ys, lx, ly, N, T, U, V, workspace,
+                                 workspace_bytes, costs, unit_grads, stream);
 }
 
 int warpctct_loss_forward_units_f32(const float *units_nat, const int *ys, const int *lx,

@@ -197,6 +197,33 @@ void dense_patch_lattice(const torch::Tensor &workspace, const torch::Tensor &ys
              "dense_patch_lattice");
 }
 
+// Compact hand-off for callers that own the joiner: costs (N,) and the unit
+// gradients (N,T,U+1,3) = d costs[n] / d joint[n,t,u,{0, y[u-1], y[u]}] (what
+// _C.ctct_loss_fwd of the reference returns, csrc/binding.cpp:31-100), from the
+// un-gathered joint; no dense gradient is formed.
+std::tuple<torch::Tensor, torch::Tensor> ctct_loss_compact_fwd(const torch::Tensor &joint,
+                                                               const torch::Tensor &ys,
+                                                               const torch::Tensor &lx,
+                                                               const torch::Tensor &ly) {
+    CHECK_CONTIGUOUS(joint);
+    CHECK_DEVICE(joint);
+    const int dtype = io_type_of(joint);
+    TORCH_CHECK(joint.dim() == 4, "log probs must have 4 dims.");
+    const int N = joint.size(0), T = joint.size(1), U = joint.size(2) - 1, V = joint.size(3);
+    check_lengths(ys, lx, ly, N, U);
+    const DeviceGuard device_guard(device_of(joint));
+    auto ws = make_workspace(joint, N, T, U);
+    const auto f32 = joint.options().dtype(at::ScalarType::Float);
+    auto costs = torch::empty({N}, f32);
+    auto grads = torch::empty({N, T, U + 1, 3}, f32);
+    check_rc(warpctct_loss_forward(joint.data_ptr(), dtype, ys.data_ptr<int>(), lx.data_ptr<int>(),
+                                   ly.data_ptr<int>(), N, T, U, V, ws.data_ptr(), ws.numel(),
+                                   costs.data_ptr<float>(), grads.data_ptr<float>(),
+                                   current_stream()),
+             "ctct_loss_compact_fwd");
+    return std::make_tuple(costs, grads);
+}
+
 // ctct_loss on logits: log_softmax over the vocabulary happens inside (the
 // caller of the reference applies it before warp_ctct.ctct_loss).  Same
 // contract as ctct_loss_joint_fwd; the workspace also holds the row-wise
@@ -551,6 +578,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           pybind11::arg("ys"), pybind11::arg("lx"), pybind11::arg("ly"),
           pybind11::arg("requires_grad"), pybind11::arg("reduction") = 0,
           pybind11::arg("average_frames") = false);
+    m.def("ctct_loss_compact_fwd", &ctct_loss_compact_fwd,
+          "Costs and compact unit gradients from the un-gathered joint.",
+          pybind11::arg("log_probs"), pybind11::arg("ys"), pybind11::arg("lx"),
+          pybind11::arg("ly"));
     m.def("ctct_loss_logits_fwd", &ctct_loss_logits_fwd,
           "CTC-Transducer loss on logits, log_softmax inside (forward).", pybind11::arg("logits"),
           pybind11::arg("ys"), pybind11::arg("lx"), pybind11::arg("ly"),

@@ -1,6 +1,7 @@
-"""In-tree build of the MI355X CTC-Transducer loss.
+"""Build of the MI355X CTC-Transducer loss.
 
-    python setup.py build_ext --inplace
+    python setup.py build_ext --inplace          # in-tree, what the tests and bench.py load
+    pip install --no-build-isolation .           # or as an installed package (wheel: bdist_wheel)
 
 1. `make` compiles the HIP kernels + C ABI into warp_ctct/libwarpctct_hip.so
    (hipcc, --offload-arch=gfx950).
@@ -40,6 +41,11 @@ setup(
     version="0.1.0",
     description="MI355X (gfx950) CTC-Transducer loss with the warp_ctct API",
     packages=["warp_ctct"],
+    # the HIP kernels + C ABI travel with the package, next to the binding that
+    # finds them through its $ORIGIN rpath
+    package_data={"warp_ctct": ["libwarpctct_hip.so"]},
+    python_requires=">=3.8",
+    install_requires=["torch>=2.0"],
     ext_modules=[ext],
     cmdclass={"build_ext": BuildWithHip.with_options(use_ninja=False)},
 )

@@ -22,7 +22,7 @@ except ImportError as exc:  # pragma: no cover - exercised only on a broken inst
         "(needs hipcc, --offload-arch=gfx950)"
     ) from exc
 
-__all__ = ["ctct_loss", "ctct_loss_with_logits", "ctct_simple_loss"]
+__all__ = ["ctct_loss", "ctct_loss_compact", "ctct_loss_with_logits", "ctct_simple_loss"]
 __version__ = core.library_version()
 
 
@@ -196,6 +196,40 @@ def ctct_loss(log_probs: torch.Tensor,
         return _CTCTLoss.apply(log_probs.contiguous(), _as_int(labels), _as_int(frames_lengths),
                                _as_int(labels_lengths), enable_grad, reduction,
                                bool(average_frames))
+
+
+def ctct_loss_compact(log_probs: torch.Tensor,
+                      labels: torch.Tensor,
+                      frames_lengths: torch.Tensor,
+                      labels_lengths: torch.Tensor):
+    """Per-sample costs and their gradient in compact form, without autograd.
+
+    For callers that own the joiner and want to apply the gradient themselves
+    instead of receiving a dense (N, T, U, V) tensor that is zero almost
+    everywhere.  Returns ``(costs, unit_grads, index)``:
+    ``costs`` (N,) float32; ``unit_grads`` (N, T, U, 3) float32 with
+    ``unit_grads[n, t, u, k] = d costs[n] / d log_probs[n, t, u, index[n, u, k]]``
+    (zero outside ``t < frames_lengths[n]``, ``u <= labels_lengths[n]``);
+    ``index`` (N, U, 3) int64 = ``[0, labels[u-1], labels[u]]`` with 0 where no
+    label exists, the gather index of the reference
+    (warp_ctct/__init__.py:124-131).  ``dense.scatter_add_(3, index[:, None]
+    .expand_as(unit_grads), unit_grads)`` rebuilds the dense gradient."""
+    assert log_probs.dim() == 4
+    assert labels.dim() == 2
+    assert log_probs.size(2) == labels.size(1) + 1
+    assert log_probs.size(0) == labels.size(0) == frames_lengths.size(0) == labels_lengths.size(0)
+    if log_probs.dtype not in _NATIVE_DTYPES:
+        log_probs = log_probs.float()
+    labels_i = _as_int(labels)
+    with torch.no_grad(), _no_autocast():
+        costs, unit_grads = core.ctct_loss_compact_fwd(
+            log_probs.detach().contiguous(), labels_i, _as_int(frames_lengths),
+            _as_int(labels_lengths))
+        n, u = labels_i.shape
+        index = torch.zeros(n, u + 1, 3, dtype=torch.long, device=labels_i.device)
+        index[:, 1:, 1] = labels_i
+        index[:, :-1, 2] = labels_i
+    return costs, unit_grads, index
 
 
 def ctct_loss_with_logits(logits: torch.Tensor,
