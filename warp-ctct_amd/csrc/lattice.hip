@@ -76,8 +76,7 @@ __device__ __forceinline__ void chunk_load(Chunk &c, const double *units_lane, s
 // what the chunked sweep must not do.
 template <int W>
 struct Relay {
-    double ring_x[W > 1 ? W - 1 : 1][kRing];
-    double ring_y[W > 1 ? W - 1 : 1][kRing];
+    double ring[W > 1 ? W - 1 : 1][kRing];
     int done[W > 1 ? W - 1 : 1];
     int taken[W > 1 ? W - 1 : 1];
 };
@@ -102,19 +101,20 @@ __device__ __forceinline__ void publish(int *counter, int value) {
 // alpha(t+1, 2u-1) =  alpha(t,2u-1) + LP(t,u,1)
 //                 (+) alpha(t,2u-2) + LP(t,u-1,2)
 //                 (+) [y[u-1] != y[u-2]] alpha(t,2u-3) + LP(t,u-1,2)
-// skip_mask is 0 where the third arc exists and -inf where it does not.
-// ext = {from 2u-2, from 2u-3} for lane 0 (from the previous wavefront, or
-// -inf); out = this lane's own contribution to context u+1.
-__device__ __forceinline__ void alpha_step(Front &f, const double *lp, double skip_mask,
-                                           double2 ext, double2 &out) {
-    const double from_e = f.e + lp[2];
-    const double from_o = f.o + lp[2];
-    out = make_double2(from_e, from_o);
-    const double pe = wave_shift_up(from_e, ext.x);
-    const double po = wave_shift_up(from_o, ext.y);
-    const double ne = lse2(f.e, f.o) + lp[0];
-    const double no = lse3(f.o + lp[1], pe, po + skip_mask);
-    f.e = ne;
+// The last two terms are what context u-1 sends to context u; with
+// L = alpha(t,2u-2) (+) alpha(t,2u-3), which context u-1 needs anyway for its
+// own blank state, they are  (skip arc ? L : alpha(t,2u-2)) + LP(t,u-1,2):
+// one semiring sum and one value to pass instead of two of each.
+// skip_next: the skip arc from this context's label state into the next
+// context exists (y[u] != y[u-1]).  ext = what lane 0 receives (from the
+// previous wavefront, or -inf); out = what this lane sends to context u+1.
+__device__ __forceinline__ void alpha_step(Front &f, const double *lp, bool skip_next, double ext,
+                                           double &out) {
+    const double both = lse2(f.e, f.o);
+    out = (skip_next ? both : f.e) + lp[2];
+    const double recv = wave_shift_up(out, ext);
+    const double no = lse2(f.o + lp[1], recv);
+    f.e = both + lp[0];
     f.o = no;
 }
 
@@ -122,17 +122,20 @@ __device__ __forceinline__ void alpha_step(Front &f, const double *lp, double sk
 // beta(t, 2u)   = beta(t+1,2u) + LP(t,u,0)  (+) [u<U] beta(t+1,2u+1) + LP(t,u,2)
 // beta(t, 2u-1) = beta(t+1,2u-1) + LP(t,u,1) (+) beta(t+1,2u) + LP(t,u,0)
 //              (+) [u<U, y[u-1] != y[u]] beta(t+1,2u+1) + LP(t,u,2)
-// o_mask is 0 for contexts that have a state 2u-1 (1 <= u <= Un), else -inf.
-// ext = beta(t+1, 2u+1) for lane 63 (from the next wavefront, or -inf);
-// out = this lane's beta(t+1, 2u-1), which context u-1 needs.
-__device__ __forceinline__ void beta_step(Front &f, const double *lp, double skip_mask,
-                                          double o_mask, double ext, double &out) {
+// The last two terms of the second line are beta(t,2u) itself when the skip
+// arc exists and its first term alone when it does not.
+// skip: y[u-1] != y[u] with 1 <= u < Un.  o_mask is 0 for contexts that have a
+// state 2u-1 (1 <= u <= Un), else -inf.  ext = beta(t+1, 2u+1) for lane 63
+// (from the next wavefront, or -inf); out = this lane's beta(t+1, 2u-1), which
+// context u-1 needs.
+__device__ __forceinline__ void beta_step(Front &f, const double *lp, bool skip, double o_mask,
+                                          double ext, double &out) {
     out = f.o;
     const double nb = wave_shift_down(f.o, ext);
     const double nxt = nb + lp[2];
     const double stay_e = f.e + lp[0];
     const double ne = lse2(stay_e, nxt);
-    const double no = lse3(f.o + lp[1], stay_e, nxt + skip_mask);
+    const double no = lse2(f.o + lp[1], skip ? ne : stay_e);
     f.e = ne;
     f.o = no + o_mask;
 }
@@ -147,17 +150,17 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, doubl
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int u = wave * 64 + lane;
-    double skip_mask, o_mask = 0.0;
+    double o_mask = 0.0;
+    bool skip;
     Front f;
     if (BETA) {
-        const bool skip = (u >= 1) && (u < Un) && (y[u - 1] != y[u]);
-        skip_mask = skip ? 0.0 : neg_inf();
+        skip = (u >= 1) && (u < Un) && (y[u - 1] != y[u]);
         o_mask = ((u >= 1) && (u <= Un)) ? 0.0 : neg_inf();
         f.e = (u == Un) ? 0.0 : neg_inf();
         f.o = (u == Un && Un >= 1) ? 0.0 : neg_inf();
     } else {
-        const bool skip = (u >= 2) && (u <= Un) && (y[u - 1] != y[u - 2]);
-        skip_mask = skip ? 0.0 : neg_inf();
+        // the skip arc from this context into context u+1
+        skip = (u >= 1) && (u < Un) && (y[u] != y[u - 1]);
         f.e = (u == 0) ? 0.0 : neg_inf();
         f.o = neg_inf();
     }
@@ -181,16 +184,13 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, doubl
         chunk_load(a, in, urow, Tn, t_start, dir);
         // one chunk: steps s0 .. s0+cnt-1 with the units in `c`
         auto run_chunk = [&](const Chunk &c, int s0, int cnt, bool full) {
-            double2 mail[R];
+            double mail[R];
 #pragma unroll
-            for (int r = 0; r < R; ++r) mail[r] = make_double2(neg_inf(), neg_inf());
+            for (int r = 0; r < R; ++r) mail[r] = neg_inf();
             if (consumes) {
                 wait_until(&relay.done[b_in], s0 + cnt);
 #pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    const int slot = (s0 + r) % kRing;
-                    mail[r] = make_double2(relay.ring_x[b_in][slot], relay.ring_y[b_in][slot]);
-                }
+                for (int r = 0; r < R; ++r) mail[r] = relay.ring[b_in][(s0 + r) % kRing];
                 publish(&relay.taken[b_in], s0 + cnt);
             }
             if (produces) wait_until(&relay.taken[b_out], s0 + cnt - kRing);
@@ -198,20 +198,15 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, doubl
             for (int r = 0; r < R; ++r) {
                 if (full || r < cnt) {
                     const int s = s0 + r;
-                    double2 mine;
+                    double mine;
                     if (BETA) {
-                        double mo;
-                        beta_step(f, c.lp[r], skip_mask, o_mask, mail[r].x, mo);
-                        mine = make_double2(mo, 0.0);
+                        beta_step(f, c.lp[r], skip, o_mask, mail[r], mine);
                         front_store(out + (size_t)(Tn - 1 - s) * srow, f);
                     } else {
-                        alpha_step(f, c.lp[r], skip_mask, mail[r], mine);
+                        alpha_step(f, c.lp[r], skip, mail[r], mine);
                         front_store(out + (size_t)(s + 1) * srow, f);
                     }
-                    if (produces && lane == edge_lane) {
-                        relay.ring_x[b_out][s % kRing] = mine.x;
-                        if (!BETA) relay.ring_y[b_out][s % kRing] = mine.y;
-                    }
+                    if (produces && lane == edge_lane) relay.ring[b_out][s % kRing] = mine;
                 }
             }
             if (produces) publish(&relay.done[b_out], s0 + cnt);
