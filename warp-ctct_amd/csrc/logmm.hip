@@ -103,6 +103,57 @@ __global__ __launch_bounds__(256) void shift_exp_kernel(const float *__restrict_
     }
 }
 
+// The same with the whole row held in registers (NV 16-byte vectors per lane,
+// K <= 256*NV): the operand is read once.  Requires contiguous, 16-byte
+// aligned rows (the launcher checks).
+template <int NV>
+__global__ __launch_bounds__(256) void shift_exp_rows_kernel(const float *__restrict__ x, long sb,
+                                                             long sr, int R, int K, int Kp,
+                                                             const int *__restrict__ len,
+                                                             int extra, float *__restrict__ mx,
+                                                             float *__restrict__ E) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r = blockIdx.x * 4 + wave;
+    const int b = blockIdx.y;
+    if (r >= R) return;
+    const int Rb = len ? min(max(len[b], 0) + extra, R) : R;
+    float *e = E + ((size_t)b * R + r) * Kp;
+    const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (r >= Rb) {
+        for (int k = lane * 4; k < Kp; k += 256) *reinterpret_cast<v4f *>(e + k) = zero;
+        if (lane == 0) mx[(size_t)b * R + r] = neg_inf_f();
+        return;
+    }
+    const float *p = x + (size_t)b * sb + (size_t)r * sr;
+    v4f v[NV];
+#pragma unroll
+    for (int j = 0; j < NV; ++j)
+        v[j] = *reinterpret_cast<const v4f *>(p + min(j * 256 + lane * 4, K - 4));
+    float m = neg_inf_f();
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        if (j * 256 + lane * 4 < K)
+            m = fmaxf(fmaxf(m, fmaxf(v[j].x, v[j].y)), fmaxf(v[j].z, v[j].w));
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    if (lane == 0) mx[(size_t)b * R + r] = m;
+    const float shift = finite_or_zero(m);
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+        const int k = j * 256 + lane * 4;
+        if (k >= Kp) continue;
+        v4f o = zero;
+        if (k < K) {
+            o.x = exp2_hw((v[j].x - shift) * kLog2eF);
+            o.y = exp2_hw((v[j].y - shift) * kLog2eF);
+            o.z = exp2_hw((v[j].z - shift) * kLog2eF);
+            o.w = exp2_hw((v[j].w - shift) * kLog2eF);
+        }
+        *reinterpret_cast<v4f *>(e + k) = o;
+    }
+}
+
 // ---- MFMA tiles ----------------------------------------------------------------
 // v_mfma_f32_16x16x4_f32: lane l supplies A[l%16][l/16] and B[l/16][l%16] and
 // holds D[4*(l/16) + r][l%16] in register r of the accumulator.
@@ -706,21 +757,49 @@ hipError_t launch_bwd(const BwdArgs &a, int B, hipStream_t stream) {
 
 }  // namespace
 
+namespace {
+
+// rows r of x[b, r, k] with strides (sb, sr, sk), see shift_exp_kernel
+void launch_shift_exp_rows(const float *x, long sb, long sr, long sk, int B, int R, int K, int Kp,
+                           const int *len, int extra, float *mx, float *E, hipStream_t stream) {
+    const dim3 grid((R + 3) / 4, B), block(256);
+    const bool rows_ok = sk == 1 && K >= 4 && (K & 3) == 0 && (sb & 3) == 0 && (sr & 3) == 0 &&
+                         (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+    if (rows_ok && K <= 1024) {
+        hipLaunchKernelGGL(shift_exp_rows_kernel<4>, grid, block, 0, stream, x, sb, sr, R, K, Kp,
+                           len, extra, mx, E);
+    } else if (rows_ok && K <= 2048) {
+        hipLaunchKernelGGL(shift_exp_rows_kernel<8>, grid, block, 0, stream, x, sb, sr, R, K, Kp,
+                           len, extra, mx, E);
+    } else if (rows_ok && K <= 4096) {
+        hipLaunchKernelGGL(shift_exp_rows_kernel<16>, grid, block, 0, stream, x, sb, sr, R, K, Kp,
+                           len, extra, mx, E);
+    } else if (rows_ok && K <= 8192) {
+        hipLaunchKernelGGL(shift_exp_rows_kernel<32>, grid, block, 0, stream, x, sb, sr, R, K, Kp,
+                           len, extra, mx, E);
+    } else {
+        hipLaunchKernelGGL(shift_exp_kernel, grid, block, 0, stream, x, sb, sr, sk, R, K, Kp, len,
+                           extra, mx, E);
+    }
+}
+
+}  // namespace
+
 hipError_t launch_logmm_shift_exp(const LogmmOperand &lhs, const LogmmOperand &rhs,
                                   const LogmmShifted &sh, int B, int M, int K, int Nn,
                                   const int *row_len, const int *col_len, hipStream_t stream) {
     const int Kp = logmm_padded_reduction(K);
     if (B == 0 || Kp == 0) return hipSuccess;
     if (M > 0) {
-        hipLaunchKernelGGL(shift_exp_kernel, dim3((M + 3) / 4, B), dim3(256), 0, stream, lhs.p,
-                           lhs.sb, lhs.s1, lhs.s2, M, K, Kp, row_len, 0, sh.lmax, sh.El);
+        launch_shift_exp_rows(lhs.p, lhs.sb, lhs.s1, lhs.s2, B, M, K, Kp, row_len, 0, sh.lmax,
+                              sh.El, stream);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
     if (Nn > 0) {
         // rhs[b,k,j]: the rows are j (stride s2), k has stride s1
-        hipLaunchKernelGGL(shift_exp_kernel, dim3((Nn + 3) / 4, B), dim3(256), 0, stream, rhs.p,
-                           rhs.sb, rhs.s2, rhs.s1, Nn, K, Kp, col_len, 1, sh.rmax, sh.Er);
+        launch_shift_exp_rows(rhs.p, rhs.sb, rhs.s2, rhs.s1, B, Nn, K, Kp, col_len, 1, sh.rmax,
+                              sh.Er, stream);
     }
     return hipGetLastError();
 }
