@@ -72,6 +72,7 @@ int forward_from_units(const Workspace &w, const int *ys, const int *lx, const i
 struct SimpleWorkspace {
     Workspace lattice;
     float *unit_grads;   // (N,T,U+1,3)
+    float *partial;      // up to 8 x (N,T,U+1): partial sums of a split log-matmul reduction
     size_t bytes;
 };
 
@@ -81,7 +82,8 @@ SimpleWorkspace carve_simple(void *base, int N, int T, int U) {
     const uintptr_t p = reinterpret_cast<uintptr_t>(base) + w.lattice.bytes;
     const size_t ug_b = align256((size_t)N * T * (U + 1) * 3 * sizeof(float));
     w.unit_grads = reinterpret_cast<float *>(p);
-    w.bytes = w.lattice.bytes + ug_b;
+    w.partial = reinterpret_cast<float *>(p + ug_b);
+    w.bytes = w.lattice.bytes + ug_b + align256((size_t)8 * N * T * (U + 1) * sizeof(float));
     return w;
 }
 
@@ -105,6 +107,7 @@ PairWorkspace carve_pairs(void *base, int B, int M, int Nn) {
 struct LogmmWorkspace {
     LogmmShifted sh;
     PairWorkspace pw;
+    float *partial;   // forward only: partial sums of a split reduction
     size_t bytes;
 };
 
@@ -122,7 +125,10 @@ LogmmWorkspace carve_logmm(void *base, int B, int M, int K, int Nn) {
     w.sh.Er = reinterpret_cast<float *>(p);
     p += align256((size_t)B * Nn * Kp * sizeof(float));
     w.pw = carve_pairs(reinterpret_cast<void *>(p), B, M, Nn);
-    w.bytes = (p - p0) + w.pw.bytes;
+    p += w.pw.bytes;
+    w.partial = reinterpret_cast<float *>(p);
+    p += align256((size_t)logmm_fwd_splits(B, M, K, Nn) * B * M * Nn * sizeof(float));
+    w.bytes = p - p0;
     return w;
 }
 
@@ -534,7 +540,7 @@ int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, c
             const LogmmShifted sh = {fmax, gmax, fexp, gexp};
             int rc = done(launch_logmm_shift_exp(lhs, rhs, sh, N, T, V, U + 1, lx, ly, st));
             if (rc != WARPCTCT_OK) return rc;
-            rc = done(launch_logmm_fwd(lhs, rhs, sh, den, N, T, V, U + 1, lx, ly, st));
+            rc = done(launch_logmm_fwd(lhs, rhs, sh, den, w.partial, N, T, V, U + 1, lx, ly, st));
             if (rc != WARPCTCT_OK) return rc;
         }
         int rc = done(launch_simple_gather_units(f, g, normalized ? den : nullptr, ys, lx, ly,
@@ -649,7 +655,7 @@ int warpctct_logmm_fwd_f32(const float *lhs, long lsb, long lsm, long lsk, const
     int rc = done(launch_logmm_shift_exp(l, r, w.sh, B, M, K, Nn, nullptr, nullptr,
                                          as_stream(stream)));
     if (rc != WARPCTCT_OK) return rc;
-    return done(launch_logmm_fwd(l, r, w.sh, res, B, M, K, Nn, nullptr, nullptr,
+    return done(launch_logmm_fwd(l, r, w.sh, res, w.partial, B, M, K, Nn, nullptr, nullptr,
                                  as_stream(stream)));
 }
 

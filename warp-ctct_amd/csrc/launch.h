@@ -128,9 +128,13 @@ struct LogmmShifted {
 hipError_t launch_logmm_shift_exp(const LogmmOperand &lhs, const LogmmOperand &rhs,
                                   const LogmmShifted &sh, int B, int M, int K, int Nn,
                                   const int *row_len, const int *col_len, hipStream_t stream);
+// partial (may be null): logmm_fwd_splits(B,M,K,Nn) * B*M*Nn floats of scratch; with it the
+// reduction of a small output is split over several workgroups per tile
+int logmm_fwd_splits(int B, int M, int K, int Nn);
 hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
-                            const LogmmShifted &sh, float *res, int B, int M, int K, int Nn,
-                            const int *row_len, const int *col_len, hipStream_t stream);
+                            const LogmmShifted &sh, float *res, float *partial, int B, int M,
+                            int K, int Nn, const int *row_len, const int *col_len,
+                            hipStream_t stream);
 // C (B,M,Nn) and flags (B,M): the pair factors go * exp(lmax + rmax - res) that
 // both gradients share, and per row whether a pair was left to the exact pass;
 // batch_scale (may be null) multiplies grad_out per batch.

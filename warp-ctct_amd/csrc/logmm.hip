@@ -233,12 +233,26 @@ struct FwdArgs {
     const float *lhs, *rhs;   // the operands themselves, for the exact fallback
     long lsb, lsm, lsk, rsb, rsk, rsn;
     float *res;               // (B,M,Nn)
+    // the reduction may be split over `splits` workgroups (more of them than a
+    // small output has tiles); then each writes its partial sums to
+    // partial (splits,B,M,Nn) and logmm_fwd_finish_kernel adds them up
+    float *partial;
+    int splits, chunks_per_split;
     int M, K, Kp, Nn;
     const int *row_len, *col_len;
 };
 
-// grid (ceil(M/TM), ceil(Nn/TN), B) with TM = 16*RB*WR rows i and TN = 16*CB*WC
-// columns j per workgroup of 64*WR*WC threads.
+// res from a sum s of shifted exponentials; the exact fallback for sums that
+// underflowed (or overflowed)
+__device__ __forceinline__ float fwd_result(const FwdArgs &a, int b, int i, int j, float s) {
+    if (s >= kTiny && s < __builtin_huge_valf())
+        return a.lmax[(size_t)b * a.M + i] + a.rmax[(size_t)b * a.Nn + j] + log2_hw(s) * kLn2F;
+    return exact_lse(a.lhs + (size_t)b * a.lsb + (size_t)i * a.lsm, a.lsk,
+                     a.rhs + (size_t)b * a.rsb + (size_t)j * a.rsn, a.rsk, a.K);
+}
+
+// grid (ceil(M/TM), ceil(Nn/TN) * splits, B) with TM = 16*RB*WR rows i and
+// TN = 16*CB*WC columns j per workgroup of 64*WR*WC threads.
 template <int RB, int CB, int WR, int WC>
 __global__ __launch_bounds__(64 * WR * WC) void logmm_fwd_kernel(const FwdArgs a) {
     constexpr int TM = 16 * RB * WR, TN = 16 * CB * WC, NT = 64 * WR * WC;
@@ -248,7 +262,8 @@ __global__ __launch_bounds__(64 * WR * WC) void logmm_fwd_kernel(const FwdArgs a
     __shared__ __attribute__((aligned(16))) float sa[2][TM][LDK];   // E_l[i][k]
     __shared__ __attribute__((aligned(16))) float sb_[2][TN][LDK];  // E_r[j][k]
     const int b = blockIdx.z;
-    const int i0 = blockIdx.x * TM, j0 = blockIdx.y * TN;
+    const int split = blockIdx.y % a.splits;
+    const int i0 = blockIdx.x * TM, j0 = (blockIdx.y / a.splits) * TN;
     const int M = a.M, Nn = a.Nn, Kp = a.Kp;
     // lengths-aware: rows >= row_len[b] and cols > col_len[b] are padding
     const int Mb = a.row_len ? min(max(a.row_len[b], 0), M) : M;
@@ -307,13 +322,15 @@ __global__ __launch_bounds__(64 * WR * WC) void logmm_fwd_kernel(const FwdArgs a
 
     // chunk j lives in register set j % kDepth and in LDS buffer j % 2; an empty
     // reduction leaves the sums at 0: log 0 below
-    const int n = Kp / TQ;
-    const int k_last = max(Kp - TQ, 0);
+    // this workgroup's share of the reduction: chunks [c_begin, c_begin + n)
+    const int c_begin = split * a.chunks_per_split;
+    const int n = max(min(Kp / TQ - c_begin, a.chunks_per_split), 0);
+    const int k_first = c_begin * TQ, k_last = max(k_first + (n - 1) * TQ, 0);
     if (n > 0) {
 #pragma unroll
-        for (int d = 0; d < kDepth; ++d) fetch(d, min(d * TQ, k_last));
+        for (int d = 0; d < kDepth; ++d) fetch(d, min(k_first + d * TQ, k_last));
         stash(0, 0);
-        fetch(0, min(kDepth * TQ, k_last));
+        fetch(0, min(k_first + kDepth * TQ, k_last));
         __syncthreads();
     }
     for (int j0 = 0; j0 < n; j0 += kDepth) {
@@ -324,13 +341,11 @@ __global__ __launch_bounds__(64 * WR * WC) void logmm_fwd_kernel(const FwdArgs a
                 tile_mfma_qq<RB, CB>(sa[d & 1], sb_[d & 1], row0, col0, lane, acc);
                 stash((d + 1) % kDepth, (d + 1) & 1);
                 // set (d+1) % kDepth is free again: refill it kDepth chunks ahead
-                fetch((d + 1) % kDepth, min((j + 1 + kDepth) * TQ, k_last));
+                fetch((d + 1) % kDepth, min(k_first + (j + 1 + kDepth) * TQ, k_last));
                 __syncthreads();
             }
         }
     }
-    const float *lm = a.lmax + (size_t)b * M;
-    const float *rm = a.rmax + (size_t)b * Nn;
 #pragma unroll
     for (int r4 = 0; r4 < RB; ++r4) {
 #pragma unroll
@@ -341,17 +356,29 @@ __global__ __launch_bounds__(64 * WR * WC) void logmm_fwd_kernel(const FwdArgs a
                 const int j = j0 + col0 + c * 16 + (lane & 15);
                 if (i >= Mb || j >= Nb) continue;
                 const float s = acc[r4][c][r];
-                float out;
-                if (s >= kTiny && s < __builtin_huge_valf()) {
-                    out = lm[i] + rm[j] + log2_hw(s) * kLn2F;
-                } else {
-                    out = exact_lse(a.lhs + (size_t)b * a.lsb + (size_t)i * a.lsm, a.lsk,
-                                    a.rhs + (size_t)b * a.rsb + (size_t)j * a.rsn, a.rsk, a.K);
-                }
-                a.res[((size_t)b * M + i) * Nn + j] = out;
+                const size_t at = ((size_t)b * M + i) * Nn + j;
+                if (a.splits > 1)
+                    a.partial[(size_t)split * gridDim.z * M * Nn + at] = s;
+                else
+                    a.res[at] = fwd_result(a, b, i, j, s);
             }
         }
     }
+}
+
+// res from the partial sums of a split reduction, added in a fixed order.
+__global__ __launch_bounds__(256) void logmm_fwd_finish_kernel(const FwdArgs a, int B) {
+    const int b = blockIdx.y;
+    const int e = blockIdx.x * 256 + threadIdx.x;
+    if (e >= a.M * a.Nn) return;
+    const int i = e / a.Nn, j = e - i * a.Nn;
+    const int Mb = a.row_len ? min(max(a.row_len[b], 0), a.M) : a.M;
+    const int Nb = a.col_len ? min(max(a.col_len[b], 0) + 1, a.Nn) : a.Nn;
+    if (i >= Mb || j >= Nb) return;
+    const size_t at = (size_t)b * a.M * a.Nn + e;
+    float s = 0.0f;
+    for (int sp = 0; sp < a.splits; ++sp) s += a.partial[(size_t)sp * B * a.M * a.Nn + at];
+    a.res[at] = fwd_result(a, b, i, j, s);
 }
 
 // ---- backward ----------------------------------------------------------------
@@ -804,11 +831,25 @@ hipError_t launch_logmm_shift_exp(const LogmmOperand &lhs, const LogmmOperand &r
     return hipGetLastError();
 }
 
+int logmm_fwd_splits(int B, int M, int K, int Nn) {
+    // enough workgroups for a few per CU, and at least 2*kDepth chunks each
+    const int chunks = logmm_padded_reduction(K) / TQ;
+    const long tiles = (long)((M + 31) / 32) * ((Nn + 95) / 96) * B;
+    int splits = 1;
+    while (splits < 8 && tiles * splits < 1024 && chunks / (splits * 2) >= 2 * kDepth) splits *= 2;
+    return splits;
+}
+
 hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
-                            const LogmmShifted &sh, float *res, int B, int M, int K, int Nn,
-                            const int *row_len, const int *col_len, hipStream_t stream) {
+                            const LogmmShifted &sh, float *res, float *partial, int B, int M,
+                            int K, int Nn, const int *row_len, const int *col_len,
+                            hipStream_t stream) {
     if (B == 0 || M == 0 || Nn == 0) return hipSuccess;
     FwdArgs a;
+    a.splits = partial ? logmm_fwd_splits(B, M, K, Nn) : 1;
+    a.partial = partial;
+    a.chunks_per_split = (logmm_padded_reduction(K) / TQ + a.splits - 1) / a.splits;
+    if (a.chunks_per_split < 1) a.chunks_per_split = 1;
     a.El = sh.El, a.Er = sh.Er, a.lmax = sh.lmax, a.rmax = sh.rmax;
     a.lhs = lhs.p, a.lsb = lhs.sb, a.lsm = lhs.s1, a.lsk = lhs.s2;
     a.rhs = rhs.p, a.rsb = rhs.sb, a.rsk = rhs.s1, a.rsn = rhs.s2;
@@ -816,12 +857,17 @@ hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
     a.row_len = row_len, a.col_len = col_len;
     // 4 wavefronts per workgroup: 32 rows i by 96 or 64 columns j
     if (prefer_96(Nn)) {
-        dim3 grid((M + 31) / 32, (Nn + 95) / 96, B);
+        dim3 grid((M + 31) / 32, (Nn + 95) / 96 * a.splits, B);
         hipLaunchKernelGGL((logmm_fwd_kernel<1, 3, 2, 2>), grid, dim3(256), 0, stream, a);
     } else {
-        dim3 grid((M + 31) / 32, (Nn + 63) / 64, B);
+        dim3 grid((M + 31) / 32, (Nn + 63) / 64 * a.splits, B);
         hipLaunchKernelGGL((logmm_fwd_kernel<1, 2, 2, 2>), grid, dim3(256), 0, stream, a);
     }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || a.splits == 1) return e;
+    const long outs = (long)M * Nn;
+    hipLaunchKernelGGL(logmm_fwd_finish_kernel, dim3((unsigned)((outs + 255) / 256), B), dim3(256),
+                       0, stream, a, B);
     return hipGetLastError();
 }
 
