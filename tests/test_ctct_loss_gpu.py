@@ -377,6 +377,69 @@ def test_compact_hand_off_rebuilds_the_dense_gradient():
         np.testing.assert_allclose(dense.cpu().numpy(), ref_dense, atol=GRAD_ATOL, rtol=0)
 
 
+def test_edge_shapes_no_labels_single_frame_and_empty_batch():
+    """U = 0 (no labels at all: only the all-blank path), samples without
+    labels next to samples with labels, a single frame, and an empty batch."""
+    import warp_ctct
+    rng = np.random.default_rng(61)
+    # no label dimension at all
+    joint = np.log(rng.dirichlet(np.ones(6), size=(3, 7, 1))).astype(np.float32)
+    ys = np.zeros((3, 0), np.int32)
+    lx, ly = np.array([7, 4, 1], np.int32), np.zeros(3, np.int32)
+    x = dev(joint).requires_grad_(True)
+    c = warp_ctct.ctct_loss(x, dev(ys), dev(lx), dev(ly), reduction="none")
+    ref = np.array([-joint[n, :lx[n], 0, 0].sum() for n in range(3)])   # blank on every frame
+    np.testing.assert_allclose(c.detach().cpu().numpy(), ref, rtol=LOSS_RTOL)
+    c.sum().backward()
+    g = x.grad.cpu().numpy()
+    for n in range(3):
+        np.testing.assert_allclose(g[n, :lx[n], 0, 0], -1.0, atol=GRAD_ATOL)
+        assert np.all(g[n, lx[n]:] == 0) and np.all(g[n, :, :, 1:] == 0)
+    # samples with zero labels inside a batch that has labels; one frame only
+    joint, ys, lx, ly = make_joint_case(62, 4, 9, 3, 8, lx=[9, 5, 1, 3], ly=[3, 0, 1, 0])
+    _, ref_dense, ref_costs = O.ctct_loss(joint, ys, lx, ly, reduction="sum")
+    x = dev(joint).requires_grad_(True)
+    c = warp_ctct.ctct_loss(x, dev(ys), dev(lx), dev(ly), reduction="none")
+    np.testing.assert_allclose(c.detach().cpu().numpy(), ref_costs, rtol=LOSS_RTOL)
+    c.sum().backward()
+    np.testing.assert_allclose(x.grad.cpu().numpy(), ref_dense, atol=GRAD_ATOL, rtol=0)
+    # empty batch: nothing to launch, empty results, torch's reductions of empty tensors
+    e = torch.zeros(0, 5, 3, 4, device="cuda", requires_grad=True)
+    ei = torch.zeros(0, 2, dtype=torch.int32, device="cuda")
+    el = torch.zeros(0, dtype=torch.int32, device="cuda")
+    out = warp_ctct.ctct_loss(e, ei, el, el, reduction="none")
+    assert tuple(out.shape) == (0,)
+    s = warp_ctct.ctct_loss(e, ei, el, el, reduction="sum")
+    assert s.item() == 0.0
+    s.backward()
+    assert tuple(e.grad.shape) == (0, 5, 3, 4)
+    assert torch.isnan(warp_ctct.ctct_loss(e, ei, el, el, reduction="mean"))
+
+
+def test_widest_lattice_eight_wavefronts():
+    """U + 1 = 512 contexts: eight wavefronts per lattice and direction, the
+    largest the kernel accepts; one more context is refused."""
+    import warp_ctct
+    T, U, V = 530, 511, 6
+    joint, ys, lx, ly = make_joint_case(63, 1, T, U, V, lx=[T], ly=[U], force_repeat=False,
+                                        zero_pad=False)
+    ys[0] = 1 + np.arange(U) % (V - 1)        # no adjacent repeats: all 511 labels fit
+    ys[0, 300] = ys[0, 299]                   # but one, in the fifth wavefront
+    ly[0] = U
+    _, ref_dense, ref_costs = O.ctct_loss(joint, ys, lx, ly, reduction="sum")
+    x = dev(joint).requires_grad_(True)
+    c = warp_ctct.ctct_loss(x, dev(ys), dev(lx), dev(ly), reduction="none")
+    np.testing.assert_allclose(c.detach().cpu().numpy(), ref_costs, rtol=LOSS_RTOL)
+    c.sum().backward()
+    got = x.grad.cpu().numpy()
+    np.testing.assert_allclose(got, ref_dense, atol=GRAD_ATOL, rtol=0)
+    assert_support(got, ref_dense, "dense gradient, 8 wavefronts")
+    too_wide = torch.zeros(1, 4, 514, 3, device="cuda")
+    with pytest.raises(RuntimeError):
+        warp_ctct.ctct_loss(too_wide, torch.ones(1, 513, dtype=torch.int32, device="cuda"),
+                            torch.tensor([4], device="cuda"), torch.tensor([2], device="cuda"))
+
+
 def test_operator_surface_on_gathered_units():
     """_C.ctct_loss_fwd keeps the reference's contract: gathered (N,T,U+1,3)
     input, (costs, grads) output, grads zero in padding, costs twice when

@@ -189,6 +189,10 @@ def ctct_loss(log_probs: torch.Tensor,
     assert log_probs.size(2) == labels.size(1) + 1
     assert log_probs.size(0) == labels.size(0) == frames_lengths.size(0) == labels_lengths.size(0)
 
+    if log_probs.size(0) == 0:
+        # nothing to launch; costs of an empty batch, still attached to the graph
+        return _reduce(log_probs.float().sum(dim=(1, 2, 3)), frames_lengths, reduction,
+                       average_frames)
     enable_grad = log_probs.requires_grad and torch.is_grad_enabled()
     if log_probs.dtype not in _NATIVE_DTYPES:
         log_probs = log_probs.float()      # as the reference does for every dtype (:135)
@@ -255,6 +259,9 @@ def ctct_loss_with_logits(logits: torch.Tensor,
     assert logits.size(2) == labels.size(1) + 1
     assert logits.size(0) == labels.size(0) == frames_lengths.size(0) == labels_lengths.size(0)
 
+    if logits.size(0) == 0:
+        return _reduce(logits.float().sum(dim=(1, 2, 3)), frames_lengths, reduction,
+                       average_frames)
     enable_grad = logits.requires_grad and torch.is_grad_enabled()
     if logits.dtype not in _NATIVE_DTYPES:
         logits = logits.float()
