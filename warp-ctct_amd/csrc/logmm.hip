@@ -832,11 +832,12 @@ hipError_t launch_logmm_shift_exp(const LogmmOperand &lhs, const LogmmOperand &r
 }
 
 int logmm_fwd_splits(int B, int M, int K, int Nn) {
-    // enough workgroups for a few per CU, and at least 2*kDepth chunks each
+    // only when there are fewer tiles than CUs (the extra pass over the partial sums costs as
+    // much as it gains otherwise), and at least 2*kDepth chunks each
     const int chunks = logmm_padded_reduction(K) / TQ;
     const long tiles = (long)((M + 31) / 32) * ((Nn + 95) / 96) * B;
     int splits = 1;
-    while (splits < 8 && tiles * splits < 1024 && chunks / (splits * 2) >= 2 * kDepth) splits *= 2;
+    while (splits < 8 && tiles * splits < 256 && chunks / (splits * 2) >= 2 * kDepth) splits *= 2;
     return splits;
 }
 

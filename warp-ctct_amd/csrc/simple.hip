@@ -12,6 +12,7 @@
 //    (SimpleCTCTLoss.backward, warp_ctct/__init__.py:76-85).
 #include "device_utils.h"
 #include "launch.h"
+#include "unit_grad.h"
 
 namespace wctct {
 
@@ -34,7 +35,9 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     const int Tn = clampi(lx[n], 0, T), Un = clampi(ly[n], 0, U);
     if (t >= Tn) return;
     double *o = units + (((size_t)n * T + t) * P + u) * 3;
-    if (u > Un) {   // padding context of a live frame: neutral units
+    // padding context of a live frame, or a cell outside the band of complete
+    // alignments (its units cannot influence costs or gradients): neutral units
+    if (u > Un || outside_band(t, u, Tn, Un)) {
         o[0] = 0.0;
         o[1] = 0.0;
         o[2] = neg_inf();
@@ -127,9 +130,12 @@ __global__ __launch_bounds__(kBlock) void simple_scatter_f_kernel(
     const int t = cell / U1, u = cell - t * U1;
     const int Tn = clampi(lx[n], 0, T), Un = clampi(ly[n], 0, U);
     if (t >= Tn || u > Un) return;
+    // cells that no complete alignment passes through hold exact zeros: no add
+    const float gv = grad_f[((size_t)n * T + t) * U1 + u];
+    if (gv == 0.0f) return;
     const float w = grad_out ? grad_out[n] : 1.0f;
     const int col = (u == 0) ? 0 : clampi(ys[(size_t)n * U + u - 1], 0, V - 1);
-    atomicAdd(dense_f + ((size_t)n * T + t) * V + col, w * grad_f[((size_t)n * T + t) * U1 + u]);
+    atomicAdd(dense_f + ((size_t)n * T + t) * V + col, w * gv);
 }
 
 // dense_g[n,u,{0,y[u-1],y[u]}] += w[n] * grad_g[n,u,k]: backward of g.gather

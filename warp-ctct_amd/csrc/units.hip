@@ -128,7 +128,8 @@ __global__ __launch_bounds__(kCellBlock) void unit_grads_kernel(
     if (!c.in_range) return;
     float *go = unit_grads + (((size_t)c.n * T + c.t) * (U + 1) + c.u) * 3;
     UnitGrad g = {0.0f, 0.0f, 0.0f};
-    if (c.live) {
+    // outside the band of complete alignments the gradient is exactly zero
+    if (c.live && !outside_band(c.t, c.u, c.Tn, c.Un)) {
         const size_t lat = (size_t)(T + 1) * P * 2;
         g = unit_grad_cell(units + (size_t)c.n * T * P * 3, alphas + (size_t)c.n * lat,
                            betas + (size_t)c.n * lat, ys + (size_t)c.n * U, c.t, c.u, c.Un, P);
