@@ -81,13 +81,36 @@ struct Relay {
     int taken[W > 1 ? W - 1 : 1];
 };
 
-__device__ __forceinline__ void wait_until(int *counter, int target) {
+// Returns the value seen (>= target unless the spin bound was hit).
+__device__ __forceinline__ int wait_until(int *counter, int target) {
+    int seen = 0;
     for (int spins = 0; spins < kMaxSpins; ++spins) {
-        const int seen = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        if (__builtin_amdgcn_readfirstlane(seen) >= target) break;
+        seen = __builtin_amdgcn_readfirstlane(
+            __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP));
+        if (seen >= target) break;
         __builtin_amdgcn_s_sleep(1);
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    return seen;
+}
+
+// Consumer side of a hand-over: the counter and the R ring slots of the chunk
+// are requested in one batch (LDS serves a wavefront's requests in order, so
+// slots read after a counter that already shows the chunk are the chunk's
+// values); only if the counter was not there yet is the batch repeated.  One
+// LDS round trip per chunk instead of two.
+__device__ __forceinline__ void wait_and_take(int *counter, int target, const double *ring,
+                                              int s0, double (&mail)[R]) {
+    for (int spins = 0; spins < kMaxSpins; ++spins) {
+        const int seen = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        __atomic_signal_fence(__ATOMIC_SEQ_CST);   // the compiler keeps the order of the requests
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            mail[r] = __hip_atomic_load(ring + (s0 + r) % kRing, __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (__builtin_amdgcn_readfirstlane(seen) >= target) break;
+        __builtin_amdgcn_s_sleep(1);
+    }
 }
 
 __device__ __forceinline__ void publish(int *counter, int value) {
@@ -182,18 +205,20 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, doubl
         const int dir = BETA ? -1 : 1;
         const int t_start = BETA ? Tn - 1 : 0;
         chunk_load(a, in, urow, Tn, t_start, dir);
+        int taken_seen = 0;
         // one chunk: steps s0 .. s0+cnt-1 with the units in `c`
         auto run_chunk = [&](const Chunk &c, int s0, int cnt, bool full) {
             double mail[R];
 #pragma unroll
             for (int r = 0; r < R; ++r) mail[r] = neg_inf();
             if (consumes) {
-                wait_until(&relay.done[b_in], s0 + cnt);
-#pragma unroll
-                for (int r = 0; r < R; ++r) mail[r] = relay.ring[b_in][(s0 + r) % kRing];
+                wait_and_take(&relay.done[b_in], s0 + cnt, relay.ring[b_in], s0, mail);
                 publish(&relay.taken[b_in], s0 + cnt);
             }
-            if (produces) wait_until(&relay.taken[b_out], s0 + cnt - kRing);
+            // the ring is four chunks deep: the consumer's progress is looked
+            // up again only when the last value seen no longer covers this chunk
+            if (produces && taken_seen < s0 + cnt - kRing)
+                taken_seen = wait_until(&relay.taken[b_out], s0 + cnt - kRing);
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 if (full || r < cnt) {
