@@ -440,6 +440,41 @@ def test_widest_lattice_eight_wavefronts():
                             torch.tensor([4], device="cuda"), torch.tensor([2], device="cuda"))
 
 
+def test_forward_and_backward_replay_from_a_hip_graph():
+    """Nothing in the path synchronises with the host or clears memory with a
+    memset, so a training step can be captured once and replayed: every replay
+    (with eager work and synchronisations in between, on fresh input values)
+    must reproduce the eager result of the same inputs bit for bit."""
+    import warp_ctct
+    joint, ys, lx, ly = make_joint_case(71, 6, 33, 9, 40, lx=range(20, 34), ly=range(3, 10))
+    d_ys, d_lx, d_ly = dev(ys), dev(lx), dev(ly)
+    static_in = dev(joint).requires_grad_(True)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                       # warm-up outside the capture
+        for _ in range(2):
+            torch.autograd.grad(warp_ctct.ctct_loss(static_in, d_ys, d_lx, d_ly), static_in)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_loss = warp_ctct.ctct_loss(static_in, d_ys, d_lx, d_ly)
+        static_grad, = torch.autograd.grad(static_loss, static_in)
+    rng = np.random.default_rng(72)
+    for replay in range(4):
+        fresh = torch.log_softmax(dev(rng.standard_normal(joint.shape).astype(np.float32)), -1)
+        with torch.no_grad():
+            static_in.copy_(fresh)
+        graph.replay()
+        torch.cuda.synchronize()
+        got_loss, got_grad = static_loss.clone(), static_grad.clone()
+        x = fresh.clone().requires_grad_(True)           # eager work between the replays
+        loss = warp_ctct.ctct_loss(x, d_ys, d_lx, d_ly)
+        grad, = torch.autograd.grad(loss, x)
+        torch.cuda.synchronize()
+        assert torch.equal(got_loss, loss), "replay %d: loss differs from eager" % replay
+        assert torch.equal(got_grad, grad), "replay %d: gradient differs from eager" % replay
+
+
 def test_operator_surface_on_gathered_units():
     """_C.ctct_loss_fwd keeps the reference's contract: gathered (N,T,U+1,3)
     input, (costs, grads) output, grads zero in padding, costs twice when

@@ -177,6 +177,45 @@ def test_public_simple_loss_and_grads(case, normalized):
         assert np.all(tg.grad[n, ly[n] + 1:].cpu().numpy() == 0)
 
 
+@pytest.mark.parametrize("normalized", [True, False])
+def test_simple_loss_replays_from_a_hip_graph(normalized):
+    """A captured ctct_simple_loss step (log-matmul, lattice, scatter) replays
+    with the eager results of the same inputs; the scatter adds atomically, so
+    gradients are compared within float32 rounding, the loss exactly."""
+    import warp_ctct
+    f, g, ys, lx, ly = make_simple_case(31, 3, 21, 6, 48, lx=range(12, 22), ly=range(2, 7),
+                                        normalized=normalized)
+    d_ys, d_lx, d_ly = dev(ys), dev(lx), dev(ly)
+    sf, sg = dev(f).requires_grad_(True), dev(g).requires_grad_(True)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            torch.autograd.grad(warp_ctct.ctct_simple_loss(sf, sg, d_ys, d_lx, d_ly,
+                                                           normalized=normalized), (sf, sg))
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        s_loss = warp_ctct.ctct_simple_loss(sf, sg, d_ys, d_lx, d_ly, normalized=normalized)
+        s_gf, s_gg = torch.autograd.grad(s_loss, (sf, sg))
+    rng = np.random.default_rng(32)
+    for replay in range(3):
+        with torch.no_grad():
+            sf.copy_(dev(rng.standard_normal(f.shape).astype(np.float32)))
+            sg.copy_(dev(rng.standard_normal(g.shape).astype(np.float32)))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = (s_loss.clone(), s_gf.clone(), s_gg.clone())
+        xf = sf.detach().clone().requires_grad_(True)
+        xg = sg.detach().clone().requires_grad_(True)
+        loss = warp_ctct.ctct_simple_loss(xf, xg, d_ys, d_lx, d_ly, normalized=normalized)
+        gf, gg = torch.autograd.grad(loss, (xf, xg))
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], loss), "replay %d" % replay
+        torch.testing.assert_close(got[1], gf, rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(got[2], gg, rtol=1e-5, atol=1e-6)
+
+
 @pytest.mark.parametrize("track", [(True, False), (False, True), (False, False)])
 def test_simple_loss_partial_tracking_and_reduction(track):
     import warp_ctct
