@@ -587,6 +587,10 @@ __global__ __launch_bounds__(64 * WR * WC) void logmm_bwd_kernel(const BwdArgs a
     }
     const bool slow = __syncthreads_or(unsafe) != 0;
     const float *eown = a.Eown + (size_t)b * P * Kp;
+    // E_own of all this lane's outputs first (clamped addresses, no branches),
+    // then one select, multiply and store per output; the exact pass is a
+    // separate, workgroup-uniform branch
+    float ev[RB][CB][4];
 #pragma unroll
     for (int r4 = 0; r4 < RB; ++r4)
 #pragma unroll
@@ -595,13 +599,19 @@ __global__ __launch_bounds__(64 * WR * WC) void logmm_bwd_kernel(const BwdArgs a
             for (int r = 0; r < 4; ++r) {
                 const int p = p0 + row0 + r4 * 16 + 4 * (lane >> 4) + r;
                 const int k = k0 + col0 + c * 16 + (lane & 15);
-                if (p >= P || k >= K) continue;
-                float v = 0.0f;
-                if (p < Pb) {
-                    v = scaled_sum(acc[r4][c][r], eown[(size_t)p * Kp + k]);
-                    if (slow) v += exact_pairs(a, b, p, k, Qb);
-                }
-                db[p * a.dsp + k * a.dsk] = v;
+                ev[r4][c][r] = eown[(size_t)min(p, P - 1) * Kp + min(k, Kp - 1)];
+            }
+#pragma unroll
+    for (int r4 = 0; r4 < RB; ++r4)
+#pragma unroll
+        for (int c = 0; c < CB; ++c)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int p = p0 + row0 + r4 * 16 + 4 * (lane >> 4) + r;
+                const int k = k0 + col0 + c * 16 + (lane & 15);
+                float v = (p < Pb) ? scaled_sum(acc[r4][c][r], ev[r4][c][r]) : 0.0f;
+                if (slow && p < Pb && k < K) v += exact_pairs(a, b, p, k, Qb);
+                if (p < P && k < K) db[p * a.dsp + k * a.dsk] = v;
             }
 }
 
@@ -721,13 +731,9 @@ __global__ __launch_bounds__(256) void logmm_bwd_resident_kernel(const BwdArgs a
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int p = my_p + r, k = k0 + c * 16 + (lane & 15);
-                if (p >= P || k >= K) continue;
-                float v = 0.0f;
-                if (p < Pb) {
-                    v = scaled_sum(acc[0][c][r], ev[c][r]);
-                    if (slow) v += exact_pairs(a, b, p, k, Qb);
-                }
-                db[p * a.dsp + k * a.dsk] = v;
+                float v = (p < Pb) ? scaled_sum(acc[0][c][r], ev[c][r]) : 0.0f;
+                if (slow && p < Pb && k < K) v += exact_pairs(a, b, p, k, Qb);   // uniform `slow`
+                if (p < P && k < K) db[p * a.dsp + k * a.dsk] = v;
             }
         __syncthreads();   // everyone is done with s_e
     }
