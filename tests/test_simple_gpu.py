@@ -116,6 +116,26 @@ def test_log_matmul_backward(B, M, K, Nn, mask):
         assert out_r is None
 
 
+def test_log_matmul_empty_extents():
+    """Empty reductions and empty operands: logsumexp over nothing is -inf,
+    its gradient zero; empty outputs stay empty."""
+    from warp_ctct import _C
+    z = lambda *shape: torch.zeros(*shape, device="cuda")
+    out = _C.log_matmul(z(2, 3, 0), z(2, 0, 4))
+    assert out.shape == (2, 3, 4) and bool(torch.isneginf(out).all())
+    assert _C.log_matmul(z(2, 0, 5), z(2, 5, 4)).shape == (2, 0, 4)
+    assert _C.log_matmul(z(2, 3, 5), z(2, 5, 0)).shape == (2, 3, 0)
+    assert _C.log_matmul(z(0, 3, 5), z(0, 5, 4)).shape == (0, 3, 4)
+    # backward: no rows on one side -> the other side's gradient is all zeros
+    gl, gr = _C.log_matmul_backward(z(2, 0, 4), z(2, 0, 5), z(2, 5, 4), z(2, 0, 4), [True, True])
+    assert gl.shape == (2, 0, 5) and gr.shape == (2, 5, 4) and bool((gr == 0).all())
+    lhs = torch.randn(2, 3, 5, device="cuda")
+    gl, gr = _C.log_matmul_backward(z(2, 3, 0), lhs, z(2, 5, 0), z(2, 3, 0), [True, True])
+    assert gr.shape == (2, 5, 0) and gl.shape == (2, 3, 5) and bool((gl == 0).all())
+    gl, gr = _C.log_matmul_backward(z(2, 3, 4), z(2, 3, 0), z(2, 0, 4), z(2, 3, 4), [True, True])
+    assert gl.shape == (2, 3, 0) and gr.shape == (2, 0, 4)
+
+
 # ------------------------------------------------ reference operator surface
 SIMPLE_CASES = [
     # name, seed, N, T, U, V, lx, ly
@@ -238,6 +258,51 @@ def test_simple_loss_partial_tracking_and_reduction(track):
         np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
     else:
         assert tg.grad is None
+
+
+@pytest.mark.parametrize("normalized", [True, False])
+def test_simple_loss_edge_shapes(normalized):
+    """No label dimension at all (g holds the one start context), samples
+    without labels beside samples with labels, a single frame, an empty batch."""
+    import warp_ctct
+    rng = np.random.default_rng(71)
+    # U = 0: only the all-blank path
+    f = rng.standard_normal((3, 7, 6)).astype(np.float32)
+    g = rng.standard_normal((3, 1, 6)).astype(np.float32)
+    ys = np.zeros((3, 0), np.int32)
+    lx, ly = np.array([7, 4, 1], np.int32), np.zeros(3, np.int32)
+    loss, gf, gg, costs = O.ctct_simple_loss(f, g, ys, lx, ly, reduction="none",
+                                             normalized=normalized, grad_output=np.ones(3))
+    tf, tg = dev(f).requires_grad_(True), dev(g).requires_grad_(True)
+    out = warp_ctct.ctct_simple_loss(tf, tg, dev(ys), dev(lx), dev(ly), reduction="none",
+                                     normalized=normalized)
+    np.testing.assert_allclose(out.detach().cpu().numpy(), costs, rtol=LOSS_RTOL)
+    out.sum().backward()
+    np.testing.assert_allclose(tf.grad.cpu().numpy(), gf, atol=GRAD_ATOL, rtol=1e-5)
+    np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
+    # zero-label samples inside a batch with labels, one of them a single frame
+    f, g, ys, lx, ly = make_simple_case(72, 4, 9, 3, 8, lx=[9, 5, 1, 3], ly=[3, 0, 1, 0],
+                                        normalized=normalized)
+    loss, gf, gg, costs = O.ctct_simple_loss(f, g, ys, lx, ly, reduction="none",
+                                             normalized=normalized, grad_output=np.ones(4))
+    tf, tg = dev(f).requires_grad_(True), dev(g).requires_grad_(True)
+    out = warp_ctct.ctct_simple_loss(tf, tg, dev(ys), dev(lx), dev(ly), reduction="none",
+                                     normalized=normalized)
+    np.testing.assert_allclose(out.detach().cpu().numpy(), costs, rtol=LOSS_RTOL)
+    out.sum().backward()
+    np.testing.assert_allclose(tf.grad.cpu().numpy(), gf, atol=GRAD_ATOL, rtol=1e-5)
+    np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
+    # empty batch
+    ef = torch.zeros(0, 5, 4, device="cuda", requires_grad=True)
+    eg = torch.zeros(0, 3, 4, device="cuda", requires_grad=True)
+    ei = torch.zeros(0, 2, dtype=torch.int32, device="cuda")
+    el = torch.zeros(0, dtype=torch.int32, device="cuda")
+    assert tuple(warp_ctct.ctct_simple_loss(ef, eg, ei, el, el, reduction="none",
+                                            normalized=normalized).shape) == (0,)
+    s_ = warp_ctct.ctct_simple_loss(ef, eg, ei, el, el, reduction="sum", normalized=normalized)
+    assert s_.item() == 0.0
+    s_.backward()
+    assert tuple(ef.grad.shape) == (0, 5, 4) and tuple(eg.grad.shape) == (0, 3, 4)
 
 
 def test_simple_loss_assertions():

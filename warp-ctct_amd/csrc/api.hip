@@ -315,9 +315,11 @@ int warpctct_dense_grad_lattice(const void *workspace, size_t workspace_bytes, c
                                 const int *lx, const int *ly, const float *grad_out,
                                 int grad_out_stride, float scale, int average_frames, void *dense,
                                 int dtype, int N, int T, int U, int V, void *stream) {
-    if (!dims_ok(N, T, U) || V < 1 || !io_valid(dtype)) return WARPCTCT_EINVAL;
+    if (!dims_ok(N, T, U) || V < 1 || grad_out_stride < 0 || !io_valid(dtype))
+        return WARPCTCT_EINVAL;
     if (N == 0 || T == 0) return WARPCTCT_OK;
-    if (!dense) return WARPCTCT_EINVAL;
+    if (!workspace || !lx || !ly || !dense || (U > 0 && !ys)) return WARPCTCT_EINVAL;
+    if (workspace_bytes < carve(nullptr, N, T, U).bytes) return WARPCTCT_EWORKSPACE;
     int rc = done(launch_zero_fill_bytes(dense, (size_t)N * T * (U + 1) * V * io_size(dtype),
                                          as_stream(stream)));
     if (rc != WARPCTCT_OK) return rc;
@@ -667,7 +669,8 @@ int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, lo
     if (B < 0 || M < 0 || K < 0 || Nn < 0 || B > kMaxGrid || K > kMaxGrid * 64)
         return WARPCTCT_EINVAL;
     if (B == 0 || K == 0) return WARPCTCT_OK;
-    if (!lhs || !rhs || !workspace || ((M > 0 && Nn > 0) && (!grad_out || !res)))
+    if (!workspace || (M > 0 && !lhs) || (Nn > 0 && !rhs) ||
+        ((M > 0 && Nn > 0) && (!grad_out || !res)))
         return WARPCTCT_EINVAL;
     const LogmmWorkspace w = carve_logmm(workspace, B, M, K, Nn);
     if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;

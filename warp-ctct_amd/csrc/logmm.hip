@@ -747,9 +747,25 @@ inline bool prefer_96(int extent) {
 bool fits_int(long extent) { return extent >= 0 && extent < 0x7fffffffL; }
 bool stride_ok(long s) { return s >= 0 && s < 0x7fffffffL; }
 
+// grad[b, p, k] = 0 through the gradient's strides: the gradient of an empty reduction
+__global__ __launch_bounds__(256) void logmm_bwd_zero_kernel(BwdArgs a) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (long)a.P * a.K) return;
+    const int p = (int)(i / a.K), k = (int)(i - (long)p * a.K);
+    a.grad[(size_t)blockIdx.y * a.dsb + (size_t)p * a.dsp + (size_t)k * a.dsk] = 0.0f;
+}
+
 // 4 wavefronts per workgroup: 64 rows p (one 16-row block per wavefront, all 64
 // columns) or 96 rows p (all rows, 16 columns per wavefront) by 64 columns k
 hipError_t launch_bwd(const BwdArgs &a, int B, hipStream_t stream) {
+    if (B == 0 || a.P == 0 || a.K == 0) return hipSuccess;
+    if (a.Q == 0) {
+        const long cells = (long)a.P * a.K;
+        if (!fits_int((cells + 255) / 256)) return hipErrorInvalidValue;
+        hipLaunchKernelGGL(logmm_bwd_zero_kernel, dim3((unsigned)((cells + 255) / 256), B),
+                           dim3(256), 0, stream, a);
+        return hipGetLastError();
+    }
     // offsets inside one batch are 32-bit in the kernel
     if (!fits_int((long)(a.P - 1) * a.osp + (long)(a.K - 1) * a.osk + 1) ||
         !fits_int((long)(a.Q - 1) * a.tsq + (long)(a.K - 1) * a.tsk + 1) ||
