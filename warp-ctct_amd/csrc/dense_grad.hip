@@ -17,10 +17,16 @@
 //    gradients (before the store, or after it with the non-zero lanes storing
 //    a second time) takes 370-480 us: a wave that waits for a load keeps its
 //    slot, and the fill lives off instant wave turnover;
-//  * the separate sparse pass (patch_kernel, one thread per live cell, <= 3
-//    scattered 4-byte stores) costs ~40 us, whether it reads ready-made unit
-//    gradients or computes them on the fly from alpha / beta; 64-byte aligned group stores
-//    instead of 4-byte ones gain little;
+//  * the separate sparse pass (patch_kernel) costs 25-35 us whether it reads
+//    ready-made unit gradients or computes them on the fly from alpha / beta.
+//    What it stores matters beyond its own duration: 4-byte stores into lines
+//    that have left the caches leave partial lines behind whose write-back
+//    (a read-modify-write on the memory side) slows whatever runs next: the
+//    following step's zero-fill took 305 us instead of 292 us, 335 us when it
+//    came right after the patch.  Whole aligned 128-byte segments, written by
+//    8 lanes x 16 bytes each, cost the fill nothing and the patch itself
+//    27 us instead of 35 us (one thread writing its row's segments alone:
+//    44 us; 64-byte segments: 28 us but the fill still suffers);
 //  * running the fill on a second stream next to the gather / lattice kernels
 //    is slower than running everything back to back.
 // Hence two launches on one stream: fill, then patch.
@@ -51,31 +57,72 @@ __global__ __launch_bounds__(kBlock) void zero_fill_vec_kernel(v4f *__restrict__
     if (i < n4) p4[i] = z;
 }
 
-// Writes (not adds) the non-zero entries of row (n,t,u) of the dense gradient:
-// columns 0, y[u-1], y[u]; columns that coincide are summed first so that
-// every element is written by exactly one store.
-template <typename IO>
-__device__ __forceinline__ void patch_row(IO *out, const int *y, int u, int Un, int V, float v0,
-                                          float v1, float v2) {
+// The non-zero entries of one row of the dense gradient, coincident columns
+// merged: v0 at column 0, v1 at column c1 (if c1 > 0), v2 at column c2 (if
+// c2 > 0); c1 != c2.
+struct RowPatch {
+    float v0, v1, v2;
+    int c1, c2;
+};
+
+// Row (n,t,u): columns 0, y[u-1], y[u] hold v0, v1, v2; columns that coincide
+// are summed so that every element is written by exactly one store.
+__device__ __forceinline__ RowPatch merge_columns(const int *y, int u, int Un, int V, float v0,
+                                                  float v1, float v2) {
     const bool has1 = (u >= 1), has2 = (u < Un);
-    const int c1 = has1 ? min(max(y[u - 1], 0), V - 1) : -1;
-    const int c2 = has2 ? min(max(y[u], 0), V - 1) : -2;
+    RowPatch r;
+    r.c1 = has1 ? min(max(y[u - 1], 0), V - 1) : -1;
+    r.c2 = has2 ? min(max(y[u], 0), V - 1) : -1;
     if (!has1) v1 = 0.0f;
     if (!has2) v2 = 0.0f;
-    if (c2 == c1) {   // y[u-1] == y[u]: both label units land in one column
+    if (r.c2 == r.c1) {   // y[u-1] == y[u]: both label units land in one column
         v1 += v2;
-        v2 = 0.0f;
+        r.c2 = -1;
     }
-    if (c1 == 0) v0 += v1;   // a label equal to the blank index
-    if (c2 == 0) v0 += v2;
-    store_from_float(out, v0);
-    if (c1 > 0) store_from_float(out + c1, v1);
-    if (c2 > 0 && c2 != c1) store_from_float(out + c2, v2);
+    if (r.c1 == 0) {      // a label equal to the blank index
+        v0 += v1;
+        r.c1 = -1;
+    }
+    if (r.c2 == 0) {
+        v0 += v2;
+        r.c2 = -1;
+    }
+    r.v0 = v0, r.v1 = v1, r.v2 = v2;
+    return r;
 }
 
-// One thread per cell (t,u) of sample blockIdx.y; FROM_LATTICE computes the
-// unit gradients on the fly from units / alpha / beta (work-buffer layout, P
-// contexts per frame), otherwise they are read from the (N,T,U+1,3) tensor.
+// Aligned piece of a row that the patch writes whole (zeros around the value).
+// A partial write of a 128-byte line costs the memory side a read-modify-write
+// whose drain slows the kernels that follow (the next zero-fill by ~15 us on
+// the 2 GB gradient of a typical batch); a whole line does not.
+constexpr int kSegment = 128;
+
+// The 16 bytes number `part` of segment `seg` of a row.
+template <typename IO>
+__device__ __forceinline__ void store_segment_part(IO *row, int seg, int part, const RowPatch &r) {
+    constexpr int W = kSegment / (int)sizeof(IO);   // elements per segment
+    constexpr int E = 16 / (int)sizeof(IO);         // elements per 16-byte store
+    const int first = seg * W + part * E;
+    alignas(16) IO vals[E];
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+        const int col = first + i;
+        float v = 0.0f;
+        if (col == 0) v = r.v0;
+        if (col == r.c1) v = r.v1;
+        if (col == r.c2) v = r.v2;
+        store_from_float(&vals[i], v);
+    }
+    *reinterpret_cast<uint4 *>(row + first) = *reinterpret_cast<const uint4 *>(vals);
+}
+
+// One thread per cell (t,u) of sample blockIdx.y computes the row's entries;
+// FROM_LATTICE computes the unit gradients on the fly from units / alpha /
+// beta (work-buffer layout, P contexts per frame), otherwise they are read
+// from the (N,T,U+1,3) tensor.  The entries are then written by the whole
+// wavefront: 8 lanes per row, each 16 bytes of a 128-byte segment, so that a
+// store instruction covers 8 whole lines (rows whose size or address does not
+// allow that are written element by element by their own thread).
 template <bool FROM_LATTICE, typename IO>
 __global__ __launch_bounds__(kBlock) void patch_kernel(
     const float *__restrict__ unit_grads, const double *__restrict__ units,
@@ -85,29 +132,66 @@ __global__ __launch_bounds__(kBlock) void patch_kernel(
     const int U1 = U + 1;
     const int n = blockIdx.y;
     const int cell = blockIdx.x * kBlock + threadIdx.x;
-    if (cell >= T * U1) return;
     const int t = cell / U1, u = cell - t * U1;
     const int lxn = lx[n];
     const int Tn = min(max(lxn, 0), T);
     const int Un = min(max(ly[n], 0), U);
-    if (t >= Tn || u > Un) return;
     // outside the band the gradient is exactly zero: the fill wrote it already
-    if (FROM_LATTICE && outside_band(t, u, Tn, Un)) return;
+    const bool live = cell < T * U1 && t < Tn && u <= Un &&
+                      !(FROM_LATTICE && outside_band(t, u, Tn, Un));
     const size_t row = ((size_t)n * T + t) * U1 + u;
-    const int *y = ys + (size_t)n * U;
-    UnitGrad g;
-    if (FROM_LATTICE) {
-        const size_t lat = (size_t)(T + 1) * P * 2;
-        g = unit_grad_cell(units + (size_t)n * T * P * 3, alphas + (size_t)n * lat,
-                           betas + (size_t)n * lat, y, t, u, Un, P);
-    } else {
-        const float *p = unit_grads + row * 3;
-        g.g0 = p[0];
-        g.g1 = p[1];
-        g.g2 = p[2];
+    RowPatch r = {0.0f, 0.0f, 0.0f, -1, -1};
+    if (live) {
+        const int *y = ys + (size_t)n * U;
+        UnitGrad g;
+        if (FROM_LATTICE) {
+            const size_t lat = (size_t)(T + 1) * P * 2;
+            g = unit_grad_cell(units + (size_t)n * T * P * 3, alphas + (size_t)n * lat,
+                               betas + (size_t)n * lat, y, t, u, Un, P);
+        } else {
+            const float *p = unit_grads + row * 3;
+            g.g0 = p[0];
+            g.g1 = p[1];
+            g.g2 = p[2];
+        }
+        const float w = sample_weight(weight, n, lxn);
+        r = merge_columns(y, u, Un, V, g.g0 * w, g.g1 * w, g.g2 * w);
     }
-    const float w = sample_weight(weight, n, lxn);
-    patch_row(dense + row * (size_t)V, y, u, Un, V, g.g0 * w, g.g1 * w, g.g2 * w);
+    // rows start on segment boundaries and hold whole segments
+    const bool segments = ((size_t)V * sizeof(IO)) % kSegment == 0 &&
+                          (reinterpret_cast<uintptr_t>(dense) & (kSegment - 1)) == 0;
+    if (!segments) {
+        if (live) {
+            IO *out = dense + row * (size_t)V;
+            store_from_float(out, r.v0);
+            if (r.c1 > 0) store_from_float(out + r.c1, r.v1);
+            if (r.c2 > 0) store_from_float(out + r.c2, r.v2);
+        }
+        return;
+    }
+    constexpr int W = kSegment / (int)sizeof(IO);
+    const int lane = threadIdx.x & 63;
+    const int part = lane & 7, group = lane >> 3;
+    // consecutive lanes hold consecutive rows: row of lane 0 of this wavefront
+    IO *wave_rows = dense + (row - lane) * (size_t)V;
+    for (int j = 0; j < 8; ++j) {
+        const int src = j * 8 + group;
+        const int src_live = __shfl((int)live, src, 64);
+        if (__ballot(src_live) == 0) continue;   // wavefront-uniform
+        RowPatch q;
+        q.v0 = __shfl(r.v0, src, 64);
+        q.v1 = __shfl(r.v1, src, 64);
+        q.v2 = __shfl(r.v2, src, 64);
+        q.c1 = __shfl(r.c1, src, 64);
+        q.c2 = __shfl(r.c2, src, 64);
+        if (src_live) {
+            IO *out = wave_rows + (size_t)src * V;
+            const int s1 = q.c1 > 0 ? q.c1 / W : 0, s2 = q.c2 > 0 ? q.c2 / W : 0;
+            store_segment_part(out, 0, part, q);
+            if (s1 > 0) store_segment_part(out, s1, part, q);
+            if (s2 > 0 && s2 != s1) store_segment_part(out, s2, part, q);
+        }
+    }
 }
 
 }  // namespace
