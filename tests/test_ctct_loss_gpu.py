@@ -267,6 +267,38 @@ def test_half_precision_joint_is_read_and_written_natively(dtype, ulp, reduction
     assert torch.equal(loss, loss32)
 
 
+@pytest.mark.parametrize("dtype,V", [(torch.float32, 96), (torch.float32, 1024), (torch.bfloat16, 192),
+                                     (torch.float16, 128), (torch.float32, 48)],
+                         ids=["f32_3_lines", "f32_32_lines", "bf16_3_lines", "f16_2_lines", "f32_not_line_sized"])
+def test_dense_gradient_rows_written_as_whole_lines(dtype, V):
+    """The sparse pass of the dense gradient writes the 128-byte line around
+    each non-zero element (rows that are not a whole number of lines: single
+    elements).  Labels are placed so that a row's non-zero columns share the
+    blank's line, share one other line, sit on both sides of a line boundary,
+    and coincide (a repeated label); every element of the result, the zeros
+    around the values included, must match the oracle."""
+    import warp_ctct
+    per_line = 128 // torch.empty(0, dtype=dtype).element_size()
+    N, T, U = 2, 14, 8
+    joint, ys, lx, ly = make_joint_case(81, N, T, U, V, lx=[14, 12], ly=[8, 7], force_repeat=False)
+    edge = min(per_line, V - 2)
+    ys[0] = [1, 2, edge - 1, edge, edge + 1, edge + 1, V - 1, 3]          # a repeat at positions 4, 5
+    ys[1] = [V - 1, V - 2, edge, 1, edge - 1, 5, 5, 0][:U]
+    ys[1, 7] = 1
+    xh = dev(joint).to(dtype).requires_grad_(True)
+    rounded = xh.detach().double().cpu().numpy()
+    w = np.array([1.5, -0.75])
+    _, ref_dense, ref_costs = O.ctct_loss(rounded, ys, lx, ly, reduction="none", grad_output=w)
+    assert np.all(np.isfinite(ref_costs))
+    loss = warp_ctct.ctct_loss(xh, dev(ys), dev(lx), dev(ly), reduction="none")
+    loss.backward(dev(w, torch.float32))
+    got = xh.grad.double().cpu().numpy()
+    ulp = {torch.float32: 2.0 ** -23, torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+    tiny = 1e-7 if dtype == torch.float16 else 1e-30
+    assert_support(got, ref_dense, "dense gradient", underflow=tiny)
+    assert np.all(np.abs(got - ref_dense) <= ulp * np.abs(ref_dense) + max(tiny, 2e-6))
+
+
 def test_double_joint_is_converted_like_the_reference():
     import warp_ctct
     joint, ys, lx, ly = make_joint_case(32, 2, 12, 4, 7)
