@@ -108,7 +108,9 @@ int warpctct_dense_grad_f32(const float *unit_grads, const int *ys, const int *l
 
 /* The sparse half of warpctct_dense_grad_f32 alone: dense must already hold
  * zeros (e.g. from warpctct_zero_fill_f32 run earlier on another stream, since
- * the fill does not depend on the lattice). */
+ * the fill does not depend on the lattice).  The non-zero elements are written,
+ * not added, and when rows are a whole number of 128-byte lines the zeros of
+ * the line around each of them are written again with it. */
 int warpctct_dense_patch_f32(const float *unit_grads, const int *ys, const int *lx, const int *ly,
                              const float *grad_out, float *dense, int N, int T, int U, int V,
                              void *stream);
