@@ -560,6 +560,40 @@ def test_infeasible_sample_has_infinite_cost():
     np.testing.assert_allclose(c[1], ref[1], rtol=LOSS_RTOL)
 
 
+def test_minus_infinity_entries_on_the_paths():
+    """Log-probabilities of -inf (masked tokens) at cells that alignments would
+    use: those alignments drop out, the rest is scored as usual; the gradient at
+    a -inf entry is 0, never NaN."""
+    import warp_ctct
+    joint, ys, lx, ly = make_joint_case(91, 4, 22, 6, 12, lx=range(14, 23), ly=range(3, 7), zero_pad=False)
+    rng = np.random.default_rng(92)
+    N, T, U1, V = joint.shape
+    for n in range(N):
+        for t in range(T):
+            for u in range(U1):
+                r = rng.random()
+                if r < 0.10:
+                    joint[n, t, u, 0] = -np.inf                       # blank masked
+                elif r < 0.20 and u < ly[n]:
+                    joint[n, t, u, ys[n, u]] = -np.inf                # next label masked
+                elif r < 0.25 and u >= 1:
+                    joint[n, t, u, ys[n, u - 1]] = -np.inf            # label repeat masked
+    joint[3, :, :, 0] = -np.inf                                       # sample 3: no blank anywhere
+    _, ref_dense, ref_costs = O.ctct_loss(joint, ys, lx, ly, reduction="none", grad_output=np.ones(N))
+    x = dev(joint).requires_grad_(True)
+    c = warp_ctct.ctct_loss(x, dev(ys), dev(lx), dev(ly), reduction="none")
+    got = c.detach().cpu().numpy()
+    fin = np.isfinite(ref_costs)
+    assert fin.sum() >= 2, "the case should leave feasible samples"
+    assert np.array_equal(np.isposinf(got), np.isposinf(ref_costs))
+    np.testing.assert_allclose(got[fin], ref_costs[fin], rtol=LOSS_RTOL)
+    c[torch.as_tensor(fin).cuda()].sum().backward()
+    g = x.grad.cpu().numpy()
+    assert np.all(np.isfinite(g[fin]))
+    np.testing.assert_allclose(g[fin], ref_dense[fin], atol=GRAD_ATOL, rtol=0)
+    assert np.all(g[fin][np.isneginf(joint[fin])] == 0)
+
+
 FULL_SIZE = [
     # name, N, T, U, V, lx range, ly range, sigma
     ("typical_asr_batch", 32, 250, 60, 1024, (150, 250), (30, 60), 1.0),
