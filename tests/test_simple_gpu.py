@@ -305,6 +305,27 @@ def test_simple_loss_edge_shapes(normalized):
     assert tuple(ef.grad.shape) == (0, 5, 4) and tuple(eg.grad.shape) == (0, 3, 4)
 
 
+@pytest.mark.parametrize("normalized", [True, False])
+def test_simple_loss_vocabulary_beyond_one_lds_row(normalized):
+    """V = 20000: a row of f no longer fits the 64 KiB that the whole-row
+    builder of the unnormalised dense gradient stages in LDS (zero-fill plus
+    atomic adds take over), and the log-matmul reduces over 625 chunks."""
+    import warp_ctct
+    f, g, ys, lx, ly = make_simple_case(73, 2, 7, 3, 20000, lx=[7, 5], ly=[3, 2], normalized=normalized)
+    ys[0] = [19999, 19999, 17000]                     # last column, a repeat
+    lx[0] = 7
+    w = np.array([0.5, -2.0])
+    loss, gf, gg, costs = O.ctct_simple_loss(f, g, ys, lx, ly, reduction="none",
+                                             normalized=normalized, grad_output=w)
+    tf, tg = dev(f).requires_grad_(True), dev(g).requires_grad_(True)
+    out = warp_ctct.ctct_simple_loss(tf, tg, dev(ys), dev(lx), dev(ly), reduction="none",
+                                     normalized=normalized)
+    np.testing.assert_allclose(out.detach().cpu().numpy(), costs, rtol=LOSS_RTOL)
+    (out * dev(w, torch.float32)).sum().backward()
+    np.testing.assert_allclose(tf.grad.cpu().numpy(), gf, atol=2 * GRAD_ATOL, rtol=1e-5)
+    np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=2 * GRAD_ATOL, rtol=1e-5)
+
+
 def test_simple_loss_assertions():
     import warp_ctct
     f, g, ys, lx, ly = make_simple_case(8, 2, 6, 2, 5)

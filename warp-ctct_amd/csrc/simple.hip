@@ -138,6 +138,43 @@ __global__ __launch_bounds__(kBlock) void simple_scatter_f_kernel(
     atomicAdd(dense_f + ((size_t)n * T + t) * V + col, w * gv);
 }
 
+// dense_f[n,t,:] as a whole row: zeros plus w[n] * grad_f[n,t,u] at idx(u), the
+// zero-fill and the scatter-add of simple_scatter_f_kernel in one pass.  One
+// workgroup per frame builds the row in LDS (repeated labels add there) and
+// writes it out with full-width stores, so no element of the row is touched
+// twice in memory and no partially written line is left behind.
+__global__ __launch_bounds__(kBlock) void simple_dense_f_rows_kernel(
+    const float *__restrict__ grad_f, const int *__restrict__ ys, const int *__restrict__ lx,
+    const int *__restrict__ ly, const float *__restrict__ grad_out, float *__restrict__ dense_f,
+    int T, int U, int V) {
+    extern __shared__ __attribute__((aligned(16))) float row[];   // V floats
+    const int U1 = U + 1;
+    const int n = blockIdx.y, t = blockIdx.x;
+    const int Tn = clampi(lx[n], 0, T), Un = clampi(ly[n], 0, U);
+    float *out = dense_f + ((size_t)n * T + t) * V;
+    const bool live = t < Tn;
+    if (live) {
+        for (int k = threadIdx.x; k < V; k += kBlock) row[k] = 0.0f;
+        __syncthreads();
+        const float w = grad_out ? grad_out[n] : 1.0f;
+        for (int u = threadIdx.x; u <= Un; u += kBlock) {
+            const float gv = grad_f[((size_t)n * T + t) * U1 + u];
+            if (gv == 0.0f) continue;
+            const int col = (u == 0) ? 0 : clampi(ys[(size_t)n * U + u - 1], 0, V - 1);
+            atomicAdd(row + col, w * gv);
+        }
+        __syncthreads();
+    }
+    if ((V & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15u) == 0) {
+        typedef float v4f __attribute__((ext_vector_type(4)));
+        const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int k = threadIdx.x * 4; k < V; k += kBlock * 4)
+            *reinterpret_cast<v4f *>(out + k) = live ? *reinterpret_cast<const v4f *>(row + k) : zero;
+    } else {
+        for (int k = threadIdx.x; k < V; k += kBlock) out[k] = live ? row[k] : 0.0f;
+    }
+}
+
 // dense_g[n,u,{0,y[u-1],y[u]}] += w[n] * grad_g[n,u,k]: backward of g.gather
 // (warp_ctct/__init__.py:211-215).  One thread per (n,u,k).
 __global__ __launch_bounds__(kBlock) void simple_scatter_g_kernel(
@@ -183,6 +220,18 @@ hipError_t launch_simple_reduce(const float *unit_grads, float *grad_f, float *g
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(simple_reduce_contexts_kernel, dim3((U + 1 + 3) / 4, N), dim3(kBlock), 0,
                        stream, unit_grads, grad_g, T, U);
+    return hipGetLastError();
+}
+
+bool simple_dense_f_rows_fit(int V) { return (size_t)V * sizeof(float) <= 64 * 1024; }
+
+hipError_t launch_simple_dense_f_rows(const float *grad_f, const int *ys, const int *lx,
+                                      const int *ly, const float *grad_out, float *dense_f, int N,
+                                      int T, int U, int V, hipStream_t stream) {
+    if (N == 0 || T == 0) return hipSuccess;
+    hipLaunchKernelGGL(simple_dense_f_rows_kernel, dim3(T, N), dim3(kBlock),
+                       (size_t)V * sizeof(float), stream, grad_f, ys, lx, ly, grad_out, dense_f, T,
+                       U, V);
     return hipGetLastError();
 }
 
