@@ -560,6 +560,29 @@ def test_infeasible_sample_has_infinite_cost():
     np.testing.assert_allclose(c[1], ref[1], rtol=LOSS_RTOL)
 
 
+def test_committed_brute_force_vectors():
+    """The HIP path against tests/golden/brute_force_cases.npz: lattices whose
+    log-likelihood and dense gradient come from enumerating every alignment
+    (no lattice recursion involved), including no labels at all, a single
+    frame, and lx = ly."""
+    import os
+    import warp_ctct
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                             "brute_force_cases.npz"))
+    x = dev(z["joint"]).requires_grad_(True)
+    c = warp_ctct.ctct_loss(x, dev(z["ys"]), dev(z["lx"]), dev(z["ly"]), reduction="none")
+    np.testing.assert_allclose(c.detach().cpu().numpy(), -z["loglik"], rtol=LOSS_RTOL)
+    c.sum().backward()
+    got = x.grad.cpu().numpy()
+    np.testing.assert_allclose(got, z["dense_grad"], atol=GRAD_ATOL, rtol=0)
+    assert_support(got, z["dense_grad"], "dense gradient")
+    # the same through the logits entry: log_softmax of log-probabilities is the identity
+    # up to rounding, its backward subtracts softmax * sum(G) = exp(joint) * (-1 per frame)
+    x2 = dev(z["joint"]).requires_grad_(True)
+    c2 = warp_ctct.ctct_loss_with_logits(x2, dev(z["ys"]), dev(z["lx"]), dev(z["ly"]), reduction="none")
+    np.testing.assert_allclose(c2.detach().cpu().numpy(), -z["loglik"], rtol=1e-4)
+
+
 def test_minus_infinity_entries_on_the_paths():
     """Log-probabilities of -inf (masked tokens) at cells that alignments would
     use: those alignments drop out, the rest is scored as usual; the gradient at

@@ -322,3 +322,21 @@ def test_c_oracle_log_matmul():
     ref = torch.logsumexp(torch.tensor(lhs)[:, :, :, None] + torch.tensor(rhs)[:, None], dim=2).numpy()
     np.testing.assert_allclose(C.log_matmul(lhs, rhs), ref, rtol=1e-13)
     np.testing.assert_allclose(C.log_matmul(lhs, rhs, dtype=np.float32), ref, rtol=2e-6)
+
+
+def test_oracle_against_committed_brute_force_vectors():
+    """tests/golden/brute_force_cases.npz holds lattices whose log-likelihood
+    and dense gradient were obtained by enumerating every alignment
+    (tests/golden/make_brute_force_fixtures.py); the oracle must reproduce them."""
+    import os
+    from oracle import c_oracle as C
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                             "brute_force_cases.npz"))
+    joint = z["joint"].astype(np.float64)
+    _, dense, costs = O.ctct_loss(joint, z["ys"], z["lx"], z["ly"], reduction="none",
+                                  grad_output=np.ones(len(z["lx"])))
+    np.testing.assert_allclose(costs, -z["loglik"], rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(dense, z["dense_grad"], rtol=0, atol=1e-12)
+    c_costs, c_dense = C.ctct_loss_dense(z["joint"], z["ys"], z["lx"], z["ly"], dtype=np.float64)
+    np.testing.assert_allclose(c_costs, -z["loglik"], rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(c_dense, z["dense_grad"], rtol=0, atol=1e-12)
