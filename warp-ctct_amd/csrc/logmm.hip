@@ -216,6 +216,33 @@ __device__ __forceinline__ void tile_mfma_qc(const float (*sa)[LDA], const float
     }
 }
 
+// ---- placement of the workgroups --------------------------------------------
+// The 8 XCDs of the GPU, each with its own 4 MB L2, receive the workgroups of a
+// launch round-robin by linear index.  Every workgroup of a batch entry re-reads
+// that entry's second operand, so the batch entries are dealt to the XCDs (entry
+// b runs on XCD b % 8) instead of being spread over all of them: an L2 then
+// serves 1/8 of the operands, not every one.  The grid is one-dimensional,
+// 8 * ceil(B/8) * tiles_x * tiles_y workgroups; tiles with b >= B do not exist.
+struct TileId {
+    int x, y, b;
+};
+__device__ __forceinline__ TileId xcd_tile(int tiles_x, int tiles_y) {
+    const int per_batch = tiles_x * tiles_y;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int w = slot % per_batch;
+    TileId t;
+    t.b = (slot / per_batch) * 8 + xcd;
+    t.x = w % tiles_x;
+    t.y = w / tiles_x;
+    return t;
+}
+inline unsigned xcd_grid(int tiles_x, int tiles_y, int B) {
+    return (unsigned)((B + 7) / 8 * 8) * tiles_x * tiles_y;
+}
+inline bool xcd_grid_fits(long tiles_x, long tiles_y, int B) {
+    return (long)((B + 7) / 8 * 8) * tiles_x * tiles_y < 0x7fffffffL;
+}
+
 // ---- forward ----------------------------------------------------------------
 __device__ float exact_lse(const float *lrow, long lsk, const float *rcol, long rsk, int K) {
     float mx = neg_inf_f();
@@ -239,6 +266,7 @@ struct FwdArgs {
     float *partial;
     int splits, chunks_per_split;
     int M, K, Kp, Nn;
+    int B, tiles_x, tiles_y;  // batch entries, row tiles, column tiles * splits
     const int *row_len, *col_len;
 };
 
@@ -261,9 +289,11 @@ __global__ __launch_bounds__(64 * WR * WC) void logmm_fwd_kernel(const FwdArgs a
     static_assert(VA % NT == 0 && VB % NT == 0, "slabs must divide over the threads");
     __shared__ __attribute__((aligned(16))) float sa[2][TM][LDK];   // E_l[i][k]
     __shared__ __attribute__((aligned(16))) float sb_[2][TN][LDK];  // E_r[j][k]
-    const int b = blockIdx.z;
-    const int split = blockIdx.y % a.splits;
-    const int i0 = blockIdx.x * TM, j0 = (blockIdx.y / a.splits) * TN;
+    const TileId tile = xcd_tile(a.tiles_x, a.tiles_y);
+    const int b = tile.b;
+    if (b >= a.B) return;
+    const int split = tile.y % a.splits;
+    const int i0 = tile.x * TM, j0 = (tile.y / a.splits) * TN;
     const int M = a.M, Nn = a.Nn, Kp = a.Kp;
     // lengths-aware: rows >= row_len[b] and cols > col_len[b] are padding
     const int Mb = a.row_len ? min(max(a.row_len[b], 0), M) : M;
@@ -358,7 +388,7 @@ __global__ __launch_bounds__(64 * WR * WC) void logmm_fwd_kernel(const FwdArgs a
                 const float s = acc[r4][c][r];
                 const size_t at = ((size_t)b * M + i) * Nn + j;
                 if (a.splits > 1)
-                    a.partial[(size_t)split * gridDim.z * M * Nn + at] = s;
+                    a.partial[(size_t)split * a.B * M * Nn + at] = s;
                 else
                     a.res[at] = fwd_result(a, b, i, j, s);
             }
@@ -441,6 +471,7 @@ struct BwdArgs {
     const int *p_len, *q_len;
     int p_extra, q_extra;
     int flags_follow_p;        // rows i are p (lhs gradient) or q (rhs gradient)
+    int B, tiles_x, tiles_y;   // batch entries, p tiles, k tiles (or groups of k tiles)
 };
 
 // E_own * sum; the sum is 0 where nothing was added: avoid 0 * inf or 0 * nan
@@ -479,8 +510,10 @@ __global__ __launch_bounds__(64 * WR * WC) void logmm_bwd_kernel(const BwdArgs a
     static_assert(TP * TQ % NT == 0 && VE % NT == 0, "slabs must divide over the threads");
     __shared__ __attribute__((aligned(16))) float s_c[2][TP][LDK];   // C[p][q]
     __shared__ __attribute__((aligned(16))) float s_e[2][TQ][LDE];   // E_oth[q][k]
-    const int b = blockIdx.z;
-    const int p0 = blockIdx.x * TP, k0 = blockIdx.y * TK;
+    const TileId tile = xcd_tile(a.tiles_x, a.tiles_y);
+    const int b = tile.b;
+    if (b >= a.B) return;
+    const int p0 = tile.x * TP, k0 = tile.y * TK;
     const int P = a.P, Q = a.Q, K = a.K, Kp = a.Kp;
     const int Pb = a.p_len ? min(max(a.p_len[b], 0) + a.p_extra, P) : P;
     const int Qb = a.q_len ? min(max(a.q_len[b], 0) + a.q_extra, Q) : Q;
@@ -632,11 +665,13 @@ __global__ __launch_bounds__(256) void logmm_bwd_resident_kernel(const BwdArgs a
     constexpr int SE = QR * TK / 4 / NT;       // E vectors per thread and tile
     __shared__ __attribute__((aligned(16))) float s_c[TP][LDC];   // C[p][q]
     __shared__ __attribute__((aligned(16))) float s_e[QR][LDE];   // E_oth[q][k]
-    const int b = blockIdx.z;
-    const int p0 = blockIdx.x * TP;
+    const TileId tile = xcd_tile(a.tiles_x, a.tiles_y);
+    const int b = tile.b;
+    if (b >= a.B) return;
+    const int p0 = tile.x * TP;
     const int P = a.P, Q = a.Q, K = a.K, Kp = a.Kp;
     const int ktiles = (K + TK - 1) / TK;
-    const int kt_begin = blockIdx.y * tiles_per_wg;
+    const int kt_begin = tile.y * tiles_per_wg;
     const int kt_end = min(kt_begin + tiles_per_wg, ktiles);
     const int Pb = a.p_len ? min(max(a.p_len[b], 0) + a.p_extra, P) : P;
     const int Qb = a.q_len ? min(max(a.q_len[b], 0) + a.q_extra, Q) : Q;
@@ -757,7 +792,9 @@ __global__ __launch_bounds__(256) void logmm_bwd_zero_kernel(BwdArgs a) {
 
 // 4 wavefronts per workgroup: 64 rows p (one 16-row block per wavefront, all 64
 // columns) or 96 rows p (all rows, 16 columns per wavefront) by 64 columns k
-hipError_t launch_bwd(const BwdArgs &a, int B, hipStream_t stream) {
+hipError_t launch_bwd(const BwdArgs &args, int B, hipStream_t stream) {
+    BwdArgs a = args;
+    a.B = B;
     if (B == 0 || a.P == 0 || a.K == 0) return hipSuccess;
     if (a.Q == 0) {
         const long cells = (long)a.P * a.K;
@@ -777,15 +814,20 @@ hipError_t launch_bwd(const BwdArgs &a, int B, hipStream_t stream) {
         const int ptiles = (a.P + 63) / 64, ktiles = (a.K + 63) / 64;
         const long wgs = (long)ptiles * ktiles * B;
         const int per = (int)std::min<long>(8, std::max<long>(1, wgs / 2048));
-        dim3 grid(ptiles, (ktiles + per - 1) / per, B);
-        hipLaunchKernelGGL(logmm_bwd_resident_kernel, grid, dim3(256), 0, stream, a, per);
+        a.tiles_x = ptiles, a.tiles_y = (ktiles + per - 1) / per;
+        if (!xcd_grid_fits(a.tiles_x, a.tiles_y, B)) return hipErrorInvalidValue;
+        hipLaunchKernelGGL(logmm_bwd_resident_kernel, dim3(xcd_grid(a.tiles_x, a.tiles_y, B)),
+                           dim3(256), 0, stream, a, per);
         return hipGetLastError();
     }
     // a reduction of up to 4 chunks (Q <= 128) is fetched whole, up front;
     // longer ones run a pipeline 3 chunks deep
     const bool short_q = a.Q <= 4 * TQ;
+    a.tiles_x = prefer_96(a.P) ? (a.P + 95) / 96 : (a.P + 63) / 64;
+    a.tiles_y = (a.K + 63) / 64;
+    if (!xcd_grid_fits(a.tiles_x, a.tiles_y, B)) return hipErrorInvalidValue;
+    const dim3 grid(xcd_grid(a.tiles_x, a.tiles_y, B));
     if (prefer_96(a.P)) {
-        dim3 grid((a.P + 95) / 96, (a.K + 63) / 64, B);
         if (short_q)
             hipLaunchKernelGGL((logmm_bwd_kernel<6, 1, 1, 4, 4, false>), grid, dim3(256), 0,
                                stream, a);
@@ -793,7 +835,6 @@ hipError_t launch_bwd(const BwdArgs &a, int B, hipStream_t stream) {
             hipLaunchKernelGGL((logmm_bwd_kernel<6, 1, 1, 4, 3, true>), grid, dim3(256), 0, stream,
                                a);
     } else {
-        dim3 grid((a.P + 63) / 64, (a.K + 63) / 64, B);
         if (short_q)
             hipLaunchKernelGGL((logmm_bwd_kernel<1, 4, 4, 1, 4, false>), grid, dim3(256), 0,
                                stream, a);
@@ -879,13 +920,15 @@ hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
     a.res = res, a.M = M, a.K = K, a.Kp = logmm_padded_reduction(K), a.Nn = Nn;
     a.row_len = row_len, a.col_len = col_len;
     // 4 wavefronts per workgroup: 32 rows i by 96 or 64 columns j
-    if (prefer_96(Nn)) {
-        dim3 grid((M + 31) / 32, (Nn + 95) / 96 * a.splits, B);
+    a.B = B;
+    a.tiles_x = (M + 31) / 32;
+    a.tiles_y = (prefer_96(Nn) ? (Nn + 95) / 96 : (Nn + 63) / 64) * a.splits;
+    if (!xcd_grid_fits(a.tiles_x, a.tiles_y, B)) return hipErrorInvalidValue;
+    const dim3 grid(xcd_grid(a.tiles_x, a.tiles_y, B));
+    if (prefer_96(Nn))
         hipLaunchKernelGGL((logmm_fwd_kernel<1, 3, 2, 2>), grid, dim3(256), 0, stream, a);
-    } else {
-        dim3 grid((M + 31) / 32, (Nn + 63) / 64 * a.splits, B);
+    else
         hipLaunchKernelGGL((logmm_fwd_kernel<1, 2, 2, 2>), grid, dim3(256), 0, stream, a);
-    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || a.splits == 1) return e;
     const long outs = (long)M * Nn;
