@@ -99,7 +99,7 @@ IO_DTYPE = {"c2_bf16": "bfloat16", "c2_f16": "float16", "c2_logits_bf16": "bfloa
 
 
 def other_config(args, torch, warp_ctct):
-    """The remaining BASELINE.json configurations: same timing discipline, a
+    """The remaining benchmark configurations: same timing discipline, a
     reduced JSON line (value, ms_per_step, per-operator HIP-event times)."""
     import numpy as np
     kind, N, T, U, V, sigma = OTHER[args.config]
@@ -221,7 +221,7 @@ def main():
     ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "c2_bf16", "c2_f16", "c2_logits",
                              "c2_logits_bf16", "c2_logits_unfused"],
                     help="workload: c2 (default) is the configuration the headline metric is "
-                         "quoted on; the others are the remaining BASELINE.json configurations "
+                         "quoted on; the others are the remaining benchmark configurations "
                          "and print a reduced line (no cpu_baseline)")
     ap.add_argument("--graph", action="store_true",
                     help="capture one step in a HIP graph and time its replays (reduced line, "
