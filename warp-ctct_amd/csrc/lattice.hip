@@ -94,20 +94,28 @@ __device__ __forceinline__ int wait_until(int *counter, int target) {
     return seen;
 }
 
-// Consumer side of a hand-over: the counter and the R ring slots of the chunk
+// Consumer side of a hand-over: the counter and the R ring slots of a chunk
 // are requested in one batch (LDS serves a wavefront's requests in order, so
 // slots read after a counter that already shows the chunk are the chunk's
-// values); only if the counter was not there yet is the batch repeated.  One
-// LDS round trip per chunk instead of two.
+// values).  peek() only issues the requests and returns the counter as read;
+// nothing waits for them until the values are used, so a peek at the chunk
+// after the current one costs the sweep no LDS round trip when the producer is
+// already that far.
+__device__ __forceinline__ int peek(int *counter, const double *ring, int s0, double (&mail)[R]) {
+    const int seen = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);   // the compiler keeps the order of the requests
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+        mail[r] = __hip_atomic_load(ring + (s0 + r) % kRing, __ATOMIC_RELAXED,
+                                    __HIP_MEMORY_SCOPE_WORKGROUP);
+    return seen;
+}
+
+// Repeats the batch until the counter shows the chunk (with a bound).
 __device__ __forceinline__ void wait_and_take(int *counter, int target, const double *ring,
                                               int s0, double (&mail)[R]) {
     for (int spins = 0; spins < kMaxSpins; ++spins) {
-        const int seen = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        __atomic_signal_fence(__ATOMIC_SEQ_CST);   // the compiler keeps the order of the requests
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-            mail[r] = __hip_atomic_load(ring + (s0 + r) % kRing, __ATOMIC_RELAXED,
-                                        __HIP_MEMORY_SCOPE_WORKGROUP);
+        const int seen = peek(counter, ring, s0, mail);
         if (__builtin_amdgcn_readfirstlane(seen) >= target) break;
         __builtin_amdgcn_s_sleep(1);
     }
@@ -206,35 +214,50 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, doubl
         const int t_start = BETA ? Tn - 1 : 0;
         chunk_load(a, in, urow, Tn, t_start, dir);
         int taken_seen = 0;
+        int ahead_seen = 0;        // counter as read by the last peek ahead
+        double ahead[R];           // ... and the slots of the chunk it looked at
+#pragma unroll
+        for (int r = 0; r < R; ++r) ahead[r] = neg_inf();
         // one chunk: steps s0 .. s0+cnt-1 with the units in `c`
         auto run_chunk = [&](const Chunk &c, int s0, int cnt, bool full) {
-            double mail[R];
+            double mail[R], mine[R];
 #pragma unroll
             for (int r = 0; r < R; ++r) mail[r] = neg_inf();
             if (consumes) {
-                wait_and_take(&relay.done[b_in], s0 + cnt, relay.ring[b_in], s0, mail);
+                // the peek of the previous chunk looked at exactly this chunk
+                if (__builtin_amdgcn_readfirstlane(ahead_seen) < s0 + cnt)
+                    wait_and_take(&relay.done[b_in], s0 + cnt, relay.ring[b_in], s0, ahead);
+#pragma unroll
+                for (int r = 0; r < R; ++r) mail[r] = ahead[r];
                 publish(&relay.taken[b_in], s0 + cnt);
+                ahead_seen = peek(&relay.done[b_in], relay.ring[b_in], s0 + cnt, ahead);
             }
-            // the ring is four chunks deep: the consumer's progress is looked
-            // up again only when the last value seen no longer covers this chunk
-            if (produces && taken_seen < s0 + cnt - kRing)
-                taken_seen = wait_until(&relay.taken[b_out], s0 + cnt - kRing);
 #pragma unroll
             for (int r = 0; r < R; ++r) {
+                mine[r] = neg_inf();
                 if (full || r < cnt) {
                     const int s = s0 + r;
-                    double mine;
                     if (BETA) {
-                        beta_step(f, c.lp[r], skip, o_mask, mail[r], mine);
+                        beta_step(f, c.lp[r], skip, o_mask, mail[r], mine[r]);
                         front_store(out + (size_t)(Tn - 1 - s) * srow, f);
                     } else {
-                        alpha_step(f, c.lp[r], skip, mail[r], mine);
+                        alpha_step(f, c.lp[r], skip, mail[r], mine[r]);
                         front_store(out + (size_t)(s + 1) * srow, f);
                     }
-                    if (produces && lane == edge_lane) relay.ring[b_out][s % kRing] = mine;
                 }
             }
-            if (produces) publish(&relay.done[b_out], s0 + cnt);
+            if (produces) {
+                // the ring is four chunks deep: the consumer's progress is looked
+                // up again only when the last value seen no longer covers this chunk
+                if (taken_seen < s0 + cnt - kRing)
+                    taken_seen = wait_until(&relay.taken[b_out], s0 + cnt - kRing);
+                if (lane == edge_lane) {
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+                        if (full || r < cnt) relay.ring[b_out][(s0 + r) % kRing] = mine[r];
+                }
+                publish(&relay.done[b_out], s0 + cnt);
+            }
         };
         int s0 = 0;
         while (s0 + 2 * R <= Tn) {
