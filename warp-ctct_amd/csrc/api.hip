@@ -136,10 +136,24 @@ LogmmWorkspace carve_logmm(void *base, int B, int M, int K, int Nn) {
 int simple_from_units(const SimpleWorkspace &w, const int *ys, const int *lx, const int *ly, int N,
                       int T, int U, float *costs, float *grad_f, float *grad_g, float *grad_den,
                       bool want_grad, hipStream_t stream) {
-    int rc = forward_from_units(w.lattice, ys, lx, ly, N, T, U, costs,
-                                want_grad ? w.unit_grads : nullptr, stream);
+    // alpha is needed only for the gradients; those are reduced straight from the
+    // lattices (the unit-gradient region of the workspace holds the partial sums)
+    LatticeArgs a = {};
+    a.units = w.lattice.units;
+    a.ys = ys;
+    a.lx = lx;
+    a.ly = ly;
+    a.alphas = w.lattice.alphas;
+    a.betas = w.lattice.betas;
+    a.costs = costs;
+    a.N = N;
+    a.T = T;
+    a.U = U;
+    a.beta_only = !want_grad;
+    int rc = done(launch_lattice(a, stream));
     if (rc != WARPCTCT_OK || !want_grad) return rc;
-    return done(launch_simple_reduce(w.unit_grads, grad_f, grad_g, grad_den, N, T, U, stream));
+    return done(launch_simple_grads(w.lattice.units, ys, lx, ly, w.lattice.alphas, w.lattice.betas,
+                                    w.unit_grads, grad_f, grad_g, grad_den, N, T, U, stream));
 }
 
 }  // namespace
@@ -549,6 +563,10 @@ int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, c
                                                  w.lattice.units, N, T, U, V, st));
         if (rc != WARPCTCT_OK) return rc;
     }
+    if (want_grad && T == 0) {   // no frames: the only gradient with elements is all zeros
+        int rc = done(launch_zero_fill(grad_g, (size_t)N * (U + 1) * 3, st));
+        if (rc != WARPCTCT_OK) return rc;
+    }
     return simple_from_units(w, ys, lx, ly, N, T, U, costs, grad_f, grad_g,
                              normalized ? grad_den : nullptr, want_grad && T > 0, st);
 }
@@ -568,6 +586,10 @@ int warpctct_simple_forward_units_f32(const float *f_g, const float *g_g, const 
     hipStream_t st = as_stream(stream);
     if (T > 0) {
         int rc = done(launch_simple_units(f_g, g_g, den, lx, ly, w.lattice.units, N, T, U, st));
+        if (rc != WARPCTCT_OK) return rc;
+    }
+    if (want_grad && T == 0) {
+        int rc = done(launch_zero_fill(grad_g, (size_t)N * (U + 1) * 3, st));
         if (rc != WARPCTCT_OK) return rc;
     }
     return simple_from_units(w, ys, lx, ly, N, T, U, costs, grad_f, grad_g,

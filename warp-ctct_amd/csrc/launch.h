@@ -91,6 +91,13 @@ hipError_t launch_logits_grad(const void *logits, int io_type, const float *lse,
 hipError_t launch_simple_gather_units(const float *f, const float *g, const float *den,
                                       const int *ys, const int *lx, const int *ly, double *units,
                                       int N, int T, int U, int V, hipStream_t stream);
+// compact gradients of the joiner path straight from the lattices: grad_f
+// (N,T,U+1), grad_g (N,U+1,3), grad_den (N,T,U+1) or null; `partial` is scratch
+// of N * ceil(T/8) * (U+1) * 3 floats
+hipError_t launch_simple_grads(const double *units, const int *ys, const int *lx, const int *ly,
+                               const double *alphas, const double *betas, float *partial,
+                               float *grad_f, float *grad_g, float *grad_den, int N, int T, int U,
+                               hipStream_t stream);
 hipError_t launch_simple_reduce(const float *unit_grads, float *grad_f, float *grad_g,
                                 float *grad_den, int N, int T, int U, hipStream_t stream);
 // dense_f of the unnormalised path in one pass (zeros + scattered compact

@@ -116,6 +116,106 @@ __global__ __launch_bounds__(kBlock) void simple_reduce_contexts_kernel(
     }
 }
 
+// Unit gradients and their reductions in one pass over the lattices: what
+// unit_grads_kernel + simple_reduce_frames_kernel + simple_reduce_contexts_kernel
+// produce, without the (N,T,U+1,3) tensor in between.  One workgroup per
+// (n, block of kFramesPerBlock frames), one thread per context:
+//   grad_den[t,u] = -(g0+g1+g2),  grad_f[t,u>=1] = g1[t,u] + g2[t,u-1],
+//   grad_f[t,0] = sum_u g0[t,u]                          (per frame)
+//   partial[n,block,u,k] = sum over the block's frames of g_k[t,u]
+// and simple_sum_partials_kernel adds the blocks up in a fixed order.
+constexpr int kFramesPerBlock = 8;
+
+__global__ __launch_bounds__(512) void simple_grads_kernel(
+    const double *__restrict__ units, const int *__restrict__ ys, const int *__restrict__ lx,
+    const int *__restrict__ ly, const double *__restrict__ alphas,
+    const double *__restrict__ betas, float *__restrict__ grad_f, float *__restrict__ grad_den,
+    float *__restrict__ partial, int T, int U, int P) {
+    constexpr int F = kFramesPerBlock;
+    __shared__ float s_g2[F][512];
+    __shared__ float s_blank[F][8];
+    const int U1 = U + 1;
+    const int n = blockIdx.y, u = threadIdx.x;
+    const int lane = u & 63, wave = u >> 6, waves = P >> 6;
+    const int Tn = clampi(lx[n], 0, T), Un = clampi(ly[n], 0, U);
+    const size_t lat = (size_t)(T + 1) * P * 2;
+    const double *units_n = units + (size_t)n * T * P * 3;
+    const double *alpha_n = alphas + (size_t)n * lat, *beta_n = betas + (size_t)n * lat;
+    const int *y = ys + (size_t)n * U;
+    const int t_begin = blockIdx.x * F;
+    // all frames of the block first (their loads are independent), then one exchange
+    UnitGrad g[F];
+    float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f;
+#pragma unroll
+    for (int f = 0; f < F; ++f) {
+        const int t = t_begin + f;
+        g[f] = UnitGrad{0.0f, 0.0f, 0.0f};
+        // padding and cells outside the band of complete alignments: exactly zero
+        if (t < Tn && u <= Un && !outside_band(t, u, Tn, Un))
+            g[f] = unit_grad_cell(units_n, alpha_n, beta_n, y, t, u, Un, P);
+        a0 += g[f].g0;
+        a1 += g[f].g1;
+        a2 += g[f].g2;
+    }
+#pragma unroll
+    for (int f = 0; f < F; ++f) {
+        float blank = g[f].g0;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) blank += __shfl_xor(blank, off, 64);
+        s_g2[f][u] = g[f].g2;
+        if (lane == 0) s_blank[f][wave] = blank;
+    }
+    __syncthreads();
+    if (u >= U1) return;
+#pragma unroll
+    for (int f = 0; f < F; ++f) {
+        const int t = t_begin + f;
+        if (t >= T) break;
+        const size_t at = ((size_t)n * T + t) * U1 + u;
+        if (grad_den) grad_den[at] = -(g[f].g0 + g[f].g1 + g[f].g2);
+        if (u >= 1) {
+            grad_f[at] = g[f].g1 + s_g2[f][u - 1];
+        } else {
+            float b = 0.0f;
+            for (int w = 0; w < waves; ++w) b += s_blank[f][w];
+            grad_f[at] = b;
+        }
+    }
+    float *o = partial + (((size_t)n * gridDim.x + blockIdx.x) * U1 + u) * 3;
+    o[0] = a0;
+    o[1] = a1;
+    o[2] = a2;
+}
+
+// grad_g[n,u,k] = sum over the frame blocks of partial[n,block,u,k]; one
+// wavefront per (n,u), lanes over the blocks, summed in a fixed order.
+__global__ __launch_bounds__(kBlock) void simple_sum_partials_kernel(
+    const float *__restrict__ partial, float *__restrict__ grad_g, int blocks, int U1) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int u = blockIdx.x * 4 + wave;
+    const int n = blockIdx.y;
+    if (u >= U1) return;
+    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f;
+    for (int b = lane; b < blocks; b += 64) {
+        const float *p = partial + (((size_t)n * blocks + b) * U1 + u) * 3;
+        s0 += p[0];
+        s1 += p[1];
+        s2 += p[2];
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        s0 += __shfl_xor(s0, off, 64);
+        s1 += __shfl_xor(s1, off, 64);
+        s2 += __shfl_xor(s2, off, 64);
+    }
+    if (lane == 0) {
+        float *o = grad_g + ((size_t)n * U1 + u) * 3;
+        o[0] = s0;
+        o[1] = s1;
+        o[2] = s2;
+    }
+}
+
 // dense_f[n,t,idx(u)] += w[n] * grad_f[n,t,u],  idx = [0, y0 .. y_{U-1}]: the
 // backward of f.gather (warp_ctct/__init__.py:205-208).  The same label may
 // occur at several u, so the adds are atomic.  Padding holds zeros: skipped.
@@ -209,6 +309,23 @@ hipError_t launch_simple_gather_units(const float *f, const float *g, const floa
     hipLaunchKernelGGL(simple_gather_units_kernel,
                        dim3((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N), dim3(kBlock),
                        0, stream, f, g, den, ys, lx, ly, units, T, U, V, P);
+    return hipGetLastError();
+}
+
+hipError_t launch_simple_grads(const double *units, const int *ys, const int *lx, const int *ly,
+                               const double *alphas, const double *betas, float *partial,
+                               float *grad_f, float *grad_g, float *grad_den, int N, int T, int U,
+                               hipStream_t stream) {
+    const int P = padded_contexts(U);
+    const int blocks = (T + kFramesPerBlock - 1) / kFramesPerBlock;
+    if (T > 0) {
+        hipLaunchKernelGGL(simple_grads_kernel, dim3(blocks, N), dim3(P), 0, stream, units, ys, lx,
+                           ly, alphas, betas, grad_f, grad_den, partial, T, U, P);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(simple_sum_partials_kernel, dim3((U + 1 + 3) / 4, N), dim3(kBlock), 0,
+                       stream, partial, grad_g, blocks, U + 1);
     return hipGetLastError();
 }
 
