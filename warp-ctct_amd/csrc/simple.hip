@@ -22,7 +22,11 @@ constexpr int kBlock = 256;
 
 __device__ __forceinline__ int clampi(int v, int lo, int hi) { return min(max(v, lo), hi); }
 
-// One thread per cell (t,u) of sample blockIdx.y.
+// One thread per cell (t,u) of sample blockIdx.y; the 64 lanes of a wavefront
+// are 64 consecutive contexts of one frame (P is a multiple of 64).  The value
+// f[t, y[u]] serves two cells, as the next label of (t,u) and as the current
+// label of (t,u+1): every lane reads it once and hands it to its neighbour
+// (one scattered read of f per cell instead of two).
 __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     const float *__restrict__ f, const float *__restrict__ g, const float *__restrict__ den,
     const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
@@ -30,33 +34,36 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     const int U1 = U + 1;
     const int n = blockIdx.y;
     const int cell = blockIdx.x * kBlock + threadIdx.x;
-    if (cell >= T * P) return;
-    const int t = cell / P, u = cell - t * P;
+    const int lane = threadIdx.x & 63;
+    const int t = cell / P, u = cell - t * P;      // t is the same for the whole wavefront
     const int Tn = clampi(lx[n], 0, T), Un = clampi(ly[n], 0, U);
-    if (t >= Tn) return;
+    if (t >= Tn) return;                           // (covers cell >= T * P)
+    const bool live = u <= Un && !outside_band(t, u, Tn, Un);
+    const float *fr = f + ((size_t)n * T + t) * V;
+    const int *y = ys + (size_t)n * U;
+    // the next label's column: wanted by this cell or by the cell of context u+1
+    const bool has2 = u < Un;
+    const int c2 = has2 ? clampi(y[u], 0, V - 1) : 0;
+    const bool wanted = has2 && (live || !outside_band(t, u + 1, Tn, Un));
+    const float f2 = wanted ? fr[c2] : 0.0f;
+    float f1 = __shfl_up(f2, 1, 64);
+    const int c1 = (u >= 1 && u <= Un) ? clampi(y[u - 1], 0, V - 1) : 0;
+    if (lane == 0 && live && u >= 1) f1 = fr[c1];  // the neighbour is in another wavefront
     double *o = units + (((size_t)n * T + t) * P + u) * 3;
     // padding context of a live frame, or a cell outside the band of complete
     // alignments (its units cannot influence costs or gradients): neutral units
-    if (u > Un || outside_band(t, u, Tn, Un)) {
+    if (!live) {
         o[0] = 0.0;
         o[1] = 0.0;
         o[2] = neg_inf();
         return;
     }
-    const float *fr = f + ((size_t)n * T + t) * V;
     const float *gr = g + ((size_t)n * U1 + u) * V;
-    const int *y = ys + (size_t)n * U;
     const double d = den ? (double)den[((size_t)n * T + t) * U1 + u] : 0.0;
     const double b = (double)fr[0] + (double)gr[0] - d;
     double cur = b, nxt = neg_inf();
-    if (u >= 1) {
-        const int c = clampi(y[u - 1], 0, V - 1);
-        cur = (double)fr[c] + (double)gr[c] - d;
-    }
-    if (u < Un) {
-        const int c = clampi(y[u], 0, V - 1);
-        nxt = ((double)fr[c] + (double)gr[c] - d) * kLog2e;
-    }
+    if (u >= 1) cur = (double)f1 + (double)gr[c1] - d;
+    if (has2) nxt = ((double)f2 + (double)gr[c2] - d) * kLog2e;
     o[0] = b * kLog2e;
     o[1] = cur * kLog2e;
     o[2] = nxt;
