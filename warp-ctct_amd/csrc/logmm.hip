@@ -195,8 +195,11 @@ __device__ __forceinline__ void tile_mfma_qq(const float (*sa)[LDK], const float
 
 // A in LDS as [row][q] (stride LDA), B as [q][column] (stride LDB): lane group
 // g takes q = 4s + g in step s; 4-byte reads, free of bank conflicts for
-// LDA = 36 and LDB = 16 (mod 64).
-template <int RB, int CB, int LDA, int LDB>
+// LDA = 36 and LDB = 16 (mod 64).  With SWAP the two values change places in
+// the instruction, which transposes the product: the lane then holds
+// D[row = l%16 of A's block][4 consecutive columns 4*(l/16) + r of B's block],
+// i.e. 16 contiguous bytes of a row-major output instead of 4 rows of one column.
+template <int RB, int CB, int LDA, int LDB, bool SWAP = false>
 __device__ __forceinline__ void tile_mfma_qc(const float (*sa)[LDA], const float (*sb)[LDB],
                                              int row0, int col0, int lane, v4f (&acc)[RB][CB]) {
     const int r = lane & 15, g = lane >> 4;
@@ -211,8 +214,10 @@ __device__ __forceinline__ void tile_mfma_qc(const float (*sa)[LDA], const float
         for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb)
-                acc[rb][cb] =
-                    __builtin_amdgcn_mfma_f32_16x16x4f32(a[rb], b[cb], acc[rb][cb], 0, 0, 0);
+                acc[rb][cb] = SWAP ? __builtin_amdgcn_mfma_f32_16x16x4f32(b[cb], a[rb],
+                                                                          acc[rb][cb], 0, 0, 0)
+                                   : __builtin_amdgcn_mfma_f32_16x16x4f32(a[rb], b[cb],
+                                                                          acc[rb][cb], 0, 0, 0);
     }
 }
 
@@ -679,7 +684,13 @@ __global__ __launch_bounds__(256) void logmm_bwd_resident_kernel(const BwdArgs a
     const int wave = tid >> 6, lane = tid & 63;
     const int row0 = wave * 16;
     float *db = a.grad + (size_t)b * a.dsb;
-    const int my_p = p0 + row0 + 4 * (lane >> 4);   // first of this lane's 4 rows
+    // The product is formed transposed (see tile_mfma_qc): this lane owns row
+    // my_p and, in each of the 4 column blocks, 4 consecutive columns from my_k
+    const int my_p = p0 + row0 + (lane & 15);
+    const int my_k = 4 * (lane >> 4);
+    // 16-byte accesses to the gradient need unit stride along k and aligned rows
+    const bool vec = a.dsk == 1 && (a.dsp & 3) == 0 && (a.dsb & 3) == 0 &&
+                     (reinterpret_cast<uintptr_t>(a.grad) & 15u) == 0;
 
     if (p0 >= Pb) {   // a tile of padding rows: zeros
         for (int kt = kt_begin; kt < kt_end; ++kt)
@@ -687,8 +698,8 @@ __global__ __launch_bounds__(256) void logmm_bwd_resident_kernel(const BwdArgs a
             for (int c = 0; c < CB; ++c)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const int p = my_p + r, k = kt * TK + c * 16 + (lane & 15);
-                    if (p < P && k < K) db[p * a.dsp + k * a.dsk] = 0.0f;
+                    const int k = kt * TK + c * 16 + my_k + r;
+                    if (my_p < P && k < K) db[my_p * a.dsp + k * a.dsk] = 0.0f;
                 }
         return;
     }
@@ -725,7 +736,7 @@ __global__ __launch_bounds__(256) void logmm_bwd_resident_kernel(const BwdArgs a
     // rows beyond Q and columns beyond Kp are clamped to valid memory (they
     // meet C = 0, or are never stored)
     const float *eo = a.Eoth + (size_t)b * Q * Kp;
-    const float *eown = a.Eown + (size_t)b * P * Kp;
+    const float *eown = a.Eown + (size_t)b * P * Kp + (size_t)min(my_p, P - 1) * Kp;
     v4f re[SE];
     auto fetch = [&](int kt) {
 #pragma unroll
@@ -747,29 +758,38 @@ __global__ __launch_bounds__(256) void logmm_bwd_resident_kernel(const BwdArgs a
         }
         __syncthreads();
         if (kt + 1 < kt_end) fetch(kt + 1);
-        float ev[CB][4];   // E_own of this lane's outputs, in flight during the MFMAs
+        // E_own of this lane's outputs, in flight during the MFMAs (Kp is a
+        // multiple of 32: the 4 columns are one aligned vector, clamped into the row)
+        v4f ev[CB];
 #pragma unroll
         for (int c = 0; c < CB; ++c)
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                ev[c][r] = eown[(size_t)min(my_p + r, P - 1) * Kp +
-                                min(k0 + c * 16 + (lane & 15), Kp - 1)];
+            ev[c] = *reinterpret_cast<const v4f *>(eown + min(k0 + c * 16 + my_k, Kp - 4));
         v4f acc[1][CB];
 #pragma unroll
         for (int c = 0; c < CB; ++c) acc[0][c] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
         for (int c3 = 0; c3 < nq; ++c3)
-            tile_mfma_qc<1, CB, LDC, LDE>(
+            tile_mfma_qc<1, CB, LDC, LDE, true>(
                 reinterpret_cast<const float (*)[LDC]>(&s_c[0][c3 * TQ]), &s_e[c3 * TQ], row0, 0,
                 lane, acc);
 #pragma unroll
-        for (int c = 0; c < CB; ++c)
+        for (int c = 0; c < CB; ++c) {
+            const int k = k0 + c * 16 + my_k;
+            float v[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int p = my_p + r, k = k0 + c * 16 + (lane & 15);
-                float v = (p < Pb) ? scaled_sum(acc[0][c][r], ev[c][r]) : 0.0f;
-                if (slow && p < Pb && k < K) v += exact_pairs(a, b, p, k, Qb);   // uniform `slow`
-                if (p < P && k < K) db[p * a.dsp + k * a.dsk] = v;
+                v[r] = (my_p < Pb) ? scaled_sum(acc[0][c][r], ev[c][r]) : 0.0f;
+                if (slow && my_p < Pb && k + r < K) v[r] += exact_pairs(a, b, my_p, k + r, Qb);
             }
+            if (my_p >= P) continue;
+            float *dst = db + my_p * a.dsp + k * a.dsk;
+            if (vec && k + 3 < K) {
+                *reinterpret_cast<v4f *>(dst) = v4f{v[0], v[1], v[2], v[3]};
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (k + r < K) dst[r * a.dsk] = v[r];
+            }
+        }
         __syncthreads();   // everyone is done with s_e
     }
 }
