@@ -57,7 +57,7 @@ def algorithmic_bytes(N, T, U, V, lx, ly):
     return dense, gathered, small
 
 
-def cpu_baseline(joint, ys, lx, ly, budget_s=20.0):
+def cpu_baseline(joint, ys, lx, ly, budget_s=10.0):
     """C oracle (oracle/ctct_oracle.c, fp32, OpenMP over lattices) on the host
     copy of the same batch: gather + lattice + dense gradient."""
     from oracle import c_oracle as C
@@ -68,7 +68,7 @@ def cpu_baseline(joint, ys, lx, ly, budget_s=20.0):
     C.ctct_loss_dense(host, ys, lx, ly)                  # warm-up (page faults, libm)
     times = []
     t_end = time.perf_counter() + budget_s
-    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 10):
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 500):
         t0 = time.perf_counter()
         C.ctct_loss_dense(host, ys, lx, ly)
         times.append(time.perf_counter() - t0)
