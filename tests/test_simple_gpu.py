@@ -143,6 +143,10 @@ SIMPLE_CASES = [
     ("ragged", 2, 5, 40, 11, 33, range(20, 41), range(3, 12)),
     ("two_contexts_per_lane", 3, 2, 140, 90, 50, [140, 120], [90, 70]),
     ("single_label", 4, 2, 5, 1, 6, [5, 2], [1, 1]),
+    # shapes that take the other log-matmul gradient kernels: more than 96
+    # contexts (no resident slab), and a frame count that tiles better by 96
+    ("wide_contexts", 5, 2, 130, 110, 40, [130, 125], [110, 100]),
+    ("ninety_frames", 6, 3, 90, 20, 70, [90, 81, 66], [20, 17, 9]),
 ]
 
 
