@@ -632,16 +632,10 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
             if (rc != WARPCTCT_OK) return rc;
         }
         if (dense_f) {
-            // where the kernel can, it adds the scattered compact gradient of f
-            // (simple_scatter_f_kernel's work) while it writes its rows
-            const LogmmSparse sp = {grad_f, ys, ly, U1};
-            const bool fold = logmm_bwd_lhs_folds_sparse(T, U1, U1);
             const LogmmGrad gl = {dense_f, (long)T * V, (long)V, 1L};
             int rc = done(launch_logmm_bwd_lhs(lhs, rhs, sh, grad_den, den, pw.factors, pw.flags,
-                                               gl, N, T, V, U1, lx, ly, grad_out,
-                                               fold ? &sp : nullptr, st));
+                                               gl, N, T, V, U1, lx, ly, grad_out, st));
             if (rc != WARPCTCT_OK) return rc;
-            if (fold) dense_f = nullptr;   // nothing left for the scatter below
         }
         if (dense_g) {
             // gradient of rhs[b,k,j] = g[b,j,k] stored straight into the (N,U+1,V) layout
@@ -722,7 +716,7 @@ int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, lo
     if (grad_lhs) {
         const LogmmGrad g = {grad_lhs, glsb, glsm, glsk};
         int rc = done(launch_logmm_bwd_lhs(l, r, w.sh, grad_out, res, w.pw.factors, w.pw.flags, g,
-                                           B, M, K, Nn, nullptr, nullptr, nullptr, nullptr, st));
+                                           B, M, K, Nn, nullptr, nullptr, nullptr, st));
         if (rc != WARPCTCT_OK) return rc;
     }
     if (grad_rhs) {

@@ -155,22 +155,11 @@ hipError_t launch_logmm_pair_factor(const float *go, const float *res, const flo
                                     const float *rmax, const float *batch_scale,
                                     const int *row_len, const int *col_len, float *C, int *flags,
                                     int B, int M, int Nn, hipStream_t stream);
-// A sparse term that the lhs gradient kernel can add while it writes its rows:
-//   grad_lhs[b, i, col(u)] += batch_scale[b] * vals[b, i, u]  for u = 0 .. len[b],
-//   col(0) = 0, col(u) = labels[b, u-1]; vals is (B,M,S), labels (B,S-1).
-// Only shapes for which logmm_bwd_lhs_folds_sparse() holds.
-struct LogmmSparse {
-    const float *vals;
-    const int *labels, *len;
-    int S;
-};
-bool logmm_bwd_lhs_folds_sparse(int M, int Nn, int S);
 hipError_t launch_logmm_bwd_lhs(const LogmmOperand &lhs, const LogmmOperand &rhs,
                                 const LogmmShifted &sh, const float *go, const float *res,
                                 const float *C, const int *flags, const LogmmGrad &grad, int B,
                                 int M, int K, int Nn, const int *row_len, const int *col_len,
-                                const float *batch_scale, const LogmmSparse *sparse,
-                                hipStream_t stream);
+                                const float *batch_scale, hipStream_t stream);
 hipError_t launch_logmm_bwd_rhs(const LogmmOperand &lhs, const LogmmOperand &rhs,
                                 const LogmmShifted &sh, const float *go, const float *res,
                                 const float *C, const int *flags, const LogmmGrad &grad, int B,

@@ -477,12 +477,6 @@ struct BwdArgs {
     int p_extra, q_extra;
     int flags_follow_p;        // rows i are p (lhs gradient) or q (rhs gradient)
     int B, tiles_x, tiles_y;   // batch entries, p tiles, k tiles (or groups of k tiles)
-    // optional sparse term (resident kernel only):
-    //   grad[b, p, col(u)] += batch_scale[b] * sp_vals[b, p, u],  u = 0 .. sp_len[b],
-    //   col(0) = 0, col(u) = sp_labels[b, u-1]; sp_S values per row, sp_S - 1 labels per entry
-    const float *sp_vals;
-    const int *sp_labels, *sp_len;
-    int sp_S;
 };
 
 // E_own * sum; the sum is 0 where nothing was added: avoid 0 * inf or 0 * nan
@@ -698,21 +692,7 @@ __global__ __launch_bounds__(256) void logmm_bwd_resident_kernel(const BwdArgs a
     const bool vec = a.dsk == 1 && (a.dsp & 3) == 0 && (a.dsb & 3) == 0 &&
                      (reinterpret_cast<uintptr_t>(a.grad) & 15u) == 0;
 
-    // sparse term: lane l keeps the columns of entries u = l and u = l + 64
-    // (-1: no such entry); sp_S <= QR + 1 entries per row
-    int sp_col0 = -1, sp_col1 = -1;
-    const float *sp_row = nullptr;
-    float sp_w = 0.0f;
-    if (a.sp_vals) {
-        const int Sb = min(max(a.sp_len[b], 0), a.sp_S - 1) + 1;
-        const int *lab = a.sp_labels + (size_t)b * (a.sp_S - 1);
-        if (lane < Sb) sp_col0 = (lane == 0) ? 0 : min(max(lab[lane - 1], 0), K - 1);
-        if (lane + 64 < Sb) sp_col1 = min(max(lab[lane + 63], 0), K - 1);
-        sp_row = a.sp_vals + ((size_t)b * P + min(my_p, P - 1)) * a.sp_S;
-        sp_w = a.batch_scale ? a.batch_scale[b] : 1.0f;
-    }
-
-    if (p0 >= Pb) {   // a tile of padding rows: zeros (the sparse term is zero there too)
+    if (p0 >= Pb) {   // a tile of padding rows: zeros
         for (int kt = kt_begin; kt < kt_end; ++kt)
 #pragma unroll
             for (int c = 0; c < CB; ++c)
@@ -791,47 +771,23 @@ __global__ __launch_bounds__(256) void logmm_bwd_resident_kernel(const BwdArgs a
             tile_mfma_qc<1, CB, LDC, LDE, true>(
                 reinterpret_cast<const float (*)[LDC]>(&s_c[0][c3 * TQ]), &s_e[c3 * TQ], row0, 0,
                 lane, acc);
-        float v[CB][4];
 #pragma unroll
         for (int c = 0; c < CB; ++c) {
             const int k = k0 + c * 16 + my_k;
+            float v[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                v[c][r] = (my_p < Pb) ? scaled_sum(acc[0][c][r], ev[c][r]) : 0.0f;
-                if (slow && my_p < Pb && k + r < K) v[c][r] += exact_pairs(a, b, my_p, k + r, Qb);
+                v[r] = (my_p < Pb) ? scaled_sum(acc[0][c][r], ev[c][r]) : 0.0f;
+                if (slow && my_p < Pb && k + r < K) v[r] += exact_pairs(a, b, my_p, k + r, Qb);
             }
-        }
-        if (a.sp_vals) {
-            // entries whose column lies in this tile (a few per tile), found by
-            // the whole wavefront at once and then applied one by one
-            unsigned long long hit0 = __ballot(sp_col0 >= k0 && sp_col0 < k0 + TK);
-            unsigned long long hit1 = __ballot(sp_col1 >= k0 && sp_col1 < k0 + TK);
-            while (hit0 | hit1) {
-                const bool first = hit0 != 0;
-                const int bit = __builtin_ctzll(first ? hit0 : hit1);
-                if (first) hit0 &= hit0 - 1; else hit1 &= hit1 - 1;
-                const int col = __builtin_amdgcn_readlane(first ? sp_col0 : sp_col1, bit);
-                const int u = bit + (first ? 0 : 64);
-                const int rel = col - k0 - my_k;     // 16 * c + r for the owner of the column
-                const float add = (my_p < Pb) ? sp_w * sp_row[u] : 0.0f;
-#pragma unroll
-                for (int c = 0; c < CB; ++c)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        if (rel == 16 * c + r) v[c][r] += add;
-            }
-        }
-#pragma unroll
-        for (int c = 0; c < CB; ++c) {
-            const int k = k0 + c * 16 + my_k;
             if (my_p >= P) continue;
             float *dst = db + my_p * a.dsp + k * a.dsk;
             if (vec && k + 3 < K) {
-                *reinterpret_cast<v4f *>(dst) = v4f{v[c][0], v[c][1], v[c][2], v[c][3]};
+                *reinterpret_cast<v4f *>(dst) = v4f{v[0], v[1], v[2], v[3]};
             } else {
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
-                    if (k + r < K) dst[r * a.dsk] = v[c][r];
+                    if (k + r < K) dst[r * a.dsk] = v[r];
             }
         }
         __syncthreads();   // everyone is done with s_e
@@ -939,11 +895,6 @@ void launch_shift_exp_rows(const float *x, long sb, long sr, long sk, int B, int
 
 }  // namespace
 
-bool logmm_bwd_lhs_folds_sparse(int M, int Nn, int S) {
-    // the resident kernel is the one that knows the sparse term (see launch_bwd)
-    return Nn >= 1 && Nn <= QR && !prefer_96(M) && S >= 1 && S <= 128;
-}
-
 hipError_t launch_logmm_shift_exp(const LogmmOperand &lhs, const LogmmOperand &rhs,
                                   const LogmmShifted &sh, int B, int M, int K, int Nn,
                                   const int *row_len, const int *col_len, hipStream_t stream) {
@@ -1020,10 +971,8 @@ hipError_t launch_logmm_bwd_lhs(const LogmmOperand &lhs, const LogmmOperand &rhs
                                 const LogmmShifted &sh, const float *go, const float *res,
                                 const float *C, const int *flags, const LogmmGrad &grad, int B,
                                 int M, int K, int Nn, const int *row_len, const int *col_len,
-                                const float *batch_scale, const LogmmSparse *sparse,
-                                hipStream_t stream) {
+                                const float *batch_scale, hipStream_t stream) {
     if (B == 0 || M == 0 || K == 0) return hipSuccess;
-    if (sparse && !logmm_bwd_lhs_folds_sparse(M, Nn, sparse->S)) return hipErrorInvalidValue;
     if (!stride_ok(lhs.s1) || !stride_ok(lhs.s2) || !stride_ok(rhs.s1) || !stride_ok(rhs.s2) ||
         !stride_ok(grad.s1) || !stride_ok(grad.s2))
         return hipErrorInvalidValue;
@@ -1039,10 +988,6 @@ hipError_t launch_logmm_bwd_lhs(const LogmmOperand &lhs, const LogmmOperand &rhs
     a.P = M, a.Q = Nn, a.K = K, a.Kp = logmm_padded_reduction(K);
     a.p_len = row_len, a.p_extra = 0, a.q_len = col_len, a.q_extra = 1;
     a.batch_scale = batch_scale;
-    a.sp_vals = sparse ? sparse->vals : nullptr;
-    a.sp_labels = sparse ? sparse->labels : nullptr;
-    a.sp_len = sparse ? sparse->len : nullptr;
-    a.sp_S = sparse ? sparse->S : 0;
     return launch_bwd(a, B, stream);
 }
 
@@ -1068,7 +1013,6 @@ hipError_t launch_logmm_bwd_rhs(const LogmmOperand &lhs, const LogmmOperand &rhs
     a.P = Nn, a.Q = M, a.K = K, a.Kp = logmm_padded_reduction(K);
     a.p_len = col_len, a.p_extra = 1, a.q_len = row_len, a.q_extra = 0;
     a.batch_scale = batch_scale;
-    a.sp_vals = nullptr, a.sp_labels = nullptr, a.sp_len = nullptr, a.sp_S = 0;
     return launch_bwd(a, B, stream);
 }
 
