@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from ctct_cases import make_simple_case
+from ctct_cases import make_joint_case, make_simple_case
 from oracle import c_oracle as C
 from oracle import ctct_oracle as O
 
@@ -134,6 +134,57 @@ def test_log_matmul_empty_extents():
     assert gr.shape == (2, 5, 0) and gl.shape == (2, 3, 5) and bool((gl == 0).all())
     gl, gr = _C.log_matmul_backward(z(2, 3, 4), z(2, 3, 0), z(2, 0, 4), z(2, 3, 4), [True, True])
     assert gl.shape == (2, 3, 0) and gr.shape == (2, 0, 4)
+
+
+def test_reference_autograd_classes_on_gathered_operands():
+    """warp_ctct.LogMMExp / CTCTLoss / SimpleCTCTLoss, the reference's
+    module-level autograd functions (warp_ctct/__init__.py:20-85), for code
+    that imports them by name: LogMMExp against torch.logsumexp and its
+    autograd, the two loss functions against the oracle on gathered operands."""
+    import warp_ctct
+    rng = np.random.default_rng(77)
+    lhs = torch.tensor(rng.standard_normal((2, 9, 21)), dtype=torch.float32, device="cuda", requires_grad=True)
+    rhs_t = torch.tensor(rng.standard_normal((2, 6, 21)), dtype=torch.float32, device="cuda", requires_grad=True)
+    w = torch.tensor(rng.standard_normal((2, 9, 6)), dtype=torch.float32, device="cuda")
+    out = warp_ctct.LogMMExp.apply(lhs, rhs_t.transpose(1, 2))
+    ref = torch.logsumexp(lhs[:, :, :, None] + rhs_t.transpose(1, 2)[:, None, :, :], dim=2)
+    torch.testing.assert_close(out, ref, rtol=1e-5, atol=1e-5)
+    gl, gr = torch.autograd.grad((out * w).sum(), (lhs, rhs_t))
+    rl, rr = torch.autograd.grad((ref * w).sum(), (lhs, rhs_t))
+    torch.testing.assert_close(gl, rl, rtol=1e-4, atol=2e-5)
+    torch.testing.assert_close(gr, rr, rtol=1e-4, atol=2e-5)
+    only_l = warp_ctct.LogMMExp.apply(lhs, rhs_t.transpose(1, 2), True, False)
+    (g_only,) = torch.autograd.grad((only_l * w).sum(), (lhs,))
+    torch.testing.assert_close(g_only, rl, rtol=1e-4, atol=2e-5)
+
+    f, g, ys, lx, ly = make_simple_case(78, 3, 14, 4, 11, lx=[14, 9, 12], ly=[4, 2, 3])
+    f_g, g_g = O.gather_separate(f, g, ys)
+    den = O.log_matmul(f, np.swapaxes(g, 1, 2)).astype(np.float32)
+    costs, gf, gg, gd = O.ctct_loss_simple_fwd(f_g, g_g, ys, den, lx, ly)
+    tf, tg, td = (dev(a).requires_grad_(True) for a in (f_g, g_g, den))
+    wn = np.array([0.5, 2.0, -1.0])
+    c = warp_ctct.SimpleCTCTLoss.apply(tf, tg, td, dev(ys), dev(lx), dev(ly), True, True)
+    np.testing.assert_allclose(c.detach().cpu().numpy(), costs, rtol=LOSS_RTOL)
+    (c * dev(wn, torch.float32)).sum().backward()
+    np.testing.assert_allclose(tf.grad.cpu().numpy(), gf * wn[:, None, None], atol=2 * GRAD_ATOL)
+    np.testing.assert_allclose(tg.grad.cpu().numpy(), gg * wn[:, None, None], atol=2 * GRAD_ATOL, rtol=1e-5)
+    np.testing.assert_allclose(td.grad.cpu().numpy(), gd * wn[:, None, None], atol=2 * GRAD_ATOL)
+    # unnormalised, gradient wanted for g only
+    costs_u, _, gg_u, _ = O.ctct_loss_simple_fwd(f_g, g_g, ys, None, lx, ly)
+    tg2 = dev(g_g).requires_grad_(True)
+    c_u = warp_ctct.SimpleCTCTLoss.apply(dev(f_g), tg2, None, dev(ys), dev(lx), dev(ly), False, True)
+    np.testing.assert_allclose(c_u.detach().cpu().numpy(), costs_u, rtol=LOSS_RTOL)
+    c_u.sum().backward()
+    np.testing.assert_allclose(tg2.grad.cpu().numpy(), gg_u, atol=2 * GRAD_ATOL, rtol=1e-5)
+
+    joint, ys, lx, ly = make_joint_case(79, 3, 12, 4, 9, lx=[12, 8, 10], ly=[4, 3, 2])
+    lp3 = O.gather_units(joint, ys)
+    costs3, ug = C.ctct_loss_fwd(lp3, ys, lx, ly, dtype=np.float64)
+    t3 = dev(lp3.astype(np.float32)).requires_grad_(True)
+    c3 = warp_ctct.CTCTLoss.apply(t3, dev(ys), dev(lx), dev(ly), True)
+    np.testing.assert_allclose(c3.detach().cpu().numpy(), costs3, rtol=LOSS_RTOL)
+    (c3 * dev(wn, torch.float32)).sum().backward()
+    np.testing.assert_allclose(t3.grad.cpu().numpy(), ug * wn[:, None, None, None], atol=2 * GRAD_ATOL)
 
 
 # ------------------------------------------------ reference operator surface

@@ -164,6 +164,73 @@ class _SimpleCTCTLoss(torch.autograd.Function):
         return dense_f, dense_g, None, None, None, None, None, None
 
 
+class CTCTLoss(torch.autograd.Function):
+    """The reference's autograd function on GATHERED log-probabilities
+    (warp_ctct/__init__.py:20-33): ``log_probs`` is (N, T, U, 3) =
+    joint[..., [0, y[u-1], y[u]]].  Kept for code that imports it by name;
+    :func:`ctct_loss` does not go through it (it works on the joint itself)."""
+
+    @staticmethod
+    def forward(ctx, log_probs, labels, lx, ly, requires_grad):
+        costs, grads = core.ctct_loss_fwd(log_probs, labels, lx, ly, requires_grad)
+        if requires_grad:
+            ctx.save_for_backward(grads)
+        return costs
+
+    @staticmethod
+    def backward(ctx, grad_outputs):
+        (grads,) = ctx.saved_tensors
+        return grad_outputs.reshape(-1, 1, 1, 1) * grads, None, None, None, None
+
+
+class LogMMExp(torch.autograd.Function):
+    """Differentiable log-semiring matrix product (warp_ctct/__init__.py:36-52
+    of the reference): ``out[b, i, j] = logsumexp_k(lhs[b, i, k] + rhs[b, k, j])``
+    for float32 operands (B, M, K) and (B, K, N); strided operands are fine."""
+
+    @staticmethod
+    def forward(ctx, lhs, rhs, track_l=True, track_r=True):
+        out = core.log_matmul(lhs, rhs)
+        if track_l or track_r:
+            ctx.save_for_backward(lhs, rhs, out)
+            ctx.track = [bool(track_l), bool(track_r)]
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_outputs):
+        lhs, rhs, out = ctx.saved_tensors
+        grad_lhs, grad_rhs = core.log_matmul_backward(grad_outputs.contiguous(), lhs, rhs, out,
+                                                      ctx.track)
+        return grad_lhs, grad_rhs, None, None
+
+
+class SimpleCTCTLoss(torch.autograd.Function):
+    """The reference's autograd function of the log-add joiner on GATHERED
+    operands (warp_ctct/__init__.py:55-85): ``f`` (N, T, U), ``g`` (N, U, 3),
+    ``den`` (N, T, U) or None for the unnormalised variant.  Kept for code that
+    imports it by name; :func:`ctct_simple_loss` works on the un-gathered
+    operands instead."""
+
+    @staticmethod
+    def forward(ctx, f, g, den, labels, lx, ly, rg_f, rg_g):
+        normalized = den is not None and den.dim() == 3
+        stand_in = den if normalized else f.new_empty(1)
+        need = bool(rg_f or rg_g)
+        costs, grad_f, grad_g, grad_den = core.ctct_loss_simple_fwd(f, g, labels, stand_in, lx, ly,
+                                                                    need)
+        ctx.which = (bool(rg_f), bool(rg_g), normalized and need)
+        ctx.save_for_backward(*[t for t, keep in zip((grad_f, grad_g, grad_den), ctx.which)
+                                if keep])
+        return costs
+
+    @staticmethod
+    def backward(ctx, grad_outputs):
+        saved = list(ctx.saved_tensors)
+        w = grad_outputs.reshape(-1, 1, 1)
+        grads = [saved.pop(0) * w if keep else None for keep in ctx.which]
+        return grads[0], grads[1], grads[2], None, None, None, None, None
+
+
 def ctct_loss(log_probs: torch.Tensor,
               labels: torch.Tensor,
               frames_lengths: torch.Tensor,
