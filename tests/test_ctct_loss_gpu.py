@@ -548,6 +548,36 @@ def test_binding_rejects_bad_tensors():
         warp_ctct.ctct_loss(dev(joint), d_ys, d_lx, d_ly, reduction="avg")
 
 
+def test_autograd_plumbing_views_non_leaf_and_repeated_backward():
+    """The joint as a non-contiguous view and as a non-leaf, backward twice
+    over a retained graph, and a loss that is only part of the objective."""
+    import warp_ctct
+    joint, ys, lx, ly = make_joint_case(93, 3, 11, 4, 10, lx=[11, 7, 9], ly=[4, 2, 3])
+    _, ref_dense, ref_costs = O.ctct_loss(joint, ys, lx, ly, reduction="none", grad_output=np.ones(3))
+    d_ys, d_lx, d_ly = dev(ys), dev(lx), dev(ly)
+    # stored as (N, U+1, T, V); the loss sees the transposed view
+    base = dev(np.ascontiguousarray(joint.transpose(0, 2, 1, 3))).requires_grad_(True)
+    view = base.transpose(1, 2)
+    assert not view.is_contiguous()
+    c = warp_ctct.ctct_loss(view, d_ys, d_lx, d_ly, reduction="none")
+    np.testing.assert_allclose(c.detach().cpu().numpy(), ref_costs, rtol=LOSS_RTOL)
+    c.sum().backward(retain_graph=True)
+    first = base.grad.clone()
+    np.testing.assert_allclose(first.transpose(1, 2).cpu().numpy(), ref_dense, atol=GRAD_ATOL, rtol=0)
+    base.grad = None
+    c.sum().backward()                                  # the saved lattices serve a second backward
+    assert torch.equal(base.grad, first)
+    # non-leaf input and an objective with another term: d/dx [2 * loss(3 * x) + sum(x)]
+    x = dev(joint).requires_grad_(True)
+    loss = warp_ctct.ctct_loss(x * 1.0, d_ys, d_lx, d_ly, reduction="sum")
+    (2.0 * loss + x.sum()).backward()
+    np.testing.assert_allclose(x.grad.cpu().numpy(), 2.0 * ref_dense + 1.0, atol=2 * GRAD_ATOL, rtol=0)
+    with torch.no_grad():
+        quiet = warp_ctct.ctct_loss(x, d_ys, d_lx, d_ly, reduction="sum")
+    assert quiet.grad_fn is None and not quiet.requires_grad
+    np.testing.assert_allclose(quiet.item(), ref_costs.sum(), rtol=LOSS_RTOL)
+
+
 def test_infeasible_sample_has_infinite_cost():
     import warp_ctct
     joint, ys, lx, ly = make_joint_case(17, 2, 6, 3, 5, force_repeat=False)
