@@ -567,7 +567,7 @@ def test_autograd_plumbing_views_non_leaf_and_repeated_backward():
     base.grad = None
     c.sum().backward()                                  # the saved lattices serve a second backward
     assert torch.equal(base.grad, first)
-    # non-leaf input and an objective with another term: d/dx [2 * loss(3 * x) + sum(x)]
+    # non-leaf input and an objective with another term: d/dx [2 * loss(x) + sum(x)]
     x = dev(joint).requires_grad_(True)
     loss = warp_ctct.ctct_loss(x * 1.0, d_ys, d_lx, d_ly, reduction="sum")
     (2.0 * loss + x.sum()).backward()
