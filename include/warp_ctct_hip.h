@@ -34,7 +34,8 @@ enum {
     WARPCTCT_EINVAL = 1,     /* null pointer, negative size, size limit exceeded */
     WARPCTCT_ELAUNCH = 2,    /* hipGetLastError() reported a failed launch */
     WARPCTCT_EWORKSPACE = 3, /* workspace smaller than warpctct_workspace_bytes() */
-    WARPCTCT_ENODEVICE = 4   /* no usable HIP device */
+    WARPCTCT_ENODEVICE = 4,  /* no usable HIP device */
+    WARPCTCT_ETOOLARGE = 5   /* needs more than WARPCTCT_STATIC_SCRATCH_BYTES of work buffers */
 };
 
 /* Human-readable text for a return code (static storage). */
@@ -168,6 +169,23 @@ int warpctct_zero_fill(void *p, size_t bytes, void *stream);
 int warpctct_loss_forward(const void *joint, int dtype, const int *ys, const int *lx,
                           const int *ly, int N, int T, int U, int V, void *workspace,
                           size_t workspace_bytes, float *costs, float *unit_grads, void *stream);
+
+/* warpctct_loss_forward without a workspace argument, for callers that cannot
+ * allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * The work buffers (units, alpha, beta) live in a device array of
+ * WARPCTCT_STATIC_SCRATCH_BYTES that is part of the library's code object, one
+ * copy per GPU, held until the process ends; the call allocates and frees
+ * nothing.  A problem whose warpctct_workspace_bytes(N,T,U) exceeds that size
+ * is refused with WARPCTCT_ETOOLARGE before anything is launched.  All calls
+ * on one GPU share that GPU's array: calls that overlap on one GPU (two
+ * streams, two host threads) race and must be serialised by the caller.  The
+ * array's address is looked up on the first call on each device
+ * (hipGetSymbolAddress); make that call outside a graph capture. */
+#define WARPCTCT_STATIC_SCRATCH_BYTES (32u << 20)
+int warpctct_loss_forward_static(const void *joint, int dtype, const int *ys, const int *lx,
+                                 const int *ly, int N, int T, int U, int V, float *costs,
+                                 float *unit_grads, void *stream);
 
 /* ---- ctct_loss on logits --------------------------------------------------
  * The step before the reference's path fused into it: a caller of the

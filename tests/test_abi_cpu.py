@@ -18,8 +18,9 @@ def test_version_and_error_strings():
     lib = hip_lib.lib()
     assert lib.warpctct_version().decode().count(".") == 2
     assert lib.warpctct_error_string(0) == b"ok"
-    for code in range(1, 5):
+    for code in range(1, 6):
         assert len(lib.warpctct_error_string(code)) > 3
+    assert lib.warpctct_error_string(99) == b"unknown error"
 
 
 def test_workspace_size_is_monotone_and_covers_buffers():
@@ -51,6 +52,16 @@ def test_invalid_arguments_are_rejected_on_the_host():
     # empty batch is a no-op
     assert lib.warpctct_loss_forward_f32(null, null, null, null, 0, 4, 2, 8, null,
                                          ctypes.c_size_t(0), null, null, null) == 0
+    # the forward on the library's own scratch array: same argument checks, and a
+    # problem larger than the array is refused before any device is touched
+    ETOOLARGE = 5
+    assert lib.warpctct_loss_forward_static(null, 0, null, null, null, 2, 4, 2, 8, null, null,
+                                            null) == EINVAL
+    assert lib.warpctct_loss_forward_static(p, 4, p, p, p, 2, 4, 2, 8, p, p, null) == EINVAL
+    assert lib.warpctct_workspace_bytes(64, 600, 60) > (32 << 20)
+    assert lib.warpctct_loss_forward_static(p, 0, p, p, p, 64, 600, 60, 8, p, p, null) == ETOOLARGE
+    assert lib.warpctct_loss_forward_static(null, 0, null, null, null, 0, 4, 2, 8, null, null,
+                                            null) == 0
 
 
 def test_generic_dtype_and_logits_entry_points_check_their_arguments():

@@ -5,7 +5,15 @@
 
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "launch.h"
+
+// Work buffers of warpctct_loss_forward_static: part of the code object, one
+// copy per GPU at its own address.  In host code this name is only a handle
+// for hipGetSymbolAddress, never a device address.  (No `used` attribute: it
+// would keep the device symbol local, and the runtime finds it by name.)
+static __device__ __align__(256) unsigned char scratch[WARPCTCT_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -132,6 +140,27 @@ LogmmWorkspace carve_logmm(void *base, int B, int M, int K, int Nn) {
     return w;
 }
 
+// Address of `scratch` on the current device, looked up once per device with
+// that device current and kept for the life of the process.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(void **out) {
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices)
+        return WARPCTCT_ENODEVICE;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p)
+            return WARPCTCT_ENODEVICE;
+        g_scratch_ptr[device] = p;
+    }
+    *out = g_scratch_ptr[device];
+    return WARPCTCT_OK;
+}
+
 // lattice + unit gradients + reductions, shared by the two simple forwards
 int simple_from_units(const SimpleWorkspace &w, const int *ys, const int *lx, const int *ly, int N,
                       int T, int U, float *costs, float *grad_f, float *grad_g, float *grad_den,
@@ -169,6 +198,9 @@ const char *warpctct_error_string(int code) {
         case WARPCTCT_ELAUNCH: return "kernel launch failed";
         case WARPCTCT_EWORKSPACE: return "workspace too small";
         case WARPCTCT_ENODEVICE: return "no usable HIP device";
+        case WARPCTCT_ETOOLARGE:
+            return "the work buffers of this problem exceed the static scratch array "
+                   "(WARPCTCT_STATIC_SCRATCH_BYTES); use the entry point with a workspace argument";
         default: return "unknown error";
     }
 }
@@ -464,6 +496,25 @@ int warpctct_loss_forward(const void *joint, int dtype, const int *ys, const int
     }
     return forward_from_units(w, ys, lx, ly, N, T, U, costs, T > 0 ? unit_grads : nullptr,
                               as_stream(stream));
+}
+
+int warpctct_loss_forward_static(const void *joint, int dtype, const int *ys, const int *lx,
+                                 const int *ly, int N, int T, int U, int V, float *costs,
+                                 float *unit_grads, void *stream) {
+    if (!dims_ok(N, T, U) || V < 1 || !io_valid(dtype)) return WARPCTCT_EINVAL;
+    if (N == 0) return WARPCTCT_OK;
+    if (!lx || !ly || !costs || (T > 0 && !joint) || (U > 0 && !ys)) return WARPCTCT_EINVAL;
+    if (carve(nullptr, N, T, U).bytes > (size_t)WARPCTCT_STATIC_SCRATCH_BYTES)
+        return WARPCTCT_ETOOLARGE;
+    void *base = nullptr;
+    const int rc = static_scratch(&base);
+    if (rc != WARPCTCT_OK) return rc;
+    // Every cell of the array that a kernel reads has been written earlier in
+    // the same call (units by the gather, alpha / beta by the lattice sweep),
+    // so what an earlier call left behind is never seen and nothing needs
+    // clearing; the arrival counter of the batch reduction is not used here.
+    return warpctct_loss_forward(joint, dtype, ys, lx, ly, N, T, U, V, base,
+                                 (size_t)WARPCTCT_STATIC_SCRATCH_BYTES, costs, unit_grads, stream);
 }
 
 int warpctct_loss_forward_f32(const float *joint, const int *ys, const int *lx, const int *ly,
