@@ -145,6 +145,17 @@ int warpctct_loss_lattice(const void *joint, int dtype, const int *ys, const int
                           size_t workspace_bytes, float *costs, int want_alpha, int reduction,
                           int average_frames, float *reduced, void *stream);
 
+/* The same for a joint that is a strided view: element [n,t,u,v] lives at
+ * joint[n*strides[0] + t*strides[1] + u*strides[2] + v*strides[3]] (in
+ * elements; strides may be zero or negative as long as every address stays
+ * inside the caller's buffer).  The reference's torch.gather works on such
+ * views directly (warp_ctct/__init__.py:131); this avoids a copy of the joint. */
+int warpctct_loss_lattice_strided(const void *joint, int dtype, const long *strides,
+                                  const int *ys, const int *lx, const int *ly, int N, int T, int U,
+                                  int V, void *workspace, size_t workspace_bytes, float *costs,
+                                  int want_alpha, int reduction, int average_frames,
+                                  float *reduced, void *stream);
+
 /* Dense gradient of type `dtype` from that workspace (see
  * warpctct_dense_grad_lattice_f32 below for the weights); values are summed in
  * fp32 and rounded once to nearest even. */

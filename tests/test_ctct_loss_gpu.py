@@ -99,6 +99,12 @@ CASES = [
     ("odd_vocab_scalar_stores", 8, 3, 17, 5, 37, range(8, 18), range(2, 6), 1.0),
     ("vocab_1024_vector_stores", 9, 2, 30, 12, 1024, [30, 21], [12, 7], 1.0),
     ("peaky", 10, 4, 60, 20, 64, range(40, 61), range(10, 21), 4.0),
+    # lattices of several wavefronts whose samples are short: fewer frames than
+    # one hand-over chunk, a single partial chunk, one frame more than a chunk,
+    # and samples with 0..2 labels (the upper wavefronts hold only padding)
+    ("two_wavefronts_short_samples", 301, 6, 20, 100, 16, [1, 5, 8, 9, 17, 20], [0, 2, 1, 5, 2, 18], 1.0),
+    ("three_wavefronts_short_samples", 302, 5, 17, 150, 8, [1, 5, 8, 9, 17], [1, 0, 2, 2, 1], 1.0),
+    ("five_wavefronts_mixed_lengths", 303, 4, 310, 300, 8, [310, 1, 5, 9], [300, 0, 2, 1], 1.0),
 ]
 
 

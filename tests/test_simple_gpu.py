@@ -116,6 +116,36 @@ def test_log_matmul_backward(B, M, K, Nn, mask):
         assert out_r is None
 
 
+def test_log_matmul_with_a_shared_right_operand():
+    """A size-1 batch of rhs is shared by all batch entries of lhs: the forward
+    broadcasts it, the backward sums its gradient over the batch (the reference
+    undoes the broadcast with a reduction, csrc/binding.cpp:283-296).  Checked
+    against torch.logsumexp and its autograd with the operand expanded."""
+    import warp_ctct
+    rng = np.random.default_rng(88)
+    B, M, K, Nn = 5, 37, 70, 11
+    lhs = torch.tensor(rng.standard_normal((B, M, K)), dtype=torch.float32, device="cuda", requires_grad=True)
+    rhs = torch.tensor(rng.standard_normal((1, K, Nn)), dtype=torch.float32, device="cuda", requires_grad=True)
+    w = torch.tensor(rng.standard_normal((B, M, Nn)), dtype=torch.float32, device="cuda")
+    out = warp_ctct.LogMMExp.apply(lhs, rhs)
+    ref = torch.logsumexp(lhs[:, :, :, None] + rhs.expand(B, K, Nn)[:, None, :, :], dim=2)
+    torch.testing.assert_close(out, ref, rtol=1e-5, atol=1e-5)
+    gl, gr = torch.autograd.grad((out * w).sum(), (lhs, rhs))
+    rl, rr = torch.autograd.grad((ref * w).sum(), (lhs, rhs))
+    assert gl.shape == lhs.shape and gr.shape == rhs.shape
+    torch.testing.assert_close(gl, rl, rtol=1e-4, atol=2e-5)
+    torch.testing.assert_close(gr, rr, rtol=1e-4, atol=5e-5)
+    # the same with lhs given as a view whose batch entries are not adjacent rows
+    base = torch.tensor(rng.standard_normal((M, B, K)), dtype=torch.float32, device="cuda")
+    view = base.transpose(0, 1).detach().requires_grad_(True)
+    out2 = warp_ctct.LogMMExp.apply(view, rhs)
+    ref2 = torch.logsumexp(view[:, :, :, None] + rhs.expand(B, K, Nn)[:, None, :, :], dim=2)
+    g2 = torch.autograd.grad((out2 * w).sum(), (view, rhs))
+    r2 = torch.autograd.grad((ref2 * w).sum(), (view, rhs))
+    torch.testing.assert_close(g2[0], r2[0], rtol=1e-4, atol=2e-5)
+    torch.testing.assert_close(g2[1], r2[1], rtol=1e-4, atol=5e-5)
+
+
 def test_log_matmul_empty_extents():
     """Empty reductions and empty operands: logsumexp over nothing is -inf,
     its gradient zero; empty outputs stay empty."""
@@ -437,6 +467,49 @@ def test_full_size_log_add_joiner_normalized():
     """N=32, T<=400, U<=80, V=2048, normalized."""
     c = _identity_check(32, 400, 80, 2048, (300, 400), (50, 80), True, 404)
     assert torch.isfinite(c).all()
+
+
+def test_full_size_log_add_joiner_against_the_float64_oracle():
+    """N=32, T<=400, U<=80, V=2048, normalized: the shapes that select the
+    production tiles of the three matrix-core kernels.  den, the loss and the
+    dense gradients wrt f and g of two batch entries (one of them the longest)
+    against the float64 oracle at the gate itself: loss 1e-5 relative,
+    gradients 1e-4 absolute."""
+    import warp_ctct
+    from warp_ctct import _C
+    N, T, U, V = 32, 400, 80, 2048
+    rng = np.random.default_rng(414)
+    gen = torch.Generator(device="cuda").manual_seed(414)
+    f = torch.randn(N, T, V, device="cuda", generator=gen).log_softmax(-1)
+    g = torch.randn(N, U + 1, V, device="cuda", generator=gen).log_softmax(-1)
+    lx = rng.integers(300, 401, N).astype(np.int32)
+    ly = rng.integers(50, 81, N).astype(np.int32)
+    lx[0], ly[0] = 400, 80
+    ys = rng.integers(1, V, (N, U)).astype(np.int32)
+    ys[:, 5] = ys[:, 4]
+    d_ys, d_lx, d_ly = dev(ys), dev(lx), dev(ly)
+    w = rng.standard_normal(N)
+    w[0], w[9] = 1.25, -0.75
+    f.requires_grad_(True)
+    g.requires_grad_(True)
+    costs = warp_ctct.ctct_simple_loss(f, g, d_ys, d_lx, d_ly, reduction="none")
+    (costs * dev(w, torch.float32)).sum().backward()
+    den = _C.ctct_simple_fwd(f.detach(), g.detach(), d_ys, d_lx, d_ly, True, False)[1]
+    for n in (0, 9):
+        fn = f[n:n + 1].detach().cpu().numpy()
+        gn = g[n:n + 1].detach().cpu().numpy()
+        t, u = int(lx[n]), int(ly[n])
+        den_ref = O.log_matmul(fn[:, :t], np.swapaxes(gn[:, :u + 1], 1, 2))
+        np.testing.assert_allclose(den[n, :t, :u + 1].cpu().numpy(), den_ref[0], rtol=1e-5, atol=1e-5)
+        loss, gf, gg, c_ref = O.ctct_simple_loss(fn, gn, ys[n:n + 1], lx[n:n + 1], ly[n:n + 1],
+                                                 reduction="none", grad_output=w[n:n + 1])
+        np.testing.assert_allclose(costs[n].item(), c_ref[0], rtol=LOSS_RTOL)
+        # an entry of these gradients is a sum over up to 400 frames (81 contexts)
+        # of terms that are each within the bound; where it reaches the hundreds,
+        # one unit in the last place of float32 is 3e-5: 1e-6 relative on top
+        np.testing.assert_allclose(f.grad[n].cpu().numpy(), gf[0], atol=GRAD_ATOL, rtol=1e-6)
+        np.testing.assert_allclose(g.grad[n].cpu().numpy(), gg[0], atol=GRAD_ATOL, rtol=1e-6)
+        assert np.all(f.grad[n, t:].cpu().numpy() == 0) and np.all(g.grad[n, u + 1:].cpu().numpy() == 0)
 
 
 def test_deep_lattice_unnormalized():

@@ -219,8 +219,8 @@ int warpctct_gather_units_f32(const float *joint, const int *ys, const int *lx, 
     if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
     if (N == 0 || T == 0) return WARPCTCT_OK;
     if (!joint || !lx || !ly || !units_out || (U > 0 && !ys)) return WARPCTCT_EINVAL;
-    return done(launch_gather_units(joint, kIoF32, ys, lx, ly, units_out, N, T, U, V, false,
-                                    nullptr, as_stream(stream)));
+    return done(launch_gather_units(joint, dense_joint_strides(T, U, V), kIoF32, ys, lx, ly,
+                                    units_out, N, T, U, V, false, nullptr, as_stream(stream)));
 }
 
 int warpctct_scale_units_f32(const float *units_nat, const int *lx, const int *ly,
@@ -298,8 +298,22 @@ int warpctct_loss_lattice(const void *joint, int dtype, const int *ys, const int
                           const int *ly, int N, int T, int U, int V, void *workspace,
                           size_t workspace_bytes, float *costs, int want_alpha, int reduction,
                           int average_frames, float *reduced, void *stream) {
-    if (!dims_ok(N, T, U) || V < 1 || !io_valid(dtype) || reduction < 0 || reduction > 2)
+    const JointStrides js = dense_joint_strides(T, U, V);
+    const long strides[4] = {js.n, js.t, js.u, js.v};
+    return warpctct_loss_lattice_strided(joint, dtype, strides, ys, lx, ly, N, T, U, V, workspace,
+                                         workspace_bytes, costs, want_alpha, reduction,
+                                         average_frames, reduced, stream);
+}
+
+int warpctct_loss_lattice_strided(const void *joint, int dtype, const long *strides,
+                                  const int *ys, const int *lx, const int *ly, int N, int T, int U,
+                                  int V, void *workspace, size_t workspace_bytes, float *costs,
+                                  int want_alpha, int reduction, int average_frames,
+                                  float *reduced, void *stream) {
+    if (!dims_ok(N, T, U) || V < 1 || !io_valid(dtype) || reduction < 0 || reduction > 2 ||
+        !strides)
         return WARPCTCT_EINVAL;
+    const JointStrides js = {strides[0], strides[1], strides[2], strides[3]};
     if (N == 0) return WARPCTCT_OK;
     if (!lx || !ly || !costs || !workspace || (T > 0 && !joint) || (U > 0 && !ys))
         return WARPCTCT_EINVAL;
@@ -309,7 +323,7 @@ int warpctct_loss_lattice(const void *joint, int dtype, const int *ys, const int
     hipStream_t st = as_stream(stream);
     unsigned *counter = reduction != 0 ? w.counter : nullptr;
     if (T > 0) {
-        int rc = done(launch_gather_units(joint, dtype, ys, lx, ly, w.units, N, T, U, V, true,
+        int rc = done(launch_gather_units(joint, js, dtype, ys, lx, ly, w.units, N, T, U, V, true,
                                           counter, st));
         if (rc != WARPCTCT_OK) return rc;
     } else if (counter) {
@@ -490,8 +504,8 @@ int warpctct_loss_forward(const void *joint, int dtype, const int *ys, const int
     const Workspace w = carve(workspace, N, T, U);
     if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
     if (T > 0) {
-        int rc = done(launch_gather_units(joint, dtype, ys, lx, ly, w.units, N, T, U, V, true,
-                                          nullptr, as_stream(stream)));
+        int rc = done(launch_gather_units(joint, dense_joint_strides(T, U, V), dtype, ys, lx, ly,
+                                          w.units, N, T, U, V, true, nullptr, as_stream(stream)));
         if (rc != WARPCTCT_OK) return rc;
     }
     return forward_from_units(w, ys, lx, ly, N, T, U, costs, T > 0 ? unit_grads : nullptr,

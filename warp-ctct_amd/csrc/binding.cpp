@@ -124,7 +124,8 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_loss_joint_fwd(const torch::Tensor
                                                              const bool requires_grad,
                                                              const int64_t reduction,
                                                              const bool average_frames) {
-    CHECK_CONTIGUOUS(joint);
+    // the joint may be any strided view (the reference's torch.gather takes
+    // views as they are, warp_ctct/__init__.py:131): no copy is made
     CHECK_DEVICE(joint);
     const int dtype = io_type_of(joint);
     TORCH_CHECK(joint.dim() == 4, "log probs must have 4 dims.");
@@ -138,13 +139,15 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_loss_joint_fwd(const torch::Tensor
     auto costs = torch::empty({N}, f32);
     torch::Tensor reduced;
     if (reduction != 0) reduced = N > 0 ? torch::empty({}, f32) : torch::zeros({}, f32);
-    check_rc(warpctct_loss_lattice(joint.data_ptr(), dtype, ys.data_ptr<int>(),
-                                   lx.data_ptr<int>(), ly.data_ptr<int>(), N, T, U, V,
-                                   ws.data_ptr(), ws.numel(), costs.data_ptr<float>(),
-                                   requires_grad ? 1 : 0, static_cast<int>(reduction),
-                                   average_frames ? 1 : 0,
-                                   reduction != 0 ? reduced.data_ptr<float>() : nullptr,
-                                   current_stream()),
+    const long strides[4] = {static_cast<long>(joint.stride(0)), static_cast<long>(joint.stride(1)),
+                             static_cast<long>(joint.stride(2)), static_cast<long>(joint.stride(3))};
+    check_rc(warpctct_loss_lattice_strided(joint.data_ptr(), dtype, strides, ys.data_ptr<int>(),
+                                           lx.data_ptr<int>(), ly.data_ptr<int>(), N, T, U, V,
+                                           ws.data_ptr(), ws.numel(), costs.data_ptr<float>(),
+                                           requires_grad ? 1 : 0, static_cast<int>(reduction),
+                                           average_frames ? 1 : 0,
+                                           reduction != 0 ? reduced.data_ptr<float>() : nullptr,
+                                           current_stream()),
              "ctct_loss_joint_fwd");
     const torch::Tensor &loss = reduction != 0 ? reduced : costs;
     if (requires_grad) return std::make_tuple(loss, ws);
@@ -545,22 +548,36 @@ std::tuple<torch::Tensor, torch::Tensor> log_matmul_backward(
                 "need cuda tensors");
     TORCH_CHECK(lhs.dim() == 3 && rhs.dim() == 3 && result.dim() == 3 && grad_out.dim() == 3,
                 "invalid sizes");
-    const int B = lhs.size(0), M = lhs.size(1), K = lhs.size(2), Nn = rhs.size(2);
-    TORCH_CHECK(rhs.size(0) == B && rhs.size(1) == K, "invalid sizes (batch broadcast is not "
-                "supported in the backward)");
+    int B = lhs.size(0), M = lhs.size(1);
+    const int K = lhs.size(2), Nn = rhs.size(2);
+    TORCH_CHECK((rhs.size(0) == B || rhs.size(0) == 1) && rhs.size(1) == K, "invalid sizes");
     TORCH_CHECK(result.size(0) == B && result.size(1) == M && result.size(2) == Nn &&
                     grad_out.sizes() == result.sizes(), "invalid sizes");
     const DeviceGuard device_guard(device_of(lhs));
     auto go = grad_out.contiguous();
     auto res = result.contiguous();
-    if (grad_input_mask[0]) grad_lhs = torch::empty({B, M, K}, lhs.options());
-    if (grad_input_mask[1]) grad_rhs = torch::empty({B, K, Nn}, rhs.options());
+    // A size-1 batch of rhs is shared by every batch entry of lhs (the
+    // reference expands it in the forward and undoes the broadcast with a
+    // reduction over the batch, csrc/binding.cpp:283-296).  With one rhs the
+    // batch of lhs is just more rows: the (B,M,K) problem is the (1,B*M,K)
+    // problem, whose rhs gradient already sums over all B*M rows.
+    torch::Tensor lhs_rows = lhs;
+    const int64_t out_B = B, out_M = M;
+    const bool shared_rhs = rhs.size(0) == 1 && B > 1;
+    if (shared_rhs) {
+        if (lhs.stride(0) != (int64_t)M * lhs.stride(1)) lhs_rows = lhs.contiguous();
+        M = B * M;
+        B = 1;
+    }
+    if (grad_input_mask[0]) grad_lhs = torch::empty({out_B, out_M, K}, lhs.options());
+    if (grad_input_mask[1]) grad_rhs = torch::empty({rhs.size(0), K, Nn}, rhs.options());
     auto ws = make_bytes(lhs, warpctct_logmm_workspace_bytes(B, M, K, Nn));
     check_rc(warpctct_logmm_bwd_f32(
-                 go.data_ptr<float>(), lhs.data_ptr<float>(), lhs.stride(0), lhs.stride(1),
-                 lhs.stride(2), rhs.data_ptr<float>(), rhs.stride(0), rhs.stride(1), rhs.stride(2),
-                 res.data_ptr<float>(), B, M, K, Nn, ws.data_ptr(), ws.numel(),
-                 grad_input_mask[0] ? grad_lhs.data_ptr<float>() : nullptr, (long)M * K, (long)K, 1L,
+                 go.data_ptr<float>(), lhs_rows.data_ptr<float>(), lhs_rows.stride(0),
+                 lhs_rows.stride(1), lhs_rows.stride(2), rhs.data_ptr<float>(), rhs.stride(0),
+                 rhs.stride(1), rhs.stride(2), res.data_ptr<float>(), B, M, K, Nn, ws.data_ptr(),
+                 ws.numel(), grad_input_mask[0] ? grad_lhs.data_ptr<float>() : nullptr,
+                 (long)M * K, (long)K, 1L,
                  grad_input_mask[1] ? grad_rhs.data_ptr<float>() : nullptr, (long)K * Nn, (long)Nn,
                  1L, current_stream()),
              "log_matmul_backward");

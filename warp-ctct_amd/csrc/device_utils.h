@@ -55,16 +55,6 @@ __device__ __forceinline__ double lse2(double x, double y) {
     return mx + (double)log2_hw(1.0f + exp2_hw(d));
 }
 
-// log2(2^x + 2^y + 2^z).  All three -inf: the sum of exponentials is 0, its
-// log2 is -inf, the result is -inf.
-__device__ __forceinline__ double lse3(double x, double y, double z) {
-    const double mx = __builtin_fmax(__builtin_fmax(x, y), z);
-    const double ms = __builtin_fmax(mx, kFloor);
-    const float s =
-        exp2_hw((float)(x - ms)) + exp2_hw((float)(y - ms)) + exp2_hw((float)(z - ms));
-    return ms + (double)log2_hw(s);
-}
-
 // Lane l receives x of lane l-1; lane 0 receives `fill`.  Two DPP moves
 // (wave_shr:1), no LDS traffic.
 __device__ __forceinline__ double wave_shift_up(double x, double fill) {

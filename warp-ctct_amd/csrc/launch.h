@@ -43,12 +43,22 @@ struct LatticeArgs {
 int lattice_max_contexts();
 hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream);
 
+// Element strides of a joint tensor (N,T,U+1,V); dense row-major is
+// {T*(U+1)*V, (U+1)*V, V, 1}.
+struct JointStrides {
+    long n, t, u, v;
+};
+inline JointStrides dense_joint_strides(int T, int U, int V) {
+    return JointStrides{(long)T * (U + 1) * V, (long)(U + 1) * V, (long)V, 1L};
+}
+
 // band_only: cells outside the band of complete alignments get neutral units
 // (same costs and gradients; alpha / beta of dead cells are not the oracle's)
 // counter (may be null): set to 0 by the kernel, for a CostReduce that follows
-hipError_t launch_gather_units(const void *joint, int io_type, const int *ys, const int *lx,
-                               const int *ly, double *units, int N, int T, int U, int V,
-                               bool band_only, unsigned *counter, hipStream_t stream);
+hipError_t launch_gather_units(const void *joint, const JointStrides &strides, int io_type,
+                               const int *ys, const int *lx, const int *ly, double *units, int N,
+                               int T, int U, int V, bool band_only, unsigned *counter,
+                               hipStream_t stream);
 hipError_t launch_clear_counter(unsigned *counter, hipStream_t stream);
 hipError_t launch_scale_units(const float *units_nat, const int *lx, const int *ly, double *units,
                               int N, int T, int U, hipStream_t stream);

@@ -25,44 +25,18 @@ constexpr int kGradWaves = 1;          // ... and backward: 4 KiB per workgroup,
 constexpr float kLog2eF = 1.4426950408889634f;
 constexpr float kLn2F = 0.6931471805599453f;
 
-template <typename IO> struct Vec4;   // 4 elements of the joint, loaded as one vector
-template <> struct Vec4<float> {
-    typedef float type __attribute__((ext_vector_type(4)));
-};
-template <> struct Vec4<__half> {
-    typedef _Float16 type __attribute__((ext_vector_type(4)));
-};
-template <> struct Vec4<__hip_bfloat16> {
-    typedef unsigned short type __attribute__((ext_vector_type(4)));
-};
-
-__device__ __forceinline__ float elem_to_float(float v) { return v; }
-__device__ __forceinline__ float elem_to_float(_Float16 v) { return (float)v; }
-__device__ __forceinline__ float elem_to_float(unsigned short v) {   // bfloat16 bits
-    return __uint_as_float((unsigned)v << 16);
+// one 16-byte vector of floats
+__device__ __forceinline__ void load4(const float *p, float (&x)[4]) {
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    const v4f v = *reinterpret_cast<const v4f *>(p);
+    x[0] = v.x;
+    x[1] = v.y;
+    x[2] = v.z;
+    x[3] = v.w;
 }
-
-template <typename IO>
-__device__ __forceinline__ void load4(const IO *p, float (&x)[4]) {
-    const typename Vec4<IO>::type v = *reinterpret_cast<const typename Vec4<IO>::type *>(p);
-    x[0] = elem_to_float(v.x);
-    x[1] = elem_to_float(v.y);
-    x[2] = elem_to_float(v.z);
-    x[3] = elem_to_float(v.w);
-}
-
 __device__ __forceinline__ void store4(float *p, const float (&x)[4]) {
     typedef float v4f __attribute__((ext_vector_type(4)));
     *reinterpret_cast<v4f *>(p) = v4f{x[0], x[1], x[2], x[3]};
-}
-__device__ __forceinline__ void store4(__half *p, const float (&x)[4]) {
-    __half h[4] = {__float2half(x[0]), __float2half(x[1]), __float2half(x[2]), __float2half(x[3])};
-    *reinterpret_cast<uint2 *>(p) = *reinterpret_cast<const uint2 *>(h);
-}
-__device__ __forceinline__ void store4(__hip_bfloat16 *p, const float (&x)[4]) {
-    __hip_bfloat16 h[4] = {__float2bfloat16(x[0]), __float2bfloat16(x[1]), __float2bfloat16(x[2]),
-                           __float2bfloat16(x[3])};
-    *reinterpret_cast<uint2 *>(p) = *reinterpret_cast<const uint2 *>(h);
 }
 
 // 16-byte vectors of 2-byte elements

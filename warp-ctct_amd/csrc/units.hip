@@ -75,20 +75,20 @@ __device__ __forceinline__ bool store_padding(double *units, const Cell &c, int 
 // kernel that follows on the same stream.
 template <bool BAND_ONLY, typename IO>
 __global__ __launch_bounds__(kCellBlock) void gather_units_kernel(
-    const IO *__restrict__ joint, const int *__restrict__ ys, const int *__restrict__ lx,
-    const int *__restrict__ ly, double *__restrict__ units, int T, int U, int V, int P,
-    unsigned *__restrict__ counter) {
+    const IO *__restrict__ joint, const JointStrides js, const int *__restrict__ ys,
+    const int *__restrict__ lx, const int *__restrict__ ly, double *__restrict__ units, int T,
+    int U, int V, int P, unsigned *__restrict__ counter) {
     if (counter && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *counter = 0u;
     Cell c = locate_cell(lx, ly, T, U, P);
     if (BAND_ONLY && c.live && outside_band(c.t, c.u, c.Tn, c.Un)) c.live = false;
     if (store_padding(units, c, T, P)) return;
-    const IO *row = joint + (((size_t)c.n * T + c.t) * (U + 1) + c.u) * (size_t)V;
+    const IO *row = joint + (long)c.n * js.n + (long)c.t * js.t + (long)c.u * js.u;
     const int *y = ys + (size_t)c.n * U;
     const float b = load_as_float(row);
     float cur = b, nxt = b;   // the reference gathers index 0 where no label exists
     // labels are clamped into [0,V) so that a corrupt label cannot fault
-    if (c.u >= 1) cur = load_as_float(row + min(max(y[c.u - 1], 0), V - 1));
-    if (c.u < c.Un) nxt = load_as_float(row + min(max(y[c.u], 0), V - 1));
+    if (c.u >= 1) cur = load_as_float(row + (long)min(max(y[c.u - 1], 0), V - 1) * js.v);
+    if (c.u < c.Un) nxt = load_as_float(row + (long)min(max(y[c.u], 0), V - 1) * js.v);
     store_units(units, c, T, P, b, cur, nxt);
 }
 
@@ -151,37 +151,38 @@ namespace {
 __global__ void clear_counter_kernel(unsigned *counter) { *counter = 0u; }
 
 template <typename IO>
-void launch_gather_typed(const void *joint, const int *ys, const int *lx, const int *ly,
-                         double *units, int N, int T, int U, int V, bool band_only,
+void launch_gather_typed(const void *joint, const JointStrides &js, const int *ys, const int *lx,
+                         const int *ly, double *units, int N, int T, int U, int V, bool band_only,
                          unsigned *counter, hipStream_t stream) {
     const int P = padded_contexts(U);
     const IO *j = static_cast<const IO *>(joint);
     if (band_only) {
         hipLaunchKernelGGL((gather_units_kernel<true, IO>), cell_grid(N, T, P), dim3(kCellBlock),
-                           0, stream, j, ys, lx, ly, units, T, U, V, P, counter);
+                           0, stream, j, js, ys, lx, ly, units, T, U, V, P, counter);
     } else {
         hipLaunchKernelGGL((gather_units_kernel<false, IO>), cell_grid(N, T, P), dim3(kCellBlock),
-                           0, stream, j, ys, lx, ly, units, T, U, V, P, counter);
+                           0, stream, j, js, ys, lx, ly, units, T, U, V, P, counter);
     }
 }
 
 }  // namespace
 
-hipError_t launch_gather_units(const void *joint, int io_type, const int *ys, const int *lx,
-                               const int *ly, double *units, int N, int T, int U, int V,
-                               bool band_only, unsigned *counter, hipStream_t stream) {
+hipError_t launch_gather_units(const void *joint, const JointStrides &js, int io_type,
+                               const int *ys, const int *lx, const int *ly, double *units, int N,
+                               int T, int U, int V, bool band_only, unsigned *counter,
+                               hipStream_t stream) {
     switch (io_type) {
         case kIoF32:
-            launch_gather_typed<float>(joint, ys, lx, ly, units, N, T, U, V, band_only, counter,
+            launch_gather_typed<float>(joint, js, ys, lx, ly, units, N, T, U, V, band_only, counter,
                                        stream);
             break;
         case kIoF16:
-            launch_gather_typed<__half>(joint, ys, lx, ly, units, N, T, U, V, band_only, counter,
-                                        stream);
+            launch_gather_typed<__half>(joint, js, ys, lx, ly, units, N, T, U, V, band_only,
+                                        counter, stream);
             break;
         case kIoBF16:
-            launch_gather_typed<__hip_bfloat16>(joint, ys, lx, ly, units, N, T, U, V, band_only,
-                                                counter, stream);
+            launch_gather_typed<__hip_bfloat16>(joint, js, ys, lx, ly, units, N, T, U, V,
+                                                band_only, counter, stream);
             break;
         default:
             return hipErrorInvalidValue;

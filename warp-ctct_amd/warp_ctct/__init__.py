@@ -23,7 +23,20 @@ except ImportError as exc:  # pragma: no cover - exercised only on a broken inst
     ) from exc
 
 __all__ = ["ctct_loss", "ctct_loss_compact", "ctct_loss_with_logits", "ctct_simple_loss"]
-__version__ = core.library_version()
+
+
+def _package_version():
+    """Version of the installed distribution (the reference reads it the same
+    way, warp_ctct/__init__.py:14); the library's own version string when the
+    package is used from a source tree without distribution metadata."""
+    try:
+        from importlib.metadata import version
+        return version("warp_ctct")
+    except Exception:
+        return core.library_version()
+
+
+__version__ = _package_version()
 
 
 # Optional observer for profiling: called as observer(kernel_name, fn) and must
@@ -264,7 +277,8 @@ def ctct_loss(log_probs: torch.Tensor,
     if log_probs.dtype not in _NATIVE_DTYPES:
         log_probs = log_probs.float()      # as the reference does for every dtype (:135)
     with _no_autocast():
-        return _CTCTLoss.apply(log_probs.contiguous(), _as_int(labels), _as_int(frames_lengths),
+        # a strided view is gathered through its strides, not copied
+        return _CTCTLoss.apply(log_probs, _as_int(labels), _as_int(frames_lengths),
                                _as_int(labels_lengths), enable_grad, reduction,
                                bool(average_frames))
 
