@@ -1,17 +1,22 @@
 #!/usr/bin/env python3
-"""Benchmark of the ctct_loss hot path on one MI355X.
+"""Benchmark of the CTC-Transducer loss hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-configs]
 
 One step = forward + backward of warp_ctct.ctct_loss on one resident batch of
 the "typical ASR batch" workload: N=32, frames 150..250, labels 30..60,
 V=1024, fp32 joint log-probs already in HBM, padded regions zero-filled.
 Prints ONE JSON line: whole-job lattices/s, the roofline of the dominant
 kernel (the zero-fill of the dense gradient, timed with HIP events on its
-stream inside the timed region) and a CPU baseline (the C oracle with OpenMP, on the host
-cores, same batch).
+stream inside the timed region), a CPU baseline (the C oracle with OpenMP, on
+the host cores, same batch) and, under "configs", the same measurement for all
+five benchmark configurations with the HIP-event duration of every kernel of
+a step (the library's own per-kernel timing, warpctct_profile).
+
+    python bench.py --config c4 [--graph]      one configuration alone (reduced line)
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -21,7 +26,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "warp-ctct_amd"))
 sys.path.insert(0, ROOT)
 
-HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix, published
 # HBM bytes per launch of zero_fill_vec_kernel from two rocprofv3 --pmc runs
 # (profiles/ctct_loss_typical_batch_pmc.md): WRITE_SIZE 1 952 000 KiB x 1.0 +
 # FETCH_SIZE 12.8 KiB x 2.0, the factors being what the same counters read for
@@ -61,7 +67,8 @@ def cpu_baseline(joint, ys, lx, ly, budget_s=10.0):
     """C oracle (oracle/ctct_oracle.c, fp32, OpenMP over lattices) on the host
     copy of the same batch: gather + lattice + dense gradient."""
     from oracle import c_oracle as C
-    threads = max(1, min(16, os.cpu_count() or 1))
+    host_cores = os.cpu_count() or 1
+    threads = max(1, min(16, host_cores))
     C.set_num_threads(threads)
     host = joint.cpu().numpy()
     N = host.shape[0]
@@ -74,15 +81,49 @@ def cpu_baseline(joint, ys, lx, ly, budget_s=10.0):
         times.append(time.perf_counter() - t0)
     times.sort()
     med = times[len(times) // 2]
-    return {"value": N / med, "unit": "lattices/s", "cores": threads, "kind": "port",
+    return {"value": N / med, "unit": "lattices/s", "cores": threads, "host_cores": host_cores,
+            "kind": "port",
             "sample": "the same N=%d batch, %d runs, median %.3f s per batch "
-                      "(C oracle, fp32, OpenMP)" % (N, len(times), med)}
+                      "(C oracle, fp32, OpenMP on %d threads; the host reports %d cores)"
+                      % (N, len(times), med, threads, host_cores)}
+
+
+# ---- per-kernel HIP-event timing through the library's own hook ---------------
+_LIB = None
+
+
+def kernel_library():
+    global _LIB
+    if _LIB is None:
+        _LIB = ctypes.CDLL(os.path.join(ROOT, "warp-ctct_amd", "warp_ctct", "libwarpctct_hip.so"))
+    return _LIB
+
+
+def profile_kernels(torch, run, steps):
+    """Average duration in microseconds, per step, of every kernel of the
+    library that `run` launches (HIP events on the stream of each launch)."""
+    lib = kernel_library()
+    torch.cuda.synchronize()
+    lib.warpctct_profile(1)
+    for _ in range(steps):
+        run()
+    torch.cuda.synchronize()
+    lib.warpctct_profile(0)
+    name, us = ctypes.c_char_p(), ctypes.c_float()
+    total, calls = {}, {}
+    for i in range(lib.warpctct_profile_count()):
+        if lib.warpctct_profile_read(i, ctypes.byref(name), ctypes.byref(us)) != 0:
+            continue
+        k = name.value.decode().strip("()")
+        total[k] = total.get(k, 0.0) + us.value
+        calls[k] = calls.get(k, 0) + 1
+    return {k: {"us_per_step": total[k] / steps, "launches_per_step": calls[k] / steps} for k in total}
 
 
 OTHER = {
     # name: (kind, N, T, U, V, sigma)
     "c1": ("full", 2, 40, 10, 32, 1.0),
-    "c2": ("full", 32, 250, 60, 1024, 1.0),   # only with --graph; the headline line is main()'s
+    "c2": ("full", 32, 250, 60, 1024, 1.0),
     "c3": ("full", 8, 500, 120, 4096, 2.0),
     "c4": ("simple_norm", 32, 400, 80, 2048, 1.0),
     "c5": ("simple_unnorm", 4, 1500, 300, 8192, 1.0),
@@ -96,21 +137,28 @@ OTHER = {
     "c2_logits_unfused": ("logits_unfused", 32, 250, 60, 1024, 1.0),
 }
 IO_DTYPE = {"c2_bf16": "bfloat16", "c2_f16": "float16", "c2_logits_bf16": "bfloat16"}
+WORKLOAD = {
+    "c1": "ctct_loss fp32, N=2, T=40, U=10, V=32, full lengths (the reference's CPU-sized case)",
+    "c2": "ctct_loss fp32, typical ASR batch: N=32, lx in [150,250], ly in [30,60], V=1024",
+    "c3": "ctct_loss fp32, large vocabulary / long lattice: N=8, lx in [400,500], ly in [80,120], V=4096, N(0,2) logits",
+    "c4": "ctct_simple_loss fp32 normalized (log-add joiner): N=32, lx in [300,400], ly in [50,80], V=2048",
+    "c5": "ctct_simple_loss fp32 unnormalized, long-utterance stress: N=4, lx in [1200,1500], ly in [250,300], V=8192",
+}
 
 
-def other_config(args, torch, warp_ctct):
-    """The remaining benchmark configurations: same timing discipline, a
-    reduced JSON line (value, ms_per_step, per-operator HIP-event times)."""
+def build_config(name, torch, warp_ctct):
+    """Synthetic inputs of one configuration, resident on the GPU.  Returns
+    (step function, facts) where facts holds sizes and algorithmic work."""
     import numpy as np
-    kind, N, T, U, V, sigma = OTHER[args.config]
+    kind, N, T, U, V, sigma = OTHER[name]
     rng = np.random.default_rng(7)
     gen = torch.Generator(device="cuda").manual_seed(7)
-    if args.config == "c1":
+    if name == "c1":
         lx = np.full(N, T, np.int32)
         ly = np.full(N, U, np.int32)
     else:
-        lo_t = {"c3": 400, "c4": 300, "c5": 1200}.get(args.config, 150)
-        lo_u = {"c3": 80, "c4": 50, "c5": 250}.get(args.config, 30)
+        lo_t = {"c3": 400, "c4": 300, "c5": 1200}.get(name, 150)
+        lo_u = {"c3": 80, "c4": 50, "c5": 250}.get(name, 30)
         lx = rng.integers(lo_t, T + 1, N).astype(np.int32)
         ly = rng.integers(lo_u, U + 1, N).astype(np.int32)
         lx[0], ly[1] = T, U
@@ -118,25 +166,29 @@ def other_config(args, torch, warp_ctct):
     ys[:, 3] = ys[:, 2]
     d_ys, d_lx, d_ly = (torch.as_tensor(a).cuda() for a in (ys, lx, ly))
     live = int(sum(int(a) * (int(b) + 1) for a, b in zip(lx, ly)))
+    facts = {"kind": kind, "N": N, "T": T, "U": U, "V": V, "max_frames": int(lx.max()),
+             "live_cells": live}
     if kind == "full":
         joint = torch.randn(N, T, U + 1, V, device="cuda", generator=gen).mul_(sigma).log_softmax(-1)
         t_idx = torch.arange(T, device="cuda")[None, :, None, None]
         u_idx = torch.arange(U + 1, device="cuda")[None, None, :, None]
         joint.masked_fill_((t_idx >= d_lx[:, None, None, None]) | (u_idx > d_ly[:, None, None, None]), 0.0)
-        io = getattr(torch, IO_DTYPE.get(args.config, "float32"))
+        io = getattr(torch, IO_DTYPE.get(name, "float32"))
         joint = joint.to(io).requires_grad_(True)
         leaves = (joint,)
-        alg_bytes = joint.element_size() * (N * T * (U + 1) * V + 3 * live) + 4 * N * (U + 3)
+        facts["algorithmic_bytes_per_step"] = (joint.element_size() * (N * T * (U + 1) * V + 3 * live)
+                                               + 4 * N * (U + 3))
+        facts["dense_gradient_bytes"] = joint.element_size() * N * T * (U + 1) * V
 
         def loss_fn():
             return warp_ctct.ctct_loss(joint, d_ys, d_lx, d_ly)
     elif kind in ("logits", "logits_unfused"):
-        io = getattr(torch, IO_DTYPE.get(args.config, "float32"))
+        io = getattr(torch, IO_DTYPE.get(name, "float32"))
         logits = torch.randn(N, T, U + 1, V, device="cuda", generator=gen).mul_(3.0).to(io)
         logits.requires_grad_(True)
         leaves = (logits,)
         # algorithmic bytes: live rows read twice (forward, backward), gradient written once
-        alg_bytes = logits.element_size() * V * (2 * live + N * T * (U + 1))
+        facts["algorithmic_bytes_per_step"] = logits.element_size() * V * (2 * live + N * T * (U + 1))
 
         if kind == "logits":
             def loss_fn():
@@ -153,26 +205,90 @@ def other_config(args, torch, warp_ctct):
         f.requires_grad_(True)
         g.requires_grad_(True)
         leaves = (f, g)
-        alg_bytes = 8 * N * V * (T + U + 1) if normalized else \
+        facts["algorithmic_bytes_per_step"] = 8 * N * V * (T + U + 1) if normalized else \
             4 * live + 12 * int(sum(int(b) + 1 for b in ly)) + 4 * N * V * (T + U + 1)
+        if normalized:
+            # log-add terms of the forward and of each of the two gradients, 2 flop each
+            facts["algorithmic_flops_per_step"] = 3 * 2 * N * T * (U + 1) * V
 
         def loss_fn():
             return warp_ctct.ctct_simple_loss(f, g, d_ys, d_lx, d_ly, normalized=normalized)
 
-    events = {}
-
-    def observer(name, fn):
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        e0.record()
-        out = fn()
-        e1.record()
-        events.setdefault(name, []).append((e0, e1))
-        return out
-
     def step():
         return torch.autograd.grad(loss_fn(), leaves)
 
+    return step, facts
+
+
+def time_steps(torch, run, steps, warmup):
+    for _ in range(warmup):
+        run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def summarise(name, facts, sec_per_step, kernels):
+    """The figures of one configuration: step time, throughput, and the
+    fraction of the roofline that bounds it."""
+    us = {k: round(v["us_per_step"], 2) for k, v in sorted(kernels.items(), key=lambda kv: -kv[1]["us_per_step"])}
+    out = {"workload": WORKLOAD.get(name, name), "ms_per_step": sec_per_step * 1e3,
+           "value": facts["N"] / sec_per_step, "unit": "lattices/s",
+           "kernel_us_per_step": us, "kernel_us_total": round(sum(us.values()), 2)}
+    if "algorithmic_bytes_per_step" in facts:
+        out["algorithmic_bytes_per_step"] = facts["algorithmic_bytes_per_step"]
+        out["step_frac_of_hbm_roofline"] = (facts["algorithmic_bytes_per_step"] / sec_per_step / 1e9
+                                            / HBM_PEAK_GBS)
+    lattice = sum(v for k, v in us.items() if k.startswith("lattice_kernel"))
+    if lattice > 0:
+        out["lattice_kernel_us"] = lattice
+        out["lattice_ns_per_frame"] = lattice * 1e3 / facts["max_frames"]
+    fill = us.get("zero_fill_vec_kernel")
+    if name == "c1" or facts["kind"] == "simple_unnorm":
+        out["roofline"] = {"bound": "latency", "kernel": "lattice_kernel",
+                           "note": "serial recursion over max_frames dependent steps; reported as "
+                                   "ns per frame, an HBM fraction would be structurally low",
+                           "max_frames": facts["max_frames"]}
+    elif facts["kind"] == "full" and fill:
+        gbs = facts["dense_gradient_bytes"] / (fill * 1e-6) / 1e9
+        out["roofline"] = {"bound": "hbm", "kernel": "zero_fill_vec_kernel", "achieved": gbs,
+                           "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                           "avg_launch_us": fill,
+                           "algorithmic_bytes_per_launch": facts["dense_gradient_bytes"]}
+    elif facts["kind"] == "simple_norm":
+        gemm = {k: v for k, v in us.items() if k.startswith(("logmm_fwd_kernel", "logmm_bwd"))
+                and "zero" not in k and "finish" not in k}
+        gemm_us = sum(gemm.values())
+        flops = facts["algorithmic_flops_per_step"]
+        tf = flops / (gemm_us * 1e-6) / 1e12 if gemm_us > 0 else 0.0
+        out["algorithmic_flops_per_step"] = flops
+        out["roofline"] = {"bound": "mfma", "kernel": "the three fp32 matrix-core GEMMs of the "
+                           "log-matmul (forward, gradient wrt f, gradient wrt g)",
+                           "achieved": tf, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                           "frac": tf / MFMA_FP32_PEAK_TFLOPS, "avg_launch_us": gemm,
+                           "algorithmic_flops_per_launch": flops // 3}
+        out["step_frac_of_mfma_roofline"] = flops / sec_per_step / 1e12 / MFMA_FP32_PEAK_TFLOPS
+    return out
+
+
+def measure_config(name, torch, warp_ctct, steps, warmup=3, profile_steps=3):
+    step, facts = build_config(name, torch, warp_ctct)
+    sec = time_steps(torch, step, steps, warmup)
+    kernels = profile_kernels(torch, step, profile_steps)
+    out = summarise(name, facts, sec, kernels)
+    out["steps"] = steps
+    del step
+    torch.cuda.empty_cache()
+    return out
+
+
+def other_config(args, torch, warp_ctct):
+    """One configuration alone: same timing discipline, a reduced JSON line."""
+    kind, N, T, U, V, sigma = OTHER[args.config]
+    step, facts = build_config(args.config, torch, warp_ctct)
     run = step
     if args.graph:
         # the whole step as one HIP graph: one submission per step instead of
@@ -185,31 +301,18 @@ def other_config(args, torch, warp_ctct):
         torch.cuda.current_stream().wait_stream(side)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            captured = step()
+            captured = step()   # noqa: F841  (keeps the captured outputs alive)
         run = graph.replay
-    for _ in range(args.warmup):
-        run()
-    torch.cuda.synchronize()
-    if not args.graph:
-        warp_ctct.set_kernel_observer(observer)
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        run()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    warp_ctct.set_kernel_observer(None)
-    ms = elapsed / args.steps * 1e3
-    ops = {k: sum(a.elapsed_time(b) for a, b in v) / len(v) * 1e3 for k, v in events.items()}
+    sec = time_steps(torch, run, args.steps, args.warmup)
+    kernels = {} if args.graph else profile_kernels(torch, step, 3)
+    out = summarise(args.config, facts, sec, kernels)
     print(json.dumps({
-        "metric": "lattices/sec (loss+grad)", "value": N * args.steps / elapsed,
+        "metric": "lattices/sec (loss+grad)", "value": out["value"],
         "unit": "lattices/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms, "higher_is_better": True, "dtype": "f32", "data": "synthetic",
-        "io_dtype": IO_DTYPE.get(args.config, "float32"), "hip_graph": bool(args.graph),
-        "config": {"workload": args.config, "kind": kind, "N": N, "T": T, "U": U, "V": V,
-                   "algorithmic_bytes_per_step": alg_bytes,
-                   "step_frac_of_hbm_roofline": alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                   "max_frames": int(lx.max()), "ns_per_frame_step": ms * 1e6 / int(lx.max())},
-        "operator_us": ops}))
+        "ms_per_step": out["ms_per_step"], "higher_is_better": True, "dtype": "f32",
+        "data": "synthetic", "io_dtype": IO_DTYPE.get(args.config, "float32"),
+        "hip_graph": bool(args.graph),
+        "config": dict(out, workload=args.config, kind=kind, N=N, T=T, U=U, V=V)}))
 
 
 def main():
@@ -218,11 +321,11 @@ def main():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "c2_bf16", "c2_f16", "c2_logits",
-                             "c2_logits_bf16", "c2_logits_unfused"],
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the per-configuration figures under \"configs\"")
+    ap.add_argument("--config", default="c2", choices=sorted(OTHER),
                     help="workload: c2 (default) is the configuration the headline metric is "
-                         "quoted on; the others are the remaining benchmark configurations "
-                         "and print a reduced line (no cpu_baseline)")
+                         "quoted on; any other prints a reduced line for that one alone")
     ap.add_argument("--graph", action="store_true",
                     help="capture one step in a HIP graph and time its replays (reduced line, "
                          "for any --config)")
@@ -313,6 +416,15 @@ def main():
     }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(joint.detach(), ys, lx, ly)
+    if not args.no_configs:
+        # every kernel of a headline step, then the other four configurations
+        kernels = profile_kernels(torch, step, 3)
+        configs = {"c2": {"workload": WORKLOAD["c2"], "ms_per_step": ms_per_step,
+                          "kernel_us_per_step": {k: round(v["us_per_step"], 2) for k, v in sorted(
+                              kernels.items(), key=lambda kv: -kv[1]["us_per_step"])}}}
+        for name, steps in (("c1", 50), ("c3", 8), ("c4", 20), ("c5", 20)):
+            configs[name] = measure_config(name, torch, warp_ctct, steps)
+        result["configs"] = configs
     print(json.dumps(result))
 
 

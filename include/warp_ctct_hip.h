@@ -354,6 +354,17 @@ int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, lo
                            float *grad_lhs, long glsb, long glsm, long glsk, float *grad_rhs,
                            long grsb, long grsk, long grsn, void *stream);
 
+/* ---- measurement aid ------------------------------------------------------
+ * No counterpart in the reference.  warpctct_profile(1) clears earlier records
+ * and starts bracketing every kernel launch of the library with two HIP events
+ * on the launch's own stream; warpctct_profile(0) stops.  After the caller has
+ * synchronised, record `index` (0 <= index < warpctct_profile_count(), in
+ * launch order) gives the kernel's name (static storage) and its duration.
+ * Creating events allocates: keep it off in production and under graph capture. */
+int warpctct_profile(int enable);
+int warpctct_profile_count(void);
+int warpctct_profile_read(int index, const char **kernel, float *microseconds);
+
 #ifdef __cplusplus
 }
 #endif

@@ -205,16 +205,16 @@ hipError_t launch_zero_fill_bytes(void *ptr, size_t bytes, hipStream_t stream) {
     const size_t n4 = (bytes - head) / 16;
     const size_t tail = bytes - head - n4 * 16;
     if (head) {
-        hipLaunchKernelGGL(zero_fill_byte_kernel, dim3(1), dim3(kBlock), 0, stream, p, head);
+        TIMED_LAUNCH(zero_fill_byte_kernel, dim3(1), dim3(kBlock), 0, stream, p, head);
     }
     if (n4) {
         const size_t blocks = (n4 + kBlock - 1) / kBlock;
         if (blocks > 0x7fffffffUL) return hipErrorInvalidValue;
-        hipLaunchKernelGGL(zero_fill_vec_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream,
+        TIMED_LAUNCH(zero_fill_vec_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream,
                            reinterpret_cast<v4f *>(p + head), n4);
     }
     if (tail) {
-        hipLaunchKernelGGL(zero_fill_byte_kernel, dim3(1), dim3(kBlock), 0, stream,
+        TIMED_LAUNCH(zero_fill_byte_kernel, dim3(1), dim3(kBlock), 0, stream,
                            p + head + n4 * 16, tail);
     }
     return hipGetLastError();
@@ -231,7 +231,7 @@ hipError_t launch_dense_patch(const float *unit_grads, const int *ys, const int 
     if (cells == 0 || N == 0) return hipSuccess;
     dim3 grid((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N);
     const Weight w = {grad_out, 1, 1.0f, 0};
-    hipLaunchKernelGGL((patch_kernel<false, float>), grid, dim3(kBlock), 0, stream, unit_grads,
+    TIMED_LAUNCH((patch_kernel<false, float>), grid, dim3(kBlock), 0, stream, unit_grads,
                        nullptr, nullptr, nullptr, ys, lx, ly, w, dense, T, U, V, 0);
     return hipGetLastError();
 }
@@ -248,17 +248,17 @@ hipError_t launch_dense_patch_lattice(const double *units, const double *alphas,
     const int P = padded_contexts(U);
     switch (io_type) {
         case kIoF32:
-            hipLaunchKernelGGL((patch_kernel<true, float>), grid, dim3(kBlock), 0, stream, nullptr,
+            TIMED_LAUNCH((patch_kernel<true, float>), grid, dim3(kBlock), 0, stream, nullptr,
                                units, alphas, betas, ys, lx, ly, w, static_cast<float *>(dense), T,
                                U, V, P);
             break;
         case kIoF16:
-            hipLaunchKernelGGL((patch_kernel<true, __half>), grid, dim3(kBlock), 0, stream,
+            TIMED_LAUNCH((patch_kernel<true, __half>), grid, dim3(kBlock), 0, stream,
                                nullptr, units, alphas, betas, ys, lx, ly, w,
                                static_cast<__half *>(dense), T, U, V, P);
             break;
         case kIoBF16:
-            hipLaunchKernelGGL((patch_kernel<true, __hip_bfloat16>), grid, dim3(kBlock), 0, stream,
+            TIMED_LAUNCH((patch_kernel<true, __hip_bfloat16>), grid, dim3(kBlock), 0, stream,
                                nullptr, units, alphas, betas, ys, lx, ly, w,
                                static_cast<__hip_bfloat16 *>(dense), T, U, V, P);
             break;

@@ -339,7 +339,7 @@ __global__ __launch_bounds__(64 * W) void lattice_kernel(const double *__restric
 template <int W>
 hipError_t launch_lattice_w(const LatticeArgs &a, hipStream_t stream) {
     dim3 grid(a.N, a.beta_only ? 1 : 2);
-    hipLaunchKernelGGL((lattice_kernel<W>), grid, dim3(64 * W), 0, stream, a.units, a.ys, a.lx,
+    TIMED_LAUNCH((lattice_kernel<W>), grid, dim3(64 * W), 0, stream, a.units, a.ys, a.lx,
                        a.ly, a.alphas, a.betas, a.costs, a.T, a.U, a.reduce);
     return hipGetLastError();
 }

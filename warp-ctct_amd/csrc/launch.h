@@ -5,6 +5,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include "profile.h"
+
 namespace wctct {
 
 // Work buffers (units, alphas, betas) hold P = padded_contexts(U) contexts per

@@ -293,7 +293,7 @@ void launch_units_typed(const void *logits, const int *ys, const int *lx, const 
     const long cells = (long)T * P;
     constexpr int ROWS = RowsPerWave<IO>::value, PER_BLOCK = kRowsPerBlock * ROWS;
     dim3 grid((unsigned)((cells + PER_BLOCK - 1) / PER_BLOCK), (unsigned)N);
-    hipLaunchKernelGGL((logits_units_kernel<IO, ROWS>), grid, dim3(64 * kRowsPerBlock), 0, stream,
+    TIMED_LAUNCH((logits_units_kernel<IO, ROWS>), grid, dim3(64 * kRowsPerBlock), 0, stream,
                        static_cast<const IO *>(logits), ys, lx, ly, units, lse, T, U, V, P,
                        counter);
 }
@@ -306,7 +306,7 @@ void launch_grad_typed(const void *logits, const float *lse, const double *units
     const long cells = (long)T * (U + 1);
     constexpr int ROWS = RowsPerWave<IO>::value, PER_BLOCK = kGradWaves * ROWS;
     dim3 grid((unsigned)((cells + PER_BLOCK - 1) / PER_BLOCK), (unsigned)N);
-    hipLaunchKernelGGL((logits_grad_kernel<IO, ROWS>), grid, dim3(64 * kGradWaves), 0, stream,
+    TIMED_LAUNCH((logits_grad_kernel<IO, ROWS>), grid, dim3(64 * kGradWaves), 0, stream,
                        static_cast<const IO *>(logits), lse, units, alphas, betas, ys, lx, ly, w,
                        static_cast<IO *>(grad), T, U, V, padded_contexts(U));
 }

@@ -819,7 +819,7 @@ hipError_t launch_bwd(const BwdArgs &args, int B, hipStream_t stream) {
     if (a.Q == 0) {
         const long cells = (long)a.P * a.K;
         if (!fits_int((cells + 255) / 256)) return hipErrorInvalidValue;
-        hipLaunchKernelGGL(logmm_bwd_zero_kernel, dim3((unsigned)((cells + 255) / 256), B),
+        TIMED_LAUNCH(logmm_bwd_zero_kernel, dim3((unsigned)((cells + 255) / 256), B),
                            dim3(256), 0, stream, a);
         return hipGetLastError();
     }
@@ -836,7 +836,7 @@ hipError_t launch_bwd(const BwdArgs &args, int B, hipStream_t stream) {
         const int per = (int)std::min<long>(8, std::max<long>(1, wgs / 2048));
         a.tiles_x = ptiles, a.tiles_y = (ktiles + per - 1) / per;
         if (!xcd_grid_fits(a.tiles_x, a.tiles_y, B)) return hipErrorInvalidValue;
-        hipLaunchKernelGGL(logmm_bwd_resident_kernel, dim3(xcd_grid(a.tiles_x, a.tiles_y, B)),
+        TIMED_LAUNCH(logmm_bwd_resident_kernel, dim3(xcd_grid(a.tiles_x, a.tiles_y, B)),
                            dim3(256), 0, stream, a, per);
         return hipGetLastError();
     }
@@ -849,17 +849,17 @@ hipError_t launch_bwd(const BwdArgs &args, int B, hipStream_t stream) {
     const dim3 grid(xcd_grid(a.tiles_x, a.tiles_y, B));
     if (prefer_96(a.P)) {
         if (short_q)
-            hipLaunchKernelGGL((logmm_bwd_kernel<6, 1, 1, 4, 4, false>), grid, dim3(256), 0,
+            TIMED_LAUNCH((logmm_bwd_kernel<6, 1, 1, 4, 4, false>), grid, dim3(256), 0,
                                stream, a);
         else
-            hipLaunchKernelGGL((logmm_bwd_kernel<6, 1, 1, 4, 3, true>), grid, dim3(256), 0, stream,
+            TIMED_LAUNCH((logmm_bwd_kernel<6, 1, 1, 4, 3, true>), grid, dim3(256), 0, stream,
                                a);
     } else {
         if (short_q)
-            hipLaunchKernelGGL((logmm_bwd_kernel<1, 4, 4, 1, 4, false>), grid, dim3(256), 0,
+            TIMED_LAUNCH((logmm_bwd_kernel<1, 4, 4, 1, 4, false>), grid, dim3(256), 0,
                                stream, a);
         else
-            hipLaunchKernelGGL((logmm_bwd_kernel<1, 4, 4, 1, 3, true>), grid, dim3(256), 0, stream,
+            TIMED_LAUNCH((logmm_bwd_kernel<1, 4, 4, 1, 3, true>), grid, dim3(256), 0, stream,
                                a);
     }
     return hipGetLastError();
@@ -876,19 +876,19 @@ void launch_shift_exp_rows(const float *x, long sb, long sr, long sk, int B, int
     const bool rows_ok = sk == 1 && K >= 4 && (K & 3) == 0 && (sb & 3) == 0 && (sr & 3) == 0 &&
                          (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
     if (rows_ok && K <= 1024) {
-        hipLaunchKernelGGL(shift_exp_rows_kernel<4>, grid, block, 0, stream, x, sb, sr, R, K, Kp,
+        TIMED_LAUNCH(shift_exp_rows_kernel<4>, grid, block, 0, stream, x, sb, sr, R, K, Kp,
                            len, extra, mx, E);
     } else if (rows_ok && K <= 2048) {
-        hipLaunchKernelGGL(shift_exp_rows_kernel<8>, grid, block, 0, stream, x, sb, sr, R, K, Kp,
+        TIMED_LAUNCH(shift_exp_rows_kernel<8>, grid, block, 0, stream, x, sb, sr, R, K, Kp,
                            len, extra, mx, E);
     } else if (rows_ok && K <= 4096) {
-        hipLaunchKernelGGL(shift_exp_rows_kernel<16>, grid, block, 0, stream, x, sb, sr, R, K, Kp,
+        TIMED_LAUNCH(shift_exp_rows_kernel<16>, grid, block, 0, stream, x, sb, sr, R, K, Kp,
                            len, extra, mx, E);
     } else if (rows_ok && K <= 8192) {
-        hipLaunchKernelGGL(shift_exp_rows_kernel<32>, grid, block, 0, stream, x, sb, sr, R, K, Kp,
+        TIMED_LAUNCH(shift_exp_rows_kernel<32>, grid, block, 0, stream, x, sb, sr, R, K, Kp,
                            len, extra, mx, E);
     } else {
-        hipLaunchKernelGGL(shift_exp_kernel, grid, block, 0, stream, x, sb, sr, sk, R, K, Kp, len,
+        TIMED_LAUNCH(shift_exp_kernel, grid, block, 0, stream, x, sb, sr, sk, R, K, Kp, len,
                            extra, mx, E);
     }
 }
@@ -946,13 +946,13 @@ hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
     if (!xcd_grid_fits(a.tiles_x, a.tiles_y, B)) return hipErrorInvalidValue;
     const dim3 grid(xcd_grid(a.tiles_x, a.tiles_y, B));
     if (prefer_96(Nn))
-        hipLaunchKernelGGL((logmm_fwd_kernel<1, 3, 2, 2>), grid, dim3(256), 0, stream, a);
+        TIMED_LAUNCH((logmm_fwd_kernel<1, 3, 2, 2>), grid, dim3(256), 0, stream, a);
     else
-        hipLaunchKernelGGL((logmm_fwd_kernel<1, 2, 2, 2>), grid, dim3(256), 0, stream, a);
+        TIMED_LAUNCH((logmm_fwd_kernel<1, 2, 2, 2>), grid, dim3(256), 0, stream, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || a.splits == 1) return e;
     const long outs = (long)M * Nn;
-    hipLaunchKernelGGL(logmm_fwd_finish_kernel, dim3((unsigned)((outs + 255) / 256), B), dim3(256),
+    TIMED_LAUNCH(logmm_fwd_finish_kernel, dim3((unsigned)((outs + 255) / 256), B), dim3(256),
                        0, stream, a, B);
     return hipGetLastError();
 }
@@ -962,7 +962,7 @@ hipError_t launch_logmm_pair_factor(const float *go, const float *res, const flo
                                     const int *row_len, const int *col_len, float *C, int *flags,
                                     int B, int M, int Nn, hipStream_t stream) {
     if (B == 0 || M == 0) return hipSuccess;
-    hipLaunchKernelGGL(logmm_pair_factor_kernel, dim3((M + 3) / 4, B), dim3(256), 0, stream, go,
+    TIMED_LAUNCH(logmm_pair_factor_kernel, dim3((M + 3) / 4, B), dim3(256), 0, stream, go,
                        res, lmax, rmax, batch_scale, row_len, col_len, C, flags, M, Nn);
     return hipGetLastError();
 }

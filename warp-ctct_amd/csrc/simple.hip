@@ -313,7 +313,7 @@ hipError_t launch_simple_gather_units(const float *f, const float *g, const floa
                                       int N, int T, int U, int V, hipStream_t stream) {
     const int P = padded_contexts(U);
     const long cells = (long)T * P;
-    hipLaunchKernelGGL(simple_gather_units_kernel,
+    TIMED_LAUNCH(simple_gather_units_kernel,
                        dim3((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N), dim3(kBlock),
                        0, stream, f, g, den, ys, lx, ly, units, T, U, V, P);
     return hipGetLastError();
@@ -326,23 +326,23 @@ hipError_t launch_simple_grads(const double *units, const int *ys, const int *lx
     const int P = padded_contexts(U);
     const int blocks = (T + kFramesPerBlock - 1) / kFramesPerBlock;
     if (T > 0) {
-        hipLaunchKernelGGL(simple_grads_kernel, dim3(blocks, N), dim3(P), 0, stream, units, ys, lx,
+        TIMED_LAUNCH(simple_grads_kernel, dim3(blocks, N), dim3(P), 0, stream, units, ys, lx,
                            ly, alphas, betas, grad_f, grad_den, partial, T, U, P);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL(simple_sum_partials_kernel, dim3((U + 1 + 3) / 4, N), dim3(kBlock), 0,
+    TIMED_LAUNCH(simple_sum_partials_kernel, dim3((U + 1 + 3) / 4, N), dim3(kBlock), 0,
                        stream, partial, grad_g, blocks, U + 1);
     return hipGetLastError();
 }
 
 hipError_t launch_simple_reduce(const float *unit_grads, float *grad_f, float *grad_g,
                                 float *grad_den, int N, int T, int U, hipStream_t stream) {
-    hipLaunchKernelGGL(simple_reduce_frames_kernel, dim3((T + 3) / 4, N), dim3(kBlock), 0, stream,
+    TIMED_LAUNCH(simple_reduce_frames_kernel, dim3((T + 3) / 4, N), dim3(kBlock), 0, stream,
                        unit_grads, grad_f, grad_den, T, U);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(simple_reduce_contexts_kernel, dim3((U + 1 + 3) / 4, N), dim3(kBlock), 0,
+    TIMED_LAUNCH(simple_reduce_contexts_kernel, dim3((U + 1 + 3) / 4, N), dim3(kBlock), 0,
                        stream, unit_grads, grad_g, T, U);
     return hipGetLastError();
 }
@@ -353,7 +353,7 @@ hipError_t launch_simple_dense_f_rows(const float *grad_f, const int *ys, const 
                                       const int *ly, const float *grad_out, float *dense_f, int N,
                                       int T, int U, int V, hipStream_t stream) {
     if (N == 0 || T == 0) return hipSuccess;
-    hipLaunchKernelGGL(simple_dense_f_rows_kernel, dim3(T, N), dim3(kBlock),
+    TIMED_LAUNCH(simple_dense_f_rows_kernel, dim3(T, N), dim3(kBlock),
                        (size_t)V * sizeof(float), stream, grad_f, ys, lx, ly, grad_out, dense_f, T,
                        U, V);
     return hipGetLastError();
@@ -364,13 +364,13 @@ hipError_t launch_simple_scatter(const float *grad_f, const float *grad_g, const
                                  float *dense_f, float *dense_g, int N, int T, int U, int V,
                                  hipStream_t stream) {
     if (dense_f) {
-        hipLaunchKernelGGL(simple_scatter_f_kernel, cell_grid(N, T, U), dim3(kBlock), 0, stream,
+        TIMED_LAUNCH(simple_scatter_f_kernel, cell_grid(N, T, U), dim3(kBlock), 0, stream,
                            grad_f, ys, lx, ly, grad_out, dense_f, T, U, V);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
     if (dense_g) {
-        hipLaunchKernelGGL(simple_scatter_g_kernel, dim3(((U + 1) * 3 + kBlock - 1) / kBlock, N),
+        TIMED_LAUNCH(simple_scatter_g_kernel, dim3(((U + 1) * 3 + kBlock - 1) / kBlock, N),
                            dim3(kBlock), 0, stream, grad_g, ys, ly, grad_out, dense_g, U, V);
         return hipGetLastError();
     }

@@ -157,10 +157,10 @@ void launch_gather_typed(const void *joint, const JointStrides &js, const int *y
     const int P = padded_contexts(U);
     const IO *j = static_cast<const IO *>(joint);
     if (band_only) {
-        hipLaunchKernelGGL((gather_units_kernel<true, IO>), cell_grid(N, T, P), dim3(kCellBlock),
+        TIMED_LAUNCH((gather_units_kernel<true, IO>), cell_grid(N, T, P), dim3(kCellBlock),
                            0, stream, j, js, ys, lx, ly, units, T, U, V, P, counter);
     } else {
-        hipLaunchKernelGGL((gather_units_kernel<false, IO>), cell_grid(N, T, P), dim3(kCellBlock),
+        TIMED_LAUNCH((gather_units_kernel<false, IO>), cell_grid(N, T, P), dim3(kCellBlock),
                            0, stream, j, js, ys, lx, ly, units, T, U, V, P, counter);
     }
 }
@@ -191,14 +191,14 @@ hipError_t launch_gather_units(const void *joint, const JointStrides &js, int io
 }
 
 hipError_t launch_clear_counter(unsigned *counter, hipStream_t stream) {
-    hipLaunchKernelGGL(clear_counter_kernel, dim3(1), dim3(1), 0, stream, counter);
+    TIMED_LAUNCH(clear_counter_kernel, dim3(1), dim3(1), 0, stream, counter);
     return hipGetLastError();
 }
 
 hipError_t launch_scale_units(const float *units_nat, const int *lx, const int *ly, double *units,
                               int N, int T, int U, hipStream_t stream) {
     const int P = padded_contexts(U);
-    hipLaunchKernelGGL(scale_units_kernel, cell_grid(N, T, P), dim3(kCellBlock), 0, stream,
+    TIMED_LAUNCH(scale_units_kernel, cell_grid(N, T, P), dim3(kCellBlock), 0, stream,
                        units_nat, lx, ly, units, T, U, P);
     return hipGetLastError();
 }
@@ -207,7 +207,7 @@ hipError_t launch_simple_units(const float *f_g, const float *g_g, const float *
                                const int *lx, const int *ly, double *units, int N, int T, int U,
                                hipStream_t stream) {
     const int P = padded_contexts(U);
-    hipLaunchKernelGGL(simple_units_kernel, cell_grid(N, T, P), dim3(kCellBlock), 0, stream, f_g,
+    TIMED_LAUNCH(simple_units_kernel, cell_grid(N, T, P), dim3(kCellBlock), 0, stream, f_g,
                        g_g, den, lx, ly, units, T, U, P);
     return hipGetLastError();
 }
@@ -215,7 +215,7 @@ hipError_t launch_simple_units(const float *f_g, const float *g_g, const float *
 hipError_t launch_unit_grads(const double *units, const int *ys, const int *lx, const int *ly,
                              const double *alphas, const double *betas, float *unit_grads, int N,
                              int T, int U, hipStream_t stream) {
-    hipLaunchKernelGGL(unit_grads_kernel, cell_grid(N, T, U + 1), dim3(kCellBlock), 0, stream,
+    TIMED_LAUNCH(unit_grads_kernel, cell_grid(N, T, U + 1), dim3(kCellBlock), 0, stream,
                        units, ys, lx, ly, alphas, betas, unit_grads, T, U, padded_contexts(U));
     return hipGetLastError();
 }
