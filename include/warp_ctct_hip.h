@@ -31,7 +31,8 @@ extern "C" {
 
 enum {
     WARPCTCT_OK = 0,
-    WARPCTCT_EINVAL = 1,     /* null pointer, negative size, size limit exceeded */
+    WARPCTCT_EINVAL = 1,     /* null pointer, negative size, or beyond N <= 65535,
+                                T * (U+1 rounded up to 64) < 2^31 */
     WARPCTCT_ELAUNCH = 2,    /* hipGetLastError() reported a failed launch */
     WARPCTCT_EWORKSPACE = 3, /* workspace smaller than warpctct_workspace_bytes() */
     WARPCTCT_ENODEVICE = 4,  /* no usable HIP device */
@@ -49,7 +50,8 @@ const char *warpctct_version(void);
 int warpctct_padded_contexts(int U);
 
 /* Bytes of device workspace the two *_forward orchestrators need
- * (units, alpha and beta lattices, all double).  Replaces the
+ * (units, alpha and beta lattices, all double, and the relay slots of
+ * lattices wider than 64 contexts).  Replaces the
  * allocations of csrc/binding.cpp:70-77 (alphas, betas, counts); needs no
  * host sync because it does not depend on max(lx-ly) (binding.cpp:68). */
 size_t warpctct_workspace_bytes(int N, int T, int U);
@@ -79,15 +81,23 @@ int warpctct_simple_units_f32(const float *f_g, const float *g_g, const float *d
                               int N, int T, int U, void *stream);
 
 /* Alpha and beta lattices of all N samples, concurrently, one wavefront per
- * (sample, direction).  Replaces run_warp_ctct (csrc/core.h:14-16,
+ * (sample, direction, 64 contexts).  Replaces run_warp_ctct (csrc/core.h:14-16,
  * csrc/gather.cu:293-309: k_warp_alphas + k_warp_betas).
  * units (N,T,P,3) f64 log2 domain; alphas, betas (N,T+1,P,2) f64 =
- * {state 2u-1, state 2u} (only t<=lx[n] is written); costs (N) f32
+ * {state 2u-1, state 2u} (only t<=lx[n], and only the 64-context blocks that
+ * hold a context u<=ly[n], are written); costs (N) f32
  * = -beta(0,0) in natural-log units (csrc/binding.cpp:86).
- * beta_only != 0 skips alpha (alphas may be NULL), as binding.cpp:84. */
+ * beta_only != 0 skips alpha (alphas may be NULL), as binding.cpp:84.
+ * relay: warpctct_lattice_relay_bytes(N,T,U) bytes of scratch, 8-byte aligned,
+ * through which the wavefronts of a lattice of more than 64 contexts hand
+ * over their boundary values (0 bytes, relay may be NULL, for U+1 <= 64; it
+ * replaces the `counts` spin-lock array of csrc/binding.cpp:77).  Should a
+ * hand-over ever not arrive within its (long) bounded wait, the cost and the
+ * lattices of that sample are NaN. */
+size_t warpctct_lattice_relay_bytes(int N, int T, int U);
 int warpctct_lattice_f32(const double *units, const int *ys, const int *lx, const int *ly,
                          double *alphas, double *betas, float *costs, int N, int T, int U,
-                         int beta_only, void *stream);
+                         int beta_only, void *relay, size_t relay_bytes, void *stream);
 
 /* d(cost)/d(unit) for every cell, natural-log units, zero outside
  * t<lx[n], u<=ly[n].  Replaces run_fill_grad + the zeros_like before it

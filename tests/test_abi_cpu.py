@@ -31,6 +31,11 @@ def test_workspace_size_is_monotone_and_covers_buffers():
     assert P == 64 and lib.warpctct_padded_contexts(64) == 128 and lib.warpctct_padded_contexts(0) == 64
     floor = 8 * N * T * P * 3 + 2 * 8 * N * (T + 1) * P * 2
     assert need >= floor and need < floor + 3 * 256
+    # wider than one wavefront: the relay slots are part of the workspace
+    lib.warpctct_lattice_relay_bytes.restype = ctypes.c_size_t
+    wide = lib.warpctct_workspace_bytes(N, T, 100)
+    floor = 8 * N * T * 128 * 3 + 2 * 8 * N * (T + 1) * 128 * 2 + lib.warpctct_lattice_relay_bytes(N, T, 100)
+    assert wide >= floor and wide < floor + 4 * 256
     assert lib.warpctct_workspace_bytes(N, T + 1, U) > need
     assert lib.warpctct_workspace_bytes(-1, T, U) == 0
 
@@ -43,10 +48,20 @@ def test_invalid_arguments_are_rejected_on_the_host():
     assert lib.warpctct_gather_units_f32(null, null, null, null, null, -1, 4, 2, 8, null) == EINVAL
     assert lib.warpctct_gather_units_f32(null, null, null, null, null, 2, 4, 2, 8, null) == EINVAL
     assert lib.warpctct_dense_grad_f32(null, null, null, null, null, null, 2, 4, 2, 8, null) == EINVAL
-    # more contexts than a wavefront can hold
     buf = (ctypes.c_float * 16)()
     p = ctypes.cast(buf, ctypes.c_void_p)
-    assert lib.warpctct_lattice_f32(p, p, p, p, p, p, p, 1, 1, 512, 0, null) == EINVAL
+    lib.warpctct_lattice_relay_bytes.restype = ctypes.c_size_t
+    # a lattice of more than 64 contexts needs relay scratch: missing or too small is refused
+    assert lib.warpctct_lattice_relay_bytes(3, 10, 63) == 0
+    need = lib.warpctct_lattice_relay_bytes(3, 10, 64)
+    assert need >= 3 * 2 * 1 * 10 * 8 and lib.warpctct_lattice_relay_bytes(3, 10, 300) == 4 * need
+    assert lib.warpctct_lattice_f32(p, p, p, p, p, p, p, 3, 10, 64, 0, null, ctypes.c_size_t(0),
+                                    null) == EINVAL
+    assert lib.warpctct_lattice_f32(p, p, p, p, p, p, p, 3, 10, 64, 0, p, ctypes.c_size_t(need - 8),
+                                    null) == EWORKSPACE
+    # sizes whose cell count does not fit 31 bits
+    assert lib.warpctct_lattice_f32(p, p, p, p, p, p, p, 1, 1 << 26, 63, 0, null,
+                                    ctypes.c_size_t(0), null) == EINVAL
     assert lib.warpctct_loss_forward_f32(p, p, p, p, 1, 1, 1, 8, p, ctypes.c_size_t(16), p, p,
                                          null) == EWORKSPACE
     # empty batch is a no-op

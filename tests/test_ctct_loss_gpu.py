@@ -59,9 +59,13 @@ def run_stages(joint, ys, lx, ly, beta_only=False):
     p = hip_lib.ptr
     hip_lib.check(lib.warpctct_gather_units_f32(p(d_joint), p(d_ys), p(d_lx), p(d_ly), p(units),
                                                 N, T, U, V, s))
+    lib.warpctct_lattice_relay_bytes.restype = ctypes.c_size_t
+    relay_bytes = lib.warpctct_lattice_relay_bytes(N, T, U)
+    relay = torch.empty(max(relay_bytes, 8), dtype=torch.uint8, device="cuda")
     hip_lib.check(lib.warpctct_lattice_f32(p(units), p(d_ys), p(d_lx), p(d_ly),
                                            p(None if beta_only else alphas), p(betas), p(costs),
-                                           N, T, U, int(beta_only), s))
+                                           N, T, U, int(beta_only), p(relay),
+                                           ctypes.c_size_t(relay_bytes), s))
     if not beta_only:
         hip_lib.check(lib.warpctct_unit_grads_f32(p(units), p(d_ys), p(d_lx), p(d_ly), p(alphas),
                                                   p(betas), p(ug), N, T, U, s))
@@ -454,16 +458,19 @@ def test_edge_shapes_no_labels_single_frame_and_empty_batch():
     assert torch.isnan(warp_ctct.ctct_loss(e, ei, el, el, reduction="mean"))
 
 
-def test_widest_lattice_eight_wavefronts():
-    """U + 1 = 512 contexts: eight wavefronts per lattice and direction, the
-    largest the kernel accepts; one more context is refused."""
+@pytest.mark.parametrize("contexts", [512, 1024])
+def test_wide_lattices_chains_of_many_wavefronts(contexts):
+    """U + 1 = 512 and 1024 contexts: chains of 8 and 16 wavefronts per lattice
+    and direction (the reference sets no limit on U: its grid is
+    (sT/32, 2U+1, N), csrc/gather.cu:293-297).  One sample fills the lattice,
+    the other is short, so most links of its chains hold only padding."""
     import warp_ctct
-    T, U, V = 530, 511, 6
-    joint, ys, lx, ly = make_joint_case(63, 1, T, U, V, lx=[T], ly=[U], force_repeat=False,
+    U, V = contexts - 1, 6
+    T = contexts + 20
+    joint, ys, lx, ly = make_joint_case(63, 2, T, U, V, lx=[T, 90], ly=[U, 70], force_repeat=False,
                                         zero_pad=False)
-    ys[0] = 1 + np.arange(U) % (V - 1)        # no adjacent repeats: all 511 labels fit
+    ys[:] = 1 + np.arange(U) % (V - 1)        # no adjacent repeats: all labels fit
     ys[0, 300] = ys[0, 299]                   # but one, in the fifth wavefront
-    ly[0] = U
     _, ref_dense, ref_costs = O.ctct_loss(joint, ys, lx, ly, reduction="sum")
     x = dev(joint).requires_grad_(True)
     c = warp_ctct.ctct_loss(x, dev(ys), dev(lx), dev(ly), reduction="none")
@@ -471,11 +478,31 @@ def test_widest_lattice_eight_wavefronts():
     c.sum().backward()
     got = x.grad.cpu().numpy()
     np.testing.assert_allclose(got, ref_dense, atol=GRAD_ATOL, rtol=0)
-    assert_support(got, ref_dense, "dense gradient, 8 wavefronts")
-    too_wide = torch.zeros(1, 4, 514, 3, device="cuda")
-    with pytest.raises(RuntimeError):
-        warp_ctct.ctct_loss(too_wide, torch.ones(1, 513, dtype=torch.int32, device="cuda"),
-                            torch.tensor([4], device="cuda"), torch.tensor([2], device="cuda"))
+    assert_support(got, ref_dense, "dense gradient, %d contexts" % contexts)
+
+
+def test_wide_lattice_log_add_joiner_beyond_512_contexts():
+    """ctct_simple_loss with 600 contexts: the compact gradients of the joiner
+    path are reduced from the unit-gradient tensor instead of inside one
+    workgroup per frame block."""
+    import warp_ctct
+    from ctct_cases import make_simple_case
+    N, T, U, V = 2, 640, 599, 9
+    f, g, ys, lx, ly = make_simple_case(64, N, T, U, V, lx=[640, 200], ly=[599, 130], normalized=False)
+    ys[:] = 1 + np.arange(U) % (V - 1)
+    for normalized in (False, True):
+        if normalized:
+            from ctct_cases import log_softmax
+            f, g = log_softmax(f).astype(np.float32), log_softmax(g).astype(np.float32)
+        loss, gf, gg, costs = O.ctct_simple_loss(f, g, ys, lx, ly, reduction="none",
+                                                 normalized=normalized, grad_output=np.ones(N))
+        tf, tg = dev(f).requires_grad_(True), dev(g).requires_grad_(True)
+        out = warp_ctct.ctct_simple_loss(tf, tg, dev(ys), dev(lx), dev(ly), reduction="none",
+                                         normalized=normalized)
+        np.testing.assert_allclose(out.detach().cpu().numpy(), costs, rtol=LOSS_RTOL)
+        out.sum().backward()
+        np.testing.assert_allclose(tf.grad.cpu().numpy(), gf, atol=GRAD_ATOL, rtol=1e-5)
+        np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
 
 
 def test_forward_and_backward_replay_from_a_hip_graph():

@@ -235,8 +235,12 @@ def test_log_add_joiner_stages(case):
         betas = nan_like(N, T + 1, P, 2, dtype=torch.float64)
         costs = nan_like(N)
         ug = nan_like(N, T, U1, 3)
+        lib.warpctct_lattice_relay_bytes.restype = ctypes.c_size_t
+        relay_bytes = lib.warpctct_lattice_relay_bytes(N, T, U)
+        relay = torch.empty(max(relay_bytes, 8), dtype=torch.uint8, device="cuda")
         hip_lib.check(lib.warpctct_lattice_f32(p(units), p(d_ys), p(d_lx), p(d_ly), p(alphas),
-                                               p(betas), p(costs), N, T, U, 0, s))
+                                               p(betas), p(costs), N, T, U, 0, p(relay),
+                                               ctypes.c_size_t(relay_bytes), s))
         hip_lib.check(lib.warpctct_unit_grads_f32(p(units), p(d_ys), p(d_lx), p(d_ly), p(alphas),
                                                   p(betas), p(ug), N, T, U, s))
         torch.cuda.synchronize()

@@ -28,9 +28,12 @@ inline int done(hipError_t e) {
     return e == hipErrorInvalidValue ? WARPCTCT_EINVAL : WARPCTCT_ELAUNCH;
 }
 
+// N is a grid dimension; cells of one sample are counted in 32 bits.  (The
+// reference has no limit of its own: its grid is (sT/32, 2U+1, N),
+// csrc/gather.cu:293-297, i.e. 2U+1 <= 65535 and N <= 65535 in practice.)
 inline bool dims_ok(int N, int T, int U) {
-    return N >= 0 && T >= 0 && U >= 0 && N <= kMaxGrid && T <= kMaxGrid &&
-           (U + 1) <= lattice_max_contexts() && (long)T * padded_contexts(U) < (1L << 31);
+    return N >= 0 && T >= 0 && U >= 0 && N <= kMaxGrid && U < (1 << 24) &&
+           (long)T * padded_contexts(U) < (1L << 31);
 }
 
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -39,6 +42,7 @@ struct Workspace {
     double *units;    // (N,T,P,3),   P = padded_contexts(U)
     double *alphas;   // (N,T+1,P,2)
     double *betas;    // (N,T+1,P,2)
+    void *relay;      // lattice_relay_slots(N,T,U) 64-bit words (none for U+1 <= 64)
     unsigned *counter;   // arrivals of the batch reduction (see CostReduce)
     size_t bytes;
 };
@@ -52,8 +56,10 @@ Workspace carve(void *base, int N, int T, int U) {
     w.units = reinterpret_cast<double *>(p);
     w.alphas = reinterpret_cast<double *>(p + units_b);
     w.betas = reinterpret_cast<double *>(p + units_b + lat_b);
-    w.counter = reinterpret_cast<unsigned *>(p + units_b + 2 * lat_b);
-    w.bytes = units_b + 2 * lat_b + 256;
+    const size_t relay_b = align256(lattice_relay_slots(N, T, U) * sizeof(unsigned long long));
+    w.relay = relay_b ? reinterpret_cast<void *>(p + units_b + 2 * lat_b) : nullptr;
+    w.counter = reinterpret_cast<unsigned *>(p + units_b + 2 * lat_b + relay_b);
+    w.bytes = units_b + 2 * lat_b + relay_b + 256;
     return w;
 }
 
@@ -66,6 +72,7 @@ int forward_from_units(const Workspace &w, const int *ys, const int *lx, const i
     a.ly = ly;
     a.alphas = w.alphas;
     a.betas = w.betas;
+    a.relay = w.relay;
     a.costs = costs;
     a.N = N;
     a.T = T;
@@ -174,6 +181,7 @@ int simple_from_units(const SimpleWorkspace &w, const int *ys, const int *lx, co
     a.ly = ly;
     a.alphas = w.lattice.alphas;
     a.betas = w.lattice.betas;
+    a.relay = w.lattice.relay;
     a.costs = costs;
     a.N = N;
     a.T = T;
@@ -193,8 +201,8 @@ const char *warpctct_error_string(int code) {
     switch (code) {
         case WARPCTCT_OK: return "ok";
         case WARPCTCT_EINVAL:
-            return "invalid argument (null pointer, negative size, or size limit: N,T <= 65535, "
-                   "U+1 <= 512)";
+            return "invalid argument (null pointer, negative size, or size limit: N <= 65535, "
+                   "T * (U+1 rounded up to 64) < 2^31)";
         case WARPCTCT_ELAUNCH: return "kernel launch failed";
         case WARPCTCT_EWORKSPACE: return "workspace too small";
         case WARPCTCT_ENODEVICE: return "no usable HIP device";
@@ -240,14 +248,23 @@ int warpctct_simple_units_f32(const float *f_g, const float *g_g, const float *d
     return done(launch_simple_units(f_g, g_g, den, lx, ly, units_out, N, T, U, as_stream(stream)));
 }
 
+size_t warpctct_lattice_relay_bytes(int N, int T, int U) {
+    if (N < 0 || T < 0 || U < 0) return 0;
+    return lattice_relay_slots(N, T, U) * sizeof(unsigned long long);
+}
+
 int warpctct_lattice_f32(const double *units, const int *ys, const int *lx, const int *ly,
                          double *alphas, double *betas, float *costs, int N, int T, int U,
-                         int beta_only, void *stream) {
+                         int beta_only, void *relay, size_t relay_bytes, void *stream) {
     if (!dims_ok(N, T, U)) return WARPCTCT_EINVAL;
     if (N == 0) return WARPCTCT_OK;
     if (!lx || !ly || !betas || !costs || (T > 0 && !units) || (U > 0 && !ys))
         return WARPCTCT_EINVAL;
     if (!beta_only && !alphas) return WARPCTCT_EINVAL;
+    const size_t relay_need = warpctct_lattice_relay_bytes(N, T, U);
+    if (relay_need > 0 && !relay) return WARPCTCT_EINVAL;
+    if (relay_bytes < relay_need) return WARPCTCT_EWORKSPACE;
+    if (relay_need > 0 && (reinterpret_cast<uintptr_t>(relay) & 7u)) return WARPCTCT_EINVAL;
     LatticeArgs a = {};
     a.units = units;
     a.ys = ys;
@@ -255,6 +272,7 @@ int warpctct_lattice_f32(const double *units, const int *ys, const int *lx, cons
     a.ly = ly;
     a.alphas = alphas;
     a.betas = betas;
+    a.relay = relay_need > 0 ? relay : nullptr;
     a.costs = costs;
     a.N = N;
     a.T = T;
@@ -337,6 +355,7 @@ int warpctct_loss_lattice_strided(const void *joint, int dtype, const long *stri
     a.ly = ly;
     a.alphas = w.alphas;
     a.betas = w.betas;
+    a.relay = w.relay;
     a.costs = costs;
     a.N = N;
     a.T = T;
@@ -459,6 +478,7 @@ int warpctct_logits_loss_lattice(const void *logits, int dtype, const int *ys, c
     a.ly = ly;
     a.alphas = w.lattice.alphas;
     a.betas = w.lattice.betas;
+    a.relay = w.lattice.relay;
     a.costs = costs;
     a.N = N;
     a.T = T;

@@ -5,13 +5,27 @@
 // so a step needs no barrier and no atomics — only one value from the
 // neighbouring context.  Every lane owns one context u and its state pair
 //     o = state 2u-1 (inside label y[u-1])      e = state 2u (blank after u labels)
-// in registers.  A lattice with up to 64 contexts is one wavefront; the value
-// of the neighbouring context moves with single-lane DPP shifts.  A wider
-// lattice (up to 512 contexts) is W = ceil((U+1)/64) wavefronts of one
-// workgroup, each sweeping its own 64 contexts: the one value that crosses a
-// wavefront boundary per step goes through a small LDS ring, published and
-// consumed a chunk of R frames at a time, so the wavefronts run skewed by one
-// chunk instead of meeting at a barrier every frame.
+// in registers; the value of the neighbouring context moves with single-lane
+// DPP shifts.
+//
+// One wavefront sweeps 64 contexts and is a workgroup of its own.  A lattice
+// with more contexts is a chain of W = ceil((U+1)/64) such workgroups, each on
+// its own compute unit (a compute unit's vector-memory path serves ~64 bytes
+// per clock: five wavefronts of one lattice sharing it ran at 178 ns per frame
+// against 92 ns for one alone).  The one value that crosses a 64-context
+// boundary per frame is handed from workgroup to workgroup through a slot in
+// device memory, one slot per (boundary, frame): the producer stores the value
+// itself, the consumer polls the slot until it no longer holds the "empty"
+// pattern.  Value and "it is there" are one 64-bit word, so the hand-over needs
+// no fences and no counters.  A consumer runs one chunk of R frames behind its
+// producer and asks for the next chunk's slots while it sweeps the current one.
+// Workgroups are ordered so that a producer always has a lower index than its
+// consumer (workgroups are dispatched in index order: a waiting consumer's
+// producer is running or done), and all links of a chain share `index % 8`,
+// i.e. the XCD and its L2, under round-robin dispatch.
+// A wait is bounded; a consumer that gives up keeps the empty pattern, which
+// is a NaN: the cost and every gradient of that lattice come out as NaN
+// instead of a plausible number.
 //
 // Values are log2 of the path mass, held in double; the exponentials and
 // logarithms of the semiring sum run on the fp32 transcendental unit (see
@@ -29,8 +43,11 @@ namespace wctct {
 namespace {
 
 constexpr int R = 8;          // frames per chunk (prefetch depth and hand-over granularity)
-constexpr int kRing = 4 * R;  // ring slots per wavefront boundary
-constexpr int kMaxSpins = 1 << 22;
+constexpr int kMaxSpins = 1 << 20;   // ~1 s of polling before a hand-over is given up
+
+// What a relay slot holds before its value has been stored: a NaN with a
+// payload that no arithmetic produces.
+constexpr unsigned long long kEmptyBits = 0x7ff8dead5107e117ULL;
 
 struct Front {
     double e, o;
@@ -66,65 +83,39 @@ __device__ __forceinline__ void chunk_load(Chunk &c, const double *units_lane, s
     }
 }
 
-// ---- hand-over between the wavefronts of one lattice -------------------------
-// Boundary b sits between wavefront b and b+1.  done[b] counts the steps whose
-// value the producer has put into ring[b]; taken[b] counts the steps the
-// consumer has read.  Both only grow; a wavefront spins (with a bound, so that
-// no input can hang the GPU) until the counter it needs has advanced.
-// The fences name the LDS address space only: a plain workgroup-scope fence
-// would also wait for the global-memory prefetch in flight, which is exactly
-// what the chunked sweep must not do.
-template <int W>
-struct Relay {
-    double ring[W > 1 ? W - 1 : 1][kRing];
-    int done[W > 1 ? W - 1 : 1];
-    int taken[W > 1 ? W - 1 : 1];
-};
-
-// Returns the value seen (>= target unless the spin bound was hit).
-__device__ __forceinline__ int wait_until(int *counter, int target) {
-    int seen = 0;
-    for (int spins = 0; spins < kMaxSpins; ++spins) {
-        seen = __builtin_amdgcn_readfirstlane(
-            __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP));
-        if (seen >= target) break;
-        __builtin_amdgcn_s_sleep(1);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-    return seen;
+// ---- hand-over between the workgroups of one lattice -------------------------
+// slots[s] belongs to step s of the sweep (s < Tn <= T); a boundary has
+// T + R of them.  Relaxed atomics at agent scope: the store goes to the L2,
+// the load comes from there.
+__device__ __forceinline__ void slot_put(unsigned long long *slot, double v) {
+    __hip_atomic_store(slot, (unsigned long long)__double_as_longlong(v), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Consumer side of a hand-over: the counter and the R ring slots of a chunk
-// are requested in one batch (LDS serves a wavefront's requests in order, so
-// slots read after a counter that already shows the chunk are the chunk's
-// values).  peek() only issues the requests and returns the counter as read;
-// nothing waits for them until the values are used, so a peek at the chunk
-// after the current one costs the sweep no LDS round trip when the producer is
-// already that far.
-__device__ __forceinline__ int peek(int *counter, const double *ring, int s0, double (&mail)[R]) {
-    const int seen = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    __atomic_signal_fence(__ATOMIC_SEQ_CST);   // the compiler keeps the order of the requests
+// Requests the slots of steps s0 .. s0+R-1 (a boundary has T + R slots, so a
+// request that starts at any step s0 <= T stays inside; what lies beyond the
+// chunk's cnt steps is not looked at).  Nothing waits for the loads until the
+// values are used.
+__device__ __forceinline__ void slots_request(const unsigned long long *slots, int s0,
+                                              unsigned long long (&bits)[R]) {
+    const unsigned long long *p = slots + s0;
 #pragma unroll
     for (int r = 0; r < R; ++r)
-        mail[r] = __hip_atomic_load(ring + (s0 + r) % kRing, __ATOMIC_RELAXED,
-                                    __HIP_MEMORY_SCOPE_WORKGROUP);
-    return seen;
+        bits[r] = __hip_atomic_load(p + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Repeats the batch until the counter shows the chunk (with a bound).
-__device__ __forceinline__ void wait_and_take(int *counter, int target, const double *ring,
-                                              int s0, double (&mail)[R]) {
-    for (int spins = 0; spins < kMaxSpins; ++spins) {
-        const int seen = peek(counter, ring, s0, mail);
-        if (__builtin_amdgcn_readfirstlane(seen) >= target) break;
-        __builtin_amdgcn_s_sleep(1);
+// All of the chunk's cnt slots hold a value: no high word is the empty
+// pattern's (no value has that high word: it is a NaN payload no arithmetic
+// produces).  The smallest of (high word xor pattern) is zero iff one is empty.
+__device__ __forceinline__ bool slots_ready(const unsigned long long (&bits)[R], int cnt) {
+    constexpr unsigned kEmptyHigh = (unsigned)(kEmptyBits >> 32);
+    unsigned least = 0xffffffffu;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const unsigned d = (unsigned)(bits[r] >> 32) ^ kEmptyHigh;
+        least = min(least, r < cnt ? d : 0xffffffffu);
     }
-}
-
-__device__ __forceinline__ void publish(int *counter, int value) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    if ((threadIdx.x & 63) == 0)
-        __hip_atomic_store(counter, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    return __builtin_amdgcn_readfirstlane((int)least) != 0;   // the same for all lanes
 }
 
 // ---- alpha ---------------------------------------------------------------
@@ -138,7 +129,7 @@ __device__ __forceinline__ void publish(int *counter, int value) {
 // one semiring sum and one value to pass instead of two of each.
 // skip_next: the skip arc from this context's label state into the next
 // context exists (y[u] != y[u-1]).  ext = what lane 0 receives (from the
-// previous wavefront, or -inf); out = what this lane sends to context u+1.
+// previous 64 contexts, or -inf); out = what this lane sends to context u+1.
 __device__ __forceinline__ void alpha_step(Front &f, const double *lp, bool skip_next, double ext,
                                            double &out) {
     const double both = lse2(f.e, f.o);
@@ -157,8 +148,8 @@ __device__ __forceinline__ void alpha_step(Front &f, const double *lp, bool skip
 // arc exists and its first term alone when it does not.
 // skip: y[u-1] != y[u] with 1 <= u < Un.  o_mask is 0 for contexts that have a
 // state 2u-1 (1 <= u <= Un), else -inf.  ext = beta(t+1, 2u+1) for lane 63
-// (from the next wavefront, or -inf); out = this lane's beta(t+1, 2u-1), which
-// context u-1 needs.
+// (from the next 64 contexts, or -inf); out = this lane's beta(t+1, 2u-1),
+// which context u-1 needs.
 __device__ __forceinline__ void beta_step(Front &f, const double *lp, bool skip, double o_mask,
                                           double ext, double &out) {
     out = f.o;
@@ -171,15 +162,17 @@ __device__ __forceinline__ void beta_step(Front &f, const double *lp, bool skip,
     f.o = no + o_mask;
 }
 
-// One direction of one lattice, swept by the W wavefronts of this workgroup.
+// One direction of the 64 contexts [64*wave, 64*wave + 64) of one lattice.
 // BETA selects the direction; step s handles frame t = s (alpha) or Tn-1-s
 // (beta) and stores the front of frame t+1 (alpha) or t (beta).
-template <int W, bool BETA>
-__device__ void sweep(const double *units_n, const int *y, int Tn, int Un, double *lat_n,
-                      float *cost_n, Relay<W> &relay) {
-    constexpr int P = 64 * W;
+// slots_in / slots_out: the T relay slots of the boundary this wavefront reads
+// (null: nothing flows in, the neighbour is -inf) and writes (null: no
+// neighbour on that side).
+template <bool BETA>
+__device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T, int P, int wave,
+                      double *lat_n, float *cost_n, const unsigned long long *slots_in,
+                      unsigned long long *slots_out) {
     const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int u = wave * 64 + lane;
     double o_mask = 0.0;
     bool skip;
@@ -200,12 +193,6 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, doubl
     double *out = lat_n + (size_t)u * 2;
     const double *in = units_n + (size_t)u * 3;
     front_store(out + (size_t)(BETA ? Tn : 0) * srow, f);
-
-    // which neighbour feeds this wavefront, and which one it feeds
-    const bool consumes = W > 1 && (BETA ? wave < W - 1 : wave > 0);
-    const bool produces = W > 1 && (BETA ? wave > 0 : wave < W - 1);
-    const int b_in = BETA ? wave : wave - 1;      // boundary this wavefront reads
-    const int b_out = BETA ? wave - 1 : wave;     // boundary this wavefront writes
     const int edge_lane = BETA ? 0 : 63;          // lane whose value crosses the boundary
 
     if (Tn > 0) {
@@ -213,24 +200,41 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, doubl
         const int dir = BETA ? -1 : 1;
         const int t_start = BETA ? Tn - 1 : 0;
         chunk_load(a, in, urow, Tn, t_start, dir);
-        int taken_seen = 0;
-        int ahead_seen = 0;        // counter as read by the last peek ahead
-        double ahead[R];           // ... and the slots of the chunk it looked at
+        // The relay slots of a chunk are requested one chunk before they are used,
+        // into two register sets used in turn (like the units): the set a chunk
+        // reads was requested while the previous chunk was swept, and is free to
+        // receive the request for the chunk after next as soon as it has been read.
+        unsigned long long ahead_a[R], ahead_b[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r) ahead[r] = neg_inf();
-        // one chunk: steps s0 .. s0+cnt-1 with the units in `c`
-        auto run_chunk = [&](const Chunk &c, int s0, int cnt, bool full) {
+        for (int r = 0; r < R; ++r) ahead_a[r] = ahead_b[r] = kEmptyBits;
+        if (slots_in) slots_request(slots_in, 0, ahead_a);
+        bool gave_up = false;            // after one wait has run out, no later one is started
+        // one chunk: steps s0 .. s0+cnt-1 with the units in `c` and the slots in
+        // `have`; the slots of the next chunk are requested into `next`
+        auto run_chunk = [&](const Chunk &c, unsigned long long (&have)[R],
+                             unsigned long long (&next)[R], int s0, int cnt, bool full) {
             double mail[R], mine[R];
 #pragma unroll
             for (int r = 0; r < R; ++r) mail[r] = neg_inf();
-            if (consumes) {
-                // the peek of the previous chunk looked at exactly this chunk
-                if (__builtin_amdgcn_readfirstlane(ahead_seen) < s0 + cnt)
-                    wait_and_take(&relay.done[b_in], s0 + cnt, relay.ring[b_in], s0, ahead);
+            if (slots_in) {
+                slots_request(slots_in, min(s0 + R, T), next);
+                // `have` was requested a chunk ago; repeat the request until the
+                // producer has got this far (with a bound: an empty slot is a NaN
+                // and poisons the lattice if the wait gives up).  The first look
+                // is kept out of the polling loop: a loop header that is also
+                // reached from the re-request would make the compiler wait for
+                // every load in flight here, the prefetched units included.
+                if (!slots_ready(have, cnt) && !gave_up) {
+                    int spins = 0;
+                    do {
+                        __builtin_amdgcn_s_sleep(2);
+                        slots_request(slots_in, s0, have);
+                        gave_up = ++spins >= kMaxSpins;
+                    } while (!slots_ready(have, cnt) && !gave_up);
+                }
 #pragma unroll
-                for (int r = 0; r < R; ++r) mail[r] = ahead[r];
-                publish(&relay.taken[b_in], s0 + cnt);
-                ahead_seen = peek(&relay.done[b_in], relay.ring[b_in], s0 + cnt, ahead);
+                for (int r = 0; r < R; ++r)
+                    if (full || r < cnt) mail[r] = __longlong_as_double((long long)have[r]);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
@@ -246,82 +250,95 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, doubl
                     }
                 }
             }
-            if (produces) {
-                // the ring is four chunks deep: the consumer's progress is looked
-                // up again only when the last value seen no longer covers this chunk
-                if (taken_seen < s0 + cnt - kRing)
-                    taken_seen = wait_until(&relay.taken[b_out], s0 + cnt - kRing);
-                if (lane == edge_lane) {
+            if (slots_out && lane == edge_lane) {
 #pragma unroll
-                    for (int r = 0; r < R; ++r)
-                        if (full || r < cnt) relay.ring[b_out][(s0 + r) % kRing] = mine[r];
-                }
-                publish(&relay.done[b_out], s0 + cnt);
+                for (int r = 0; r < R; ++r)
+                    if (full || r < cnt) slot_put(slots_out + s0 + r, mine[r]);
             }
         };
         int s0 = 0;
         while (s0 + 2 * R <= Tn) {
             chunk_load(b, in, urow, Tn, t_start + dir * (s0 + R), dir);
-            run_chunk(a, s0, R, true);
+            run_chunk(a, ahead_a, ahead_b, s0, R, true);
             chunk_load(a, in, urow, Tn, t_start + dir * (s0 + 2 * R), dir);
-            run_chunk(b, s0 + R, R, true);
+            run_chunk(b, ahead_b, ahead_a, s0 + R, R, true);
             s0 += 2 * R;
         }
         // fewer than 2R frames left
         chunk_load(b, in, urow, Tn, t_start + dir * (s0 + R), dir);
         const int rest = Tn - s0;
-        if (rest > 0) run_chunk(a, s0, min(rest, R), false);
-        if (rest > R) run_chunk(b, s0 + R, rest - R, false);
+        if (rest > 0) run_chunk(a, ahead_a, ahead_b, s0, min(rest, R), false);
+        if (rest > R) run_chunk(b, ahead_b, ahead_a, s0 + R, rest - R, false);
     }
     // cost = -beta(0, state 0) in natural-log units (csrc/binding.cpp:86)
     if (BETA && u == 0) *cost_n = (float)(-f.e * kLn2);
 }
 
-// grid = (N, beta_only ? 1 : 2), block = 64*W.  blockIdx.y == 0 runs beta (it
-// also produces the cost), blockIdx.y == 1 runs alpha.
-template <int W>
-__global__ __launch_bounds__(64 * W) void lattice_kernel(const double *__restrict__ units,
-                                                         const int *__restrict__ ys,
-                                                         const int *__restrict__ lx,
-                                                         const int *__restrict__ ly,
-                                                         double *__restrict__ alphas,
-                                                         double *__restrict__ betas,
-                                                         float *__restrict__ costs, int T, int U,
-                                                         const CostReduce red) {
-    __shared__ Relay<W> relay;
-    const int n = blockIdx.x;
-    constexpr int P = 64 * W;
-    if (W > 1) {
-        if (threadIdx.x < W - 1) {
-            relay.done[threadIdx.x] = 0;
-            relay.taken[threadIdx.x] = 0;
-        }
-        __syncthreads();
-    }
+// Every relay slot = empty, before the sweeps of a launch.
+__global__ __launch_bounds__(256) void relay_clear_kernel(unsigned long long *slots, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) slots[i] = kEmptyBits;
+}
+
+// One wavefront per workgroup.  Workgroup index = link * chains_pad + chain with
+// chain = n * dirs + d (d = 0: beta, which also produces the cost; d = 1:
+// alpha), chains_pad = the number of chains rounded up to a multiple of 8 (the
+// surplus workgroups exit), link = position in the chain of W workgroups, first
+// producer first: alpha starts at contexts 0..63, beta at the last 64.
+__global__ __launch_bounds__(64) void lattice_kernel(const double *__restrict__ units,
+                                                     const int *__restrict__ ys,
+                                                     const int *__restrict__ lx,
+                                                     const int *__restrict__ ly,
+                                                     double *__restrict__ alphas,
+                                                     double *__restrict__ betas,
+                                                     float *__restrict__ costs,
+                                                     unsigned long long *__restrict__ relay, int N,
+                                                     int T, int U, int W, int dirs, int chains_pad,
+                                                     const CostReduce red) {
+    const int chain = blockIdx.x % chains_pad, link = blockIdx.x / chains_pad;
+    if (chain >= N * dirs) return;
+    const int n = chain / dirs;
+    const bool beta = (chain % dirs) == 0;
+    const int wave = beta ? W - 1 - link : link;
+    const int P = 64 * W;
     // lengths outside the allocation are clamped: nothing is ever read or
     // written beyond (T, U), whatever the length tensors hold
     const int Tn = min(max(lx[n], 0), T);
     const int Un = min(max(ly[n], 0), U);
+    // 64 contexts that lie entirely beyond this sample's last context hold no
+    // state that anything reads, and pass nothing on: -inf flows in from them
+    if (wave * 64 > Un) return;
     const double *units_n = units + (size_t)n * T * P * 3;
     const int *y = ys + (size_t)n * U;
     const size_t lat = (size_t)(T + 1) * P * 2;
-    if (blockIdx.y != 0) {
-        sweep<W, false>(units_n, y, Tn, Un, alphas + (size_t)n * lat, nullptr, relay);
+    // boundary b lies between contexts 64b+63 and 64b+64; its slots for one
+    // direction of one sample: relay[((n*2 + direction)*(W-1) + b) * (T+R) ...]
+    const size_t TS = (size_t)T + R;
+    unsigned long long *slots_n =
+        relay ? relay + ((size_t)n * 2 + (beta ? 0 : 1)) * (size_t)(W - 1) * TS : nullptr;
+    if (!beta) {
+        const unsigned long long *in = wave > 0 ? slots_n + (size_t)(wave - 1) * TS : nullptr;
+        unsigned long long *out = (wave + 1) * 64 <= Un ? slots_n + (size_t)wave * TS : nullptr;
+        sweep<false>(units_n, y, Tn, Un, T, P, wave, alphas + (size_t)n * lat, nullptr, in, out);
         return;
     }
-    sweep<W, true>(units_n, y, Tn, Un, betas + (size_t)n * lat, costs + n, relay);
-    if (threadIdx.x >= 64) return;
+    {
+        const unsigned long long *in = (wave + 1) * 64 <= Un ? slots_n + (size_t)wave * TS : nullptr;
+        unsigned long long *out = wave > 0 ? slots_n + (size_t)(wave - 1) * TS : nullptr;
+        sweep<true>(units_n, y, Tn, Un, T, P, wave, betas + (size_t)n * lat, costs + n, in, out);
+    }
+    if (wave != 0) return;
     // thread 0 (context 0) has just written costs[n]
-    if (red.average_frames && threadIdx.x == 0) costs[n] /= (float)lx[n];
+    const int lane = threadIdx.x;
+    if (red.average_frames && lane == 0) costs[n] /= (float)lx[n];
     if (red.reduced == nullptr) return;
     // Reduction over the batch (warp_ctct/__init__.py:142-147 of the reference)
     // by the workgroup that finishes last: every workgroup publishes its cost
     // (release fence), then counts itself; the one that sees N-1 earlier
     // arrivals reads all N costs (acquire fence) and adds them in a fixed
     // order, so the result does not depend on the order of arrival.
-    const int N = gridDim.x;
     int last = 0;
-    if (threadIdx.x == 0) {
+    if (lane == 0) {
         __threadfence();
         last = (atomicAdd(red.counter, 1u) == (unsigned)(N - 1)) ? 1 : 0;
     }
@@ -329,38 +346,44 @@ __global__ __launch_bounds__(64 * W) void lattice_kernel(const double *__restric
     if (!last) return;
     __threadfence();
     float s = 0.0f;
-    for (int i = threadIdx.x; i < N; i += 64)
+    for (int i = lane; i < N; i += 64)
         s += __hip_atomic_load(costs + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) s += __shfl_xor(s, off, 64);
-    if (threadIdx.x == 0) *red.reduced = (red.mode == 2) ? s / (float)N : s;
-}
-
-template <int W>
-hipError_t launch_lattice_w(const LatticeArgs &a, hipStream_t stream) {
-    dim3 grid(a.N, a.beta_only ? 1 : 2);
-    TIMED_LAUNCH((lattice_kernel<W>), grid, dim3(64 * W), 0, stream, a.units, a.ys, a.lx,
-                       a.ly, a.alphas, a.betas, a.costs, a.T, a.U, a.reduce);
-    return hipGetLastError();
+    if (lane == 0) *red.reduced = (red.mode == 2) ? s / (float)N : s;
 }
 
 }  // namespace
 
-int lattice_max_contexts() { return 64 * 8; }
+size_t lattice_relay_slots(int N, int T, int U) {
+    const int W = (U + 1 + 63) / 64;
+    return (size_t)N * 2 * (size_t)(W - 1) * ((size_t)T + R);
+}
 
 hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream) {
+    if (a.N == 0) return hipSuccess;
     const int W = (a.U + 1 + 63) / 64;
-    switch (W) {
-        case 1: return launch_lattice_w<1>(a, stream);
-        case 2: return launch_lattice_w<2>(a, stream);
-        case 3: return launch_lattice_w<3>(a, stream);
-        case 4: return launch_lattice_w<4>(a, stream);
-        case 5: return launch_lattice_w<5>(a, stream);
-        case 6: return launch_lattice_w<6>(a, stream);
-        case 7: return launch_lattice_w<7>(a, stream);
-        case 8: return launch_lattice_w<8>(a, stream);
-        default: return hipErrorInvalidValue;
+    const size_t slots = lattice_relay_slots(a.N, a.T, a.U);
+    unsigned long long *relay = reinterpret_cast<unsigned long long *>(a.relay);
+    if (slots > 0) {
+        if (!relay) return hipErrorInvalidValue;
+        const size_t blocks = (slots + 255) / 256;
+        if (blocks > 0x7fffffffUL) return hipErrorInvalidValue;
+        TIMED_LAUNCH(relay_clear_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, relay,
+                     slots);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    } else {
+        relay = nullptr;
     }
+    const int dirs = a.beta_only ? 1 : 2;
+    const long chains = (long)a.N * dirs;
+    const long chains_pad = (chains + 7) / 8 * 8;
+    if (chains_pad * W > 0x7fffffffL) return hipErrorInvalidValue;
+    TIMED_LAUNCH(lattice_kernel, dim3((unsigned)(chains_pad * W)), dim3(64), 0, stream, a.units,
+                 a.ys, a.lx, a.ly, a.alphas, a.betas, a.costs, relay, a.N, a.T, a.U, W, dirs,
+                 (int)chains_pad, a.reduce);
+    return hipGetLastError();
 }
 
 }  // namespace wctct

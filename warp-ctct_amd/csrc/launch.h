@@ -37,12 +37,16 @@ struct LatticeArgs {
     double *alphas;       // (N,T+1,P,2) log2 units, or null if beta_only
     double *betas;        // (N,T+1,P,2) log2 units
     float *costs;         // (N)
+    void *relay;          // lattice_relay_slots(N,T,U) 64-bit words, or null if there are none
     int N, T, U;
     bool beta_only;
     CostReduce reduce;    // zero-initialise for plain per-sample costs
 };
 
-int lattice_max_contexts();
+// A lattice of more than 64 contexts is swept by a chain of workgroups that
+// hand one value per frame and 64-context boundary through device memory:
+// the number of 64-bit slots that takes (0 for U + 1 <= 64).
+size_t lattice_relay_slots(int N, int T, int U);
 hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream);
 
 // Element strides of a joint tensor (N,T,U+1,V); dense row-major is
@@ -105,7 +109,8 @@ hipError_t launch_simple_gather_units(const float *f, const float *g, const floa
                                       int N, int T, int U, int V, hipStream_t stream);
 // compact gradients of the joiner path straight from the lattices: grad_f
 // (N,T,U+1), grad_g (N,U+1,3), grad_den (N,T,U+1) or null; `partial` is scratch
-// of N * ceil(T/8) * (U+1) * 3 floats
+// of N * T * (U+1) * 3 floats (partial sums over blocks of 8 frames, or, for
+// lattices of more than 512 contexts, the unit gradients themselves)
 hipError_t launch_simple_grads(const double *units, const int *ys, const int *lx, const int *ly,
                                const double *alphas, const double *betas, float *partial,
                                float *grad_f, float *grad_g, float *grad_den, int N, int T, int U,

@@ -324,6 +324,14 @@ hipError_t launch_simple_grads(const double *units, const int *ys, const int *lx
                                float *grad_f, float *grad_g, float *grad_den, int N, int T, int U,
                                hipStream_t stream) {
     const int P = padded_contexts(U);
+    if (P > 512) {
+        // more contexts than one workgroup of the fused kernel holds: unit
+        // gradients into `partial` (it has room for all of them), then the two
+        // reductions over them
+        hipError_t e = launch_unit_grads(units, ys, lx, ly, alphas, betas, partial, N, T, U, stream);
+        if (e != hipSuccess) return e;
+        return launch_simple_reduce(partial, grad_f, grad_g, grad_den, N, T, U, stream);
+    }
     const int blocks = (T + kFramesPerBlock - 1) / kFramesPerBlock;
     if (T > 0) {
         TIMED_LAUNCH(simple_grads_kernel, dim3(blocks, N), dim3(P), 0, stream, units, ys, lx,
