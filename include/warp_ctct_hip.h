@@ -166,6 +166,21 @@ int warpctct_loss_lattice_strided(const void *joint, int dtype, const long *stri
                                   int want_alpha, int reduction, int average_frames,
                                   float *reduced, void *stream);
 
+/* warpctct_loss_lattice_strided that also clears the buffer of the dense
+ * gradient, dense_bytes bytes at `dense`, for warpctct_dense_patch_lattice to
+ * write into later (the reference forms its dense gradient inside autograd:
+ * the backward of torch.gather, warp_ctct/__init__.py:131, zero-fills the
+ * joint's shape and scatters into it).  The clear rides in the launch of the
+ * lattice kernel, as extra workgroups behind the sweeps: those wait on chains
+ * of dependent arithmetic and leave the memory system idle, the clear is pure
+ * write traffic, so the sweeps cost no time of their own.  Everything runs on
+ * `stream`.  dense == NULL or dense_bytes == 0: nothing to clear. */
+int warpctct_loss_lattice_clearing(const void *joint, int dtype, const long *strides,
+                                   const int *ys, const int *lx, const int *ly, int N, int T,
+                                   int U, int V, void *workspace, size_t workspace_bytes,
+                                   float *costs, int want_alpha, int reduction, int average_frames,
+                                   float *reduced, void *dense, size_t dense_bytes, void *stream);
+
 /* Dense gradient of type `dtype` from that workspace (see
  * warpctct_dense_grad_lattice_f32 below for the weights); values are summed in
  * fp32 and rounded once to nearest even. */
@@ -370,8 +385,12 @@ int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, lo
  * on the launch's own stream; warpctct_profile(0) stops.  After the caller has
  * synchronised, record `index` (0 <= index < warpctct_profile_count(), in
  * launch order) gives the kernel's name (static storage) and its duration.
+ * warpctct_profile_filter(text) limits the bracketing to kernels whose name
+ * contains `text` (at most 63 characters; NULL or "": every kernel), so that
+ * one kernel can be timed inside a timed region at the cost of two events.
  * Creating events allocates: keep it off in production and under graph capture. */
 int warpctct_profile(int enable);
+int warpctct_profile_filter(const char *text);
 int warpctct_profile_count(void);
 int warpctct_profile_read(int index, const char **kernel, float *microseconds);
 

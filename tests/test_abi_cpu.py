@@ -98,6 +98,14 @@ def test_generic_dtype_and_logits_entry_points_check_their_arguments():
     assert lib.warpctct_loss_lattice(p, 2, p, p, p, 1, 1, 1, 8, p, small, p, 1, 2, 0, p, null) == EWORKSPACE
     assert lib.warpctct_logits_loss_lattice(p, 1, p, p, p, 1, 1, 1, 8, p, small, p, 1, 0, 0, null,
                                             null) == EWORKSPACE
+    # the clearing form refuses the same things, before it forks its stream
+    strides = (ctypes.c_long * 4)(16, 16, 8, 1)
+    assert lib.warpctct_loss_lattice_clearing(p, 7, strides, p, p, p, 1, 1, 1, 8, p, small, p, 1, 0,
+                                              0, null, p, small, null) == EINVAL
+    assert lib.warpctct_loss_lattice_clearing(p, 0, null, p, p, p, 1, 1, 1, 8, p, small, p, 1, 0,
+                                              0, null, p, small, null) == EINVAL
+    assert lib.warpctct_loss_lattice_clearing(p, 2, strides, p, p, p, 1, 1, 1, 8, p, small, p, 1, 2,
+                                              0, p, p, small, null) == EWORKSPACE
     assert lib.warpctct_logits_grad_lattice(p, small, p, 0, p, p, p, p, 1, f(1.0), 0, p, 1, 1, 1, 8,
                                             null) == EWORKSPACE
     assert lib.warpctct_logits_grad_lattice(p, small, p, 5, p, p, p, p, 1, f(1.0), 0, p, 1, 1, 1, 8,

@@ -611,6 +611,33 @@ def test_autograd_plumbing_views_non_leaf_and_repeated_backward():
     np.testing.assert_allclose(quiet.item(), ref_costs.sum(), rtol=LOSS_RTOL)
 
 
+def test_gradient_buffer_cleared_in_the_forward_or_in_the_backward():
+    """ctct_loss clears the joint's gradient beside the lattices in the forward
+    (warp_ctct.CLEAR_GRADIENT_IN_FORWARD) or, with the switch off, in the
+    backward: losses and gradients are the same bit for bit, for float32 and
+    bfloat16 joints; without a gradient no buffer is made."""
+    import warp_ctct
+    joint, ys, lx, ly = make_joint_case(95, 5, 41, 12, 96, lx=[41, 30, 22, 41, 7], ly=[12, 5, 9, 1, 3])
+    d_ys, d_lx, d_ly = dev(ys), dev(lx), dev(ly)
+    _, ref_dense, ref_costs = O.ctct_loss(joint, ys, lx, ly, reduction="sum", grad_output=np.ones(5))
+    assert warp_ctct.CLEAR_GRADIENT_IN_FORWARD
+    try:
+        for dtype in (torch.float32, torch.bfloat16):
+            got = []
+            for switch in (True, False):
+                warp_ctct.CLEAR_GRADIENT_IN_FORWARD = switch
+                x = dev(joint).to(dtype).requires_grad_(True)
+                loss = warp_ctct.ctct_loss(x, d_ys, d_lx, d_ly, reduction="sum")
+                loss.backward()
+                got.append((loss.detach().clone(), x.grad.clone()))
+            assert torch.equal(got[0][0], got[1][0]) and torch.equal(got[0][1], got[1][1])
+            if dtype == torch.float32:
+                np.testing.assert_allclose(got[0][0].item(), ref_costs.sum(), rtol=LOSS_RTOL)
+                np.testing.assert_allclose(got[0][1].cpu().numpy(), ref_dense, atol=GRAD_ATOL, rtol=0)
+    finally:
+        warp_ctct.CLEAR_GRADIENT_IN_FORWARD = True
+
+
 def test_infeasible_sample_has_infinite_cost():
     import warp_ctct
     joint, ys, lx, ly = make_joint_case(17, 2, 6, 3, 5, force_repeat=False)

@@ -167,6 +167,61 @@ def test_scale_units_and_orchestrators_in_float32_form():
     assert torch.equal(costs2, costs)
 
 
+def test_forward_that_clears_the_gradient_buffer_beside_the_lattices():
+    """warpctct_loss_lattice_clearing + warpctct_dense_patch_lattice against
+    warpctct_loss_lattice + warpctct_dense_grad_lattice: same costs and the same
+    dense gradient bit for bit, on a buffer that held NaNs, for a narrow and for
+    a two-wavefront lattice, with and without a buffer to clear, for a strided
+    joint."""
+    lib = hip_lib.lib()
+    p, s = hip_lib.ptr, hip_lib.stream_ptr()
+    one = ctypes.c_float(1.0)
+    for seed, N, T, U, V, lx, ly in [(231, 4, 37, 9, 1024, [37, 20, 31, 9], [9, 4, 7, 1]),
+                                     (232, 2, 21, 70, 48, [21, 15], [70, 33])]:
+        joint, ys, lx, ly = make_joint_case(seed, N, T, U, V, lx=lx, ly=ly)
+        w = np.random.default_rng(seed).standard_normal(N).astype(np.float32)
+        _, ref_dense, ref_costs = O.ctct_loss(joint, ys, lx, ly, reduction="none", grad_output=w)
+        need = lib.warpctct_workspace_bytes(N, T, U)
+        d_ys, d_lx, d_ly, d_w = dev(ys), dev(lx), dev(ly), dev(w)
+        # the joint stored as (N, U+1, T, V): the entry point sees it through strides
+        stored = dev(np.ascontiguousarray(joint.transpose(0, 2, 1, 3)))
+        view = stored.transpose(1, 2)
+        strides = (ctypes.c_long * 4)(*view.stride())
+        ws_a = torch.empty(need, dtype=torch.uint8, device="cuda")
+        ws_b = torch.empty(need, dtype=torch.uint8, device="cuda")
+        costs_a, costs_b, costs_c = nan_like(N), nan_like(N), nan_like(N)
+        dense_a, dense_b = nan_like(N, T, U + 1, V), nan_like(N, T, U + 1, V)
+        nbytes = ctypes.c_size_t(dense_a.numel() * 4)
+        hip_lib.check(lib.warpctct_loss_lattice_strided(p(stored), 0, strides, p(d_ys), p(d_lx),
+                                                        p(d_ly), N, T, U, V, p(ws_a),
+                                                        ctypes.c_size_t(need), p(costs_a), 1, 0, 0,
+                                                        None, s))
+        hip_lib.check(lib.warpctct_dense_grad_lattice(p(ws_a), ctypes.c_size_t(need), p(d_ys),
+                                                      p(d_lx), p(d_ly), p(d_w), 1, one, 0,
+                                                      p(dense_a), 0, N, T, U, V, s))
+        hip_lib.check(lib.warpctct_loss_lattice_clearing(p(stored), 0, strides, p(d_ys), p(d_lx),
+                                                         p(d_ly), N, T, U, V, p(ws_b),
+                                                         ctypes.c_size_t(need), p(costs_b), 1, 0, 0,
+                                                         None, p(dense_b), nbytes, s))
+        # work queued on the caller's stream afterwards sees the cleared buffer
+        cleared = dense_b.clone()
+        hip_lib.check(lib.warpctct_dense_patch_lattice(p(ws_b), ctypes.c_size_t(need), p(d_ys),
+                                                       p(d_lx), p(d_ly), p(d_w), 1, one, 0,
+                                                       p(dense_b), 0, N, T, U, V, s))
+        # nothing to clear: the plain forward
+        hip_lib.check(lib.warpctct_loss_lattice_clearing(p(stored), 0, strides, p(d_ys), p(d_lx),
+                                                         p(d_ly), N, T, U, V, p(ws_b),
+                                                         ctypes.c_size_t(need), p(costs_c), 1, 0, 0,
+                                                         None, None, ctypes.c_size_t(0), s))
+        torch.cuda.synchronize()
+        assert torch.count_nonzero(cleared).item() == 0 and not torch.isnan(cleared).any()
+        assert torch.equal(costs_b, costs_a) and torch.equal(costs_c, costs_a)
+        assert torch.equal(dense_b, dense_a)
+        np.testing.assert_allclose(costs_b.cpu().numpy(), ref_costs, rtol=LOSS_RTOL)
+        scale = max(1.0, float(np.abs(w).max()))
+        np.testing.assert_allclose(dense_b.cpu().numpy(), ref_dense, atol=GRAD_ATOL * scale, rtol=0)
+
+
 SIMPLE_STAGE_CASES = [
     # name, seed, N, T, U, V, lx, ly, normalized
     ("normalized", 221, 3, 23, 7, 29, [23, 12, 17], [7, 3, 5], True),

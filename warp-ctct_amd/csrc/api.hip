@@ -323,22 +323,31 @@ int warpctct_loss_lattice(const void *joint, int dtype, const int *ys, const int
                                          average_frames, reduced, stream);
 }
 
-int warpctct_loss_lattice_strided(const void *joint, int dtype, const long *strides,
-                                  const int *ys, const int *lx, const int *ly, int N, int T, int U,
-                                  int V, void *workspace, size_t workspace_bytes, float *costs,
-                                  int want_alpha, int reduction, int average_frames,
-                                  float *reduced, void *stream) {
+namespace {
+
+// What warpctct_loss_lattice_strided refuses, before anything is launched.
+int check_loss_lattice(const void *joint, int dtype, const long *strides, const int *ys,
+                       const int *lx, const int *ly, int N, int T, int U, int V,
+                       const void *workspace, size_t workspace_bytes, const float *costs,
+                       int reduction, const float *reduced) {
     if (!dims_ok(N, T, U) || V < 1 || !io_valid(dtype) || reduction < 0 || reduction > 2 ||
         !strides)
         return WARPCTCT_EINVAL;
-    const JointStrides js = {strides[0], strides[1], strides[2], strides[3]};
     if (N == 0) return WARPCTCT_OK;
     if (!lx || !ly || !costs || !workspace || (T > 0 && !joint) || (U > 0 && !ys))
         return WARPCTCT_EINVAL;
     if (reduction != 0 && !reduced) return WARPCTCT_EINVAL;
+    if (workspace_bytes < carve(nullptr, N, T, U).bytes) return WARPCTCT_EWORKSPACE;
+    return WARPCTCT_OK;
+}
+
+// gather + lattices, with `fill` cleared inside the lattice kernel's launch
+int loss_lattice_run(const void *joint, int dtype, const long *strides, const int *ys,
+                     const int *lx, const int *ly, int N, int T, int U, int V, void *workspace,
+                     float *costs, int want_alpha, int reduction, int average_frames,
+                     float *reduced, const FillTail &fill, hipStream_t st) {
+    const JointStrides js = {strides[0], strides[1], strides[2], strides[3]};
     const Workspace w = carve(workspace, N, T, U);
-    if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
-    hipStream_t st = as_stream(stream);
     unsigned *counter = reduction != 0 ? w.counter : nullptr;
     if (T > 0) {
         int rc = done(launch_gather_units(joint, js, dtype, ys, lx, ly, w.units, N, T, U, V, true,
@@ -365,7 +374,50 @@ int warpctct_loss_lattice_strided(const void *joint, int dtype, const long *stri
     a.reduce.counter = counter;
     a.reduce.mode = reduction;
     a.reduce.average_frames = average_frames != 0;
+    a.fill = fill;
     return done(launch_lattice(a, st));
+}
+
+}  // namespace
+
+int warpctct_loss_lattice_clearing(const void *joint, int dtype, const long *strides,
+                                   const int *ys, const int *lx, const int *ly, int N, int T,
+                                   int U, int V, void *workspace, size_t workspace_bytes,
+                                   float *costs, int want_alpha, int reduction, int average_frames,
+                                   float *reduced, void *dense, size_t dense_bytes, void *stream) {
+    int rc = check_loss_lattice(joint, dtype, strides, ys, lx, ly, N, T, U, V, workspace,
+                                workspace_bytes, costs, reduction, reduced);
+    if (rc != WARPCTCT_OK) return rc;
+    hipStream_t st = as_stream(stream);
+    if (!dense) dense_bytes = 0;
+    if (N == 0) return done(launch_zero_fill_bytes(dense, dense_bytes, st));
+    // the 16-byte vectors of the buffer ride in the lattice kernel's launch;
+    // the few bytes before and after them (if any) are cleared on their own
+    unsigned char *p = static_cast<unsigned char *>(dense);
+    size_t head = (16 - (reinterpret_cast<uintptr_t>(p) & 15u)) & 15u;
+    if (head > dense_bytes) head = dense_bytes;
+    FillTail fill;
+    fill.p = p + head;
+    fill.n4 = (dense_bytes - head) / 16;
+    const size_t tail = dense_bytes - head - fill.n4 * 16;
+    if ((rc = done(launch_zero_fill_bytes(p, head, st))) != WARPCTCT_OK) return rc;
+    if ((rc = done(launch_zero_fill_bytes(p + head + fill.n4 * 16, tail, st))) != WARPCTCT_OK)
+        return rc;
+    return loss_lattice_run(joint, dtype, strides, ys, lx, ly, N, T, U, V, workspace, costs,
+                            want_alpha, reduction, average_frames, reduced, fill, st);
+}
+
+int warpctct_loss_lattice_strided(const void *joint, int dtype, const long *strides,
+                                  const int *ys, const int *lx, const int *ly, int N, int T, int U,
+                                  int V, void *workspace, size_t workspace_bytes, float *costs,
+                                  int want_alpha, int reduction, int average_frames,
+                                  float *reduced, void *stream) {
+    const int ok = check_loss_lattice(joint, dtype, strides, ys, lx, ly, N, T, U, V, workspace,
+                                      workspace_bytes, costs, reduction, reduced);
+    if (ok != WARPCTCT_OK || N == 0) return ok;
+    return loss_lattice_run(joint, dtype, strides, ys, lx, ly, N, T, U, V, workspace, costs,
+                            want_alpha, reduction, average_frames, reduced, FillTail(),
+                            as_stream(stream));
 }
 
 int warpctct_loss_lattice_f32(const float *joint, const int *ys, const int *lx, const int *ly,

@@ -117,13 +117,10 @@ int io_type_of(const torch::Tensor &t) {
 // always float32; the workspace (units, alpha, beta) is what
 // dense_patch_lattice needs in backward; without requires_grad only beta runs
 // and loss is returned twice (as the reference does, binding.cpp:98).
-std::tuple<torch::Tensor, torch::Tensor> ctct_loss_joint_fwd(const torch::Tensor &joint,
-                                                             const torch::Tensor &ys,
-                                                             const torch::Tensor &lx,
-                                                             const torch::Tensor &ly,
-                                                             const bool requires_grad,
-                                                             const int64_t reduction,
-                                                             const bool average_frames) {
+std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> ctct_loss_joint_fwd(
+    const torch::Tensor &joint, const torch::Tensor &ys, const torch::Tensor &lx,
+    const torch::Tensor &ly, const bool requires_grad, const int64_t reduction,
+    const bool average_frames, const bool clear_gradient) {
     // the joint may be any strided view (the reference's torch.gather takes
     // views as they are, warp_ctct/__init__.py:131): no copy is made
     CHECK_DEVICE(joint);
@@ -141,17 +138,25 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_loss_joint_fwd(const torch::Tensor
     if (reduction != 0) reduced = N > 0 ? torch::empty({}, f32) : torch::zeros({}, f32);
     const long strides[4] = {static_cast<long>(joint.stride(0)), static_cast<long>(joint.stride(1)),
                              static_cast<long>(joint.stride(2)), static_cast<long>(joint.stride(3))};
-    check_rc(warpctct_loss_lattice_strided(joint.data_ptr(), dtype, strides, ys.data_ptr<int>(),
-                                           lx.data_ptr<int>(), ly.data_ptr<int>(), N, T, U, V,
-                                           ws.data_ptr(), ws.numel(), costs.data_ptr<float>(),
-                                           requires_grad ? 1 : 0, static_cast<int>(reduction),
-                                           average_frames ? 1 : 0,
-                                           reduction != 0 ? reduced.data_ptr<float>() : nullptr,
-                                           current_stream()),
+    // With clear_gradient the buffer of the dense gradient is allocated now and
+    // cleared beside the gather and the lattices; the backward then only
+    // patches it (dense_patch_lattice).  Otherwise `dense` comes back empty.
+    torch::Tensor dense;
+    if (requires_grad && clear_gradient)
+        dense = torch::empty({N, T, U + 1, V}, joint.options());
+    else
+        dense = torch::empty({0}, joint.options());
+    check_rc(warpctct_loss_lattice_clearing(
+                 joint.data_ptr(), dtype, strides, ys.data_ptr<int>(), lx.data_ptr<int>(),
+                 ly.data_ptr<int>(), N, T, U, V, ws.data_ptr(), ws.numel(),
+                 costs.data_ptr<float>(), requires_grad ? 1 : 0, static_cast<int>(reduction),
+                 average_frames ? 1 : 0, reduction != 0 ? reduced.data_ptr<float>() : nullptr,
+                 dense.numel() > 0 ? dense.data_ptr() : nullptr,
+                 static_cast<size_t>(dense.numel()) * dense.element_size(), current_stream()),
              "ctct_loss_joint_fwd");
     const torch::Tensor &loss = reduction != 0 ? reduced : costs;
-    if (requires_grad) return std::make_tuple(loss, ws);
-    return std::make_tuple(loss, loss);
+    if (requires_grad) return std::make_tuple(loss, ws, dense);
+    return std::make_tuple(loss, loss, dense);
 }
 
 // The two halves of the dense gradient as separate operators, so that a caller
@@ -594,7 +599,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           "CTC-Transducer loss on the un-gathered joint (forward).", pybind11::arg("log_probs"),
           pybind11::arg("ys"), pybind11::arg("lx"), pybind11::arg("ly"),
           pybind11::arg("requires_grad"), pybind11::arg("reduction") = 0,
-          pybind11::arg("average_frames") = false);
+          pybind11::arg("average_frames") = false, pybind11::arg("clear_gradient") = false);
     m.def("ctct_loss_compact_fwd", &ctct_loss_compact_fwd,
           "Costs and compact unit gradients from the un-gathered joint.",
           pybind11::arg("log_probs"), pybind11::arg("ys"), pybind11::arg("lx"),

@@ -28,8 +28,22 @@
 //    27 us instead of 35 us (one thread writing its row's segments alone:
 //    44 us; 64-byte segments: 28 us but the fill still suffers);
 //  * running the fill on a second stream next to the gather / lattice kernels
-//    is slower than running everything back to back.
-// Hence two launches on one stream: fill, then patch.
+//    is no faster than running everything back to back (the fill takes 330 us
+//    instead of 290 us, and forking and joining the streams costs ~30 us, which
+//    a small batch feels most);
+//  * the fill does not need every wave slot: at 4 (or 2) wavefronts per SIMD
+//    it takes 280 us, at all 8 it takes 289 us, at 1 it takes 460 us; 64-thread
+//    workgroups take 415 us, 512 threads 289 us, 1024 threads 313 us;
+//  * workgroups of the fill appended to the LATTICE kernel's launch (see
+//    lattice_fill_kernel) run beside the sweeps at the fill's own speed
+//    (282 us for both): the sweeps wait on chains of dependent arithmetic and
+//    hardly touch memory.  The same trick with the gather kernel gains nothing
+//    (its workgroups in front: they run first, then the fill) or loses (spread
+//    between the fill's: scattered reads between the writes slow the fill by
+//    half).
+// Hence: the forward clears the buffer inside the lattice kernel's launch when
+// the caller hands it over (warpctct_loss_lattice_clearing) and the backward
+// only patches; or, on a buffer of the backward's own, fill then patch.
 #include "device_utils.h"
 #include "launch.h"
 #include "unit_grad.h"
@@ -50,8 +64,11 @@ __global__ __launch_bounds__(kBlock) void zero_fill_byte_kernel(unsigned char *_
     if (i < n) p[i] = 0;
 }
 
-// p4[i] = 0 for i < n4: one store per thread, no loop.
-__global__ __launch_bounds__(kBlock) void zero_fill_vec_kernel(v4f *__restrict__ p4, size_t n4) {
+// p4[i] = 0 for i < n4: one store per thread, no loop; at most 4 wavefronts per
+// SIMD (with all 8 the memory side queues up and the fill takes 3 % longer;
+// 2 are as good as 4, 1 is far too few).
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) void
+zero_fill_vec_kernel(v4f *__restrict__ p4, size_t n4) {
     const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
     const v4f z = {0.0f, 0.0f, 0.0f, 0.0f};
     if (i < n4) p4[i] = z;

@@ -285,16 +285,16 @@ __global__ __launch_bounds__(256) void relay_clear_kernel(unsigned long long *sl
 // alpha), chains_pad = the number of chains rounded up to a multiple of 8 (the
 // surplus workgroups exit), link = position in the chain of W workgroups, first
 // producer first: alpha starts at contexts 0..63, beta at the last 64.
-__global__ __launch_bounds__(64) void lattice_kernel(const double *__restrict__ units,
-                                                     const int *__restrict__ ys,
-                                                     const int *__restrict__ lx,
-                                                     const int *__restrict__ ly,
-                                                     double *__restrict__ alphas,
-                                                     double *__restrict__ betas,
-                                                     float *__restrict__ costs,
-                                                     unsigned long long *__restrict__ relay, int N,
-                                                     int T, int U, int W, int dirs, int chains_pad,
-                                                     const CostReduce red) {
+__device__ __forceinline__ void lattice_block(const double *__restrict__ units,
+                                              const int *__restrict__ ys,
+                                              const int *__restrict__ lx,
+                                              const int *__restrict__ ly,
+                                              double *__restrict__ alphas,
+                                              double *__restrict__ betas,
+                                              float *__restrict__ costs,
+                                              unsigned long long *__restrict__ relay, int N, int T,
+                                              int U, int W, int dirs, int chains_pad,
+                                              const CostReduce &red) {
     const int chain = blockIdx.x % chains_pad, link = blockIdx.x / chains_pad;
     if (chain >= N * dirs) return;
     const int n = chain / dirs;
@@ -353,6 +353,40 @@ __global__ __launch_bounds__(64) void lattice_kernel(const double *__restrict__ 
     if (lane == 0) *red.reduced = (red.mode == 2) ? s / (float)N : s;
 }
 
+__global__ __launch_bounds__(64) void lattice_kernel(const double *__restrict__ units,
+                                                     const int *__restrict__ ys,
+                                                     const int *__restrict__ lx,
+                                                     const int *__restrict__ ly,
+                                                     double *__restrict__ alphas,
+                                                     double *__restrict__ betas,
+                                                     float *__restrict__ costs,
+                                                     unsigned long long *__restrict__ relay, int N,
+                                                     int T, int U, int W, int dirs, int chains_pad,
+                                                     const CostReduce red) {
+    lattice_block(units, ys, lx, ly, alphas, betas, costs, relay, N, T, U, W, dirs, chains_pad, red);
+}
+
+// The same sweeps with a memory clear riding along: workgroups of 256 threads,
+// of which the first lattice_blocks are the sweeps (their first wavefront; the
+// other three retire at once) and every later one stores 256 zero vectors of
+// 16 bytes and retires.  The sweeps wait on a chain of dependent arithmetic
+// and leave the memory system idle; the clear is pure write traffic.
+typedef float v4f_fill __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void lattice_fill_kernel(
+    const double *__restrict__ units, const int *__restrict__ ys, const int *__restrict__ lx,
+    const int *__restrict__ ly, double *__restrict__ alphas, double *__restrict__ betas,
+    float *__restrict__ costs, unsigned long long *__restrict__ relay, int N, int T, int U, int W,
+    int dirs, int chains_pad, const CostReduce red, v4f_fill *__restrict__ fill, size_t n4,
+    unsigned lattice_blocks) {
+    if (blockIdx.x >= lattice_blocks) {
+        const size_t i = (size_t)(blockIdx.x - lattice_blocks) * 256 + threadIdx.x;
+        if (i < n4) fill[i] = v4f_fill{0.0f, 0.0f, 0.0f, 0.0f};
+        return;
+    }
+    if (threadIdx.x >= 64) return;
+    lattice_block(units, ys, lx, ly, alphas, betas, costs, relay, N, T, U, W, dirs, chains_pad, red);
+}
+
 }  // namespace
 
 size_t lattice_relay_slots(int N, int T, int U) {
@@ -380,6 +414,15 @@ hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream) {
     const long chains = (long)a.N * dirs;
     const long chains_pad = (chains + 7) / 8 * 8;
     if (chains_pad * W > 0x7fffffffL) return hipErrorInvalidValue;
+    if (a.fill.n4 > 0) {
+        const size_t blocks = (size_t)(chains_pad * W) + (a.fill.n4 + 255) / 256;
+        if (blocks > 0x7fffffffUL) return hipErrorInvalidValue;
+        TIMED_LAUNCH(lattice_fill_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a.units,
+                     a.ys, a.lx, a.ly, a.alphas, a.betas, a.costs, relay, a.N, a.T, a.U, W, dirs,
+                     (int)chains_pad, a.reduce, static_cast<v4f_fill *>(a.fill.p), a.fill.n4,
+                     (unsigned)(chains_pad * W));
+        return hipGetLastError();
+    }
     TIMED_LAUNCH(lattice_kernel, dim3((unsigned)(chains_pad * W)), dim3(64), 0, stream, a.units,
                  a.ys, a.lx, a.ly, a.alphas, a.betas, a.costs, relay, a.N, a.T, a.U, W, dirs,
                  (int)chains_pad, a.reduce);

@@ -29,6 +29,15 @@ struct CostReduce {
     int average_frames;   // costs[n] /= lx[n] before anything else
 };
 
+// Memory to clear inside another kernel's launch: n4 vectors of 16 bytes at p
+// (16-byte aligned).  Workgroups appended to that launch each store 256 vectors
+// and retire, while the kernel's own workgroups, which are bound by latency and
+// leave the memory system idle, do their work.
+struct FillTail {
+    void *p = nullptr;
+    size_t n4 = 0;
+};
+
 struct LatticeArgs {
     const double *units;  // (N,T,P,3) log2 units, neutral values in the padding
     const int *ys;        // (N,U)
@@ -41,6 +50,7 @@ struct LatticeArgs {
     int N, T, U;
     bool beta_only;
     CostReduce reduce;    // zero-initialise for plain per-sample costs
+    FillTail fill;        // cleared beside the sweeps (default: nothing)
 };
 
 // A lattice of more than 64 contexts is swept by a chain of workgroups that

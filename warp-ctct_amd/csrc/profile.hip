@@ -2,6 +2,7 @@
 #include "profile.h"
 
 #include <atomic>
+#include <cstring>
 #include <mutex>
 #include <vector>
 
@@ -22,6 +23,7 @@ struct Record {
 std::atomic<bool> g_enabled{false};
 std::mutex g_mutex;
 std::vector<Record> g_records;
+char g_filter[64] = "";   // bracket only kernels whose name contains this
 
 void drop_records() {
     for (Record &r : g_records) {
@@ -38,6 +40,7 @@ bool profile_enabled() { return g_enabled.load(std::memory_order_relaxed); }
 void profile_begin(const char *kernel, hipStream_t stream, int *slot) {
     std::lock_guard<std::mutex> lock(g_mutex);
     if ((int)g_records.size() >= kMaxRecords) return;
+    if (g_filter[0] && !std::strstr(kernel, g_filter)) return;
     Record r = {kernel, nullptr, nullptr, false};
     if (hipEventCreate(&r.begin) != hipSuccess) return;
     if (hipEventCreate(&r.end) != hipSuccess) {
@@ -68,6 +71,14 @@ int warpctct_profile(int enable) {
     std::lock_guard<std::mutex> lock(g_mutex);
     if (enable) drop_records();
     g_enabled.store(enable != 0, std::memory_order_relaxed);
+    return WARPCTCT_OK;
+}
+
+int warpctct_profile_filter(const char *text) {
+    using namespace wctct;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (text && std::strlen(text) >= sizeof(g_filter)) return WARPCTCT_EINVAL;
+    std::strcpy(g_filter, text ? text : "");
     return WARPCTCT_OK;
 }
 

@@ -52,6 +52,13 @@ def set_kernel_observer(observer):
     _kernel_observer = observer
 
 
+# ctct_loss allocates and clears the joint's gradient during the forward (in the
+# lattice kernel's launch, beside the sweeps) when the joint requires a gradient.  The
+# buffer then lives from the forward to the backward; set this to False to
+# allocate and clear it in the backward instead.
+CLEAR_GRADIENT_IN_FORWARD = True
+
+
 def _run(name, fn):
     if _kernel_observer is None:
         return fn()
@@ -89,21 +96,29 @@ class _CTCTLoss(torch.autograd.Function):
     Counterpart of the reference's gather (warp_ctct/__init__.py:124-131), the
     cast to float (:135), CTCTLoss (:20-33) and the reduction (:138-147).
     Forward runs gather, both lattices and the batch reduction on the GPU and
-    keeps their workspace; backward zero-fills the dense gradient at full HBM
-    write bandwidth and then writes the <= 3 non-zero entries per live row,
-    already weighted by the upstream gradient and by the reduction's own
-    factor (1/N, 1/lx[n]), so autograd launches nothing else.  A float16 or
-    bfloat16 joint is read as it is and its gradient is written in the same
-    type (the lattice itself always runs in float32 / float64)."""
+    keeps their workspace.  The dense gradient is all zeros but <= 3 entries
+    per live row, so its buffer is allocated in the forward and cleared, at
+    HBM write bandwidth, inside the launch of the lattice kernel (whose sweeps
+    are bound by latency and leave the memory system idle); backward then only
+    writes the non-zero entries, already weighted by the upstream gradient and by the
+    reduction's own factor (1/N, 1/lx[n]), so autograd launches nothing else.
+    A float16 or bfloat16 joint is read as it is and its gradient is written
+    in the same type (the lattice itself always runs in float32 / float64).
+
+    The cleared buffer serves one backward: a second backward through the same
+    graph (retain_graph=True) clears and fills a buffer of its own."""
 
     @staticmethod
     def forward(ctx, joint, labels, lx, ly, requires_grad, reduction, average_frames):
-        loss, workspace = _run("loss_forward", lambda: core.ctct_loss_joint_fwd(
-            joint, labels, lx, ly, requires_grad, _REDUCTION_CODE[reduction], average_frames))
+        clear = bool(requires_grad and CLEAR_GRADIENT_IN_FORWARD)
+        loss, workspace, dense = _run("loss_forward", lambda: core.ctct_loss_joint_fwd(
+            joint, labels, lx, ly, requires_grad, _REDUCTION_CODE[reduction], average_frames,
+            clear))
         if requires_grad:
             ctx.save_for_backward(workspace, labels, lx, ly)
             ctx.shape = tuple(joint.shape)
             ctx.like = joint.new_empty(0)
+            ctx.dense = dense if clear else None
             ctx.scale = 1.0 / joint.size(0) if reduction == "mean" else 1.0
             ctx.average_frames = bool(average_frames)
         return loss
@@ -113,7 +128,9 @@ class _CTCTLoss(torch.autograd.Function):
         workspace, labels, lx, ly = ctx.saved_tensors
         n, t, u1, v = ctx.shape
         grad_outputs = grad_outputs.reshape(-1).float().contiguous()
-        dense = _run("dense_zero_fill", lambda: core.dense_zero_fill(ctx.like, n, t, u1, v))
+        dense, ctx.dense = ctx.dense, None
+        if dense is None:
+            dense = _run("dense_zero_fill", lambda: core.dense_zero_fill(ctx.like, n, t, u1, v))
         _run("dense_patch", lambda: core.dense_patch_lattice(
             workspace, labels, lx, ly, grad_outputs, ctx.scale, ctx.average_frames, dense))
         return dense, None, None, None, None, None, None
