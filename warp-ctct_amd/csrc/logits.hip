@@ -99,107 +99,240 @@ __device__ __forceinline__ bool rows_vectorised(const IO *base, int V) {
     return (V % (16 / (int)sizeof(IO))) == 0 && (reinterpret_cast<uintptr_t>(base) & 15u) == 0;
 }
 
-// ROWS rows per wavefront (64 / ROWS lanes each): one for 4-byte elements, two
-// for 2-byte ones, so that a wavefront has 4 KiB of loads in flight either way.
-// Each group of lanes owns one cell (t,u) of the work buffer (P contexts per
-// frame) of sample blockIdx.y.  Live cells inside the band: logsumexp of the
-// row in one pass (running maximum and rescaled sum per lane, combined over
-// the group), then the three units.  Other cells of live frames: neutral
-// units, as gather_units_kernel.
-template <typename IO, int ROWS>
-__global__ __launch_bounds__(64 * kRowsPerBlock) void logits_units_kernel(
-    const IO *__restrict__ logits, const int *__restrict__ ys, const int *__restrict__ lx,
-    const int *__restrict__ ly, double *__restrict__ units, float *__restrict__ lse, int T, int U,
-    int V, int P, unsigned *__restrict__ counter) {
-    constexpr int LANES = 64 / ROWS;            // lanes per row
-    constexpr int EV = 16 / (int)sizeof(IO);    // elements per 16-byte vector
-    constexpr int NV = 1024 / (LANES * EV);     // vectors per lane and round of 1024 elements
-    if (counter && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *counter = 0u;
-    const int n = blockIdx.y;
-    const int lane = threadIdx.x & 63, hl = lane % LANES;
-    const int cell = (blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6)) * ROWS + lane / LANES;
-    const int t = cell / P, u = cell - t * P;
-    const int Tn = min(max(lx[n], 0), T), Un = min(max(ly[n], 0), U);
-    if (cell >= T * P || t >= Tn) return;
-    double *o = units + (((size_t)n * T + t) * P + u) * 3;
-    // The groups of a wavefront part ways here; what follows (loads, the
-    // reductions over LANES lanes) involves the lanes of one group only.
-    if (u > Un || outside_band(t, u, Tn, Un)) {
-        if (hl == 0) {
-            o[0] = 0.0;
-            o[1] = 0.0;
-            o[2] = neg_inf();
-        }
-        return;
-    }
-    const size_t r = ((size_t)n * T + t) * (U + 1) + u;
-    const IO *row = logits + r * (size_t)V;
-    // the three logits that become units are requested now (every lane of the
-    // group the same address), so that their latency runs in parallel with the
-    // row's instead of after the reduction
-    const int *y = ys + (size_t)n * U;
-    const int c1 = (u >= 1) ? min(max(y[u - 1], 0), V - 1) : 0;
-    const int c2 = (u < Un) ? min(max(y[u], 0), V - 1) : 0;
-    const float xb = load_as_float(row), x1 = load_as_float(row + c1), x2 = load_as_float(row + c2);
-    // running maximum m and sum s of 2^(x*log2e - m) over this lane's elements
-    float m = -__builtin_huge_valf(), s = 0.0f;
-    if (rows_vectorised(logits, V)) {
-        // 1024 elements per round: NV 16-byte vectors per lane, all loads issued
-        // before anything is computed (addresses past the row are clamped into
-        // it and the values dropped)
-        for (int k0 = 0; k0 < V; k0 += 1024) {
-            float x[NV][EV];
+// A 16-byte vector as loaded, and its EV elements as floats: a vector that is
+// still in flight costs 4 registers in this form, whatever the element type.
+typedef unsigned int raw16 __attribute__((ext_vector_type(4)));
+template <typename IO>
+__device__ __forceinline__ raw16 load_raw(const IO *p) {
+    return *reinterpret_cast<const raw16 *>(p);
+}
+__device__ __forceinline__ void unpack(const float *, const raw16 &v, float (&x)[4]) {
 #pragma unroll
-            for (int j = 0; j < NV; ++j)
-                load_vec(row + min(k0 + (j * LANES + hl) * EV, V - EV), x[j]);
-            float mn = m;
+    for (int i = 0; i < 4; ++i) x[i] = __uint_as_float(v[i]);
+}
+__device__ __forceinline__ void unpack(const __half *, const raw16 &v, float (&x)[8]) {
+    typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const v2h h = __builtin_bit_cast(v2h, v[i]);
+        x[2 * i] = (float)h[0];
+        x[2 * i + 1] = (float)h[1];
+    }
+}
+__device__ __forceinline__ void unpack(const __hip_bfloat16 *, const raw16 &v, float (&x)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        x[2 * i] = __uint_as_float(v[i] << 16);
+        x[2 * i + 1] = __uint_as_float(v[i] & 0xffff0000u);
+    }
+}
+
+// The element at byte offset `at` (0 or 2 for the 2-byte types) of a 32-bit word.
+__device__ __forceinline__ float word_element(const float *, unsigned word, unsigned) {
+    return __uint_as_float(word);
+}
+__device__ __forceinline__ float word_element(const __half *, unsigned word, unsigned at) {
+    const unsigned short bits = (unsigned short)(word >> (at * 8));
+    return (float)__builtin_bit_cast(_Float16, bits);
+}
+__device__ __forceinline__ float word_element(const __hip_bfloat16 *, unsigned word, unsigned at) {
+    return __uint_as_float((word >> (at * 8)) << 16);
+}
+
+// One workgroup of 4 wavefronts per frame (n, t) = (blockIdx.y, blockIdx.x).
+// Frames of padding cost one workgroup that retires at once.  The cells of a
+// live frame outside the band of complete alignments get neutral units, as in
+// gather_units_kernel, written by the whole workgroup in one sweep.  The rows
+// inside the band, u in [max(0, Un - (Tn - t)), min(Un, t)], are dealt to the
+// wavefronts round-robin; a wavefront walks over its rows in rounds of 1024
+// elements (NV 16-byte vectors per lane) and requests the next round before it
+// works on the present one, so that it always has a round in flight: logsumexp
+// of the row in one pass (running maximum and rescaled sum per lane, combined
+// over the wavefront at the end of the row), then the three units.
+template <typename IO, bool STAGED>
+__global__ __launch_bounds__(64 * kRowsPerBlock)
+    __attribute__((amdgpu_waves_per_eu(sizeof(IO) == 4 ? 6 : 8, 8))) void
+    logits_units_kernel(const IO *__restrict__ logits, const int *__restrict__ ys,
+                    const int *__restrict__ lx, const int *__restrict__ ly,
+                    double *__restrict__ units, float *__restrict__ lse, int T, int U, int V, int P,
+                    unsigned *__restrict__ counter) {
+    constexpr int EV = 16 / (int)sizeof(IO);    // elements per 16-byte vector
+    constexpr int NV = 1024 / (64 * EV);        // vectors per lane and round of 1024 elements
+    if (counter && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *counter = 0u;
+    const int n = blockIdx.y, t = blockIdx.x;
+    const int Tn = min(max(lx[n], 0), T), Un = min(max(ly[n], 0), U);
+    if (t >= Tn) return;
+    // the wavefront's index as a scalar: rows, labels and the three logits that
+    // become units are then addressed (and the latter two loaded) by the scalar
+    // unit, whose loads do not queue behind the row's vector loads
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ulo = max(0, Un - (Tn - t)), uhi = min(Un, t);
+    double *frame = units + ((size_t)n * T + t) * P * 3;
+    // STAGED: the frame's units (P x 3 doubles, neutral outside the band) and
+    // logsumexps (P floats) are put together in LDS and written out in one
+    // sweep at the end.  A global store inside the loop over the rows would
+    // make every re-use of its data registers wait for the store, and with it
+    // for the loads of the next round, which must stay in flight.
+    extern __shared__ double staged[];
+    double *frame_out = STAGED ? staged : frame;
+    float *lse_out = STAGED ? reinterpret_cast<float *>(staged + (size_t)P * 3)
+                            : lse + ((size_t)n * T + t) * (U + 1);
+    for (int i = threadIdx.x; i < P * 3; i += 64 * kRowsPerBlock) {
+        const int u = i / 3;
+        if (STAGED || u < ulo || u > uhi) frame_out[i] = (i - u * 3 == 2) ? neg_inf() : 0.0;
+    }
+    if (STAGED) __syncthreads();
+    const int *y = ys + (size_t)n * U;
+    const size_t r0 = ((size_t)n * T + t) * (U + 1);
+    const bool vec = rows_vectorised(logits, V);
+
+    // the end of a row: every lane holds m (maximum of its raw values) and s
+    // (sum of e^(x - m)); xb, x1, x2 are the logits that become units
+    auto finish_row = [&](int u, float m, float s, float xb, float x1, float x2) {
+        const float M = group_max<64>(m);
+        const float Mf = fmaxf(M, -2.0e38f);
+        const float S = group_sum<64>(s * exp2_hw((m - Mf) * kLog2eF));
+        if (lane != 0) return;
+        const float l = M + log2_hw(S) * kLn2F;   // natural-log logsumexp of the row
+        lse_out[u] = l;
+        double *o = frame_out + (size_t)u * 3;
+        const double b = (double)xb - (double)l;
+        double cur = b, nxt = neg_inf();
+        if (u >= 1) cur = (double)x1 - (double)l;
+        if (u < Un) nxt = ((double)x2 - (double)l) * kLog2e;
+        o[0] = b * kLog2e;
+        o[1] = cur * kLog2e;
+        o[2] = nxt;
+    };
+    if (!vec) {   // rows that cannot be read as 16-byte vectors: element by element
+        for (int u = ulo + wave; u <= uhi; u += kRowsPerBlock) {
+            const IO *row = logits + (r0 + u) * (size_t)V;
+            const int c1 = (u >= 1) ? min(max(y[u - 1], 0), V - 1) : 0;
+            const int c2 = (u < Un) ? min(max(y[u], 0), V - 1) : 0;
+            const float xb = load_as_float(row), x1 = load_as_float(row + c1),
+                        x2 = load_as_float(row + c2);
+            float m = -__builtin_huge_valf(), s = 0.0f;
+            for (int k = lane; k < V; k += 64) {
+                const float x = load_as_float(row + k);
+                const float mn = fmaxf(m, x);
+                const float mf = fmaxf(mn, -2.0e38f);
+                s = s * exp2_hw((m - mf) * kLog2eF) + exp2_hw((x - mf) * kLog2eF);
+                m = mn;
+            }
+            finish_row(u, m, s, xb, x1, x2);
+        }
+    }
+    // One step = one round of one row.  Two register sets hold the step being
+    // worked on and the one in flight.
+    struct Step {
+        int u, k0;
+    };
+    auto next_step = [&](Step at) {
+        Step nx = {at.u, at.k0 + 1024};
+        if (nx.k0 >= V) nx = Step{at.u + kRowsPerBlock, 0};
+        return nx;
+    };
+    // One element at a wavefront-uniform index: the aligned 32-bit word that
+    // holds it (a scalar load; the tensor starts on a 16-byte boundary here),
+    // then the element out of the word.
+    const unsigned *words = reinterpret_cast<const unsigned *>(logits);
+    auto uniform_element = [&](size_t index) {
+        const size_t byte = index * sizeof(IO);
+        return word_element(logits, words[byte >> 2], (unsigned)(byte & 3u));
+    };
+    // A step past the last row asks for the last row again (and is dropped):
+    // every step issues the same vector loads, so that the wait for a step's
+    // vectors can leave exactly the next step's in flight.  The three logits
+    // that become units come through the scalar unit (every lane would ask for
+    // the same address), which keeps them out of that count.
+    auto request = [&](Step at, raw16 (&raw)[NV], float (&side)[3]) {
+        const int u = min(at.u, uhi);
+        const size_t first = (r0 + u) * (size_t)V;
+        const IO *row = logits + first;
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+            raw[j] = load_raw(row + min(at.k0 + (j * 64 + lane) * EV, V - EV));
+        if (at.k0 == 0) {
+            const int c1 = (u >= 1) ? min(max(y[u - 1], 0), V - 1) : 0;
+            const int c2 = (u < Un) ? min(max(y[u], 0), V - 1) : 0;
+            side[0] = uniform_element(first);
+            side[1] = uniform_element(first + c1);
+            side[2] = uniform_element(first + c2);
+        }
+    };
+    float m = -__builtin_huge_valf(), s = 0.0f;
+    float xb = 0.0f, x1 = 0.0f, x2 = 0.0f;
+    auto work = [&](Step at, const raw16 (&raw)[NV], const float (&side)[3]) {
+        if (at.k0 == 0) xb = side[0], x1 = side[1], x2 = side[2];
+        float x[NV][EV];
+#pragma unroll
+        for (int j = 0; j < NV; ++j) unpack(logits, raw[j], x[j]);
+        if (at.k0 + 1024 > V) {   // the last, partial round: drop what lies past the row
 #pragma unroll
             for (int j = 0; j < NV; ++j) {
-                const bool in = (k0 + (j * LANES + hl) * EV) < V;
+                const bool in = (at.k0 + (j * 64 + lane) * EV) < V;
 #pragma unroll
-                for (int i = 0; i < EV; ++i) {
-                    x[j][i] = in ? x[j][i] * kLog2eF : -__builtin_huge_valf();
-                    mn = fmaxf(mn, x[j][i]);
-                }
+                for (int i = 0; i < EV; ++i) x[j][i] = in ? x[j][i] : -__builtin_huge_valf();
             }
-            // mn = -inf only while everything seen is -inf: keep s = 0
-            const float mf = fmaxf(mn, -3.0e38f);
-            float acc = s * exp2_hw(m - mf);
-#pragma unroll
-            for (int j = 0; j < NV; ++j)
-#pragma unroll
-                for (int i = 0; i < EV; ++i) acc += exp2_hw(x[j][i] - mf);
-            s = acc;
-            m = mn;
         }
-    } else {
-        for (int k = hl; k < V; k += LANES) {
-            const float x = load_as_float(row + k) * kLog2eF;
-            const float mn = fmaxf(m, x);
-            const float mf = fmaxf(mn, -3.0e38f);
-            s = s * exp2_hw(m - mf) + exp2_hw(x - mf);
-            m = mn;
+        float mn = m;
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+#pragma unroll
+            for (int i = 0; i < EV; ++i) mn = fmaxf(mn, x[j][i]);
+        // mn = -inf only while everything seen is -inf: keep s = 0 (the floor
+        // times log2(e) must stay finite)
+        const float mf = fmaxf(mn, -2.0e38f);
+        const float shift = -mf * kLog2eF;
+        float acc = s * exp2_hw((m - mf) * kLog2eF);
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+#pragma unroll
+            for (int i = 0; i < EV; ++i) acc += exp2_hw(fmaf(x[j][i], kLog2eF, shift));
+        s = acc;
+        m = mn;
+        if (at.k0 + 1024 >= V) {
+            finish_row(at.u, m, s, xb, x1, x2);
+            m = -__builtin_huge_valf(), s = 0.0f;
         }
+    };
+    raw16 raw_a[NV], raw_b[NV];
+    float side_a[3] = {0.0f, 0.0f, 0.0f}, side_b[3] = {0.0f, 0.0f, 0.0f};
+    Step sa = {ulo + wave, 0};
+    if (vec && sa.u <= uhi) {
+        // Both register sets are kept in flight: a set is asked for again as soon
+        // as its step has been worked on.  The steps of this wavefront are
+        // counted beforehand and walked in pairs without a branch in between
+        // (with one, the compiler's count of outstanding loads turns cautious
+        // and it waits for both sets at once).
+        const int rounds = (V + 1023) / 1024;
+        const int steps = ((uhi - sa.u) / kRowsPerBlock + 1) * rounds;
+        Step sb = next_step(sa);
+        request(sa, raw_a, side_a);
+        request(sb, raw_b, side_b);
+        int i = 0;
+        for (; i + 2 <= steps; i += 2) {
+            work(sa, raw_a, side_a);
+            sa = next_step(sb);
+            request(sa, raw_a, side_a);
+            work(sb, raw_b, side_b);
+            sb = next_step(sa);
+            request(sb, raw_b, side_b);
+        }
+        if (i < steps) work(sa, raw_a, side_a);
     }
-    const float M = group_max<LANES>(m);
-    const float Mf = fmaxf(M, -3.0e38f);
-    const float S = group_sum<LANES>(s * exp2_hw(m - Mf));
-    if (hl != 0) return;
-    const float l = (M + log2_hw(S)) * kLn2F;   // natural-log logsumexp of the row
-    lse[r] = l;
-    const double b = (double)xb - (double)l;
-    double cur = b, nxt = neg_inf();
-    if (u >= 1) cur = (double)x1 - (double)l;
-    if (u < Un) nxt = ((double)x2 - (double)l) * kLog2e;
-    o[0] = b * kLog2e;
-    o[1] = cur * kLog2e;
-    o[2] = nxt;
+    if (!STAGED) return;
+    __syncthreads();
+    for (int i = threadIdx.x; i < P * 3; i += 64 * kRowsPerBlock) frame[i] = staged[i];
+    float *lse_row = lse + ((size_t)n * T + t) * (U + 1);
+    for (int u = ulo + threadIdx.x; u <= uhi; u += 64 * kRowsPerBlock) lse_row[u] = lse_out[u];
 }
 
 // ROWS rows (n,t,u) of the gradient per wavefront, 64 / ROWS lanes each (see
 // logits_units_kernel); blockIdx.y = n.
 template <typename IO, int ROWS>
-__global__ __launch_bounds__(64 * kGradWaves) void logits_grad_kernel(
+__global__ __launch_bounds__(64 * kGradWaves) __attribute__((amdgpu_waves_per_eu(8, 8))) void
+logits_grad_kernel(
     const IO *__restrict__ logits, const float *__restrict__ lse, const double *__restrict__ units,
     const double *__restrict__ alphas, const double *__restrict__ betas,
     const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
@@ -248,6 +381,7 @@ __global__ __launch_bounds__(64 * kGradWaves) void logits_grad_kernel(
     const int c1 = (u >= 1) ? min(max(y[u - 1], 0), V - 1) : -1;
     const int c2 = (u < Un) ? min(max(y[u], 0), V - 1) : -1;
     const float shift = lse[r] * kLog2eF;
+    const float neg_shift = -shift, neg_total = -total;
     if (vec) {
         for (int k0 = 0; k0 < V; k0 += ROUND) {
             if (k0 > 0) {
@@ -260,13 +394,21 @@ __global__ __launch_bounds__(64 * kGradWaves) void logits_grad_kernel(
                 const int k = k0 + (j * LANES + hl) * EV;
                 if (k >= V) continue;
 #pragma unroll
-                for (int i = 0; i < EV; ++i) {
-                    float v = -total * exp2_hw(x[j][i] * kLog2eF - shift);
-                    const int col = k + i;
-                    if (col == 0) v += g0;
-                    if (col == c1) v += g1;
-                    if (col == c2) v += g2;
-                    x[j][i] = v;
+                for (int i = 0; i < EV; ++i)
+                    x[j][i] = neg_total * exp2_hw(fmaf(x[j][i], kLog2eF, neg_shift));
+                // the <= 3 columns that also receive a unit gradient: looked for
+                // per vector, not per element (few lanes ever find one)
+                if ((unsigned)(0 - k) < (unsigned)EV || (unsigned)(c1 - k) < (unsigned)EV ||
+                    (unsigned)(c2 - k) < (unsigned)EV) {
+#pragma unroll
+                    for (int i = 0; i < EV; ++i) {
+                        const int col = k + i;
+                        float add = 0.0f;
+                        if (col == 0) add += g0;
+                        if (col == c1) add += g1;
+                        if (col == c2) add += g2;
+                        x[j][i] += add;
+                    }
                 }
                 store_vec(out + k, x[j]);
             }
@@ -290,12 +432,16 @@ void launch_units_typed(const void *logits, const int *ys, const int *lx, const 
                         double *units, float *lse, int N, int T, int U, int V, unsigned *counter,
                         hipStream_t stream) {
     const int P = padded_contexts(U);
-    const long cells = (long)T * P;
-    constexpr int ROWS = RowsPerWave<IO>::value, PER_BLOCK = kRowsPerBlock * ROWS;
-    dim3 grid((unsigned)((cells + PER_BLOCK - 1) / PER_BLOCK), (unsigned)N);
-    TIMED_LAUNCH((logits_units_kernel<IO, ROWS>), grid, dim3(64 * kRowsPerBlock), 0, stream,
-                       static_cast<const IO *>(logits), ys, lx, ly, units, lse, T, U, V, P,
-                       counter);
+    const size_t staged = (size_t)P * (3 * sizeof(double) + sizeof(float));
+    if (staged <= 64 * 1024) {
+        TIMED_LAUNCH((logits_units_kernel<IO, true>), dim3((unsigned)T, (unsigned)N),
+                     dim3(64 * kRowsPerBlock), staged, stream, static_cast<const IO *>(logits), ys,
+                     lx, ly, units, lse, T, U, V, P, counter);
+    } else {   // a frame too wide for LDS: results stored row by row
+        TIMED_LAUNCH((logits_units_kernel<IO, false>), dim3((unsigned)T, (unsigned)N),
+                     dim3(64 * kRowsPerBlock), 0, stream, static_cast<const IO *>(logits), ys, lx,
+                     ly, units, lse, T, U, V, P, counter);
+    }
 }
 
 template <typename IO>
