@@ -7,8 +7,9 @@ One step = forward + backward of warp_ctct.ctct_loss on one resident batch of
 the "typical ASR batch" workload: N=32, frames 150..250, labels 30..60,
 V=1024, fp32 joint log-probs already in HBM, padded regions zero-filled.
 Prints ONE JSON line: whole-job lattices/s, the roofline of the dominant
-kernel (the zero-fill of the dense gradient, timed with HIP events on its
-stream inside the timed region), a CPU baseline (the C oracle with OpenMP, on
+kernel (lattice_fill_kernel: the clear of the dense gradient with the lattice
+sweeps riding in the same launch, timed with HIP events on its stream inside
+the timed region), a CPU baseline (the C oracle with OpenMP, on
 the host cores, same batch) and, under "configs", the same measurement for all
 five benchmark configurations with the HIP-event duration of every kernel of
 a step (the library's own per-kernel timing, warpctct_profile).
@@ -28,12 +29,13 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix, published
-# HBM bytes per launch of zero_fill_vec_kernel from two rocprofv3 --pmc runs
-# (profiles/ctct_loss_typical_batch_pmc.md): WRITE_SIZE 1 952 000 KiB x 1.0 +
-# FETCH_SIZE 12.8 KiB x 2.0, the factors being what the same counters read for
-# a plain 1 GiB -> 1 GiB elementwise kernel (WRITE_SIZE 1 048 576, FETCH_SIZE
-# 524 300 KiB).
-ZERO_FILL_TRAFFIC_BYTES = 1952000 * 1024 + int(12.8 * 2 * 1024)
+# HBM bytes per launch of lattice_fill_kernel (the clear of the dense gradient
+# with the lattice sweeps in the same launch) from two rocprofv3 --pmc runs
+# (profiles/ctct_loss_typical_batch_pmc.md): WRITE_SIZE 1 964 748 KiB x 1.0 +
+# FETCH_SIZE 9 710.3 KiB x 2.0, the factors being what the same counters read
+# for a plain 1 GiB -> 1 GiB elementwise kernel (WRITE_SIZE 1 048 576,
+# FETCH_SIZE 524 300 KiB).
+LATTICE_FILL_TRAFFIC_BYTES = 1964748 * 1024 + int(9710.3 * 2 * 1024)
 
 
 def make_batch(torch, N, T, U, V, seed=2024):
@@ -244,11 +246,13 @@ def summarise(name, facts, sec_per_step, kernels):
         out["algorithmic_bytes_per_step"] = facts["algorithmic_bytes_per_step"]
         out["step_frac_of_hbm_roofline"] = (facts["algorithmic_bytes_per_step"] / sec_per_step / 1e9
                                             / HBM_PEAK_GBS)
+    # (lattice_fill_kernel, the sweeps with the clear of the dense gradient in
+    # the same launch, is as long as the clear: no figure per frame from it)
     lattice = sum(v for k, v in us.items() if k.startswith("lattice_kernel"))
     if lattice > 0:
         out["lattice_kernel_us"] = lattice
         out["lattice_ns_per_frame"] = lattice * 1e3 / facts["max_frames"]
-    fill = us.get("zero_fill_vec_kernel")
+    fill = us.get("lattice_fill_kernel")
     if name == "c1" or facts["kind"] == "simple_unnorm":
         out["roofline"] = {"bound": "latency", "kernel": "lattice_kernel",
                            "note": "serial recursion over max_frames dependent steps; reported as "
@@ -256,7 +260,7 @@ def summarise(name, facts, sec_per_step, kernels):
                            "max_frames": facts["max_frames"]}
     elif facts["kind"] == "full" and fill:
         gbs = facts["dense_gradient_bytes"] / (fill * 1e-6) / 1e9
-        out["roofline"] = {"bound": "hbm", "kernel": "zero_fill_vec_kernel", "achieved": gbs,
+        out["roofline"] = {"bound": "hbm", "kernel": "lattice_fill_kernel", "achieved": gbs,
                            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
                            "avg_launch_us": fill,
                            "algorithmic_bytes_per_launch": facts["dense_gradient_bytes"]}
@@ -413,7 +417,7 @@ def main():
                        (dense_b + gathered_b + small_b) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS},
         "roofline": {"bound": "hbm", "kernel": "lattice_fill_kernel", "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": ZERO_FILL_TRAFFIC_BYTES, "avg_launch_us": dense_ms * 1e3,
+                     "traffic": LATTICE_FILL_TRAFFIC_BYTES, "avg_launch_us": dense_ms * 1e3,
                      "algorithmic_bytes_per_launch": dense_b},
         "loss": float(loss),
     }
