@@ -34,9 +34,12 @@ __device__ __forceinline__ void load4(const float *p, float (&x)[4]) {
     x[2] = v.z;
     x[3] = v.w;
 }
+// (the stores of the gradient are non-temporal: it is not read again by this
+// path, and written the ordinary way 2 GB of it linger in the caches and are
+// written back while the next forward runs: 231 us instead of 188 us there)
 __device__ __forceinline__ void store4(float *p, const float (&x)[4]) {
     typedef float v4f __attribute__((ext_vector_type(4)));
-    *reinterpret_cast<v4f *>(p) = v4f{x[0], x[1], x[2], x[3]};
+    __builtin_nontemporal_store(v4f{x[0], x[1], x[2], x[3]}, reinterpret_cast<v4f *>(p));
 }
 
 // 16-byte vectors of 2-byte elements
@@ -68,7 +71,8 @@ __device__ __forceinline__ void store8(IO *p, const float (&x)[8]) {
     v.y = pack2(p, x[2], x[3]);
     v.z = pack2(p, x[4], x[5]);
     v.w = pack2(p, x[6], x[7]);
-    *reinterpret_cast<uint4 *>(p) = v;
+    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+    __builtin_nontemporal_store(u4{v.x, v.y, v.z, v.w}, reinterpret_cast<u4 *>(p));
 }
 // EV elements = one 16-byte vector of the element type
 __device__ __forceinline__ void load_vec(const float *p, float (&x)[4]) { load4(p, x); }
@@ -356,8 +360,9 @@ logits_grad_kernel(
         if (vec) {
             // zeros in 16-byte pieces whatever the element type
             constexpr int E16 = 16 / (int)sizeof(IO);
-            const uint4 zero = {0u, 0u, 0u, 0u};
-            for (int k = hl * E16; k < V; k += LANES * E16) *reinterpret_cast<uint4 *>(out + k) = zero;
+            typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+            for (int k = hl * E16; k < V; k += LANES * E16)
+                __builtin_nontemporal_store(u4{0u, 0u, 0u, 0u}, reinterpret_cast<u4 *>(out + k));
         } else {
             for (int k = hl; k < V; k += LANES) store_from_float(out + k, 0.0f);
         }
