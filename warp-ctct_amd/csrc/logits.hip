@@ -25,10 +25,13 @@ constexpr int kGradWaves = 1;          // ... and backward: 4 KiB per workgroup,
 constexpr float kLog2eF = 1.4426950408889634f;
 constexpr float kLn2F = 0.6931471805599453f;
 
-// one 16-byte vector of floats
+// one 16-byte vector of floats (these loads serve the backward, which is the
+// last to read a row: non-temporal, 503 -> 475 us for the typical batch; the
+// forward's loads stay ordinary, the backward finds part of its rows in the
+// memory-side cache because of them)
 __device__ __forceinline__ void load4(const float *p, float (&x)[4]) {
     typedef float v4f __attribute__((ext_vector_type(4)));
-    const v4f v = *reinterpret_cast<const v4f *>(p);
+    const v4f v = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(p));
     x[0] = v.x;
     x[1] = v.y;
     x[2] = v.z;
@@ -45,13 +48,13 @@ __device__ __forceinline__ void store4(float *p, const float (&x)[4]) {
 // 16-byte vectors of 2-byte elements
 __device__ __forceinline__ void load8(const __half *p, float (&x)[8]) {
     typedef _Float16 v8h __attribute__((ext_vector_type(8)));
-    const v8h v = *reinterpret_cast<const v8h *>(p);
+    const v8h v = __builtin_nontemporal_load(reinterpret_cast<const v8h *>(p));
 #pragma unroll
     for (int i = 0; i < 8; ++i) x[i] = (float)v[i];
 }
 __device__ __forceinline__ void load8(const __hip_bfloat16 *p, float (&x)[8]) {
     typedef unsigned short v8u __attribute__((ext_vector_type(8)));
-    const v8u v = *reinterpret_cast<const v8u *>(p);
+    const v8u v = __builtin_nontemporal_load(reinterpret_cast<const v8u *>(p));
 #pragma unroll
     for (int i = 0; i < 8; ++i) x[i] = __uint_as_float((unsigned)v[i] << 16);
 }
