@@ -276,7 +276,10 @@ __global__ __launch_bounds__(kBlock) void simple_dense_f_rows_kernel(
         typedef float v4f __attribute__((ext_vector_type(4)));
         const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
         for (int k = threadIdx.x * 4; k < V; k += kBlock * 4)
-            *reinterpret_cast<v4f *>(out + k) = live ? *reinterpret_cast<const v4f *>(row + k) : zero;
+            // (non-temporal: nothing of this path reads the rows again, and their
+            // write-back would run into the next step's gather)
+            __builtin_nontemporal_store(live ? *reinterpret_cast<const v4f *>(row + k) : zero,
+                                        reinterpret_cast<v4f *>(out + k));
     } else {
         for (int k = threadIdx.x; k < V; k += kBlock) out[k] = live ? row[k] : 0.0f;
     }
