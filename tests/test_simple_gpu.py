@@ -25,7 +25,14 @@ def dev(a, dtype=None):
 
 
 # ------------------------------------------------------------------ log matmul
-@pytest.mark.parametrize("B,M,K,Nn", [(1, 1, 1, 1), (2, 5, 7, 3), (3, 70, 100, 33), (2, 130, 257, 81)])
+@pytest.mark.parametrize("B,M,K,Nn", [
+    (1, 1, 1, 1), (2, 5, 7, 3), (3, 70, 100, 33), (2, 130, 257, 81),
+    # long reductions: the form that keeps a slab of the right operand in LDS
+    # (512 <= K rounded up to 32 <= 2048): whole and partial slabs, one to three
+    # column tiles, fewer rows than a row block and a ragged last block
+    (2, 37, 512, 81), (1, 130, 777, 100), (2, 21, 2048, 200), (1, 5, 1500, 3), (3, 16, 1024, 64),
+    # and just beyond it
+    (1, 9, 2049, 7)])
 @pytest.mark.parametrize("layout", ["contiguous", "transposed_view"])
 def test_log_matmul_forward(B, M, K, Nn, layout):
     from warp_ctct import _C

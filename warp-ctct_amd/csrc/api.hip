@@ -87,7 +87,7 @@ int forward_from_units(const Workspace &w, const int *ys, const int *lx, const i
 struct SimpleWorkspace {
     Workspace lattice;
     float *unit_grads;   // (N,T,U+1,3)
-    float *partial;      // up to 8 x (N,T,U+1): partial sums of a split log-matmul reduction
+    float *partial;      // logmm_fwd_partial_floats: partial sums of a split log-matmul reduction
     size_t bytes;
 };
 
@@ -98,7 +98,7 @@ SimpleWorkspace carve_simple(void *base, int N, int T, int U) {
     const size_t ug_b = align256((size_t)N * T * (U + 1) * 3 * sizeof(float));
     w.unit_grads = reinterpret_cast<float *>(p);
     w.partial = reinterpret_cast<float *>(p + ug_b);
-    w.bytes = w.lattice.bytes + ug_b + align256((size_t)8 * N * T * (U + 1) * sizeof(float));
+    w.bytes = w.lattice.bytes + ug_b + align256(logmm_fwd_partial_floats(N, T, U + 1) * sizeof(float));
     return w;
 }
 
@@ -142,7 +142,7 @@ LogmmWorkspace carve_logmm(void *base, int B, int M, int K, int Nn) {
     w.pw = carve_pairs(reinterpret_cast<void *>(p), B, M, Nn);
     p += w.pw.bytes;
     w.partial = reinterpret_cast<float *>(p);
-    p += align256((size_t)logmm_fwd_splits(B, M, K, Nn) * B * M * Nn * sizeof(float));
+    p += align256(logmm_fwd_partial_floats(B, M, Nn) * sizeof(float));
     w.bytes = p - p0;
     return w;
 }

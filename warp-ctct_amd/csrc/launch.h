@@ -168,9 +168,11 @@ struct LogmmShifted {
 hipError_t launch_logmm_shift_exp(const LogmmOperand &lhs, const LogmmOperand &rhs,
                                   const LogmmShifted &sh, int B, int M, int K, int Nn,
                                   const int *row_len, const int *col_len, hipStream_t stream);
-// partial (may be null): logmm_fwd_splits(B,M,K,Nn) * B*M*Nn floats of scratch; with it the
+// partial (may be null): logmm_fwd_partial_floats(B,M,Nn) floats of scratch; with it the
 // reduction of a small output is split over several workgroups per tile
 int logmm_fwd_splits(int B, int M, int K, int Nn);
+// floats of `partial` that launch_logmm_fwd may use, whatever K is
+size_t logmm_fwd_partial_floats(int B, int M, int Nn);
 hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
                             const LogmmShifted &sh, float *res, float *partial, int B, int M,
                             int K, int Nn, const int *row_len, const int *col_len,

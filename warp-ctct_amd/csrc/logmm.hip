@@ -270,6 +270,7 @@ struct FwdArgs {
     // partial (splits,B,M,Nn) and logmm_fwd_finish_kernel adds them up
     float *partial;
     int splits, chunks_per_split;
+    int pM, pN;               // rows and row length of one partial sum (>= M, Nn)
     int M, K, Kp, Nn;
     int B, tiles_x, tiles_y;  // batch entries, row tiles, column tiles * splits
     const int *row_len, *col_len;
@@ -401,6 +402,174 @@ __global__ __launch_bounds__(64 * WR * WC) void logmm_fwd_kernel(const FwdArgs a
     }
 }
 
+// ---- fp32 products on the bfloat16 matrix cores -------------------------------
+// An fp32 value x is split into three bfloat16 values h + m + l (each rounded to
+// nearest even from what the ones before left over): 24 bits of mantissa, i.e.
+// all of x but for values near the bottom of the fp32 range.  A product of two
+// such sums, cut after the terms of order 2^-16 (lh, hl, mm, mh, hm, hh; small
+// ones first), is as accurate as an fp32 product: measured relative error of a
+// dot product of length 2048: 4e-8 (plain fp32 accumulation: 2e-6).  Six
+// v_mfma_f32_16x16x32_bf16 do per 32 reduction indices what eight
+// v_mfma_f32_16x16x4_f32 do per 32 in fp32, in 96 instead of 256 cycles.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+
+struct Split3 {
+    __bf16 h, m, l;
+};
+__device__ __forceinline__ Split3 split3(float x) {
+    Split3 s;
+    s.h = (__bf16)x;
+    const float r1 = x - (float)s.h;
+    s.m = (__bf16)r1;
+    s.l = (__bf16)(r1 - (float)s.m);
+    return s;
+}
+// acc += x * y for 16x16 outputs over 32 reduction indices, x and y given as
+// their three planes (each lane holds 8 consecutive reduction indices of its
+// row / column)
+__device__ __forceinline__ v4f mfma6(const bf16x8 (&x)[3], const bf16x8 (&y)[3], v4f acc) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(x[2], y[0], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(x[0], y[2], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(x[1], y[1], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(x[1], y[0], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(x[0], y[1], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(x[0], y[0], acc, 0, 0, 0);
+    return acc;
+}
+
+// The forward for few columns (Nn up to a few hundred: the label axis of a
+// joiner) and a long reduction: the product is bound by streaming E_l once, as
+// long as E_r stays on the chip.  A workgroup of 4 wavefronts takes one batch
+// entry, one tile of 16*CB columns and one slab of kSlab reduction indices;
+// that slab of E_r is split into its three bfloat16 planes and put into LDS
+// once (3 x 16*CB x kSlab bfloat16, ~150 KB), and all rows of E_l pass through
+// registers against it: a wavefront walks over blocks of 16 rows, a lane loads
+// its 8 consecutive k of a row and chunk of 32 as two 16-byte vectors of fp32
+// and splits them in registers, and half a block's vectors (4 chunks) are
+// requested again as soon as they have been multiplied.  No barrier and no LDS
+// write inside the loop.  Each slab writes its partial sums;
+// logmm_fwd_finish_kernel adds them in a fixed order.
+constexpr int kSlab = 256;
+constexpr int kSlabLd = kSlab + 8;   // bfloat16 per LDS row: 16-byte aligned, rows 4 banks apart
+constexpr int kSlabWaves = 8;        // two wavefronts per SIMD: one's matrix instructions cover the other's waits
+
+template <int CB>
+__global__ __launch_bounds__(64 * kSlabWaves) void logmm_fwd_slab_kernel(const FwdArgs a, int slabs) {
+    constexpr int TN = 16 * CB, NW = kSlabWaves, NT = 64 * NW;
+    constexpr int CH = kSlab / TQ / 2;                  // chunks of 32 per half slab
+    constexpr int GB = CB / 2;                          // column blocks per group
+    extern __shared__ __attribute__((aligned(16))) __bf16 s_b[];   // [3][TN][kSlabLd]
+    const int b = blockIdx.y;
+    const int slab = blockIdx.x % slabs, j0 = (blockIdx.x / slabs) * TN;
+    const int M = a.M, Nn = a.Nn, Kp = a.Kp;
+    const int Mb = a.row_len ? min(max(a.row_len[b], 0), M) : M;
+    const int Nb = a.col_len ? min(max(a.col_len[b], 0) + 1, Nn) : Nn;
+    if (Mb <= 0 || j0 >= Nb) return;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, g = lane >> 4;
+    const int row_blocks = (Mb + 15) / 16;
+    const int steps = (row_blocks - wave + NW - 1) / NW;   // row blocks of this wavefront
+    // one partial sum is (pM, pN) floats, whole row blocks and column tiles: the
+    // stores below need no conditions (and are then counted exactly by the
+    // compiler when it waits for the loads in flight around them)
+    float *part = a.partial + ((size_t)slab * a.B + b) * a.pM * a.pN;
+    const int k0 = slab * kSlab;
+    for (int e = tid; e < TN * (kSlab / 4); e += NT) {
+        const int row = e / (kSlab / 4), c4 = e - row * (kSlab / 4);
+        const int k = k0 + c4 * 4;
+        v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (k < Kp)
+            v = *reinterpret_cast<const v4f *>(a.Er + ((size_t)b * Nn + min(j0 + row, Nn - 1)) * Kp + k);
+        bf16x4 h, m, l;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const Split3 sp = split3(v[i]);
+            h[i] = sp.h, m[i] = sp.m, l[i] = sp.l;
+        }
+        __bf16 *at = s_b + (size_t)row * kSlabLd + c4 * 4;
+        *reinterpret_cast<bf16x4 *>(at) = h;
+        *reinterpret_cast<bf16x4 *>(at + (size_t)TN * kSlabLd) = m;
+        *reinterpret_cast<bf16x4 *>(at + (size_t)2 * TN * kSlabLd) = l;
+    }
+    __syncthreads();
+    if (steps <= 0) return;
+    // Two register sets, each one half (4 chunks = 8 vectors per lane) of a row
+    // block's share of the slab; a half is requested for the next row block as
+    // soon as it has been multiplied, so both are always in flight, and a row
+    // block is walked without a branch (the waits are then counted exactly).
+    // Vectors past the reduction are clamped into it (they meet zeros of the
+    // slab), row blocks past the last repeat it (and are dropped).
+    auto request = [&](int st, int half, v4f (&A)[2 * CH]) {
+        const int rb = wave + NW * min(st, steps - 1);
+        const float *row = a.El + ((size_t)b * M + min(rb * 16 + r, M - 1)) * Kp;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int k = min(k0 + TQ * (half * CH + c) + 8 * g, Kp - 8);
+            A[2 * c] = *reinterpret_cast<const v4f *>(row + k);
+            A[2 * c + 1] = *reinterpret_cast<const v4f *>(row + k + 4);
+        }
+    };
+    v4f acc[CB];
+    // E_r's planes are read from LDS right before the matrix instructions that
+    // use them, one group of GB column blocks at a time (the scheduler is held to
+    // that: left alone it hoists all reads of a half and spills); the other
+    // wavefront of the SIMD covers the wait.
+    auto multiply = [&](int half, const v4f (&A)[2 * CH]) {
+        bf16x8 xp[3];
+#pragma unroll
+        for (int item = 0; item < 2 * CH; ++item) {
+            const int c = item >> 1, grp = item & 1;
+            bf16x8 bq[GB][3];
+#pragma unroll
+            for (int cb = 0; cb < GB; ++cb)
+#pragma unroll
+                for (int p = 0; p < 3; ++p)
+                    bq[cb][p] = *reinterpret_cast<const bf16x8 *>(
+                        s_b + ((size_t)p * TN + (grp * GB + cb) * 16 + r) * kSlabLd +
+                        TQ * (half * CH + c) + 8 * g);
+            if (grp == 0) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const Split3 sp = split3(i < 4 ? A[2 * c][i] : A[2 * c + 1][i - 4]);
+                    xp[0][i] = sp.h, xp[1][i] = sp.m, xp[2][i] = sp.l;
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int cb = 0; cb < GB; ++cb)
+                acc[grp * GB + cb] = mfma6(xp, bq[cb], acc[grp * GB + cb]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    v4f A0[2 * CH], A1[2 * CH];
+    request(0, 0, A0);
+    // (the two halves in this order, as in the loop: the waits for a half are
+    // counted from the loads issued after it)
+    __builtin_amdgcn_sched_barrier(0);
+    request(0, 1, A1);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int st = 0; st < steps; ++st) {
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) acc[cb] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        multiply(0, A0);
+        request(st + 1, 0, A0);
+        multiply(1, A1);
+        // lane l holds D[4*(l/16) + q][l%16] of each block in register q; the
+        // stores come before the second request, so that at the head of the
+        // loop nothing but the two halves is outstanding
+        const int i0 = (wave + NW * st) * 16 + 4 * g;
+        float *at = part + (size_t)i0 * a.pN + j0 + r;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) at[(size_t)q * a.pN + cb * 16] = acc[cb][q];
+        __builtin_amdgcn_sched_barrier(0);
+        request(st + 1, 1, A1);
+    }
+}
+
 // res from the partial sums of a split reduction, added in a fixed order.
 __global__ __launch_bounds__(256) void logmm_fwd_finish_kernel(const FwdArgs a, int B) {
     const int b = blockIdx.y;
@@ -410,10 +579,11 @@ __global__ __launch_bounds__(256) void logmm_fwd_finish_kernel(const FwdArgs a, 
     const int Mb = a.row_len ? min(max(a.row_len[b], 0), a.M) : a.M;
     const int Nb = a.col_len ? min(max(a.col_len[b], 0) + 1, a.Nn) : a.Nn;
     if (i >= Mb || j >= Nb) return;
-    const size_t at = (size_t)b * a.M * a.Nn + e;
+    const size_t per = (size_t)a.pM * a.pN;
+    const float *p = a.partial + (size_t)b * per + (size_t)i * a.pN + j;
     float s = 0.0f;
-    for (int sp = 0; sp < a.splits; ++sp) s += a.partial[(size_t)sp * B * a.M * a.Nn + at];
-    a.res[at] = fwd_result(a, b, i, j, s);
+    for (int sp = 0; sp < a.splits; ++sp) s += p[(size_t)sp * B * per];
+    a.res[(size_t)b * a.M * a.Nn + e] = fwd_result(a, b, i, j, s);
 }
 
 // ---- backward ----------------------------------------------------------------
@@ -914,6 +1084,12 @@ hipError_t launch_logmm_shift_exp(const LogmmOperand &lhs, const LogmmOperand &r
     return hipGetLastError();
 }
 
+size_t logmm_fwd_partial_floats(int B, int M, int Nn) {
+    // up to 8 partial sums of whole row blocks (16) and column tiles (96 or 64)
+    const int tn = prefer_96(Nn) ? 96 : 64;
+    return (size_t)8 * B * ((M + 15) / 16 * 16) * ((Nn + tn - 1) / tn * tn);
+}
+
 int logmm_fwd_splits(int B, int M, int K, int Nn) {
     // only when there are fewer tiles than CUs (the extra pass over the partial sums costs as
     // much as it gains otherwise), and at least 2*kDepth chunks each
@@ -938,9 +1114,33 @@ hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
     a.lhs = lhs.p, a.lsb = lhs.sb, a.lsm = lhs.s1, a.lsk = lhs.s2;
     a.rhs = rhs.p, a.rsb = rhs.sb, a.rsk = rhs.s1, a.rsn = rhs.s2;
     a.res = res, a.M = M, a.K = K, a.Kp = logmm_padded_reduction(K), a.Nn = Nn;
+    a.pM = M, a.pN = Nn;
     a.row_len = row_len, a.col_len = col_len;
-    // 4 wavefronts per workgroup: 32 rows i by 96 or 64 columns j
     a.B = B;
+    // few columns, long reduction, room for the partial sums: one slab of E_r
+    // resident per workgroup, E_l streamed once
+    const bool slab_form = partial && a.Kp >= 2 * kSlab && a.Kp <= 8 * kSlab && Nn <= 8 * 96 &&
+                           B <= 65535;
+    if (slab_form) {
+        const int slabs = (a.Kp + kSlab - 1) / kSlab;   // <= 8: one partial sum each
+        a.splits = slabs;
+        const bool wide = prefer_96(Nn);
+        const int tn = wide ? 96 : 64;
+        a.pM = (M + 15) / 16 * 16, a.pN = (Nn + tn - 1) / tn * tn;
+        const dim3 grid((unsigned)(slabs * ((Nn + tn - 1) / tn)), (unsigned)B);
+        const size_t lds = (size_t)3 * tn * kSlabLd * sizeof(__bf16);
+        if (wide)
+            TIMED_LAUNCH((logmm_fwd_slab_kernel<6>), grid, dim3(64 * kSlabWaves), lds, stream, a, slabs);
+        else
+            TIMED_LAUNCH((logmm_fwd_slab_kernel<4>), grid, dim3(64 * kSlabWaves), lds, stream, a, slabs);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        const long outs = (long)M * Nn;
+        TIMED_LAUNCH(logmm_fwd_finish_kernel, dim3((unsigned)((outs + 255) / 256), B), dim3(256),
+                     0, stream, a, B);
+        return hipGetLastError();
+    }
+    // 4 wavefronts per workgroup: 32 rows i by 96 or 64 columns j
     a.tiles_x = (M + 31) / 32;
     a.tiles_y = (prefer_96(Nn) ? (Nn + 95) / 96 : (Nn + 63) / 64) * a.splits;
     if (!xcd_grid_fits(a.tiles_x, a.tiles_y, B)) return hipErrorInvalidValue;
