@@ -83,6 +83,30 @@ def test_log_matmul_infinities_and_far_apart_maxima():
     assert abs(gl[1, 4, 0]) + abs(gl[1, 4, 7]) > 1e-3      # the far-apart pair carries gradient
 
 
+def test_log_matmul_far_apart_maxima_in_a_long_reduction():
+    """The pairs left to the exact per-term pass, in the shapes that take the
+    slab-resident kernels (reduction of 512, whole and ragged row blocks)."""
+    from warp_ctct import _C
+    rng = np.random.default_rng(5)
+    for B, M, K, Nn in ((2, 32, 512, 40), (1, 21, 300, 9)):
+        lhs = rng.standard_normal((B, M, K)).astype(np.float32)
+        rhs = rng.standard_normal((B, K, Nn)).astype(np.float32)
+        lhs[0, 4, 0] = 300.0              # row maximum at k = 0
+        rhs[0, 7, 3] = 300.0              # column maximum at k = 7: pair (4, 3) underflows
+        lhs[B - 1, M - 1, K - 1] = 250.0
+        rhs[B - 1, 2, Nn - 1] = 250.0
+        ref = C.log_matmul(lhs, rhs)
+        d_lhs, d_rhs = dev(lhs), dev(rhs)
+        d_res = _C.log_matmul(d_lhs, d_rhs)
+        np.testing.assert_allclose(d_res.cpu().numpy(), ref, rtol=1e-5, atol=1e-4)
+        go = rng.standard_normal((B, M, Nn)).astype(np.float32)
+        gl, gr = O.log_matmul_backward(go, lhs, rhs, ref)
+        out_l, out_r = _C.log_matmul_backward(dev(go), d_lhs, d_rhs, d_res, [True, True])
+        np.testing.assert_allclose(out_l.cpu().numpy(), gl, atol=2e-5, rtol=1e-4)
+        np.testing.assert_allclose(out_r.cpu().numpy(), gr, atol=2e-5, rtol=1e-4)
+        assert abs(gl[0, 4, 0]) + abs(gl[0, 4, 7]) > 1e-3
+
+
 def test_log_matmul_rejects_bad_arguments():
     from warp_ctct import _C
     a = torch.zeros(2, 3, 4, device="cuda")
@@ -96,7 +120,12 @@ def test_log_matmul_rejects_bad_arguments():
         _C.log_matmul(a[0], torch.zeros(4, 3, device="cuda"))
 
 
-@pytest.mark.parametrize("B,M,K,Nn", [(2, 5, 7, 3), (2, 45, 130, 40), (1, 33, 65, 17)])
+@pytest.mark.parametrize("B,M,K,Nn", [
+    (2, 5, 7, 3), (2, 45, 130, 40), (1, 33, 65, 17),
+    # reductions of 256 and more with at most 96 columns: the gradient of lhs keeps
+    # a slab of the right operand in LDS; one, two and three chunks of columns,
+    # ragged and whole row blocks, ragged and whole slabs
+    (2, 37, 300, 81), (1, 48, 512, 33), (2, 20, 260, 7), (3, 64, 384, 96)])
 @pytest.mark.parametrize("mask", [(True, True), (True, False), (False, True)])
 def test_log_matmul_backward(B, M, K, Nn, mask):
     from warp_ctct import _C

@@ -102,7 +102,7 @@ SimpleWorkspace carve_simple(void *base, int N, int T, int U) {
     return w;
 }
 
-// Work buffers of the log-matmul backward: pair factors (B,M,Nn) and row flags (B,M).
+// Work buffers of the log-matmul backward: pair factors (B,M,logmm_pair_row(Nn)) and row flags (B,M).
 struct PairWorkspace {
     float *factors;
     int *flags;
@@ -111,7 +111,7 @@ struct PairWorkspace {
 
 PairWorkspace carve_pairs(void *base, int B, int M, int Nn) {
     PairWorkspace w;
-    const size_t fb = align256((size_t)B * M * Nn * sizeof(float));
+    const size_t fb = align256((size_t)B * M * logmm_pair_row(Nn) * sizeof(float));
     w.factors = reinterpret_cast<float *>(base);
     w.flags = reinterpret_cast<int *>(reinterpret_cast<uintptr_t>(base) + fb);
     w.bytes = fb + align256((size_t)B * M * sizeof(int));

@@ -171,13 +171,16 @@ hipError_t launch_logmm_shift_exp(const LogmmOperand &lhs, const LogmmOperand &r
 // partial (may be null): logmm_fwd_partial_floats(B,M,Nn) floats of scratch; with it the
 // reduction of a small output is split over several workgroups per tile
 int logmm_fwd_splits(int B, int M, int K, int Nn);
+// Row length, in floats, of the pair-factor buffer C of the backward: Nn rounded
+// up to the reduction chunk (32), zeros in the padding.
+__host__ __device__ inline int logmm_pair_row(int Nn) { return (Nn + 31) / 32 * 32; }
 // floats of `partial` that launch_logmm_fwd may use, whatever K is
 size_t logmm_fwd_partial_floats(int B, int M, int Nn);
 hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
                             const LogmmShifted &sh, float *res, float *partial, int B, int M,
                             int K, int Nn, const int *row_len, const int *col_len,
                             hipStream_t stream);
-// C (B,M,Nn) and flags (B,M): the pair factors go * exp(lmax + rmax - res) that
+// C (B,M,logmm_pair_row(Nn)) and flags (B,M): the pair factors go * exp(lmax + rmax - res) that
 // both gradients share, and per row whether a pair was left to the exact pass;
 // batch_scale (may be null) multiplies grad_out per batch.
 hipError_t launch_logmm_pair_factor(const float *go, const float *res, const float *lmax,

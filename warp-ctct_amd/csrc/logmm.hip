@@ -460,8 +460,12 @@ __global__ __launch_bounds__(64 * kSlabWaves) void logmm_fwd_slab_kernel(const F
     constexpr int CH = kSlab / TQ / 2;                  // chunks of 32 per half slab
     constexpr int GB = CB / 2;                          // column blocks per group
     extern __shared__ __attribute__((aligned(16))) __bf16 s_b[];   // [3][TN][kSlabLd]
-    const int b = blockIdx.y;
-    const int slab = blockIdx.x % slabs, j0 = (blockIdx.x / slabs) * TN;
+    // the slabs of one batch entry on one XCD, next to each other in time (see
+    // xcd_tile): together they read whole rows of E_l, through one L2
+    const TileId tile = xcd_tile(a.tiles_x, a.tiles_y);
+    const int b = tile.b;
+    if (b >= a.B) return;
+    const int slab = tile.x, j0 = tile.y * TN;
     const int M = a.M, Nn = a.Nn, Kp = a.Kp;
     const int Mb = a.row_len ? min(max(a.row_len[b], 0), M) : M;
     const int Nb = a.col_len ? min(max(a.col_len[b], 0) + 1, Nn) : Nn;
@@ -591,7 +595,8 @@ __global__ __launch_bounds__(256) void logmm_fwd_finish_kernel(const FwdArgs a, 
 // that a pair (i,j) contributes to both gradients; 0 for padding, for a zero
 // grad_out and for an all -inf row (no gradient).  A pair whose exponent
 // exceeds 2^60 is stored as 0 and its row is flagged: flags[b,i] = 1 makes the
-// gradient kernels add such pairs term by term.  One wavefront per row i.
+// gradient kernels add such pairs term by term.  Rows of C are logmm_pair_row(Nn)
+// floats long, zeros in the padding.  One wavefront per row i.
 __global__ __launch_bounds__(256) void logmm_pair_factor_kernel(
     const float *__restrict__ go, const float *__restrict__ res, const float *__restrict__ lmax,
     const float *__restrict__ rmax, const float *__restrict__ batch_scale,
@@ -604,9 +609,11 @@ __global__ __launch_bounds__(256) void logmm_pair_factor_kernel(
     const int Nb = col_len ? min(max(col_len[b], 0) + 1, Nn) : Nn;
     const float scale = batch_scale ? batch_scale[b] : 1.0f;
     const size_t row = ((size_t)b * M + i) * Nn;
+    const int Cq = logmm_pair_row(Nn);
+    float *crow = C + ((size_t)b * M + i) * Cq;
     const float ml = lmax[(size_t)b * M + i];
     int unsafe = 0;
-    for (int j = lane; j < Nn; j += 64) {
+    for (int j = lane; j < Cq; j += 64) {
         float cv = 0.0f;
         if (i < Mb && j < Nb) {
             const float gv = go[row + j] * scale, rr = res[row + j];
@@ -618,7 +625,7 @@ __global__ __launch_bounds__(256) void logmm_pair_factor_kernel(
                     unsafe = 1;
             }
         }
-        C[row + j] = cv;
+        crow[j] = cv;
     }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) unsafe |= __shfl_xor(unsafe, off, 64);
@@ -642,6 +649,8 @@ struct BwdArgs {
     float *grad;
     long osb, tsb, gsb, dsb;   // batch strides
     int osp, osk, tsq, tsk, gp, gq, dsp, dsk;
+    long csb;                  // C: batch stride and element strides along p and q (its rows
+    int cgp, cgq;              // are padded to logmm_pair_row(Nn) floats, zeros in the padding)
     int P, Q, K, Kp;
     const int *p_len, *q_len;
     int p_extra, q_extra;
@@ -695,7 +704,7 @@ __global__ __launch_bounds__(64 * WR * WC) void logmm_bwd_kernel(const BwdArgs a
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int row0 = (wave % WR) * 16 * RB, col0 = (wave / WR) * 16 * CB;
-    const float *cb = a.C + (size_t)b * a.gsb;
+    const float *cb = a.C + (size_t)b * a.csb;
     const float *eo = a.Eoth + (size_t)b * Q * Kp;
     float *db = a.grad + (size_t)b * a.dsb;
 
@@ -729,17 +738,17 @@ __global__ __launch_bounds__(64 * WR * WC) void logmm_bwd_kernel(const BwdArgs a
             ek[s] = (e % (TK / 4)) * 4;
             pe[s] = eo + min(k0 + ek[s], Kp - 4);
         }
-        const int c_last = (Q - 1) * a.gq;
+        const int c_last = (Q - 1) * a.cgq;
         int cp[SC], cq[SC];
         bool cp_ok[SC];
         const float *c_row[SC];
 #pragma unroll
         for (int s = 0; s < SC; ++s) {
             const int e = tid + NT * s;
-            cp[s] = (a.gq == 1) ? e / TQ : e % TP;
-            cq[s] = (a.gq == 1) ? e % TQ : e / TP;
+            cp[s] = (a.cgq == 1) ? e / TQ : e % TP;
+            cq[s] = (a.cgq == 1) ? e % TQ : e / TP;
             cp_ok[s] = (p0 + cp[s]) < Pb;
-            c_row[s] = cb + min(p0 + cp[s], P - 1) * a.gp;
+            c_row[s] = cb + min(p0 + cp[s], P - 1) * a.cgp;
         }
         v4f re[DEPTH][SE];
         float rc[DEPTH][SC];
@@ -750,7 +759,7 @@ __global__ __launch_bounds__(64 * WR * WC) void logmm_bwd_kernel(const BwdArgs a
                     pe[s] + (size_t)min(q0 + eq[s], Q - 1) * Kp);
 #pragma unroll
             for (int s = 0; s < SC; ++s)
-                rc[set][s] = c_row[s][min((q0 + cq[s]) * a.gq, c_last)];
+                rc[set][s] = c_row[s][min((q0 + cq[s]) * a.cgq, c_last)];
         };
         auto stash = [&](int set, int buf, int q0) {
 #pragma unroll
@@ -886,19 +895,19 @@ __global__ __launch_bounds__(256) void logmm_bwd_resident_kernel(const BwdArgs a
     // C slab, whole reduction: element e = tid + NT*s is (p, q) = (e / QR, e % QR)
     // when q is the contiguous index of C, else (e % TP, e / TP)
     {
-        const float *cb = a.C + (size_t)b * a.gsb;
-        const int c_last = (Q - 1) * a.gq;
+        const float *cb = a.C + (size_t)b * a.csb;
+        const int c_last = (Q - 1) * a.cgq;
         float rc[SC];
 #pragma unroll
         for (int s = 0; s < SC; ++s) {
             const int e = tid + NT * s;
-            const int cp = (a.gq == 1) ? e / QR : e % TP, cq = (a.gq == 1) ? e % QR : e / TP;
-            rc[s] = cb[min(p0 + cp, P - 1) * a.gp + min(cq * a.gq, c_last)];
+            const int cp = (a.cgq == 1) ? e / QR : e % TP, cq = (a.cgq == 1) ? e % QR : e / TP;
+            rc[s] = cb[min(p0 + cp, P - 1) * a.cgp + min(cq * a.cgq, c_last)];
         }
 #pragma unroll
         for (int s = 0; s < SC; ++s) {
             const int e = tid + NT * s;
-            const int cp = (a.gq == 1) ? e / QR : e % TP, cq = (a.gq == 1) ? e % QR : e / TP;
+            const int cp = (a.cgq == 1) ? e / QR : e % TP, cq = (a.cgq == 1) ? e % QR : e / TP;
             s_c[cp][cq] = ((p0 + cp) < Pb && cq < Qb) ? rc[s] : 0.0f;
         }
     }
@@ -964,6 +973,140 @@ __global__ __launch_bounds__(256) void logmm_bwd_resident_kernel(const BwdArgs a
     }
 }
 
+// The gradient of the operand with many rows and a SHORT reduction (the f of a
+// joiner: P = frames, Q = labels + 1 <= 96, K = vocabulary):
+//   grad[b,p,k] = E_own[p,k] * sum_q C[p,q] * E_oth[q,k].
+// The product is bound by reading E_own and writing the gradient once, as long
+// as E_oth stays on the chip.  A workgroup of 4 wavefronts takes one batch entry
+// and kBwdSlab columns k; that slab of E_oth is split into three bfloat16
+// planes and put into LDS once, transposed ([k][q]: the reduction index is then
+// contiguous for the matrix instruction).  A wavefront walks over blocks of 16
+// rows p: it splits the block's rows of C in registers (QC chunks of 32) and
+// multiplies them with every 16 columns of the slab.  The product is formed
+// transposed (E_oth^T first), so that a lane ends up with 4 consecutive k of one
+// row p: one 16-byte load of E_own and one 16-byte store of the gradient.
+constexpr int kBwdSlab = 128;
+
+constexpr int kBwdWaves = 4;
+
+template <int QC, bool FAST>
+__global__ __launch_bounds__(64 * kBwdWaves) void logmm_bwd_lhs_slab_kernel(const BwdArgs a) {
+    constexpr int QLD = QC * TQ + 8;            // bfloat16 per LDS row: rows 4 banks apart
+    constexpr int KB = kBwdSlab / 16, NW = kBwdWaves, NT = 64 * NW;
+    extern __shared__ __attribute__((aligned(16))) __bf16 s_e[];   // [3][kBwdSlab][QLD]
+    // the slabs of one batch entry on one XCD, next to each other in time (see
+    // xcd_tile): together they read whole rows of E_own and write whole rows of
+    // the gradient, through one L2
+    const TileId tile = xcd_tile(a.tiles_x, 1);
+    const int b = tile.b, k0 = tile.x * kBwdSlab;
+    if (b >= a.B) return;
+    const int P = a.P, Q = a.Q, K = a.K, Kp = a.Kp;
+    const int Pb = a.p_len ? min(max(a.p_len[b], 0) + a.p_extra, P) : P;
+    const int Qb = a.q_len ? min(max(a.q_len[b], 0) + a.q_extra, Q) : Q;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c = lane & 15, g = lane >> 4;
+    float *db = a.grad + (size_t)b * a.dsb;
+    const bool vec = a.dsk == 1 && (a.dsp & 3) == 0 && (a.dsb & 3) == 0 &&
+                     (reinterpret_cast<uintptr_t>(a.grad) & 15u) == 0;
+    // the slab of E_oth, transposed and split: element e is (row q, 4 columns k),
+    // q the fast index: neighbouring lanes then write neighbouring bfloat16 of an
+    // LDS row (with k the fast index all lanes of a store hit 4 banks)
+    for (int e = tid; e < QC * TQ * (kBwdSlab / 4); e += NT) {
+        const int k4 = (e / (QC * TQ)) * 4, q = e % (QC * TQ);
+        v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (q < Qb && k0 + k4 < Kp)
+            v = *reinterpret_cast<const v4f *>(a.Eoth + ((size_t)b * Q + q) * Kp + k0 + k4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const Split3 sp = split3(v[i]);
+            __bf16 *at = s_e + (size_t)(k4 + i) * QLD + q;
+            at[0] = sp.h;
+            at[(size_t)kBwdSlab * QLD] = sp.m;
+            at[(size_t)2 * kBwdSlab * QLD] = sp.l;
+        }
+    }
+    __syncthreads();
+    const int row_blocks = (P + 15) / 16;
+    const int *fl = a.flags + (size_t)b * P;
+    const int Cq = a.cgp;                       // row length of C
+    // A wavefront asks for everything a block of rows needs (its rows of C, and
+    // E_own at its lane's 4 columns of every 16) at the top of the block; the
+    // second workgroup of the CU covers the wait.  Measured and dropped: a second
+    // set of registers, so that a block's rows are requested while the block
+    // before it is worked on (64 us instead of 62: what a wavefront waits for is
+    // mostly its own earlier stores, which retire in order with its loads), and
+    // 8 wavefronts with E_own requested per 16 columns (73 us).
+    for (int rb = wave; rb < row_blocks; rb += NW) {
+        const int p = rb * 16 + c, pl = min(p, P - 1);
+        const float *crow = a.C + (size_t)b * a.csb + (size_t)pl * Cq + 8 * g;
+        v4f cv[2 * QC], ev[KB];
+#pragma unroll
+        for (int ch = 0; ch < QC; ++ch) {
+            cv[2 * ch] = *reinterpret_cast<const v4f *>(crow + TQ * ch);
+            cv[2 * ch + 1] = *reinterpret_cast<const v4f *>(crow + TQ * ch + 4);
+        }
+        const float *erow = a.Eown + ((size_t)b * P + pl) * Kp;
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+            ev[kb] = *reinterpret_cast<const v4f *>(erow + min(k0 + kb * 16 + 4 * g, Kp - 4));
+        bf16x8 cp[QC][3];
+#pragma unroll
+        for (int ch = 0; ch < QC; ++ch)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const Split3 sp = split3(i < 4 ? cv[2 * ch][i] : cv[2 * ch + 1][i - 4]);
+                cp[ch][0][i] = sp.h, cp[ch][1][i] = sp.m, cp[ch][2][i] = sp.l;
+            }
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+            v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int ch = 0; ch < QC; ++ch) {
+                bf16x8 ep[3];
+#pragma unroll
+                for (int pn = 0; pn < 3; ++pn)
+                    ep[pn] = *reinterpret_cast<const bf16x8 *>(
+                        s_e + ((size_t)pn * kBwdSlab + kb * 16 + c) * QLD + TQ * ch + 8 * g);
+                acc = mfma6(ep, cp[ch], acc);
+            }
+            // register q holds (k = k0 + kb*16 + 4g + q, row p)
+            const int k = k0 + kb * 16 + 4 * g;
+            v4f v;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] = scaled_sum(acc[q], ev[kb][q]);
+            float *dst = db + (size_t)p * a.dsp + (size_t)k * a.dsk;
+            if (FAST) {
+                *reinterpret_cast<v4f *>(dst) = v;
+            } else if (p < P && k < K) {
+                if (vec && k + 3 < K) {
+                    *reinterpret_cast<v4f *>(dst) = v;
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        if (k + q < K) dst[(size_t)q * a.dsk] = v[q];
+                }
+            }
+            // (left alone the scheduler hoists the LDS reads of all 16-column
+            // blocks to the top and spills)
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    // rows with pairs that C left out (exponent beyond the shifted range): their
+    // terms are added one by one, to what this lane has stored
+    for (int rb = wave; rb < row_blocks; rb += NW) {
+        const int p = rb * 16 + c;
+        const int flagged = (p < Pb) ? fl[min(p, P - 1)] : 0;
+        if (!__any(flagged)) continue;
+        if (!flagged) continue;
+        for (int kb = 0; kb < KB; ++kb)
+            for (int q = 0; q < 4; ++q) {
+                const int k = k0 + kb * 16 + 4 * g + q;
+                if (k < K) db[(size_t)p * a.dsp + (size_t)k * a.dsk] += exact_pairs(a, b, p, k, Qb);
+            }
+    }
+}
+
 // Tiles of 64 or 96 along an extent, whichever pads the tiled extent less.
 inline bool prefer_96(int extent) {
     return (extent + 95) / 96 * 96 < (extent + 63) / 64 * 64;
@@ -999,6 +1142,37 @@ hipError_t launch_bwd(const BwdArgs &args, int B, hipStream_t stream) {
         !fits_int((long)(a.P - 1) * a.dsp + (long)(a.K - 1) * a.dsk + 1) ||
         !fits_int((long)a.P * a.Q))
         return hipErrorInvalidValue;
+    if (a.cgq == 1 && a.Q <= 3 * TQ && a.Kp >= 2 * kBwdSlab) {
+        // short reduction, rows of C contiguous in it (the gradient of the operand
+        // with many rows): the slab of E_oth resident, E_own and the gradient
+        // streamed once
+        const int qc = (a.Q + TQ - 1) / TQ;
+        a.tiles_x = (a.Kp + kBwdSlab - 1) / kBwdSlab, a.tiles_y = 1;
+        if (!xcd_grid_fits(a.tiles_x, 1, B)) return hipErrorInvalidValue;
+        const dim3 grid(xcd_grid(a.tiles_x, 1, B));
+        const size_t lds = (size_t)3 * kBwdSlab * (qc * TQ + 8) * sizeof(__bf16);
+        // whole blocks of rows and whole slabs of columns, 16-byte stores: no
+        // bounds to check in the kernel
+        const bool fast = a.P % 16 == 0 && a.K % kBwdSlab == 0 && a.dsk == 1 && (a.dsp & 3) == 0 &&
+                          (a.dsb & 3) == 0 && (reinterpret_cast<uintptr_t>(a.grad) & 15u) == 0;
+#define LAUNCH_LHS_SLAB(QCN)                                                                   \
+    do {                                                                                       \
+        if (fast)                                                                              \
+            TIMED_LAUNCH((logmm_bwd_lhs_slab_kernel<QCN, true>), grid, dim3(64 * kBwdWaves), lds, \
+                         stream, a);                                                           \
+        else                                                                                   \
+            TIMED_LAUNCH((logmm_bwd_lhs_slab_kernel<QCN, false>), grid, dim3(64 * kBwdWaves), lds, \
+                         stream, a);                                                           \
+    } while (0)
+        if (qc == 1)
+            LAUNCH_LHS_SLAB(1);
+        else if (qc == 2)
+            LAUNCH_LHS_SLAB(2);
+        else
+            LAUNCH_LHS_SLAB(3);
+#undef LAUNCH_LHS_SLAB
+        return hipGetLastError();
+    }
     if (a.Q <= QR && !prefer_96(a.P)) {
         // short reduction, many rows: C slab resident, a few k tiles per workgroup
         const int ptiles = (a.P + 63) / 64, ktiles = (a.K + 63) / 64;
@@ -1119,15 +1293,16 @@ hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
     a.B = B;
     // few columns, long reduction, room for the partial sums: one slab of E_r
     // resident per workgroup, E_l streamed once
-    const bool slab_form = partial && a.Kp >= 2 * kSlab && a.Kp <= 8 * kSlab && Nn <= 8 * 96 &&
-                           B <= 65535;
+    const bool slab_form = partial && a.Kp >= 2 * kSlab && a.Kp <= 8 * kSlab && Nn <= 8 * 96;
     if (slab_form) {
         const int slabs = (a.Kp + kSlab - 1) / kSlab;   // <= 8: one partial sum each
         a.splits = slabs;
         const bool wide = prefer_96(Nn);
         const int tn = wide ? 96 : 64;
         a.pM = (M + 15) / 16 * 16, a.pN = (Nn + tn - 1) / tn * tn;
-        const dim3 grid((unsigned)(slabs * ((Nn + tn - 1) / tn)), (unsigned)B);
+        a.tiles_x = slabs, a.tiles_y = (Nn + tn - 1) / tn;
+        if (!xcd_grid_fits(a.tiles_x, a.tiles_y, B)) return hipErrorInvalidValue;
+        const dim3 grid(xcd_grid(a.tiles_x, a.tiles_y, B));
         const size_t lds = (size_t)3 * tn * kSlabLd * sizeof(__bf16);
         if (wide)
             TIMED_LAUNCH((logmm_fwd_slab_kernel<6>), grid, dim3(64 * kSlabWaves), lds, stream, a, slabs);
@@ -1183,6 +1358,7 @@ hipError_t launch_logmm_bwd_lhs(const LogmmOperand &lhs, const LogmmOperand &rhs
     a.oth = rhs.p, a.tsb = rhs.sb, a.tsq = (int)rhs.s2, a.tsk = (int)rhs.s1;
     a.own_max = sh.lmax, a.oth_max = sh.rmax;
     a.C = C, a.go = go, a.res = res, a.gsb = (long)M * Nn, a.gp = Nn, a.gq = 1;
+    a.csb = (long)M * logmm_pair_row(Nn), a.cgp = logmm_pair_row(Nn), a.cgq = 1;
     a.flags = flags, a.flags_follow_p = 1;
     a.grad = grad.p, a.dsb = grad.sb, a.dsp = (int)grad.s1, a.dsk = (int)grad.s2;
     a.P = M, a.Q = Nn, a.K = K, a.Kp = logmm_padded_reduction(K);
@@ -1208,6 +1384,7 @@ hipError_t launch_logmm_bwd_rhs(const LogmmOperand &lhs, const LogmmOperand &rhs
     a.oth = lhs.p, a.tsb = lhs.sb, a.tsq = (int)lhs.s1, a.tsk = (int)lhs.s2;
     a.own_max = sh.rmax, a.oth_max = sh.lmax;
     a.C = C, a.go = go, a.res = res, a.gsb = (long)M * Nn, a.gp = 1, a.gq = Nn;
+    a.csb = (long)M * logmm_pair_row(Nn), a.cgp = 1, a.cgq = logmm_pair_row(Nn);
     a.flags = flags, a.flags_follow_p = 0;
     a.grad = grad.p, a.dsb = grad.sb, a.dsp = (int)grad.s2, a.dsk = (int)grad.s1;
     a.P = Nn, a.Q = M, a.K = K, a.Kp = logmm_padded_reduction(K);
