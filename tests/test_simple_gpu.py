@@ -88,7 +88,7 @@ def test_log_matmul_far_apart_maxima_in_a_long_reduction():
     slab-resident kernels (reduction of 512, whole and ragged row blocks)."""
     from warp_ctct import _C
     rng = np.random.default_rng(5)
-    for B, M, K, Nn in ((2, 32, 512, 40), (1, 21, 300, 9)):
+    for B, M, K, Nn in ((2, 32, 512, 40), (1, 21, 300, 9), (2, 140, 512, 40)):
         lhs = rng.standard_normal((B, M, K)).astype(np.float32)
         rhs = rng.standard_normal((B, K, Nn)).astype(np.float32)
         lhs[0, 4, 0] = 300.0              # row maximum at k = 0
@@ -125,7 +125,10 @@ def test_log_matmul_rejects_bad_arguments():
     # reductions of 256 and more with at most 96 columns: the gradient of lhs keeps
     # a slab of the right operand in LDS; one, two and three chunks of columns,
     # ragged and whole row blocks, ragged and whole slabs
-    (2, 37, 300, 81), (1, 48, 512, 33), (2, 20, 260, 7), (3, 64, 384, 96)])
+    (2, 37, 300, 81), (1, 48, 512, 33), (2, 20, 260, 7), (3, 64, 384, 96),
+    # 128 and more rows as well: the gradient of rhs keeps its sums in registers and
+    # streams lhs once; one to six blocks of 16 columns, ragged chunks of rows
+    (2, 150, 300, 81), (1, 400, 512, 96), (2, 129, 260, 7), (1, 200, 777, 33), (1, 128, 256, 50)])
 @pytest.mark.parametrize("mask", [(True, True), (True, False), (False, True)])
 def test_log_matmul_backward(B, M, K, Nn, mask):
     from warp_ctct import _C

@@ -1107,6 +1107,141 @@ __global__ __launch_bounds__(64 * kBwdWaves) void logmm_bwd_lhs_slab_kernel(cons
     }
 }
 
+// The gradient of the operand with FEW rows and a LONG reduction (the g of a
+// joiner: P = labels + 1 <= 96, Q = frames, K = vocabulary):
+//   grad[b,p,k] = E_own[p,k] * sum_q C[q,p] * E_oth[q,k].
+// The output is small; the product is bound by streaming E_oth once.  A
+// workgroup of 4 wavefronts takes one batch entry and kRhsSlab columns k and
+// keeps its (16*UB x kRhsSlab) sums in registers (a wavefront: 32 columns).  The
+// reduction runs in chunks of 32 rows q.  Both operands have q as their ROW
+// index in memory, the matrix instruction wants 8 consecutive q per lane: a
+// thread loads 4 rows x 4 columns (16-byte vectors), splits the 16 values into
+// bfloat16 planes and writes them to LDS transposed, 4 consecutive q at a time
+// (8-byte stores; lanes run along q first, which keeps the stores free of bank
+// conflicts).  The next chunk is loaded while the present one is multiplied.
+constexpr int kRhsSlab = 128;
+constexpr int kRhsLd = TQ + 8;       // bfloat16 per LDS row (80 bytes)
+
+template <int UB>
+__global__ __launch_bounds__(256) void logmm_bwd_rhs_slab_kernel(const BwdArgs a) {
+    constexpr int NT = 256;
+    __shared__ __attribute__((aligned(16))) __bf16 s_el[3][kRhsSlab][kRhsLd];   // E_oth^T planes
+    __shared__ __attribute__((aligned(16))) __bf16 s_ct[3][16 * UB][kRhsLd];    // C^T planes
+    __shared__ int s_unsafe;
+    const TileId tile = xcd_tile(a.tiles_x, 1);
+    const int b = tile.b, k0 = tile.x * kRhsSlab;
+    if (b >= a.B) return;
+    const int P = a.P, Q = a.Q, K = a.K, Kp = a.Kp;
+    const int Pb = a.p_len ? min(max(a.p_len[b], 0) + a.p_extra, P) : P;
+    const int Qb = a.q_len ? min(max(a.q_len[b], 0) + a.q_extra, Q) : Q;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c = lane & 15, g = lane >> 4;
+    // rows q flagged by the pair-factor kernel (pairs left to the exact pass)
+    if (tid == 0) s_unsafe = 0;
+    __syncthreads();
+    {
+        const int *fl = a.flags + (size_t)b * Q;
+        int unsafe = 0;
+        for (int q = tid; q < Qb; q += NT) unsafe |= fl[q];
+        if (unsafe) s_unsafe = 1;
+    }
+    // staging roles: 4 rows q (tg) x 4 columns (k4 of the slab / u4 of C)
+    const int tg = tid & 7, k4 = tid >> 3, u4 = tid >> 3;
+    const bool has_c = u4 < 4 * UB;
+    const float *el_base = a.Eoth + (size_t)b * Q * Kp + min(k0 + 4 * k4, Kp - 4);
+    const float *c_base = a.C + (size_t)b * a.csb + 4 * u4;
+    v4f el[4], cv[4];
+    auto fetch = [&](int chunk) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int q = chunk * TQ + 4 * tg + j;
+            el[j] = *reinterpret_cast<const v4f *>(el_base + (size_t)min(q, Q - 1) * Kp);
+            cv[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            if (has_c && q < Qb) cv[j] = *reinterpret_cast<const v4f *>(c_base + (size_t)q * a.cgq);
+        }
+    };
+    // 4 rows x 4 columns -> per column the 4 rows as bfloat16 planes, 8 bytes each
+    auto stash = [&]() {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            bf16x4 h, m, l;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const Split3 sp = split3(el[j][i]);
+                h[j] = sp.h, m[j] = sp.m, l[j] = sp.l;
+            }
+            *reinterpret_cast<bf16x4 *>(&s_el[0][4 * k4 + i][4 * tg]) = h;
+            *reinterpret_cast<bf16x4 *>(&s_el[1][4 * k4 + i][4 * tg]) = m;
+            *reinterpret_cast<bf16x4 *>(&s_el[2][4 * k4 + i][4 * tg]) = l;
+        }
+        if (has_c) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                bf16x4 h, m, l;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const Split3 sp = split3(cv[j][i]);
+                    h[j] = sp.h, m[j] = sp.m, l[j] = sp.l;
+                }
+                *reinterpret_cast<bf16x4 *>(&s_ct[0][4 * u4 + i][4 * tg]) = h;
+                *reinterpret_cast<bf16x4 *>(&s_ct[1][4 * u4 + i][4 * tg]) = m;
+                *reinterpret_cast<bf16x4 *>(&s_ct[2][4 * u4 + i][4 * tg]) = l;
+            }
+        }
+    };
+    v4f acc[2][UB];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int ub = 0; ub < UB; ++ub) acc[kk][ub] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    const int n = (Qb + TQ - 1) / TQ;
+    if (n > 0) fetch(0);
+    for (int chunk = 0; chunk < n; ++chunk) {
+        __syncthreads();                    // the chunk before is no longer read
+        stash();
+        __syncthreads();
+        if (chunk + 1 < n) fetch(chunk + 1);
+        bf16x8 bk[2][3];
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+            for (int pn = 0; pn < 3; ++pn)
+                bk[kk][pn] = *reinterpret_cast<const bf16x8 *>(&s_el[pn][(2 * wave + kk) * 16 + c][8 * g]);
+#pragma unroll
+        for (int ub = 0; ub < UB; ++ub) {
+            bf16x8 au[3];
+#pragma unroll
+            for (int pn = 0; pn < 3; ++pn)
+                au[pn] = *reinterpret_cast<const bf16x8 *>(&s_ct[pn][ub * 16 + c][8 * g]);
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) acc[kk][ub] = mfma6(au, bk[kk], acc[kk][ub]);
+        }
+    }
+    __syncthreads();
+    const bool slow = s_unsafe != 0;
+    // lane l holds D[p = ub*16 + 4*(l/16) + q][k = kb*16 + l%16] in register q
+    float *db = a.grad + (size_t)b * a.dsb;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+        const int k = k0 + (2 * wave + kk) * 16 + c;
+        if (k >= K) continue;
+#pragma unroll
+        for (int ub = 0; ub < UB; ++ub)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int p = ub * 16 + 4 * g + q;
+                if (p >= P) continue;
+                float v = 0.0f;
+                if (p < Pb) {
+                    v = scaled_sum(acc[kk][ub][q], a.Eown[((size_t)b * P + p) * Kp + k]);
+                    if (slow) v += exact_pairs(a, b, p, k, Qb);
+                }
+                db[(size_t)p * a.dsp + (size_t)k * a.dsk] = v;
+            }
+    }
+}
+
 // Tiles of 64 or 96 along an extent, whichever pads the tiled extent less.
 inline bool prefer_96(int extent) {
     return (extent + 95) / 96 * 96 < (extent + 63) / 64 * 64;
@@ -1171,6 +1306,25 @@ hipError_t launch_bwd(const BwdArgs &args, int B, hipStream_t stream) {
         else
             LAUNCH_LHS_SLAB(3);
 #undef LAUNCH_LHS_SLAB
+        return hipGetLastError();
+    }
+    if (a.cgp == 1 && a.P <= 96 && a.Kp >= 2 * kRhsSlab && a.Q >= 4 * TQ &&
+        !getenv("WARPCTCT_NO_RHS_SLAB")) {
+        // few rows, long reduction with the reduction index as the row index of C
+        // (the gradient of the operand with few rows): sums in registers, E_oth
+        // streamed once
+        const int ub = (a.P + 15) / 16;
+        a.tiles_x = (a.Kp + kRhsSlab - 1) / kRhsSlab, a.tiles_y = 1;
+        if (!xcd_grid_fits(a.tiles_x, 1, B)) return hipErrorInvalidValue;
+        const dim3 grid(xcd_grid(a.tiles_x, 1, B));
+        switch (ub) {
+            case 1: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<1>), grid, dim3(256), 0, stream, a); break;
+            case 2: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<2>), grid, dim3(256), 0, stream, a); break;
+            case 3: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<3>), grid, dim3(256), 0, stream, a); break;
+            case 4: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<4>), grid, dim3(256), 0, stream, a); break;
+            case 5: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<5>), grid, dim3(256), 0, stream, a); break;
+            default: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<6>), grid, dim3(256), 0, stream, a); break;
+        }
         return hipGetLastError();
     }
     if (a.Q <= QR && !prefer_96(a.P)) {
