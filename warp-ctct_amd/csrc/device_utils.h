@@ -55,6 +55,19 @@ __device__ __forceinline__ double lse2(double x, double y) {
     return mx + (double)log2_hw(1.0f + exp2_hw(d));
 }
 
+// log2((1 + 2^-|d|) / 2), in [-1, 0]: the correction term of a semiring sum
+// whose operands are d apart, less one.  log2(2^x + 2^y) is then
+// (max(x, y) + 1) + this, where the first sum does not wait for the
+// transcendental unit.  d = NaN (the difference of two -inf) gives -inf: the
+// clamp of the multiply-add turns NaN into 0 (kernels run with DX10 clamping).
+// Three instructions between the difference and the result.
+__device__ __forceinline__ float half_sum_log2(float d) {
+    const float e = exp2_hw(-__builtin_fabsf(d));
+    // median of (x, 0, 1) on a multiply-add: folded into the instruction's clamp
+    const float t = __builtin_amdgcn_fmed3f(__builtin_fmaf(e, 0.5f, 0.5f), 0.0f, 1.0f);
+    return log2_hw(t);
+}
+
 // Lane l receives x of lane l-1; lane 0 receives `fill`.  Two DPP moves
 // (wave_shr:1), no LDS traffic.
 __device__ __forceinline__ double wave_shift_up(double x, double fill) {

@@ -83,6 +83,23 @@ __device__ __forceinline__ void chunk_load(Chunk &c, const double *units_lane, s
     }
 }
 
+// The same for R frames that all exist: `frame` points at the first one's row
+// (the same for all lanes) and moves on by `step` bytes per frame; a lane adds
+// its own 32-bit offset.  Two scalar additions per frame instead of a clamp and
+// a 64-bit product: a lone wavefront issues one instruction at a time, so the
+// address arithmetic of a frame costs as much as its semiring sums.
+__device__ __forceinline__ void chunk_load_walk(Chunk &c, const char *&frame, unsigned lane_bytes,
+                                                ptrdiff_t step) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const double *p = reinterpret_cast<const double *>(frame + lane_bytes);
+        c.lp[r][0] = p[0];
+        c.lp[r][1] = p[1];
+        c.lp[r][2] = p[2];
+        frame += step;
+    }
+}
+
 // ---- hand-over between the workgroups of one lattice -------------------------
 // slots[s] belongs to step s of the sweep (s < Tn <= T); a boundary has
 // T + R of them.  Relaxed atomics at agent scope: the store goes to the L2,
@@ -132,12 +149,14 @@ __device__ __forceinline__ bool slots_ready(const unsigned long long (&bits)[R],
 // previous 64 contexts, or -inf); out = what this lane sends to context u+1.
 __device__ __forceinline__ void alpha_step(Front &f, const double *lp, bool skip_next, double ext,
                                            double &out) {
-    const double both = lse2(f.e, f.o);
-    out = (skip_next ? both : f.e) + lp[2];
+    const double top = __builtin_fmax(f.e, f.o) + 1.0;
+    const double l = (double)half_sum_log2((float)(f.e - f.o));      // both = top + l
+    out = skip_next ? (top + lp[2]) + l : f.e + lp[2];
     const double recv = wave_shift_up(out, ext);
-    const double no = lse2(f.o + lp[1], recv);
-    f.e = both + lp[0];
-    f.o = no;
+    const double stay = f.o + lp[1];
+    const double l2 = (double)half_sum_log2((float)(recv - stay));
+    f.e = (top + lp[0]) + l;
+    f.o = (__builtin_fmax(stay, recv) + 1.0) + l2;
 }
 
 // ---- beta ----------------------------------------------------------------
@@ -156,10 +175,13 @@ __device__ __forceinline__ void beta_step(Front &f, const double *lp, bool skip,
     const double nb = wave_shift_down(f.o, ext);
     const double nxt = nb + lp[2];
     const double stay_e = f.e + lp[0];
-    const double ne = lse2(stay_e, nxt);
-    const double no = lse2(f.o + lp[1], skip ? ne : stay_e);
+    const double l = (double)half_sum_log2((float)(stay_e - nxt));
+    const double ne = (__builtin_fmax(stay_e, nxt) + 1.0) + l;
+    const double sel = skip ? ne : stay_e;
+    const double stay_o = f.o + lp[1];
+    const double l2 = (double)half_sum_log2((float)(stay_o - sel));
     f.e = ne;
-    f.o = no + o_mask;
+    f.o = (__builtin_fmax(stay_o, sel) + (1.0 + o_mask)) + l2;
 }
 
 // One direction of the 64 contexts [64*wave, 64*wave + 64) of one lattice.
@@ -193,6 +215,12 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T
     double *out = lat_n + (size_t)u * 2;
     const double *in = units_n + (size_t)u * 3;
     front_store(out + (size_t)(BETA ? Tn : 0) * srow, f);
+    // the row a step stores to, the same for all lanes, walked frame by frame
+    const unsigned out_lane = (unsigned)u * 2u * (unsigned)sizeof(double);
+    const unsigned in_lane = (unsigned)u * 3u * (unsigned)sizeof(double);
+    const ptrdiff_t out_step = (BETA ? -1 : 1) * (ptrdiff_t)(srow * sizeof(double));
+    const ptrdiff_t in_step = (BETA ? -1 : 1) * (ptrdiff_t)(urow * sizeof(double));
+    char *out_row = reinterpret_cast<char *>(lat_n) + (size_t)(BETA ? Tn - 1 : 1) * srow * sizeof(double);
     const int edge_lane = BETA ? 0 : 63;          // lane whose value crosses the boundary
 
     if (Tn > 0) {
@@ -240,14 +268,10 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T
             for (int r = 0; r < R; ++r) {
                 mine[r] = neg_inf();
                 if (full || r < cnt) {
-                    const int s = s0 + r;
-                    if (BETA) {
-                        beta_step(f, c.lp[r], skip, o_mask, mail[r], mine[r]);
-                        front_store(out + (size_t)(Tn - 1 - s) * srow, f);
-                    } else {
-                        alpha_step(f, c.lp[r], skip, mail[r], mine[r]);
-                        front_store(out + (size_t)(s + 1) * srow, f);
-                    }
+                    if (BETA) beta_step(f, c.lp[r], skip, o_mask, mail[r], mine[r]);
+                    else alpha_step(f, c.lp[r], skip, mail[r], mine[r]);
+                    front_store(reinterpret_cast<double *>(out_row + out_lane), f);
+                    out_row += out_step;
                 }
             }
             if (slots_out && lane == edge_lane) {
@@ -257,6 +281,18 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T
             }
         };
         int s0 = 0;
+        // while the chunk after next lies inside the sample, its rows need no clamp
+        if (3 * R <= Tn) {
+            const char *frame = reinterpret_cast<const char *>(units_n) +
+                                (size_t)(t_start + dir * R) * urow * sizeof(double);
+            do {
+                chunk_load_walk(b, frame, in_lane, in_step);
+                run_chunk(a, ahead_a, ahead_b, s0, R, true);
+                chunk_load_walk(a, frame, in_lane, in_step);
+                run_chunk(b, ahead_b, ahead_a, s0 + R, R, true);
+                s0 += 2 * R;
+            } while (s0 + 3 * R <= Tn);
+        }
         while (s0 + 2 * R <= Tn) {
             chunk_load(b, in, urow, Tn, t_start + dir * (s0 + R), dir);
             run_chunk(a, ahead_a, ahead_b, s0, R, true);

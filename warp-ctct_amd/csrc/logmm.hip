@@ -425,6 +425,24 @@ __device__ __forceinline__ Split3 split3(float x) {
     s.l = (__bf16)(r1 - (float)s.m);
     return s;
 }
+// Two values -> their three planes by truncation, each plane as two packed
+// bfloat16 (integer instructions only; x = h + m + l exactly, as with rounding,
+// since three 8-bit pieces cover the 24 bits of an fp32 significand)
+struct Pair3 {
+    unsigned h, m, l;
+};
+__device__ __forceinline__ Pair3 split3_pair(float x0, float x1) {
+    const unsigned top = 0xffff0000u;
+    const float h0 = __uint_as_float(__float_as_uint(x0) & top), h1 = __uint_as_float(__float_as_uint(x1) & top);
+    const float r0 = x0 - h0, r1 = x1 - h1;
+    const float m0 = __uint_as_float(__float_as_uint(r0) & top), m1 = __uint_as_float(__float_as_uint(r1) & top);
+    const float s0 = r0 - m0, s1 = r1 - m1;
+    Pair3 p;
+    p.h = __builtin_amdgcn_perm(__float_as_uint(x1), __float_as_uint(x0), 0x07060302u);
+    p.m = __builtin_amdgcn_perm(__float_as_uint(r1), __float_as_uint(r0), 0x07060302u);
+    p.l = __builtin_amdgcn_perm(__float_as_uint(s1), __float_as_uint(s0), 0x07060302u);
+    return p;
+}
 // acc += x * y for 16x16 outputs over 32 reduction indices, x and y given as
 // their three planes (each lane holds 8 consecutive reduction indices of its
 // row / column)
@@ -1121,9 +1139,13 @@ __global__ __launch_bounds__(64 * kBwdWaves) void logmm_bwd_lhs_slab_kernel(cons
 // conflicts).  The next chunk is loaded while the present one is multiplied.
 constexpr int kRhsSlab = 128;
 constexpr int kRhsLd = TQ + 8;       // bfloat16 per LDS row (80 bytes)
+#ifndef RHS_DEPTH
+#define RHS_DEPTH 3
+#endif
+constexpr int kRhsDepth = RHS_DEPTH;
 
-template <int UB>
-__global__ __launch_bounds__(256) void logmm_bwd_rhs_slab_kernel(const BwdArgs a) {
+template <int UB, int DEPTH>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void logmm_bwd_rhs_slab_kernel(const BwdArgs a) {
     constexpr int NT = 256;
     __shared__ __attribute__((aligned(16))) __bf16 s_el[3][kRhsSlab][kRhsLd];   // E_oth^T planes
     __shared__ __attribute__((aligned(16))) __bf16 s_ct[3][16 * UB][kRhsLd];    // C^T planes
@@ -1151,42 +1173,33 @@ __global__ __launch_bounds__(256) void logmm_bwd_rhs_slab_kernel(const BwdArgs a
     const bool has_c = u4 < 4 * UB;
     const float *el_base = a.Eoth + (size_t)b * Q * Kp + min(k0 + 4 * k4, Kp - 4);
     const float *c_base = a.C + (size_t)b * a.csb + 4 * u4;
-    v4f el[4], cv[4];
-    auto fetch = [&](int chunk) {
+    v4f el[DEPTH][4], cv[DEPTH][4];
+    // rows beyond the reduction: E_oth clamped to a valid row, C = 0
+    auto fetch = [&](int chunk, v4f (&e)[4], v4f (&cc)[4]) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int q = chunk * TQ + 4 * tg + j;
-            el[j] = *reinterpret_cast<const v4f *>(el_base + (size_t)min(q, Q - 1) * Kp);
-            cv[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-            if (has_c && q < Qb) cv[j] = *reinterpret_cast<const v4f *>(c_base + (size_t)q * a.cgq);
+            e[j] = *reinterpret_cast<const v4f *>(el_base + (size_t)min(q, Q - 1) * Kp);
+            cc[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            if (has_c && q < Qb) cc[j] = *reinterpret_cast<const v4f *>(c_base + (size_t)q * a.cgq);
         }
     };
     // 4 rows x 4 columns -> per column the 4 rows as bfloat16 planes, 8 bytes each
-    auto stash = [&]() {
+    auto stash = [&](const v4f (&e)[4], const v4f (&cc)[4]) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            bf16x4 h, m, l;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const Split3 sp = split3(el[j][i]);
-                h[j] = sp.h, m[j] = sp.m, l[j] = sp.l;
-            }
-            *reinterpret_cast<bf16x4 *>(&s_el[0][4 * k4 + i][4 * tg]) = h;
-            *reinterpret_cast<bf16x4 *>(&s_el[1][4 * k4 + i][4 * tg]) = m;
-            *reinterpret_cast<bf16x4 *>(&s_el[2][4 * k4 + i][4 * tg]) = l;
+            const Pair3 lo = split3_pair(e[0][i], e[1][i]), hi = split3_pair(e[2][i], e[3][i]);
+            *reinterpret_cast<uint2 *>(&s_el[0][4 * k4 + i][4 * tg]) = make_uint2(lo.h, hi.h);
+            *reinterpret_cast<uint2 *>(&s_el[1][4 * k4 + i][4 * tg]) = make_uint2(lo.m, hi.m);
+            *reinterpret_cast<uint2 *>(&s_el[2][4 * k4 + i][4 * tg]) = make_uint2(lo.l, hi.l);
         }
         if (has_c) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                bf16x4 h, m, l;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const Split3 sp = split3(cv[j][i]);
-                    h[j] = sp.h, m[j] = sp.m, l[j] = sp.l;
-                }
-                *reinterpret_cast<bf16x4 *>(&s_ct[0][4 * u4 + i][4 * tg]) = h;
-                *reinterpret_cast<bf16x4 *>(&s_ct[1][4 * u4 + i][4 * tg]) = m;
-                *reinterpret_cast<bf16x4 *>(&s_ct[2][4 * u4 + i][4 * tg]) = l;
+                const Pair3 lo = split3_pair(cc[0][i], cc[1][i]), hi = split3_pair(cc[2][i], cc[3][i]);
+                *reinterpret_cast<uint2 *>(&s_ct[0][4 * u4 + i][4 * tg]) = make_uint2(lo.h, hi.h);
+                *reinterpret_cast<uint2 *>(&s_ct[1][4 * u4 + i][4 * tg]) = make_uint2(lo.m, hi.m);
+                *reinterpret_cast<uint2 *>(&s_ct[2][4 * u4 + i][4 * tg]) = make_uint2(lo.l, hi.l);
             }
         }
     };
@@ -1196,26 +1209,33 @@ __global__ __launch_bounds__(256) void logmm_bwd_rhs_slab_kernel(const BwdArgs a
 #pragma unroll
         for (int ub = 0; ub < UB; ++ub) acc[kk][ub] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
     const int n = (Qb + TQ - 1) / TQ;
-    if (n > 0) fetch(0);
-    for (int chunk = 0; chunk < n; ++chunk) {
-        __syncthreads();                    // the chunk before is no longer read
-        stash();
-        __syncthreads();
-        if (chunk + 1 < n) fetch(chunk + 1);
-        bf16x8 bk[2][3];
+    // DEPTH chunks are on their way while one is multiplied: a chunk's phases
+    // (split and store, multiply) take about a microsecond, a load takes longer
 #pragma unroll
-        for (int kk = 0; kk < 2; ++kk)
+    for (int d = 0; d < DEPTH; ++d) fetch(d, el[d], cv[d]);
+    for (int chunk = 0; chunk < n; chunk += DEPTH) {
 #pragma unroll
-            for (int pn = 0; pn < 3; ++pn)
-                bk[kk][pn] = *reinterpret_cast<const bf16x8 *>(&s_el[pn][(2 * wave + kk) * 16 + c][8 * g]);
+        for (int d = 0; d < DEPTH; ++d) {
+            if (chunk + d >= n) break;
+            __syncthreads();                    // the chunk before is no longer read
+            stash(el[d], cv[d]);
+            __syncthreads();
+            fetch(chunk + d + DEPTH, el[d], cv[d]);
+            bf16x8 bk[2][3];
 #pragma unroll
-        for (int ub = 0; ub < UB; ++ub) {
-            bf16x8 au[3];
+            for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-            for (int pn = 0; pn < 3; ++pn)
-                au[pn] = *reinterpret_cast<const bf16x8 *>(&s_ct[pn][ub * 16 + c][8 * g]);
+                for (int pn = 0; pn < 3; ++pn)
+                    bk[kk][pn] = *reinterpret_cast<const bf16x8 *>(&s_el[pn][(2 * wave + kk) * 16 + c][8 * g]);
 #pragma unroll
-            for (int kk = 0; kk < 2; ++kk) acc[kk][ub] = mfma6(au, bk[kk], acc[kk][ub]);
+            for (int ub = 0; ub < UB; ++ub) {
+                bf16x8 au[3];
+#pragma unroll
+                for (int pn = 0; pn < 3; ++pn)
+                    au[pn] = *reinterpret_cast<const bf16x8 *>(&s_ct[pn][ub * 16 + c][8 * g]);
+#pragma unroll
+                for (int kk = 0; kk < 2; ++kk) acc[kk][ub] = mfma6(au, bk[kk], acc[kk][ub]);
+            }
         }
     }
     __syncthreads();
@@ -1317,13 +1337,35 @@ hipError_t launch_bwd(const BwdArgs &args, int B, hipStream_t stream) {
         a.tiles_x = (a.Kp + kRhsSlab - 1) / kRhsSlab, a.tiles_y = 1;
         if (!xcd_grid_fits(a.tiles_x, 1, B)) return hipErrorInvalidValue;
         const dim3 grid(xcd_grid(a.tiles_x, 1, B));
+        const char *dep_s = getenv("WARPCTCT_RHS_DEPTH");
+        const int dep = dep_s ? atoi(dep_s) : kRhsDepth;
+        if (dep == 2) {
         switch (ub) {
-            case 1: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<1>), grid, dim3(256), 0, stream, a); break;
-            case 2: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<2>), grid, dim3(256), 0, stream, a); break;
-            case 3: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<3>), grid, dim3(256), 0, stream, a); break;
-            case 4: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<4>), grid, dim3(256), 0, stream, a); break;
-            case 5: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<5>), grid, dim3(256), 0, stream, a); break;
-            default: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<6>), grid, dim3(256), 0, stream, a); break;
+            case 1: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<1, 2>), grid, dim3(256), 0, stream, a); break;
+            case 2: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<2, 2>), grid, dim3(256), 0, stream, a); break;
+            case 3: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<3, 2>), grid, dim3(256), 0, stream, a); break;
+            case 4: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<4, 2>), grid, dim3(256), 0, stream, a); break;
+            case 5: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<5, 2>), grid, dim3(256), 0, stream, a); break;
+            default: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<6, 2>), grid, dim3(256), 0, stream, a); break;
+        }
+        } else if (dep == 4) {
+        switch (ub) {
+            case 1: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<1, 4>), grid, dim3(256), 0, stream, a); break;
+            case 2: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<2, 4>), grid, dim3(256), 0, stream, a); break;
+            case 3: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<3, 4>), grid, dim3(256), 0, stream, a); break;
+            case 4: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<4, 4>), grid, dim3(256), 0, stream, a); break;
+            case 5: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<5, 4>), grid, dim3(256), 0, stream, a); break;
+            default: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<6, 4>), grid, dim3(256), 0, stream, a); break;
+        }
+        } else {
+        switch (ub) {
+            case 1: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<1, 3>), grid, dim3(256), 0, stream, a); break;
+            case 2: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<2, 3>), grid, dim3(256), 0, stream, a); break;
+            case 3: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<3, 3>), grid, dim3(256), 0, stream, a); break;
+            case 4: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<4, 3>), grid, dim3(256), 0, stream, a); break;
+            case 5: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<5, 3>), grid, dim3(256), 0, stream, a); break;
+            default: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<6, 3>), grid, dim3(256), 0, stream, a); break;
+        }
         }
         return hipGetLastError();
     }
