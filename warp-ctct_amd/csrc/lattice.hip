@@ -83,21 +83,43 @@ __device__ __forceinline__ void chunk_load(Chunk &c, const double *units_lane, s
     }
 }
 
-// The same for R frames that all exist: `frame` points at the first one's row
-// (the same for all lanes) and moves on by `step` bytes per frame; a lane adds
-// its own 32-bit offset.  Two scalar additions per frame instead of a clamp and
-// a 64-bit product: a lone wavefront issues one instruction at a time, so the
-// address arithmetic of a frame costs as much as its semiring sums.
+// A lone wavefront issues one instruction at a time, so the address arithmetic
+// of a frame costs as much as its semiring sums.  Rows are therefore walked:
+// loads follow a pointer that moves by one row per frame (two scalar additions
+// instead of a clamp and a 64-bit product), stores go through a buffer
+// descriptor: descriptor (the chunk's row of lowest address, in scalar
+// registers) + scalar byte offset of the frame + the lane's own 32-bit offset,
+// all inside the store instruction.  The descriptor's range is left open
+// (offsets stay inside the rows by construction).  Loads through a descriptor
+// were measured too: chains of five workgroups ran 10 % slower with them.
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t rows_from(const void *lowest) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(lowest), 0, 0xffffffffu, 0x00020000);
+}
+
+// The units of R frames that all exist.  `frame` points at the row of the
+// chunk's first frame (the same for all lanes) and is moved on by the chunk;
+// `step` = bytes per frame; DOWN: frames run towards lower addresses.
+template <bool DOWN>
 __device__ __forceinline__ void chunk_load_walk(Chunk &c, const char *&frame, unsigned lane_bytes,
-                                                ptrdiff_t step) {
+                                                unsigned step) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const double *p = reinterpret_cast<const double *>(frame + lane_bytes);
         c.lp[r][0] = p[0];
         c.lp[r][1] = p[1];
         c.lp[r][2] = p[2];
-        frame += step;
+        frame = DOWN ? frame - step : frame + step;
     }
+}
+
+__device__ __forceinline__ void front_store_at(__amdgpu_buffer_rsrc_t rows, unsigned lane_bytes,
+                                               unsigned at, const Front &f) {
+    v4u w;
+    w[0] = __double2loint(f.o), w[1] = __double2hiint(f.o);
+    w[2] = __double2loint(f.e), w[3] = __double2hiint(f.e);
+    __builtin_amdgcn_raw_buffer_store_b128(w, rows, lane_bytes, at, 0);
 }
 
 // ---- hand-over between the workgroups of one lattice -------------------------
@@ -218,8 +240,8 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T
     // the row a step stores to, the same for all lanes, walked frame by frame
     const unsigned out_lane = (unsigned)u * 2u * (unsigned)sizeof(double);
     const unsigned in_lane = (unsigned)u * 3u * (unsigned)sizeof(double);
-    const ptrdiff_t out_step = (BETA ? -1 : 1) * (ptrdiff_t)(srow * sizeof(double));
-    const ptrdiff_t in_step = (BETA ? -1 : 1) * (ptrdiff_t)(urow * sizeof(double));
+    const unsigned out_step = (unsigned)(srow * sizeof(double));     // bytes per frame
+    const unsigned in_step = (unsigned)(urow * sizeof(double));
     char *out_row = reinterpret_cast<char *>(lat_n) + (size_t)(BETA ? Tn - 1 : 1) * srow * sizeof(double);
     const int edge_lane = BETA ? 0 : 63;          // lane whose value crosses the boundary
 
@@ -264,16 +286,22 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T
                 for (int r = 0; r < R; ++r)
                     if (full || r < cnt) mail[r] = __longlong_as_double((long long)have[r]);
             }
+            // the chunk's rows of the lattice, lowest address first
+            const int rows_here = full ? R : cnt;
+            const __amdgpu_buffer_rsrc_t rows =
+                rows_from(BETA ? out_row - (size_t)(rows_here - 1) * out_step : out_row);
+            unsigned at = BETA ? (unsigned)(rows_here - 1) * out_step : 0u;
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 mine[r] = neg_inf();
                 if (full || r < cnt) {
                     if (BETA) beta_step(f, c.lp[r], skip, o_mask, mail[r], mine[r]);
                     else alpha_step(f, c.lp[r], skip, mail[r], mine[r]);
-                    front_store(reinterpret_cast<double *>(out_row + out_lane), f);
-                    out_row += out_step;
+                    front_store_at(rows, out_lane, at, f);
+                    at = BETA ? at - out_step : at + out_step;
                 }
             }
+            out_row = BETA ? out_row - (size_t)rows_here * out_step : out_row + (size_t)rows_here * out_step;
             if (slots_out && lane == edge_lane) {
 #pragma unroll
                 for (int r = 0; r < R; ++r)
@@ -286,9 +314,9 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T
             const char *frame = reinterpret_cast<const char *>(units_n) +
                                 (size_t)(t_start + dir * R) * urow * sizeof(double);
             do {
-                chunk_load_walk(b, frame, in_lane, in_step);
+                chunk_load_walk<BETA>(b, frame, in_lane, in_step);
                 run_chunk(a, ahead_a, ahead_b, s0, R, true);
-                chunk_load_walk(a, frame, in_lane, in_step);
+                chunk_load_walk<BETA>(a, frame, in_lane, in_step);
                 run_chunk(b, ahead_b, ahead_a, s0 + R, R, true);
                 s0 += 2 * R;
             } while (s0 + 3 * R <= Tn);
