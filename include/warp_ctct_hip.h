@@ -92,9 +92,20 @@ int warpctct_simple_units_f32(const float *f_g, const float *g_g, const float *d
  * through which the wavefronts of a lattice of more than 64 contexts hand
  * over their boundary values (0 bytes, relay may be NULL, for U+1 <= 64; it
  * replaces the `counts` spin-lock array of csrc/binding.cpp:77).  Should a
- * hand-over ever not arrive within its (long) bounded wait, the cost and the
- * lattices of that sample are NaN. */
+ * hand-over ever not arrive within its bounded wait, the workgroup that waited
+ * stops, writes NaN into the rows of alpha / beta that it has not swept and
+ * tells the workgroups behind it in the chain, which do the same: every
+ * gradient computed from those rows is NaN, and so is the cost when the beta
+ * chain is affected.  No plausible number comes out of a lattice that was not
+ * swept to the end.
+ * warpctct_lattice_wait_limit(spins): how often a waiting workgroup asks again
+ * before it gives up (0: the first look decides; negative: back to the default,
+ * about a second of polling); applies to launches made afterwards, returns the
+ * previous limit.  It has no counterpart in the reference, whose spin lock
+ * (csrc/gather.cu:88, :106, :171) is unbounded; tests use it to exercise the give-up
+ * path with kernels that still run to their end. */
 size_t warpctct_lattice_relay_bytes(int N, int T, int U);
+int warpctct_lattice_wait_limit(int spins);
 int warpctct_lattice_f32(const double *units, const int *ys, const int *lx, const int *ly,
                          double *alphas, double *betas, float *costs, int N, int T, int U,
                          int beta_only, void *relay, size_t relay_bytes, void *stream);

@@ -115,6 +115,10 @@ def test_generic_dtype_and_logits_entry_points_check_their_arguments():
     assert lib.warpctct_loss_forward(p, 9, p, p, p, 1, 1, 1, 8, p, small, p, p, null) == EINVAL
     assert lib.warpctct_zero_fill(null, ctypes.c_size_t(64), null) == EINVAL
     assert lib.warpctct_zero_fill(null, ctypes.c_size_t(0), null) == 0
+    # the wait limit of the chained lattice: a process-wide setting, returned on change
+    default = lib.warpctct_lattice_wait_limit(5)
+    assert default > 1000 and lib.warpctct_lattice_wait_limit(-1) == 5
+    assert lib.warpctct_lattice_wait_limit(-1) == default
     # workspace sizes: logits = lattice + one float per row; log-matmul grows with K
     N, T, U = 4, 50, 20
     lat = lib.warpctct_workspace_bytes(N, T, U)

@@ -481,6 +481,52 @@ def test_wide_lattices_chains_of_many_wavefronts(contexts):
     assert_support(got, ref_dense, "dense gradient, %d contexts" % contexts)
 
 
+def test_lost_hand_over_never_yields_a_plausible_number():
+    """A workgroup of a chain whose wait for its neighbour's boundary values runs
+    out stops and poisons what depends on it.  The wait limit is set to zero from
+    the host (the first look decides), so consumers that have caught up with their
+    producer give up at once and every kernel still runs to its end: each cost is
+    then either NaN or the right number, the gradient of a sample with a NaN cost
+    holds NaN, a sample whose lattice fits one wavefront is untouched, and with
+    the default limit restored the same call is right again."""
+    import warp_ctct
+    lib = hip_lib.lib()
+    N, T, U, V = 6, 200, 300, 6
+    ly = [300, 290, 10, 280, 64, 200]
+    joint, ys, lx, ly = make_joint_case(71, N, T, U, V, lx=[200, 190, 60, 200, 150, 180], ly=ly,
+                                        force_repeat=False, zero_pad=False)
+    ys[:] = 1 + np.arange(U) % (V - 1)
+    _, ref_dense, ref_costs = O.ctct_loss(joint, ys, lx, ly, reduction="sum")
+    d_ys, d_lx, d_ly = dev(ys), dev(lx), dev(ly)
+
+    def run():
+        x = dev(joint).requires_grad_(True)
+        c = warp_ctct.ctct_loss(x, d_ys, d_lx, d_ly, reduction="none")
+        c.sum().backward()
+        torch.cuda.synchronize()
+        return c.detach().cpu().numpy(), x.grad.cpu().numpy()
+
+    default = lib.warpctct_lattice_wait_limit(0)
+    try:
+        assert default > 1000
+        costs, grad = run()
+    finally:
+        assert lib.warpctct_lattice_wait_limit(-1) == 0
+    lost = np.isnan(costs)
+    assert lost[[0, 1, 3, 4, 5]].any(), "no consumer ever caught up with its producer"
+    assert not lost[2]                                   # 11 contexts: one wavefront, no hand-over
+    np.testing.assert_allclose(costs[~lost], ref_costs[~lost], rtol=LOSS_RTOL)
+    for n in range(N):
+        if lost[n]:
+            assert np.isnan(grad[n]).any()
+        elif not np.isnan(grad[n]).any():
+            # (a finite cost with NaN in the gradient: only the alpha chain lost its input)
+            np.testing.assert_allclose(grad[n], ref_dense[n], atol=GRAD_ATOL, rtol=0)
+    costs, grad = run()
+    np.testing.assert_allclose(costs, ref_costs, rtol=LOSS_RTOL)
+    np.testing.assert_allclose(grad, ref_dense, atol=GRAD_ATOL, rtol=0)
+
+
 def test_wide_lattice_log_add_joiner_beyond_512_contexts():
     """ctct_simple_loss with 600 contexts: the compact gradients of the joiner
     path are reduced from the unit-gradient tensor instead of inside one

@@ -248,6 +248,8 @@ int warpctct_simple_units_f32(const float *f_g, const float *g_g, const float *d
     return done(launch_simple_units(f_g, g_g, den, lx, ly, units_out, N, T, U, as_stream(stream)));
 }
 
+int warpctct_lattice_wait_limit(int spins) { return lattice_wait_limit(spins); }
+
 size_t warpctct_lattice_relay_bytes(int N, int T, int U) {
     if (N < 0 || T < 0 || U < 0) return 0;
     return lattice_relay_slots(N, T, U) * sizeof(unsigned long long);

@@ -35,6 +35,8 @@
 // Math restated from ref_ctct.py:6-74 of the reference (alpha :6-37, beta
 // :40-74); this kernel replaces k_warp_alphas / k_warp_betas
 // (csrc/gather.cu:36-291) and their global-memory spin-lock row pipeline.
+#include <atomic>
+
 #include "device_utils.h"
 #include "launch.h"
 
@@ -43,11 +45,15 @@ namespace wctct {
 namespace {
 
 constexpr int R = 8;          // frames per chunk (prefetch depth and hand-over granularity)
-constexpr int kMaxSpins = 1 << 20;   // ~1 s of polling before a hand-over is given up
+constexpr int kMaxSpins = 1 << 20;   // ~1 s of polling before a hand-over is given up (default)
 
 // What a relay slot holds before its value has been stored: a NaN with a
 // payload that no arithmetic produces.
 constexpr unsigned long long kEmptyBits = 0x7ff8dead5107e117ULL;
+// What a workgroup that has lost its input (its wait ran out, or its producer
+// lost its own) stores instead of values: another such NaN, one bit away in the
+// high word, so that one comparison tells empty, lost and value apart.
+constexpr unsigned long long kLostBits = kEmptyBits ^ (1ULL << 32);
 
 struct Front {
     double e, o;
@@ -143,10 +149,11 @@ __device__ __forceinline__ void slots_request(const unsigned long long *slots, i
         bits[r] = __hip_atomic_load(p + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// All of the chunk's cnt slots hold a value: no high word is the empty
-// pattern's (no value has that high word: it is a NaN payload no arithmetic
-// produces).  The smallest of (high word xor pattern) is zero iff one is empty.
-__device__ __forceinline__ bool slots_ready(const unsigned long long (&bits)[R], int cnt) {
+// State of the chunk's cnt slots: the smallest of (high word xor the empty
+// pattern's).  0: one is still empty; 1: none is empty and one says "lost";
+// anything else: all hold values (no value has either high word: they are NaN
+// payloads no arithmetic produces).  The same for all lanes.
+__device__ __forceinline__ unsigned slots_state(const unsigned long long (&bits)[R], int cnt) {
     constexpr unsigned kEmptyHigh = (unsigned)(kEmptyBits >> 32);
     unsigned least = 0xffffffffu;
 #pragma unroll
@@ -154,7 +161,7 @@ __device__ __forceinline__ bool slots_ready(const unsigned long long (&bits)[R],
         const unsigned d = (unsigned)(bits[r] >> 32) ^ kEmptyHigh;
         least = min(least, r < cnt ? d : 0xffffffffu);
     }
-    return __builtin_amdgcn_readfirstlane((int)least) != 0;   // the same for all lanes
+    return (unsigned)__builtin_amdgcn_readfirstlane((int)least);
 }
 
 // ---- alpha ---------------------------------------------------------------
@@ -215,7 +222,7 @@ __device__ __forceinline__ void beta_step(Front &f, const double *lp, bool skip,
 template <bool BETA>
 __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T, int P, int wave,
                       double *lat_n, float *cost_n, const unsigned long long *slots_in,
-                      unsigned long long *slots_out) {
+                      unsigned long long *slots_out, int max_spins) {
     const int lane = threadIdx.x & 63;
     const int u = wave * 64 + lane;
     double o_mask = 0.0;
@@ -258,7 +265,14 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T
 #pragma unroll
         for (int r = 0; r < R; ++r) ahead_a[r] = ahead_b[r] = kEmptyBits;
         if (slots_in) slots_request(slots_in, 0, ahead_a);
-        bool gave_up = false;            // after one wait has run out, no later one is started
+        // The input is lost: a wait has run out, or the producer says that it lost
+        // its own (lost_from = the first step without input).  The sweep goes on to
+        // its end without waiting again and without handing anything over (leaving
+        // the loop early, or a branch around a chunk, costs the common path 15 %:
+        // the compiler then waits for every load in flight where the paths join);
+        // what it has computed since is overwritten afterwards.
+        bool lost = false;
+        int lost_from = 0;
         // one chunk: steps s0 .. s0+cnt-1 with the units in `c` and the slots in
         // `have`; the slots of the next chunk are requested into `next`
         auto run_chunk = [&](const Chunk &c, unsigned long long (&have)[R],
@@ -269,19 +283,20 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T
             if (slots_in) {
                 slots_request(slots_in, min(s0 + R, T), next);
                 // `have` was requested a chunk ago; repeat the request until the
-                // producer has got this far (with a bound: an empty slot is a NaN
-                // and poisons the lattice if the wait gives up).  The first look
-                // is kept out of the polling loop: a loop header that is also
+                // producer has got this far, max_spins times at most.  The first
+                // look is kept out of the polling loop: a loop header that is also
                 // reached from the re-request would make the compiler wait for
                 // every load in flight here, the prefetched units included.
-                if (!slots_ready(have, cnt) && !gave_up) {
+                unsigned state = slots_state(have, cnt);
+                if (state == 0 && max_spins > 0 && !lost) {
                     int spins = 0;
                     do {
                         __builtin_amdgcn_s_sleep(2);
                         slots_request(slots_in, s0, have);
-                        gave_up = ++spins >= kMaxSpins;
-                    } while (!slots_ready(have, cnt) && !gave_up);
+                        state = slots_state(have, cnt);
+                    } while (state == 0 && ++spins < max_spins);
                 }
+                if (state <= 1 && !lost) lost = true, lost_from = s0;
 #pragma unroll
                 for (int r = 0; r < R; ++r)
                     if (full || r < cnt) mail[r] = __longlong_as_double((long long)have[r]);
@@ -302,7 +317,7 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T
                 }
             }
             out_row = BETA ? out_row - (size_t)rows_here * out_step : out_row + (size_t)rows_here * out_step;
-            if (slots_out && lane == edge_lane) {
+            if (slots_out && !lost && lane == edge_lane) {
 #pragma unroll
                 for (int r = 0; r < R; ++r)
                     if (full || r < cnt) slot_put(slots_out + s0 + r, mine[r]);
@@ -333,6 +348,19 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T
         const int rest = Tn - s0;
         if (rest > 0) run_chunk(a, ahead_a, ahead_b, s0, min(rest, R), false);
         if (rest > R) run_chunk(b, ahead_b, ahead_a, s0 + R, rest - R, false);
+        if (lost) {
+            // Nothing plausible may come out of this lattice: the rows from the
+            // first step without input on are NaN (so is every gradient computed
+            // from them, and the cost if this is the end of the beta chain), and
+            // the consumer, which has been waiting since, is told.
+            f.e = f.o = __longlong_as_double(0x7ff8000000000000LL);
+            for (int s = lost_from; s < Tn; ++s)
+                front_store(out + (size_t)(BETA ? Tn - 1 - s : s + 1) * srow, f);
+            if (slots_out && lane == edge_lane)
+                for (int s = lost_from; s < Tn; ++s)
+                    __hip_atomic_store(slots_out + s, kLostBits, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
     // cost = -beta(0, state 0) in natural-log units (csrc/binding.cpp:86)
     if (BETA && u == 0) *cost_n = (float)(-f.e * kLn2);
@@ -358,7 +386,7 @@ __device__ __forceinline__ void lattice_block(const double *__restrict__ units,
                                               float *__restrict__ costs,
                                               unsigned long long *__restrict__ relay, int N, int T,
                                               int U, int W, int dirs, int chains_pad,
-                                              const CostReduce &red) {
+                                              const CostReduce &red, int max_spins) {
     const int chain = blockIdx.x % chains_pad, link = blockIdx.x / chains_pad;
     if (chain >= N * dirs) return;
     const int n = chain / dirs;
@@ -383,13 +411,15 @@ __device__ __forceinline__ void lattice_block(const double *__restrict__ units,
     if (!beta) {
         const unsigned long long *in = wave > 0 ? slots_n + (size_t)(wave - 1) * TS : nullptr;
         unsigned long long *out = (wave + 1) * 64 <= Un ? slots_n + (size_t)wave * TS : nullptr;
-        sweep<false>(units_n, y, Tn, Un, T, P, wave, alphas + (size_t)n * lat, nullptr, in, out);
+        sweep<false>(units_n, y, Tn, Un, T, P, wave, alphas + (size_t)n * lat, nullptr, in, out,
+                     max_spins);
         return;
     }
     {
         const unsigned long long *in = (wave + 1) * 64 <= Un ? slots_n + (size_t)wave * TS : nullptr;
         unsigned long long *out = wave > 0 ? slots_n + (size_t)(wave - 1) * TS : nullptr;
-        sweep<true>(units_n, y, Tn, Un, T, P, wave, betas + (size_t)n * lat, costs + n, in, out);
+        sweep<true>(units_n, y, Tn, Un, T, P, wave, betas + (size_t)n * lat, costs + n, in, out,
+                    max_spins);
     }
     if (wave != 0) return;
     // thread 0 (context 0) has just written costs[n]
@@ -426,8 +456,9 @@ __global__ __launch_bounds__(64) void lattice_kernel(const double *__restrict__ 
                                                      float *__restrict__ costs,
                                                      unsigned long long *__restrict__ relay, int N,
                                                      int T, int U, int W, int dirs, int chains_pad,
-                                                     const CostReduce red) {
-    lattice_block(units, ys, lx, ly, alphas, betas, costs, relay, N, T, U, W, dirs, chains_pad, red);
+                                                     const CostReduce red, int max_spins) {
+    lattice_block(units, ys, lx, ly, alphas, betas, costs, relay, N, T, U, W, dirs, chains_pad, red,
+                  max_spins);
 }
 
 // The same sweeps with a memory clear riding along: workgroups of 256 threads,
@@ -440,18 +471,27 @@ __global__ __launch_bounds__(256) void lattice_fill_kernel(
     const double *__restrict__ units, const int *__restrict__ ys, const int *__restrict__ lx,
     const int *__restrict__ ly, double *__restrict__ alphas, double *__restrict__ betas,
     float *__restrict__ costs, unsigned long long *__restrict__ relay, int N, int T, int U, int W,
-    int dirs, int chains_pad, const CostReduce red, v4f_fill *__restrict__ fill, size_t n4,
-    unsigned lattice_blocks) {
+    int dirs, int chains_pad, const CostReduce red, int max_spins, v4f_fill *__restrict__ fill,
+    size_t n4, unsigned lattice_blocks) {
     if (blockIdx.x >= lattice_blocks) {
         const size_t i = (size_t)(blockIdx.x - lattice_blocks) * 256 + threadIdx.x;
         if (i < n4) fill[i] = v4f_fill{0.0f, 0.0f, 0.0f, 0.0f};
         return;
     }
     if (threadIdx.x >= 64) return;
-    lattice_block(units, ys, lx, ly, alphas, betas, costs, relay, N, T, U, W, dirs, chains_pad, red);
+    lattice_block(units, ys, lx, ly, alphas, betas, costs, relay, N, T, U, W, dirs, chains_pad, red,
+                  max_spins);
 }
 
 }  // namespace
+
+namespace {
+std::atomic<int> g_wait_limit{kMaxSpins};
+}
+
+int lattice_wait_limit(int spins) {
+    return g_wait_limit.exchange(spins < 0 ? kMaxSpins : spins, std::memory_order_relaxed);
+}
 
 size_t lattice_relay_slots(int N, int T, int U) {
     const int W = (U + 1 + 63) / 64;
@@ -474,6 +514,7 @@ hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream) {
     } else {
         relay = nullptr;
     }
+    const int max_spins = g_wait_limit.load(std::memory_order_relaxed);
     const int dirs = a.beta_only ? 1 : 2;
     const long chains = (long)a.N * dirs;
     const long chains_pad = (chains + 7) / 8 * 8;
@@ -483,13 +524,13 @@ hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream) {
         if (blocks > 0x7fffffffUL) return hipErrorInvalidValue;
         TIMED_LAUNCH(lattice_fill_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a.units,
                      a.ys, a.lx, a.ly, a.alphas, a.betas, a.costs, relay, a.N, a.T, a.U, W, dirs,
-                     (int)chains_pad, a.reduce, static_cast<v4f_fill *>(a.fill.p), a.fill.n4,
+                     (int)chains_pad, a.reduce, max_spins, static_cast<v4f_fill *>(a.fill.p), a.fill.n4,
                      (unsigned)(chains_pad * W));
         return hipGetLastError();
     }
     TIMED_LAUNCH(lattice_kernel, dim3((unsigned)(chains_pad * W)), dim3(64), 0, stream, a.units,
                  a.ys, a.lx, a.ly, a.alphas, a.betas, a.costs, relay, a.N, a.T, a.U, W, dirs,
-                 (int)chains_pad, a.reduce);
+                 (int)chains_pad, a.reduce, max_spins);
     return hipGetLastError();
 }
 

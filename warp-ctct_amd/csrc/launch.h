@@ -57,6 +57,11 @@ struct LatticeArgs {
 // hand one value per frame and 64-context boundary through device memory:
 // the number of 64-bit slots that takes (0 for U + 1 <= 64).
 size_t lattice_relay_slots(int N, int T, int U);
+// How often a consumer asks again for a hand-over that has not arrived before
+// it declares its input lost (0: the first look decides; negative: the
+// default, about a second).  Applies to launches made afterwards; returns the
+// previous limit.
+int lattice_wait_limit(int spins);
 hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream);
 
 // Element strides of a joint tensor (N,T,U+1,V); dense row-major is
