@@ -23,9 +23,10 @@
 // consumer (workgroups are dispatched in index order: a waiting consumer's
 // producer is running or done), and all links of a chain share `index % 8`,
 // i.e. the XCD and its L2, under round-robin dispatch.
-// A wait is bounded; a consumer that gives up keeps the empty pattern, which
-// is a NaN: the cost and every gradient of that lattice come out as NaN
-// instead of a plausible number.
+// A wait is bounded; a consumer whose wait runs out fills the rows it could not
+// sweep properly with NaN and stores a "lost" pattern instead of values, which
+// makes the workgroups behind it do the same: the gradients, and the cost when
+// the beta chain is hit, come out as NaN instead of a plausible number.
 //
 // Values are log2 of the path mass, held in double; the exponentials and
 // logarithms of the semiring sum run on the fp32 transcendental unit (see
@@ -219,7 +220,11 @@ __device__ __forceinline__ void beta_step(Front &f, const double *lp, bool skip,
 // slots_in / slots_out: the T relay slots of the boundary this wavefront reads
 // (null: nothing flows in, the neighbour is -inf) and writes (null: no
 // neighbour on that side).
-template <bool BETA>
+// HAS_IN: boundary values flow in (slots_in is not null).  A template argument
+// rather than a test of the pointer: with both cases in one body the values
+// that enter lane 0 / lane 63 are copied once more per frame, and a lone
+// wavefront pays for every instruction (chains of five: 199 -> 182 us).
+template <bool BETA, bool HAS_IN>
 __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T, int P, int wave,
                       double *lat_n, float *cost_n, const unsigned long long *slots_in,
                       unsigned long long *slots_out, int max_spins) {
@@ -264,7 +269,7 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T
         unsigned long long ahead_a[R], ahead_b[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) ahead_a[r] = ahead_b[r] = kEmptyBits;
-        if (slots_in) slots_request(slots_in, 0, ahead_a);
+        if (HAS_IN) slots_request(slots_in, 0, ahead_a);
         // The input is lost: a wait has run out, or the producer says that it lost
         // its own (lost_from = the first step without input).  The sweep goes on to
         // its end without waiting again and without handing anything over (leaving
@@ -280,7 +285,7 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T
             double mail[R], mine[R];
 #pragma unroll
             for (int r = 0; r < R; ++r) mail[r] = neg_inf();
-            if (slots_in) {
+            if (HAS_IN) {
                 slots_request(slots_in, min(s0 + R, T), next);
                 // `have` was requested a chunk ago; repeat the request until the
                 // producer has got this far, max_spins times at most.  The first
@@ -411,15 +416,15 @@ __device__ __forceinline__ void lattice_block(const double *__restrict__ units,
     if (!beta) {
         const unsigned long long *in = wave > 0 ? slots_n + (size_t)(wave - 1) * TS : nullptr;
         unsigned long long *out = (wave + 1) * 64 <= Un ? slots_n + (size_t)wave * TS : nullptr;
-        sweep<false>(units_n, y, Tn, Un, T, P, wave, alphas + (size_t)n * lat, nullptr, in, out,
-                     max_spins);
+        if (in) sweep<false, true>(units_n, y, Tn, Un, T, P, wave, alphas + (size_t)n * lat, nullptr, in, out, max_spins);
+        else sweep<false, false>(units_n, y, Tn, Un, T, P, wave, alphas + (size_t)n * lat, nullptr, in, out, max_spins);
         return;
     }
     {
         const unsigned long long *in = (wave + 1) * 64 <= Un ? slots_n + (size_t)wave * TS : nullptr;
         unsigned long long *out = wave > 0 ? slots_n + (size_t)(wave - 1) * TS : nullptr;
-        sweep<true>(units_n, y, Tn, Un, T, P, wave, betas + (size_t)n * lat, costs + n, in, out,
-                    max_spins);
+        if (in) sweep<true, true>(units_n, y, Tn, Un, T, P, wave, betas + (size_t)n * lat, costs + n, in, out, max_spins);
+        else sweep<true, false>(units_n, y, Tn, Un, T, P, wave, betas + (size_t)n * lat, costs + n, in, out, max_spins);
     }
     if (wave != 0) return;
     // thread 0 (context 0) has just written costs[n]
