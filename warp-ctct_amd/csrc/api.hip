@@ -171,7 +171,7 @@ int static_scratch(void **out) {
 // lattice + unit gradients + reductions, shared by the two simple forwards
 int simple_from_units(const SimpleWorkspace &w, const int *ys, const int *lx, const int *ly, int N,
                       int T, int U, float *costs, float *grad_f, float *grad_g, float *grad_den,
-                      bool want_grad, hipStream_t stream) {
+                      bool want_grad, bool relay_is_clear, hipStream_t stream) {
     // alpha is needed only for the gradients; those are reduced straight from the
     // lattices (the unit-gradient region of the workspace holds the partial sums)
     LatticeArgs a = {};
@@ -182,6 +182,7 @@ int simple_from_units(const SimpleWorkspace &w, const int *ys, const int *lx, co
     a.alphas = w.lattice.alphas;
     a.betas = w.lattice.betas;
     a.relay = w.lattice.relay;
+    a.relay_is_clear = relay_is_clear;
     a.costs = costs;
     a.N = N;
     a.T = T;
@@ -228,7 +229,8 @@ int warpctct_gather_units_f32(const float *joint, const int *ys, const int *lx, 
     if (N == 0 || T == 0) return WARPCTCT_OK;
     if (!joint || !lx || !ly || !units_out || (U > 0 && !ys)) return WARPCTCT_EINVAL;
     return done(launch_gather_units(joint, dense_joint_strides(T, U, V), kIoF32, ys, lx, ly,
-                                    units_out, N, T, U, V, false, nullptr, as_stream(stream)));
+                                    units_out, N, T, U, V, false, nullptr, RelaySlots{},
+                                    as_stream(stream)));
 }
 
 int warpctct_scale_units_f32(const float *units_nat, const int *lx, const int *ly,
@@ -353,7 +355,7 @@ int loss_lattice_run(const void *joint, int dtype, const long *strides, const in
     unsigned *counter = reduction != 0 ? w.counter : nullptr;
     if (T > 0) {
         int rc = done(launch_gather_units(joint, js, dtype, ys, lx, ly, w.units, N, T, U, V, true,
-                                          counter, st));
+                                          counter, relay_slots_of(w.relay, N, T, U), st));
         if (rc != WARPCTCT_OK) return rc;
     } else if (counter) {
         int rc = done(launch_clear_counter(counter, st));
@@ -367,6 +369,7 @@ int loss_lattice_run(const void *joint, int dtype, const long *strides, const in
     a.alphas = w.alphas;
     a.betas = w.betas;
     a.relay = w.relay;
+    a.relay_is_clear = T > 0;             // by the gather kernel
     a.costs = costs;
     a.N = N;
     a.T = T;
@@ -579,7 +582,8 @@ int warpctct_loss_forward(const void *joint, int dtype, const int *ys, const int
     if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
     if (T > 0) {
         int rc = done(launch_gather_units(joint, dense_joint_strides(T, U, V), dtype, ys, lx, ly,
-                                          w.units, N, T, U, V, true, nullptr, as_stream(stream)));
+                                          w.units, N, T, U, V, true, nullptr, RelaySlots{},
+                                          as_stream(stream)));
         if (rc != WARPCTCT_OK) return rc;
     }
     return forward_from_units(w, ys, lx, ly, N, T, U, costs, T > 0 ? unit_grads : nullptr,
@@ -637,7 +641,7 @@ int warpctct_simple_gather_units_f32(const float *f, const float *g, const float
     if (N == 0 || T == 0) return WARPCTCT_OK;
     if (!f || !g || !lx || !ly || !units_out || (U > 0 && !ys)) return WARPCTCT_EINVAL;
     return done(launch_simple_gather_units(f, g, den, ys, lx, ly, units_out, N, T, U, V,
-                                           as_stream(stream)));
+                                           RelaySlots{}, as_stream(stream)));
 }
 
 int warpctct_simple_reduce_f32(const float *unit_grads, float *grad_f, float *grad_g,
@@ -699,7 +703,8 @@ int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, c
             if (rc != WARPCTCT_OK) return rc;
         }
         int rc = done(launch_simple_gather_units(f, g, normalized ? den : nullptr, ys, lx, ly,
-                                                 w.lattice.units, N, T, U, V, st));
+                                                 w.lattice.units, N, T, U, V,
+                                                 relay_slots_of(w.lattice.relay, N, T, U), st));
         if (rc != WARPCTCT_OK) return rc;
     }
     if (want_grad && T == 0) {   // no frames: the only gradient with elements is all zeros
@@ -707,7 +712,7 @@ int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, c
         if (rc != WARPCTCT_OK) return rc;
     }
     return simple_from_units(w, ys, lx, ly, N, T, U, costs, grad_f, grad_g,
-                             normalized ? grad_den : nullptr, want_grad && T > 0, st);
+                             normalized ? grad_den : nullptr, want_grad && T > 0, T > 0, st);
 }
 
 int warpctct_simple_forward_units_f32(const float *f_g, const float *g_g, const float *den,
@@ -732,7 +737,7 @@ int warpctct_simple_forward_units_f32(const float *f_g, const float *g_g, const 
         if (rc != WARPCTCT_OK) return rc;
     }
     return simple_from_units(w, ys, lx, ly, N, T, U, costs, grad_f, grad_g,
-                             den ? grad_den : nullptr, want_grad && T > 0, st);
+                             den ? grad_den : nullptr, want_grad && T > 0, false, st);
 }
 
 size_t warpctct_simple_backward_workspace_bytes(int N, int T, int U) {

@@ -50,7 +50,7 @@ constexpr int kMaxSpins = 1 << 20;   // ~1 s of polling before a hand-over is gi
 
 // What a relay slot holds before its value has been stored: a NaN with a
 // payload that no arithmetic produces.
-constexpr unsigned long long kEmptyBits = 0x7ff8dead5107e117ULL;
+constexpr unsigned long long kEmptyBits = kRelayEmpty;
 // What a workgroup that has lost its input (its wait ran out, or its producer
 // lost its own) stores instead of values: another such NaN, one bit away in the
 // high word, so that one comparison tells empty, lost and value apart.
@@ -508,7 +508,9 @@ hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream) {
     const int W = (a.U + 1 + 63) / 64;
     const size_t slots = lattice_relay_slots(a.N, a.T, a.U);
     unsigned long long *relay = reinterpret_cast<unsigned long long *>(a.relay);
-    if (slots > 0) {
+    if (slots > 0 && a.relay_is_clear) {
+        if (!relay) return hipErrorInvalidValue;
+    } else if (slots > 0) {
         if (!relay) return hipErrorInvalidValue;
         const size_t blocks = (slots + 255) / 256;
         if (blocks > 0x7fffffffUL) return hipErrorInvalidValue;

@@ -47,6 +47,7 @@ struct LatticeArgs {
     double *betas;        // (N,T+1,P,2) log2 units
     float *costs;         // (N)
     void *relay;          // lattice_relay_slots(N,T,U) 64-bit words, or null if there are none
+    bool relay_is_clear;  // every slot already holds kRelayEmpty (see RelaySlots)
     int N, T, U;
     bool beta_only;
     CostReduce reduce;    // zero-initialise for plain per-sample costs
@@ -57,6 +58,32 @@ struct LatticeArgs {
 // hand one value per frame and 64-context boundary through device memory:
 // the number of 64-bit slots that takes (0 for U + 1 <= 64).
 size_t lattice_relay_slots(int N, int T, int U);
+// What a slot holds before its value has been stored: a NaN with a payload that
+// no arithmetic produces.
+constexpr unsigned long long kRelayEmpty = 0x7ff8dead5107e117ULL;
+// The slots of a lattice launch, for the kernel that runs before it on the same
+// stream to clear on the side (a launch of its own for a few hundred KB costs
+// more than the stores): every thread of that kernel's grid calls
+// relay_clear_share first thing, before it may return.
+struct RelaySlots {
+    unsigned long long *p = nullptr;
+    size_t n = 0;
+};
+inline RelaySlots relay_slots_of(void *relay, int N, int T, int U) {
+    RelaySlots r;
+    r.n = relay ? lattice_relay_slots(N, T, U) : 0;
+    r.p = r.n ? static_cast<unsigned long long *>(relay) : nullptr;
+    return r;
+}
+__device__ __forceinline__ void relay_clear_share(const RelaySlots &r) {
+    if (r.n == 0) return;
+    const size_t block = (size_t)blockIdx.z * gridDim.y * gridDim.x + (size_t)blockIdx.y * gridDim.x + blockIdx.x;
+    const size_t threads = (size_t)blockDim.x * blockDim.y * blockDim.z;
+    const size_t me = block * threads + (size_t)threadIdx.z * blockDim.y * blockDim.x +
+                      (size_t)threadIdx.y * blockDim.x + threadIdx.x;
+    const size_t all = threads * gridDim.x * gridDim.y * gridDim.z;
+    for (size_t i = me; i < r.n; i += all) r.p[i] = kRelayEmpty;
+}
 // How often a consumer asks again for a hand-over that has not arrived before
 // it declares its input lost (0: the first look decides; negative: the
 // default, about a second).  Applies to launches made afterwards; returns the
@@ -75,11 +102,12 @@ inline JointStrides dense_joint_strides(int T, int U, int V) {
 
 // band_only: cells outside the band of complete alignments get neutral units
 // (same costs and gradients; alpha / beta of dead cells are not the oracle's)
-// counter (may be null): set to 0 by the kernel, for a CostReduce that follows
+// counter (may be null): set to 0 by the kernel, for a CostReduce that follows;
+// relay: slots cleared by the kernel, for the lattice launch that follows
 hipError_t launch_gather_units(const void *joint, const JointStrides &strides, int io_type,
                                const int *ys, const int *lx, const int *ly, double *units, int N,
                                int T, int U, int V, bool band_only, unsigned *counter,
-                               hipStream_t stream);
+                               const RelaySlots &relay, hipStream_t stream);
 hipError_t launch_clear_counter(unsigned *counter, hipStream_t stream);
 hipError_t launch_scale_units(const float *units_nat, const int *lx, const int *ly, double *units,
                               int N, int T, int U, hipStream_t stream);
@@ -121,7 +149,8 @@ hipError_t launch_logits_grad(const void *logits, int io_type, const float *lse,
 // ---- log-add joiner path -------------------------------------------------
 hipError_t launch_simple_gather_units(const float *f, const float *g, const float *den,
                                       const int *ys, const int *lx, const int *ly, double *units,
-                                      int N, int T, int U, int V, hipStream_t stream);
+                                      int N, int T, int U, int V, const RelaySlots &relay,
+                                      hipStream_t stream);
 // compact gradients of the joiner path straight from the lattices: grad_f
 // (N,T,U+1), grad_g (N,U+1,3), grad_den (N,T,U+1) or null; `partial` is scratch
 // of N * T * (U+1) * 3 floats (partial sums over blocks of 8 frames, or, for

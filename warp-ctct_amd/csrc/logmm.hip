@@ -1054,7 +1054,8 @@ __global__ __launch_bounds__(64 * kBwdWaves) void logmm_bwd_lhs_slab_kernel(cons
     // set of registers, so that a block's rows are requested while the block
     // before it is worked on (64 us instead of 62: what a wavefront waits for is
     // mostly its own earlier stores, which retire in order with its loads), and
-    // 8 wavefronts with E_own requested per 16 columns (73 us).
+    // 8 wavefronts with E_own requested per 16 columns (73 us), and slabs of 64
+    // columns, which let three workgroups share a compute unit (71 us).
     for (int rb = wave; rb < row_blocks; rb += NW) {
         const int p = rb * 16 + c, pl = min(p, P - 1);
         const float *crow = a.C + (size_t)b * a.csb + (size_t)pl * Cq + 8 * g;

@@ -30,7 +30,8 @@ __device__ __forceinline__ int clampi(int v, int lo, int hi) { return min(max(v,
 __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     const float *__restrict__ f, const float *__restrict__ g, const float *__restrict__ den,
     const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
-    double *__restrict__ units, int T, int U, int V, int P) {
+    double *__restrict__ units, int T, int U, int V, int P, const RelaySlots relay) {
+    relay_clear_share(relay);
     const int U1 = U + 1;
     const int n = blockIdx.y;
     const int cell = blockIdx.x * kBlock + threadIdx.x;
@@ -313,12 +314,13 @@ inline dim3 cell_grid(int N, int T, int U) {
 
 hipError_t launch_simple_gather_units(const float *f, const float *g, const float *den,
                                       const int *ys, const int *lx, const int *ly, double *units,
-                                      int N, int T, int U, int V, hipStream_t stream) {
+                                      int N, int T, int U, int V, const RelaySlots &relay,
+                                      hipStream_t stream) {
     const int P = padded_contexts(U);
     const long cells = (long)T * P;
     TIMED_LAUNCH(simple_gather_units_kernel,
                        dim3((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N), dim3(kBlock),
-                       0, stream, f, g, den, ys, lx, ly, units, T, U, V, P);
+                       0, stream, f, g, den, ys, lx, ly, units, T, U, V, P, relay);
     return hipGetLastError();
 }
 

@@ -89,8 +89,9 @@ template <bool BAND_ONLY, typename IO>
 __global__ __launch_bounds__(kCellBlock) void gather_units_kernel(
     const IO *__restrict__ joint, const JointStrides js, const int *__restrict__ ys,
     const int *__restrict__ lx, const int *__restrict__ ly, double *__restrict__ units, int T,
-    int U, int V, int P, unsigned *__restrict__ counter) {
+    int U, int V, int P, unsigned *__restrict__ counter, const RelaySlots relay) {
     if (counter && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *counter = 0u;
+    relay_clear_share(relay);
     Cell c = locate_cell(lx, ly, T, U, P);
     if (BAND_ONLY && c.live && outside_band(c.t, c.u, c.Tn, c.Un)) c.live = false;
     if (store_padding(units, c, T, P)) return;
@@ -165,15 +166,15 @@ __global__ void clear_counter_kernel(unsigned *counter) { *counter = 0u; }
 template <typename IO>
 void launch_gather_typed(const void *joint, const JointStrides &js, const int *ys, const int *lx,
                          const int *ly, double *units, int N, int T, int U, int V, bool band_only,
-                         unsigned *counter, hipStream_t stream) {
+                         unsigned *counter, const RelaySlots &relay, hipStream_t stream) {
     const int P = padded_contexts(U);
     const IO *j = static_cast<const IO *>(joint);
     if (band_only) {
         TIMED_LAUNCH((gather_units_kernel<true, IO>), cell_grid(N, T, P), dim3(kCellBlock),
-                           0, stream, j, js, ys, lx, ly, units, T, U, V, P, counter);
+                           0, stream, j, js, ys, lx, ly, units, T, U, V, P, counter, relay);
     } else {
         TIMED_LAUNCH((gather_units_kernel<false, IO>), cell_grid(N, T, P), dim3(kCellBlock),
-                           0, stream, j, js, ys, lx, ly, units, T, U, V, P, counter);
+                           0, stream, j, js, ys, lx, ly, units, T, U, V, P, counter, relay);
     }
 }
 
@@ -182,19 +183,17 @@ void launch_gather_typed(const void *joint, const JointStrides &js, const int *y
 hipError_t launch_gather_units(const void *joint, const JointStrides &js, int io_type,
                                const int *ys, const int *lx, const int *ly, double *units, int N,
                                int T, int U, int V, bool band_only, unsigned *counter,
-                               hipStream_t stream) {
+                               const RelaySlots &relay, hipStream_t stream) {
     switch (io_type) {
         case kIoF32:
-            launch_gather_typed<float>(joint, js, ys, lx, ly, units, N, T, U, V, band_only, counter,
-                                       stream);
+            launch_gather_typed<float>(joint, js, ys, lx, ly, units, N, T, U, V, band_only, counter, relay, stream);
             break;
         case kIoF16:
-            launch_gather_typed<__half>(joint, js, ys, lx, ly, units, N, T, U, V, band_only,
-                                        counter, stream);
+            launch_gather_typed<__half>(joint, js, ys, lx, ly, units, N, T, U, V, band_only, counter, relay, stream);
             break;
         case kIoBF16:
             launch_gather_typed<__hip_bfloat16>(joint, js, ys, lx, ly, units, N, T, U, V,
-                                                band_only, counter, stream);
+                                                band_only, counter, relay, stream);
             break;
         default:
             return hipErrorInvalidValue;
