@@ -1140,10 +1140,7 @@ __global__ __launch_bounds__(64 * kBwdWaves) void logmm_bwd_lhs_slab_kernel(cons
 // conflicts).  The next chunk is loaded while the present one is multiplied.
 constexpr int kRhsSlab = 128;
 constexpr int kRhsLd = TQ + 8;       // bfloat16 per LDS row (80 bytes)
-#ifndef RHS_DEPTH
-#define RHS_DEPTH 3
-#endif
-constexpr int kRhsDepth = RHS_DEPTH;
+constexpr int kRhsDepth = 3;          // chunks on their way while one is multiplied
 
 template <int UB, int DEPTH>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void logmm_bwd_rhs_slab_kernel(const BwdArgs a) {
@@ -1329,8 +1326,7 @@ hipError_t launch_bwd(const BwdArgs &args, int B, hipStream_t stream) {
 #undef LAUNCH_LHS_SLAB
         return hipGetLastError();
     }
-    if (a.cgp == 1 && a.P <= 96 && a.Kp >= 2 * kRhsSlab && a.Q >= 4 * TQ &&
-        !getenv("WARPCTCT_NO_RHS_SLAB")) {
+    if (a.cgp == 1 && a.P <= 96 && a.Kp >= 2 * kRhsSlab && a.Q >= 4 * TQ) {
         // few rows, long reduction with the reduction index as the row index of C
         // (the gradient of the operand with few rows): sums in registers, E_oth
         // streamed once
@@ -1338,35 +1334,13 @@ hipError_t launch_bwd(const BwdArgs &args, int B, hipStream_t stream) {
         a.tiles_x = (a.Kp + kRhsSlab - 1) / kRhsSlab, a.tiles_y = 1;
         if (!xcd_grid_fits(a.tiles_x, 1, B)) return hipErrorInvalidValue;
         const dim3 grid(xcd_grid(a.tiles_x, 1, B));
-        const char *dep_s = getenv("WARPCTCT_RHS_DEPTH");
-        const int dep = dep_s ? atoi(dep_s) : kRhsDepth;
-        if (dep == 2) {
         switch (ub) {
-            case 1: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<1, 2>), grid, dim3(256), 0, stream, a); break;
-            case 2: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<2, 2>), grid, dim3(256), 0, stream, a); break;
-            case 3: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<3, 2>), grid, dim3(256), 0, stream, a); break;
-            case 4: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<4, 2>), grid, dim3(256), 0, stream, a); break;
-            case 5: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<5, 2>), grid, dim3(256), 0, stream, a); break;
-            default: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<6, 2>), grid, dim3(256), 0, stream, a); break;
-        }
-        } else if (dep == 4) {
-        switch (ub) {
-            case 1: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<1, 4>), grid, dim3(256), 0, stream, a); break;
-            case 2: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<2, 4>), grid, dim3(256), 0, stream, a); break;
-            case 3: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<3, 4>), grid, dim3(256), 0, stream, a); break;
-            case 4: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<4, 4>), grid, dim3(256), 0, stream, a); break;
-            case 5: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<5, 4>), grid, dim3(256), 0, stream, a); break;
-            default: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<6, 4>), grid, dim3(256), 0, stream, a); break;
-        }
-        } else {
-        switch (ub) {
-            case 1: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<1, 3>), grid, dim3(256), 0, stream, a); break;
-            case 2: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<2, 3>), grid, dim3(256), 0, stream, a); break;
-            case 3: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<3, 3>), grid, dim3(256), 0, stream, a); break;
-            case 4: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<4, 3>), grid, dim3(256), 0, stream, a); break;
-            case 5: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<5, 3>), grid, dim3(256), 0, stream, a); break;
-            default: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<6, 3>), grid, dim3(256), 0, stream, a); break;
-        }
+            case 1: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<1, kRhsDepth>), grid, dim3(256), 0, stream, a); break;
+            case 2: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<2, kRhsDepth>), grid, dim3(256), 0, stream, a); break;
+            case 3: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<3, kRhsDepth>), grid, dim3(256), 0, stream, a); break;
+            case 4: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<4, kRhsDepth>), grid, dim3(256), 0, stream, a); break;
+            case 5: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<5, kRhsDepth>), grid, dim3(256), 0, stream, a); break;
+            default: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<6, kRhsDepth>), grid, dim3(256), 0, stream, a); break;
         }
         return hipGetLastError();
     }
