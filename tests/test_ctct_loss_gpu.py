@@ -684,6 +684,30 @@ def test_gradient_buffer_cleared_in_the_forward_or_in_the_backward():
         warp_ctct.CLEAR_GRADIENT_IN_FORWARD = True
 
 
+def test_label_range_check_is_opt_in():
+    """Labels outside [0, V) are clamped by the kernels (no fault, a finite loss);
+    with warp_ctct.CHECK_LABEL_RANGE the call raises as torch.gather does in the
+    reference (warp_ctct/__init__.py:131)."""
+    import warp_ctct
+    joint, ys, lx, ly = make_joint_case(77, 2, 9, 4, 7)
+    ys[0, 1] = 7                              # == V
+    ys[1, 0] = -1
+    x, d_ys, d_lx, d_ly = dev(joint), dev(ys), dev(lx), dev(ly)
+    assert torch.isfinite(warp_ctct.ctct_loss(x, d_ys, d_lx, d_ly, reduction="none")).all()
+    warp_ctct.CHECK_LABEL_RANGE = True
+    try:
+        with pytest.raises(IndexError):
+            warp_ctct.ctct_loss(x, d_ys, d_lx, d_ly)
+        with pytest.raises(IndexError):
+            warp_ctct.ctct_loss_with_logits(x, d_ys, d_lx, d_ly)
+        with pytest.raises(IndexError):
+            warp_ctct.ctct_simple_loss(x[:, :, 0], x[:, 0], d_ys, d_lx, d_ly)
+        ys[0, 1], ys[1, 0] = 6, 0
+        assert torch.isfinite(warp_ctct.ctct_loss(x, dev(ys), d_lx, d_ly, reduction="none")).all()
+    finally:
+        warp_ctct.CHECK_LABEL_RANGE = False
+
+
 def test_infeasible_sample_has_infinite_cost():
     import warp_ctct
     joint, ys, lx, ly = make_joint_case(17, 2, 6, 3, 5, force_repeat=False)

@@ -58,6 +58,21 @@ def set_kernel_observer(observer):
 # allocate and clear it in the backward instead.
 CLEAR_GRADIENT_IN_FORWARD = True
 
+# The kernels clamp labels into [0, V) before they use them as column indices,
+# so that a corrupt label cannot make the GPU fault; the reference's
+# torch.gather raises on such an index (warp_ctct/__init__.py:131).  Set this
+# to True to get that behaviour back while debugging a data pipeline: every
+# call then checks its labels on the host (one device-to-host synchronisation).
+CHECK_LABEL_RANGE = False
+
+
+def _check_labels(labels, vocabulary):
+    if CHECK_LABEL_RANGE and labels.numel() > 0:
+        lo, hi = int(labels.min()), int(labels.max())
+        if lo < 0 or hi >= vocabulary:
+            raise IndexError("labels must lie in [0, %d): found values from %d to %d"
+                             % (vocabulary, lo, hi))
+
 
 def _run(name, fn):
     if _kernel_observer is None:
@@ -290,6 +305,7 @@ def ctct_loss(log_probs: torch.Tensor,
         # nothing to launch; costs of an empty batch, still attached to the graph
         return _reduce(log_probs.float().sum(dim=(1, 2, 3)), frames_lengths, reduction,
                        average_frames)
+    _check_labels(labels, log_probs.size(3))
     enable_grad = log_probs.requires_grad and torch.is_grad_enabled()
     if log_probs.dtype not in _NATIVE_DTYPES:
         log_probs = log_probs.float()      # as the reference does for every dtype (:135)
@@ -360,6 +376,7 @@ def ctct_loss_with_logits(logits: torch.Tensor,
     if logits.size(0) == 0:
         return _reduce(logits.float().sum(dim=(1, 2, 3)), frames_lengths, reduction,
                        average_frames)
+    _check_labels(labels, logits.size(3))
     enable_grad = logits.requires_grad and torch.is_grad_enabled()
     if logits.dtype not in _NATIVE_DTYPES:
         logits = logits.float()
@@ -394,6 +411,7 @@ def ctct_simple_loss(f: torch.Tensor,
     assert g.size(1) == labels.size(1) + 1
     assert f.size(0) == g.size(0) == labels.size(0) == frames_lengths.size(0) == labels_lengths.size(0)
 
+    _check_labels(labels, f.size(-1))
     track_f = f.requires_grad and torch.is_grad_enabled()
     track_g = g.requires_grad and torch.is_grad_enabled()
     with _no_autocast():
