@@ -385,6 +385,38 @@ def test_simple_loss_partial_tracking_and_reduction(track):
 
 
 @pytest.mark.parametrize("normalized", [True, False])
+@pytest.mark.parametrize("case", [(3, 15, 5, 12, [15, 11, 8], [5, 3, 4]),
+                                  (2, 140, 80, 9, [140, 125], [80, 70]),       # chains of two
+                                  (2, 9, 4, 7, [9, 1], [4, 0])])
+def test_simple_loss_repeated_labels_weighted_and_backward_twice(case, normalized):
+    """Every other label repeats its neighbour (their columns of the dense gradients
+    coincide and add), per-sample weights, and a second backward over a retained
+    graph, which must give the same gradients again."""
+    import warp_ctct
+    N, T, U, V, lx, ly = case
+    f, g, ys, lx, ly = make_simple_case(17, N, T, U, V, lx=lx, ly=ly, normalized=normalized)
+    k = ys[:, 1::2].shape[1]
+    ys[:, 1::2] = ys[:, 0::2][:, :k]
+    w = np.linspace(0.5, 2.0, N)
+    _, gf, gg, costs = O.ctct_simple_loss(f, g, ys, lx, ly, reduction="none",
+                                          normalized=normalized, grad_output=w)
+    tf, tg = dev(f).requires_grad_(True), dev(g).requires_grad_(True)
+    out = warp_ctct.ctct_simple_loss(tf, tg, dev(ys), dev(lx), dev(ly), reduction="none",
+                                     normalized=normalized)
+    fin = np.isfinite(costs)
+    np.testing.assert_allclose(out.detach().cpu().numpy()[fin], costs[fin], rtol=LOSS_RTOL)
+    assert fin.all()
+    (out * dev(w, torch.float32)).sum().backward(retain_graph=True)
+    first = (tf.grad.clone(), tg.grad.clone())
+    tf.grad, tg.grad = None, None
+    (out * dev(w, torch.float32)).sum().backward()
+    for a, b in zip(first, (tf.grad, tg.grad)):
+        torch.testing.assert_close(a, b, atol=1e-6, rtol=1e-6)
+    np.testing.assert_allclose(first[0].cpu().numpy(), gf, atol=GRAD_ATOL, rtol=1e-5)
+    np.testing.assert_allclose(first[1].cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
+
+
+@pytest.mark.parametrize("normalized", [True, False])
 def test_simple_loss_edge_shapes(normalized):
     """No label dimension at all (g holds the one start context), samples
     without labels beside samples with labels, a single frame, an empty batch."""
