@@ -1142,9 +1142,9 @@ constexpr int kRhsSlab = 128;
 constexpr int kRhsLd = TQ + 8;       // bfloat16 per LDS row (80 bytes)
 constexpr int kRhsDepth = 3;          // chunks on their way while one is multiplied
 
-template <int UB, int DEPTH>
+template <int UB>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void logmm_bwd_rhs_slab_kernel(const BwdArgs a) {
-    constexpr int NT = 256;
+    constexpr int NT = 256, DEPTH = kRhsDepth;
     __shared__ __attribute__((aligned(16))) __bf16 s_el[3][kRhsSlab][kRhsLd];   // E_oth^T planes
     __shared__ __attribute__((aligned(16))) __bf16 s_ct[3][16 * UB][kRhsLd];    // C^T planes
     __shared__ int s_unsafe;
@@ -1335,12 +1335,12 @@ hipError_t launch_bwd(const BwdArgs &args, int B, hipStream_t stream) {
         if (!xcd_grid_fits(a.tiles_x, 1, B)) return hipErrorInvalidValue;
         const dim3 grid(xcd_grid(a.tiles_x, 1, B));
         switch (ub) {
-            case 1: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<1, kRhsDepth>), grid, dim3(256), 0, stream, a); break;
-            case 2: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<2, kRhsDepth>), grid, dim3(256), 0, stream, a); break;
-            case 3: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<3, kRhsDepth>), grid, dim3(256), 0, stream, a); break;
-            case 4: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<4, kRhsDepth>), grid, dim3(256), 0, stream, a); break;
-            case 5: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<5, kRhsDepth>), grid, dim3(256), 0, stream, a); break;
-            default: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<6, kRhsDepth>), grid, dim3(256), 0, stream, a); break;
+            case 1: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<1>), grid, dim3(256), 0, stream, a); break;
+            case 2: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<2>), grid, dim3(256), 0, stream, a); break;
+            case 3: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<3>), grid, dim3(256), 0, stream, a); break;
+            case 4: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<4>), grid, dim3(256), 0, stream, a); break;
+            case 5: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<5>), grid, dim3(256), 0, stream, a); break;
+            default: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<6>), grid, dim3(256), 0, stream, a); break;
         }
         return hipGetLastError();
     }
