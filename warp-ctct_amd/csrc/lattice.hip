@@ -45,7 +45,7 @@ namespace wctct {
 
 namespace {
 
-constexpr int R = 8;          // frames per chunk (prefetch depth and hand-over granularity)
+constexpr int kRelayPad = 16;   // slots behind a boundary's T: a request may start at any step <= T
 constexpr int kMaxSpins = 1 << 20;   // ~1 s of polling before a hand-over is given up (default)
 
 // What a relay slot holds before its value has been stored: a NaN with a
@@ -71,25 +71,6 @@ __device__ __forceinline__ void front_store(double *dst, const Front &f) {
     *reinterpret_cast<double2 *>(dst) = make_double2(f.o, f.e);
 }
 
-struct Chunk {
-    double lp[R][3];
-};
-
-// Units of frames t_first + dir*r, r in [0,R); the frame index is clamped into
-// [0, Tn-1] so that a prefetch past the end re-reads a valid row (its values
-// are then not used).
-__device__ __forceinline__ void chunk_load(Chunk &c, const double *units_lane, size_t row, int Tn,
-                                           int t_first, int dir) {
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int t = min(max(t_first + dir * r, 0), Tn - 1);
-        const double *p = units_lane + (size_t)t * row;
-        c.lp[r][0] = p[0];
-        c.lp[r][1] = p[1];
-        c.lp[r][2] = p[2];
-    }
-}
-
 // A lone wavefront issues one instruction at a time, so the address arithmetic
 // of a frame costs as much as its semiring sums.  Rows are therefore walked:
 // loads follow a pointer that moves by one row per frame (two scalar additions
@@ -105,22 +86,6 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t rows_from(const void *lowest) 
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(lowest), 0, 0xffffffffu, 0x00020000);
 }
 
-// The units of R frames that all exist.  `frame` points at the row of the
-// chunk's first frame (the same for all lanes) and is moved on by the chunk;
-// `step` = bytes per frame; DOWN: frames run towards lower addresses.
-template <bool DOWN>
-__device__ __forceinline__ void chunk_load_walk(Chunk &c, const char *&frame, unsigned lane_bytes,
-                                                unsigned step) {
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const double *p = reinterpret_cast<const double *>(frame + lane_bytes);
-        c.lp[r][0] = p[0];
-        c.lp[r][1] = p[1];
-        c.lp[r][2] = p[2];
-        frame = DOWN ? frame - step : frame + step;
-    }
-}
-
 __device__ __forceinline__ void front_store_at(__amdgpu_buffer_rsrc_t rows, unsigned lane_bytes,
                                                unsigned at, const Front &f) {
     v4u w;
@@ -131,38 +96,11 @@ __device__ __forceinline__ void front_store_at(__amdgpu_buffer_rsrc_t rows, unsi
 
 // ---- hand-over between the workgroups of one lattice -------------------------
 // slots[s] belongs to step s of the sweep (s < Tn <= T); a boundary has
-// T + R of them.  Relaxed atomics at agent scope: the store goes to the L2,
+// T + kRelayPad of them.  Relaxed atomics at agent scope: the store goes to the L2,
 // the load comes from there.
 __device__ __forceinline__ void slot_put(unsigned long long *slot, double v) {
     __hip_atomic_store(slot, (unsigned long long)__double_as_longlong(v), __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Requests the slots of steps s0 .. s0+R-1 (a boundary has T + R slots, so a
-// request that starts at any step s0 <= T stays inside; what lies beyond the
-// chunk's cnt steps is not looked at).  Nothing waits for the loads until the
-// values are used.
-__device__ __forceinline__ void slots_request(const unsigned long long *slots, int s0,
-                                              unsigned long long (&bits)[R]) {
-    const unsigned long long *p = slots + s0;
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-        bits[r] = __hip_atomic_load(p + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// State of the chunk's cnt slots: the smallest of (high word xor the empty
-// pattern's).  0: one is still empty; 1: none is empty and one says "lost";
-// anything else: all hold values (no value has either high word: they are NaN
-// payloads no arithmetic produces).  The same for all lanes.
-__device__ __forceinline__ unsigned slots_state(const unsigned long long (&bits)[R], int cnt) {
-    constexpr unsigned kEmptyHigh = (unsigned)(kEmptyBits >> 32);
-    unsigned least = 0xffffffffu;
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const unsigned d = (unsigned)(bits[r] >> 32) ^ kEmptyHigh;
-        least = min(least, r < cnt ? d : 0xffffffffu);
-    }
-    return (unsigned)__builtin_amdgcn_readfirstlane((int)least);
 }
 
 // ---- alpha ---------------------------------------------------------------
@@ -214,6 +152,82 @@ __device__ __forceinline__ void beta_step(Front &f, const double *lp, bool skip,
     f.o = (__builtin_fmax(stay_o, sel) + (1.0 + o_mask)) + l2;
 }
 
+// Every relay slot = empty, before the sweeps of a launch.
+__global__ __launch_bounds__(256) void relay_clear_kernel(unsigned long long *slots, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) slots[i] = kEmptyBits;
+}
+
+// Everything that depends on the chunk size R (frames per chunk: prefetch depth
+// and hand-over granularity).  Two sizes are in use: 16 for the plain lattice
+// launch (units asked for two microseconds ahead: 3-7 % faster sweeps), 8 for the
+// launch that also clears memory, whose clearing workgroups share the kernel's
+// register count and need four wavefronts per SIMD (at 16 the kernel takes 256
+// registers and the clear twice its time).
+template <int R>
+struct Chunked {
+struct Chunk {
+    double lp[R][3];
+};
+
+// Units of frames t_first + dir*r, r in [0,R); the frame index is clamped into
+// [0, Tn-1] so that a prefetch past the end re-reads a valid row (its values
+// are then not used).
+static __device__ __forceinline__ void chunk_load(Chunk &c, const double *units_lane, size_t row, int Tn,
+                                           int t_first, int dir) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int t = min(max(t_first + dir * r, 0), Tn - 1);
+        const double *p = units_lane + (size_t)t * row;
+        c.lp[r][0] = p[0];
+        c.lp[r][1] = p[1];
+        c.lp[r][2] = p[2];
+    }
+}
+
+// The units of R frames that all exist.  `frame` points at the row of the
+// chunk's first frame (the same for all lanes) and is moved on by the chunk;
+// `step` = bytes per frame; DOWN: frames run towards lower addresses.
+template <bool DOWN>
+static __device__ __forceinline__ void chunk_load_walk(Chunk &c, const char *&frame, unsigned lane_bytes,
+                                                unsigned step) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const double *p = reinterpret_cast<const double *>(frame + lane_bytes);
+        c.lp[r][0] = p[0];
+        c.lp[r][1] = p[1];
+        c.lp[r][2] = p[2];
+        frame = DOWN ? frame - step : frame + step;
+    }
+}
+
+// Requests the slots of steps s0 .. s0+R-1 (a boundary has T + kRelayPad slots, so a
+// request that starts at any step s0 <= T stays inside; what lies beyond the
+// chunk's cnt steps is not looked at).  Nothing waits for the loads until the
+// values are used.
+static __device__ __forceinline__ void slots_request(const unsigned long long *slots, int s0,
+                                              unsigned long long (&bits)[R]) {
+    const unsigned long long *p = slots + s0;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+        bits[r] = __hip_atomic_load(p + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// State of the chunk's cnt slots: the smallest of (high word xor the empty
+// pattern's).  0: one is still empty; 1: none is empty and one says "lost";
+// anything else: all hold values (no value has either high word: they are NaN
+// payloads no arithmetic produces).  The same for all lanes.
+static __device__ __forceinline__ unsigned slots_state(const unsigned long long (&bits)[R], int cnt) {
+    constexpr unsigned kEmptyHigh = (unsigned)(kEmptyBits >> 32);
+    unsigned least = 0xffffffffu;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const unsigned d = (unsigned)(bits[r] >> 32) ^ kEmptyHigh;
+        least = min(least, r < cnt ? d : 0xffffffffu);
+    }
+    return (unsigned)__builtin_amdgcn_readfirstlane((int)least);
+}
+
 // One direction of the 64 contexts [64*wave, 64*wave + 64) of one lattice.
 // BETA selects the direction; step s handles frame t = s (alpha) or Tn-1-s
 // (beta) and stores the front of frame t+1 (alpha) or t (beta).
@@ -225,7 +239,7 @@ __device__ __forceinline__ void beta_step(Front &f, const double *lp, bool skip,
 // that enter lane 0 / lane 63 are copied once more per frame, and a lone
 // wavefront pays for every instruction (chains of five: 199 -> 182 us).
 template <bool BETA, bool HAS_IN>
-__device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T, int P, int wave,
+static __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T, int P, int wave,
                       double *lat_n, float *cost_n, const unsigned long long *slots_in,
                       unsigned long long *slots_out, int max_spins) {
     const int lane = threadIdx.x & 63;
@@ -371,18 +385,12 @@ __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T
     if (BETA && u == 0) *cost_n = (float)(-f.e * kLn2);
 }
 
-// Every relay slot = empty, before the sweeps of a launch.
-__global__ __launch_bounds__(256) void relay_clear_kernel(unsigned long long *slots, size_t n) {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) slots[i] = kEmptyBits;
-}
-
 // One wavefront per workgroup.  Workgroup index = link * chains_pad + chain with
 // chain = n * dirs + d (d = 0: beta, which also produces the cost; d = 1:
 // alpha), chains_pad = the number of chains rounded up to a multiple of 8 (the
 // surplus workgroups exit), link = position in the chain of W workgroups, first
 // producer first: alpha starts at contexts 0..63, beta at the last 64.
-__device__ __forceinline__ void lattice_block(const double *__restrict__ units,
+static __device__ __forceinline__ void lattice_block(const double *__restrict__ units,
                                               const int *__restrict__ ys,
                                               const int *__restrict__ lx,
                                               const int *__restrict__ ly,
@@ -409,8 +417,8 @@ __device__ __forceinline__ void lattice_block(const double *__restrict__ units,
     const int *y = ys + (size_t)n * U;
     const size_t lat = (size_t)(T + 1) * P * 2;
     // boundary b lies between contexts 64b+63 and 64b+64; its slots for one
-    // direction of one sample: relay[((n*2 + direction)*(W-1) + b) * (T+R) ...]
-    const size_t TS = (size_t)T + R;
+    // direction of one sample: relay[((n*2 + direction)*(W-1) + b) * (T + kRelayPad) ...]
+    const size_t TS = (size_t)T + kRelayPad;
     unsigned long long *slots_n =
         relay ? relay + ((size_t)n * 2 + (beta ? 0 : 1)) * (size_t)(W - 1) * TS : nullptr;
     if (!beta) {
@@ -452,6 +460,8 @@ __device__ __forceinline__ void lattice_block(const double *__restrict__ units,
     if (lane == 0) *red.reduced = (red.mode == 2) ? s / (float)N : s;
 }
 
+};
+
 __global__ __launch_bounds__(64) void lattice_kernel(const double *__restrict__ units,
                                                      const int *__restrict__ ys,
                                                      const int *__restrict__ lx,
@@ -462,8 +472,8 @@ __global__ __launch_bounds__(64) void lattice_kernel(const double *__restrict__ 
                                                      unsigned long long *__restrict__ relay, int N,
                                                      int T, int U, int W, int dirs, int chains_pad,
                                                      const CostReduce red, int max_spins) {
-    lattice_block(units, ys, lx, ly, alphas, betas, costs, relay, N, T, U, W, dirs, chains_pad, red,
-                  max_spins);
+    Chunked<16>::lattice_block(units, ys, lx, ly, alphas, betas, costs, relay, N, T, U, W, dirs,
+                               chains_pad, red, max_spins);
 }
 
 // The same sweeps with a memory clear riding along: workgroups of 256 threads,
@@ -484,8 +494,8 @@ __global__ __launch_bounds__(256) void lattice_fill_kernel(
         return;
     }
     if (threadIdx.x >= 64) return;
-    lattice_block(units, ys, lx, ly, alphas, betas, costs, relay, N, T, U, W, dirs, chains_pad, red,
-                  max_spins);
+    Chunked<8>::lattice_block(units, ys, lx, ly, alphas, betas, costs, relay, N, T, U, W, dirs,
+                              chains_pad, red, max_spins);
 }
 
 }  // namespace
@@ -500,7 +510,7 @@ int lattice_wait_limit(int spins) {
 
 size_t lattice_relay_slots(int N, int T, int U) {
     const int W = (U + 1 + 63) / 64;
-    return (size_t)N * 2 * (size_t)(W - 1) * ((size_t)T + R);
+    return (size_t)N * 2 * (size_t)(W - 1) * ((size_t)T + kRelayPad);
 }
 
 hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream) {
