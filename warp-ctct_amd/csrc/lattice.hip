@@ -159,11 +159,12 @@ __global__ __launch_bounds__(256) void relay_clear_kernel(unsigned long long *sl
 }
 
 // Everything that depends on the chunk size R (frames per chunk: prefetch depth
-// and hand-over granularity).  Two sizes are in use: 16 for the plain lattice
-// launch (units asked for two microseconds ahead: 3-7 % faster sweeps), 8 for the
-// launch that also clears memory, whose clearing workgroups share the kernel's
-// register count and need four wavefronts per SIMD (at 16 the kernel takes 256
-// registers and the clear twice its time).
+// and hand-over granularity).  Two sizes are in use: 12 for the plain lattice
+// launch (units asked for 1.5 us ahead: 3-7 % faster sweeps than with 8; 16 is the
+// same within noise at the register limit, 24 slower), 8 for the launch that also
+// clears memory, whose clearing workgroups share the kernel's register count and
+// need four wavefronts per SIMD (at 16 the kernel takes 256 registers and the
+// clear twice its time).
 template <int R>
 struct Chunked {
 struct Chunk {
@@ -472,7 +473,7 @@ __global__ __launch_bounds__(64) void lattice_kernel(const double *__restrict__ 
                                                      unsigned long long *__restrict__ relay, int N,
                                                      int T, int U, int W, int dirs, int chains_pad,
                                                      const CostReduce red, int max_spins) {
-    Chunked<16>::lattice_block(units, ys, lx, ly, alphas, betas, costs, relay, N, T, U, W, dirs,
+    Chunked<12>::lattice_block(units, ys, lx, ly, alphas, betas, costs, relay, N, T, U, W, dirs,
                                chains_pad, red, max_spins);
 }
 
