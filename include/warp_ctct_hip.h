@@ -324,9 +324,18 @@ size_t warpctct_simple_workspace_bytes(int N, int T, int U);
  * (csrc/binding.cpp:103-222).  When normalized != 0, these are outputs that
  * the backward needs (otherwise they are ignored): den (N,T,U+1; only
  * t<lx[n], u<=ly[n] is written), fmax (N,T) = max_v f, gmax (N,U+1) = max_v g,
- * fexp (N,T,Vp) = exp(f - fmax) and gexp (N,U+1,Vp) = exp(g - gmax) with
+ * fexp (N,T,Vp) = exp(f - fmax) (see warpctct_simple_needs_fexp) and
+ * gexp (N,U+1,Vp) = exp(g - gmax) with
  * Vp = warpctct_logmm_padded_reduction(V), zero in the padding.
  * grad_f/grad_g/grad_den may all be NULL (no-grad mode). */
+/* 0 where the log-matmul kernels of the normalised path read f itself and form
+ * exp(f - fmax) on the way (U+1 <= 96 contexts, 512 <= V <= 2048 in whole
+ * multiples of 32, T >= 128, f aligned to 16 bytes): fexp is then neither
+ * written by the forward nor read by the backward and may be NULL in both.
+ * 1 otherwise.  No counterpart in the reference (which recomputes every
+ * exponential in every kernel, csrc/logmatmul.cu:44-146). */
+int warpctct_simple_needs_fexp(const float *f, int T, int U, int V);
+
 int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, const int *lx,
                                 const int *ly, int N, int T, int U, int V, int normalized,
                                 void *workspace, size_t workspace_bytes, float *den, float *fmax,

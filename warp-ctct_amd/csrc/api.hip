@@ -676,6 +676,12 @@ size_t warpctct_simple_workspace_bytes(int N, int T, int U) {
     return carve_simple(nullptr, N, T, U).bytes;
 }
 
+int warpctct_simple_needs_fexp(const float *f, int T, int U, int V) {
+    if (T < 0 || U < 0 || V < 1) return 1;
+    const LogmmOperand lhs = {f, (long)T * V, (long)V, 1L};
+    return logmm_reads_lhs_itself(lhs, T, V, U + 1) ? 0 : 1;
+}
+
 int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, const int *lx,
                                 const int *ly, int N, int T, int U, int V, int normalized,
                                 void *workspace, size_t workspace_bytes, float *den, float *fmax,
@@ -687,7 +693,10 @@ int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, c
     if (!g || !lx || !ly || !costs || !workspace || (T > 0 && !f) || (U > 0 && !ys))
         return WARPCTCT_EINVAL;
     if (want_grad && (!grad_f || !grad_g || (normalized && !grad_den))) return WARPCTCT_EINVAL;
-    if (normalized && T > 0 && (!den || !fmax || !gmax || !fexp || !gexp)) return WARPCTCT_EINVAL;
+    // where the log-matmul kernels read f itself, exp(f - fmax) is not stored
+    const bool keeps_fexp = warpctct_simple_needs_fexp(f, T, U, V) != 0;
+    if (normalized && T > 0 && (!den || !fmax || !gmax || !gexp || (keeps_fexp && !fexp)))
+        return WARPCTCT_EINVAL;
     const SimpleWorkspace w = carve_simple(workspace, N, T, U);
     if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
     hipStream_t st = as_stream(stream);
@@ -696,7 +705,7 @@ int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, c
             // den[n,t,u] = logsumexp_v(f[n,t,v] + g[n,u,v]):  lhs = f, rhs[b,k,j] = g[b,j,k]
             const LogmmOperand lhs = {f, (long)T * V, (long)V, 1L};
             const LogmmOperand rhs = {g, (long)(U + 1) * V, 1L, (long)V};
-            const LogmmShifted sh = {fmax, gmax, fexp, gexp};
+            const LogmmShifted sh = {fmax, gmax, keeps_fexp ? fexp : nullptr, gexp};
             int rc = done(launch_logmm_shift_exp(lhs, rhs, sh, N, T, V, U + 1, lx, ly, st));
             if (rc != WARPCTCT_OK) return rc;
             rc = done(launch_logmm_fwd(lhs, rhs, sh, den, w.partial, N, T, V, U + 1, lx, ly, st));
@@ -757,7 +766,9 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
     if (N == 0) return WARPCTCT_OK;
     if (!lx || !ly || (U > 0 && !ys) || (dense_f && !grad_f) || (dense_g && !grad_g))
         return WARPCTCT_EINVAL;
-    if (den && (!f || !g || !grad_den || !fmax || !gmax || !fexp || !gexp || !workspace))
+    const bool keeps_fexp = warpctct_simple_needs_fexp(f, T, U, V) != 0;
+    if (den && (!f || !g || !grad_den || !fmax || !gmax || !gexp || !workspace ||
+                (keeps_fexp && !fexp)))
         return WARPCTCT_EINVAL;
     if (den && workspace_bytes < warpctct_simple_backward_workspace_bytes(N, T, U))
         return WARPCTCT_EWORKSPACE;
@@ -769,7 +780,8 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
         const LogmmOperand rhs = {g, (long)U1 * V, 1L, (long)V};
         const PairWorkspace pw = carve_pairs(workspace, N, T, U1);
         const LogmmShifted sh = {const_cast<float *>(fmax), const_cast<float *>(gmax),
-                                 const_cast<float *>(fexp), const_cast<float *>(gexp)};
+                                 keeps_fexp ? const_cast<float *>(fexp) : nullptr,
+                                 const_cast<float *>(gexp)};
         if (T > 0) {
             int rc = done(launch_logmm_pair_factor(grad_den, den, fmax, gmax, grad_out, lx, ly,
                                                    pw.factors, pw.flags, N, T, U1, st));

@@ -413,7 +413,9 @@ ctct_simple_fwd(const torch::Tensor &f, const torch::Tensor &g, const torch::Ten
         den = torch::empty({N, T, U + 1}, f.options());
         fmax = torch::empty({N, T}, f.options());
         gmax = torch::empty({N, U + 1}, f.options());
-        fexp = torch::empty({N, T, Vp}, f.options());
+        // (not needed where the kernels read f itself)
+        const bool keeps = warpctct_simple_needs_fexp(f.data_ptr<float>(), T, U, V) != 0;
+        fexp = keeps ? torch::empty({N, T, Vp}, f.options()) : torch::empty({0}, f.options());
         gexp = torch::empty({N, U + 1, Vp}, f.options());
         shifted = {fmax, gmax, fexp, gexp};
     }
@@ -428,7 +430,7 @@ ctct_simple_fwd(const torch::Tensor &f, const torch::Tensor &g, const torch::Ten
                  normalized ? den.data_ptr<float>() : nullptr,
                  normalized ? fmax.data_ptr<float>() : nullptr,
                  normalized ? gmax.data_ptr<float>() : nullptr,
-                 normalized ? fexp.data_ptr<float>() : nullptr,
+                 (normalized && fexp.numel() > 0) ? fexp.data_ptr<float>() : nullptr,
                  normalized ? gexp.data_ptr<float>() : nullptr, costs.data_ptr<float>(),
                  requires_grad ? grad_f.data_ptr<float>() : nullptr,
                  requires_grad ? grad_g.data_ptr<float>() : nullptr,
@@ -487,7 +489,8 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_simple_bwd(
         TORCH_CHECK(shifted[0].numel() == (int64_t)N * T &&
                         shifted[1].numel() == (int64_t)N * (U + 1),
                     "fmax must be (N,T), gmax (N,U+1)");
-        TORCH_CHECK(shifted[2].numel() == (int64_t)N * T * Vp &&
+        const bool keeps = warpctct_simple_needs_fexp(f.data_ptr<float>(), T, U, V) != 0;
+        TORCH_CHECK((shifted[2].numel() == (int64_t)N * T * Vp || !keeps) &&
                         shifted[3].numel() == (int64_t)N * (U + 1) * Vp,
                     "fexp must be (N,T,Vp), gexp (N,U+1,Vp)");
     }
@@ -501,7 +504,7 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_simple_bwd(
                  normalized ? den->data_ptr<float>() : nullptr,
                  normalized ? shifted[0].data_ptr<float>() : nullptr,
                  normalized ? shifted[1].data_ptr<float>() : nullptr,
-                 normalized ? shifted[2].data_ptr<float>() : nullptr,
+                 (normalized && shifted[2].numel() > 0) ? shifted[2].data_ptr<float>() : nullptr,
                  normalized ? shifted[3].data_ptr<float>() : nullptr, grad_f_g.data_ptr<float>(),
                  grad_g_g.data_ptr<float>(), normalized ? grad_den->data_ptr<float>() : nullptr,
                  ys.data_ptr<int>(), lx.data_ptr<int>(), ly.data_ptr<int>(),

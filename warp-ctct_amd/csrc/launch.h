@@ -196,6 +196,11 @@ inline int logmm_padded_reduction(int K) { return (K + 31) / 32 * 32; }
 struct LogmmShifted {
     float *lmax, *rmax, *El, *Er;
 };
+// El may be null where logmm_reads_lhs_itself(...) holds: launch_logmm_shift_exp
+// then writes the maxima only, and the forward (with `partial`) and both gradients
+// read lhs itself and exponentiate it on the way (one pass over lhs less per
+// forward, and no (B,M,Kp) buffer).
+bool logmm_reads_lhs_itself(const LogmmOperand &lhs, int M, int K, int Nn);
 
 // row_len / col_len (may be null): per-batch number of valid rows of lhs and
 // index of the last valid column of rhs; outputs outside are not computed.

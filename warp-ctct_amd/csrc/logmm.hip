@@ -65,7 +65,8 @@ __global__ __launch_bounds__(256) void shift_exp_kernel(const float *__restrict_
     float *e = E + ((size_t)b * R + r) * Kp;
     const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
     if (r >= Rb) {
-        for (int k = lane * 4; k < Kp; k += 256) *reinterpret_cast<v4f *>(e + k) = zero;
+        if (E)
+            for (int k = lane * 4; k < Kp; k += 256) *reinterpret_cast<v4f *>(e + k) = zero;
         if (lane == 0) mx[(size_t)b * R + r] = neg_inf_f();
         return;
     }
@@ -84,6 +85,7 @@ __global__ __launch_bounds__(256) void shift_exp_kernel(const float *__restrict_
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
     if (lane == 0) mx[(size_t)b * R + r] = m;
+    if (!E) return;                                   // the maxima only
     const float shift = finite_or_zero(m);
     if (vec) {
         for (int k = lane * 4; k < Kp; k += 256) {
@@ -120,7 +122,8 @@ __global__ __launch_bounds__(256) void shift_exp_rows_kernel(const float *__rest
     float *e = E + ((size_t)b * R + r) * Kp;
     const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
     if (r >= Rb) {
-        for (int k = lane * 4; k < Kp; k += 256) *reinterpret_cast<v4f *>(e + k) = zero;
+        if (E)
+            for (int k = lane * 4; k < Kp; k += 256) *reinterpret_cast<v4f *>(e + k) = zero;
         if (lane == 0) mx[(size_t)b * R + r] = neg_inf_f();
         return;
     }
@@ -138,6 +141,7 @@ __global__ __launch_bounds__(256) void shift_exp_rows_kernel(const float *__rest
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
     if (lane == 0) mx[(size_t)b * R + r] = m;
+    if (!E) return;                                   // the maxima only
     const float shift = finite_or_zero(m);
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
@@ -472,7 +476,11 @@ constexpr int kSlab = 256;
 constexpr int kSlabLd = kSlab + 8;   // bfloat16 per LDS row: 16-byte aligned, rows 4 banks apart
 constexpr int kSlabWaves = 8;        // two wavefronts per SIMD: one's matrix instructions cover the other's waits
 
-template <int CB>
+// RAW: E_l is not in memory; the kernel reads lhs itself (k contiguous, K a
+// multiple of 32) and forms exp(lhs - lmax) in registers on the way to the
+// split (the maxima come from a pass of their own).  E_l is then never
+// written: one pass over lhs less per step, and its memory.
+template <int CB, bool RAW>
 __global__ __launch_bounds__(64 * kSlabWaves) void logmm_fwd_slab_kernel(const FwdArgs a, int slabs) {
     constexpr int TN = 16 * CB, NW = kSlabWaves, NT = 64 * NW;
     constexpr int CH = kSlab / TQ / 2;                  // chunks of 32 per half slab
@@ -523,9 +531,12 @@ __global__ __launch_bounds__(64 * kSlabWaves) void logmm_fwd_slab_kernel(const F
     // block is walked without a branch (the waits are then counted exactly).
     // Vectors past the reduction are clamped into it (they meet zeros of the
     // slab), row blocks past the last repeat it (and are dropped).
-    auto request = [&](int st, int half, v4f (&A)[2 * CH]) {
+    auto request = [&](int st, int half, v4f (&A)[2 * CH], float &shift) {
         const int rb = wave + NW * min(st, steps - 1);
-        const float *row = a.El + ((size_t)b * M + min(rb * 16 + r, M - 1)) * Kp;
+        const int i = min(rb * 16 + r, M - 1);
+        const float *row = RAW ? a.lhs + (size_t)b * a.lsb + (size_t)i * a.lsm
+                               : a.El + ((size_t)b * M + i) * Kp;
+        if (RAW) shift = finite_or_zero(a.lmax[(size_t)b * M + i]);
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             const int k = min(k0 + TQ * (half * CH + c) + 8 * g, Kp - 8);
@@ -538,7 +549,7 @@ __global__ __launch_bounds__(64 * kSlabWaves) void logmm_fwd_slab_kernel(const F
     // use them, one group of GB column blocks at a time (the scheduler is held to
     // that: left alone it hoists all reads of a half and spills); the other
     // wavefront of the SIMD covers the wait.
-    auto multiply = [&](int half, const v4f (&A)[2 * CH]) {
+    auto multiply = [&](int half, const v4f (&A)[2 * CH], float shift) {
         bf16x8 xp[3];
 #pragma unroll
         for (int item = 0; item < 2 * CH; ++item) {
@@ -554,7 +565,9 @@ __global__ __launch_bounds__(64 * kSlabWaves) void logmm_fwd_slab_kernel(const F
             if (grp == 0) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    const Split3 sp = split3(i < 4 ? A[2 * c][i] : A[2 * c + 1][i - 4]);
+                    float x = i < 4 ? A[2 * c][i] : A[2 * c + 1][i - 4];
+                    if (RAW) x = exp2_hw((x - shift) * kLog2eF);
+                    const Split3 sp = split3(x);
                     xp[0][i] = sp.h, xp[1][i] = sp.m, xp[2][i] = sp.l;
                 }
             }
@@ -566,18 +579,19 @@ __global__ __launch_bounds__(64 * kSlabWaves) void logmm_fwd_slab_kernel(const F
         }
     };
     v4f A0[2 * CH], A1[2 * CH];
-    request(0, 0, A0);
+    float shift0 = 0.0f, shift1 = 0.0f;
+    request(0, 0, A0, shift0);
     // (the two halves in this order, as in the loop: the waits for a half are
     // counted from the loads issued after it)
     __builtin_amdgcn_sched_barrier(0);
-    request(0, 1, A1);
+    request(0, 1, A1, shift1);
     __builtin_amdgcn_sched_barrier(0);
     for (int st = 0; st < steps; ++st) {
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) acc[cb] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-        multiply(0, A0);
-        request(st + 1, 0, A0);
-        multiply(1, A1);
+        multiply(0, A0, shift0);
+        request(st + 1, 0, A0, shift0);
+        multiply(1, A1, shift1);
         // lane l holds D[4*(l/16) + q][l%16] of each block in register q; the
         // stores come before the second request, so that at the head of the
         // loop nothing but the two halves is outstanding
@@ -588,7 +602,7 @@ __global__ __launch_bounds__(64 * kSlabWaves) void logmm_fwd_slab_kernel(const F
 #pragma unroll
             for (int q = 0; q < 4; ++q) at[(size_t)q * a.pN + cb * 16] = acc[cb][q];
         __builtin_amdgcn_sched_barrier(0);
-        request(st + 1, 1, A1);
+        request(st + 1, 1, A1, shift1);
     }
 }
 
@@ -1007,7 +1021,9 @@ constexpr int kBwdSlab = 128;
 
 constexpr int kBwdWaves = 4;
 
-template <int QC, bool FAST>
+// RAW: E_own is not in memory; the kernel reads the operand itself (k contiguous,
+// K a multiple of 32) and forms exp(own - own_max) where it needs it.
+template <int QC, bool FAST, bool RAW>
 __global__ __launch_bounds__(64 * kBwdWaves) void logmm_bwd_lhs_slab_kernel(const BwdArgs a) {
     constexpr int QLD = QC * TQ + 8;            // bfloat16 per LDS row: rows 4 banks apart
     constexpr int KB = kBwdSlab / 16, NW = kBwdWaves, NT = 64 * NW;
@@ -1065,7 +1081,9 @@ __global__ __launch_bounds__(64 * kBwdWaves) void logmm_bwd_lhs_slab_kernel(cons
             cv[2 * ch] = *reinterpret_cast<const v4f *>(crow + TQ * ch);
             cv[2 * ch + 1] = *reinterpret_cast<const v4f *>(crow + TQ * ch + 4);
         }
-        const float *erow = a.Eown + ((size_t)b * P + pl) * Kp;
+        const float *erow = RAW ? a.own + (size_t)b * a.osb + (size_t)pl * a.osp
+                                : a.Eown + ((size_t)b * P + pl) * Kp;
+        const float own_shift = RAW ? finite_or_zero(a.own_max[(size_t)b * P + pl]) : 0.0f;
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
             ev[kb] = *reinterpret_cast<const v4f *>(erow + min(k0 + kb * 16 + 4 * g, Kp - 4));
@@ -1093,7 +1111,8 @@ __global__ __launch_bounds__(64 * kBwdWaves) void logmm_bwd_lhs_slab_kernel(cons
             const int k = k0 + kb * 16 + 4 * g;
             v4f v;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) v[q] = scaled_sum(acc[q], ev[kb][q]);
+            for (int q = 0; q < 4; ++q)
+                v[q] = scaled_sum(acc[q], RAW ? exp2_hw((ev[kb][q] - own_shift) * kLog2eF) : ev[kb][q]);
             float *dst = db + (size_t)p * a.dsp + (size_t)k * a.dsk;
             if (FAST) {
                 *reinterpret_cast<v4f *>(dst) = v;
@@ -1142,7 +1161,9 @@ constexpr int kRhsSlab = 128;
 constexpr int kRhsLd = TQ + 8;       // bfloat16 per LDS row (80 bytes)
 constexpr int kRhsDepth = 3;          // chunks on their way while one is multiplied
 
-template <int UB>
+// RAW: E_oth is not in memory; the kernel reads the long operand itself (k
+// contiguous, K a multiple of 32) and forms exp(oth - oth_max) before the split.
+template <int UB, bool RAW>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void logmm_bwd_rhs_slab_kernel(const BwdArgs a) {
     constexpr int NT = 256, DEPTH = kRhsDepth;
     __shared__ __attribute__((aligned(16))) __bf16 s_el[3][kRhsSlab][kRhsLd];   // E_oth^T planes
@@ -1169,24 +1190,36 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // staging roles: 4 rows q (tg) x 4 columns (k4 of the slab / u4 of C)
     const int tg = tid & 7, k4 = tid >> 3, u4 = tid >> 3;
     const bool has_c = u4 < 4 * UB;
-    const float *el_base = a.Eoth + (size_t)b * Q * Kp + min(k0 + 4 * k4, Kp - 4);
+    const float *el_base = (RAW ? a.oth + (size_t)b * a.tsb : a.Eoth + (size_t)b * Q * Kp) +
+                           min(k0 + 4 * k4, Kp - 4);
+    const size_t el_row = RAW ? (size_t)a.tsq : (size_t)Kp;
+    const float *shifts = a.oth_max + (size_t)b * Q;
     const float *c_base = a.C + (size_t)b * a.csb + 4 * u4;
     v4f el[DEPTH][4], cv[DEPTH][4];
-    // rows beyond the reduction: E_oth clamped to a valid row, C = 0
-    auto fetch = [&](int chunk, v4f (&e)[4], v4f (&cc)[4]) {
+    float sh[DEPTH][4];
+    // rows beyond the reduction: E_oth clamped to a valid row, C = 0 (RAW: to a
+    // row within the entry's own length, whose values and maximum are real ones;
+    // what lies in the padding of the operand is never looked at)
+    const int q_last = RAW ? max(Qb - 1, 0) : Q - 1;
+    auto fetch = [&](int chunk, v4f (&e)[4], v4f (&cc)[4], float (&shift)[4]) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int q = chunk * TQ + 4 * tg + j;
-            e[j] = *reinterpret_cast<const v4f *>(el_base + (size_t)min(q, Q - 1) * Kp);
+            e[j] = *reinterpret_cast<const v4f *>(el_base + (size_t)min(q, q_last) * el_row);
+            if (RAW) shift[j] = finite_or_zero(shifts[min(q, q_last)]);
             cc[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
             if (has_c && q < Qb) cc[j] = *reinterpret_cast<const v4f *>(c_base + (size_t)q * a.cgq);
         }
     };
     // 4 rows x 4 columns -> per column the 4 rows as bfloat16 planes, 8 bytes each
-    auto stash = [&](const v4f (&e)[4], const v4f (&cc)[4]) {
+    auto stash = [&](const v4f (&e)[4], const v4f (&cc)[4], const float (&shift)[4]) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const Pair3 lo = split3_pair(e[0][i], e[1][i]), hi = split3_pair(e[2][i], e[3][i]);
+            float x[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                x[j] = RAW ? exp2_hw((e[j][i] - shift[j]) * kLog2eF) : e[j][i];
+            const Pair3 lo = split3_pair(x[0], x[1]), hi = split3_pair(x[2], x[3]);
             *reinterpret_cast<uint2 *>(&s_el[0][4 * k4 + i][4 * tg]) = make_uint2(lo.h, hi.h);
             *reinterpret_cast<uint2 *>(&s_el[1][4 * k4 + i][4 * tg]) = make_uint2(lo.m, hi.m);
             *reinterpret_cast<uint2 *>(&s_el[2][4 * k4 + i][4 * tg]) = make_uint2(lo.l, hi.l);
@@ -1210,15 +1243,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // DEPTH chunks are on their way while one is multiplied: a chunk's phases
     // (split and store, multiply) take about a microsecond, a load takes longer
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) fetch(d, el[d], cv[d]);
+    for (int d = 0; d < DEPTH; ++d) fetch(d, el[d], cv[d], sh[d]);
     for (int chunk = 0; chunk < n; chunk += DEPTH) {
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {
             if (chunk + d >= n) break;
             __syncthreads();                    // the chunk before is no longer read
-            stash(el[d], cv[d]);
+            stash(el[d], cv[d], sh[d]);
             __syncthreads();
-            fetch(chunk + d + DEPTH, el[d], cv[d]);
+            fetch(chunk + d + DEPTH, el[d], cv[d], sh[d]);
             bf16x8 bk[2][3];
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk)
@@ -1308,14 +1341,22 @@ hipError_t launch_bwd(const BwdArgs &args, int B, hipStream_t stream) {
         // bounds to check in the kernel
         const bool fast = a.P % 16 == 0 && a.K % kBwdSlab == 0 && a.dsk == 1 && (a.dsp & 3) == 0 &&
                           (a.dsb & 3) == 0 && (reinterpret_cast<uintptr_t>(a.grad) & 15u) == 0;
+        const bool raw = a.Eown == nullptr;
+        if (!a.Eoth || (raw && (a.osk != 1 || a.K != a.Kp))) return hipErrorInvalidValue;
 #define LAUNCH_LHS_SLAB(QCN)                                                                   \
     do {                                                                                       \
-        if (fast)                                                                              \
-            TIMED_LAUNCH((logmm_bwd_lhs_slab_kernel<QCN, true>), grid, dim3(64 * kBwdWaves), lds, \
-                         stream, a);                                                           \
+        if (fast && raw)                                                                       \
+            TIMED_LAUNCH((logmm_bwd_lhs_slab_kernel<QCN, true, true>), grid, dim3(64 * kBwdWaves), \
+                         lds, stream, a);                                                      \
+        else if (fast)                                                                         \
+            TIMED_LAUNCH((logmm_bwd_lhs_slab_kernel<QCN, true, false>), grid, dim3(64 * kBwdWaves), \
+                         lds, stream, a);                                                      \
+        else if (raw)                                                                          \
+            TIMED_LAUNCH((logmm_bwd_lhs_slab_kernel<QCN, false, true>), grid, dim3(64 * kBwdWaves), \
+                         lds, stream, a);                                                      \
         else                                                                                   \
-            TIMED_LAUNCH((logmm_bwd_lhs_slab_kernel<QCN, false>), grid, dim3(64 * kBwdWaves), lds, \
-                         stream, a);                                                           \
+            TIMED_LAUNCH((logmm_bwd_lhs_slab_kernel<QCN, false, false>), grid, dim3(64 * kBwdWaves), \
+                         lds, stream, a);                                                      \
     } while (0)
         if (qc == 1)
             LAUNCH_LHS_SLAB(1);
@@ -1334,16 +1375,27 @@ hipError_t launch_bwd(const BwdArgs &args, int B, hipStream_t stream) {
         a.tiles_x = (a.Kp + kRhsSlab - 1) / kRhsSlab, a.tiles_y = 1;
         if (!xcd_grid_fits(a.tiles_x, 1, B)) return hipErrorInvalidValue;
         const dim3 grid(xcd_grid(a.tiles_x, 1, B));
+        const bool raw = a.Eoth == nullptr;
+        if (!a.Eown || (raw && (a.tsk != 1 || a.K != a.Kp))) return hipErrorInvalidValue;
+#define RHS_SLAB(UBN)                                                                          \
+    do {                                                                                       \
+        if (raw)                                                                               \
+            TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<UBN, true>), grid, dim3(256), 0, stream, a); \
+        else                                                                                   \
+            TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<UBN, false>), grid, dim3(256), 0, stream, a); \
+    } while (0)
         switch (ub) {
-            case 1: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<1>), grid, dim3(256), 0, stream, a); break;
-            case 2: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<2>), grid, dim3(256), 0, stream, a); break;
-            case 3: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<3>), grid, dim3(256), 0, stream, a); break;
-            case 4: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<4>), grid, dim3(256), 0, stream, a); break;
-            case 5: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<5>), grid, dim3(256), 0, stream, a); break;
-            default: TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<6>), grid, dim3(256), 0, stream, a); break;
+            case 1: RHS_SLAB(1); break;
+            case 2: RHS_SLAB(2); break;
+            case 3: RHS_SLAB(3); break;
+            case 4: RHS_SLAB(4); break;
+            case 5: RHS_SLAB(5); break;
+            default: RHS_SLAB(6); break;
         }
+#undef RHS_SLAB
         return hipGetLastError();
     }
+    if (!a.Eown || !a.Eoth) return hipErrorInvalidValue;   // only the slab kernels read an operand itself
     if (a.Q <= QR && !prefer_96(a.P)) {
         // short reduction, many rows: C slab resident, a few k tiles per workgroup
         const int ptiles = (a.P + 63) / 64, ktiles = (a.K + 63) / 64;
@@ -1410,6 +1462,16 @@ void launch_shift_exp_rows(const float *x, long sb, long sr, long sk, int B, int
 
 }  // namespace
 
+// Whether all three products of these shapes go to the slab kernels, which can
+// read lhs itself: few columns, a reduction of 512..2048 in whole chunks, at
+// least 128 rows, lhs contiguous along the reduction in 16-byte aligned rows.
+// (Mirrors the conditions in launch_logmm_fwd and launch_bwd.)
+bool logmm_reads_lhs_itself(const LogmmOperand &lhs, int M, int K, int Nn) {
+    return Nn >= 1 && Nn <= 3 * TQ && K >= 2 * kSlab && K <= 8 * kSlab && K % TQ == 0 &&
+           M >= 4 * TQ && lhs.s2 == 1 && (lhs.s1 & 3) == 0 && (lhs.sb & 3) == 0 &&
+           (reinterpret_cast<uintptr_t>(lhs.p) & 15u) == 0;
+}
+
 hipError_t launch_logmm_shift_exp(const LogmmOperand &lhs, const LogmmOperand &rhs,
                                   const LogmmShifted &sh, int B, int M, int K, int Nn,
                                   const int *row_len, const int *col_len, hipStream_t stream) {
@@ -1475,10 +1537,16 @@ hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
         if (!xcd_grid_fits(a.tiles_x, a.tiles_y, B)) return hipErrorInvalidValue;
         const dim3 grid(xcd_grid(a.tiles_x, a.tiles_y, B));
         const size_t lds = (size_t)3 * tn * kSlabLd * sizeof(__bf16);
-        if (wide)
-            TIMED_LAUNCH((logmm_fwd_slab_kernel<6>), grid, dim3(64 * kSlabWaves), lds, stream, a, slabs);
+        const bool raw = a.El == nullptr;
+        if (raw && (a.lsk != 1 || a.K != a.Kp)) return hipErrorInvalidValue;
+        if (wide && raw)
+            TIMED_LAUNCH((logmm_fwd_slab_kernel<6, true>), grid, dim3(64 * kSlabWaves), lds, stream, a, slabs);
+        else if (wide)
+            TIMED_LAUNCH((logmm_fwd_slab_kernel<6, false>), grid, dim3(64 * kSlabWaves), lds, stream, a, slabs);
+        else if (raw)
+            TIMED_LAUNCH((logmm_fwd_slab_kernel<4, true>), grid, dim3(64 * kSlabWaves), lds, stream, a, slabs);
         else
-            TIMED_LAUNCH((logmm_fwd_slab_kernel<4>), grid, dim3(64 * kSlabWaves), lds, stream, a, slabs);
+            TIMED_LAUNCH((logmm_fwd_slab_kernel<4, false>), grid, dim3(64 * kSlabWaves), lds, stream, a, slabs);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         const long outs = (long)M * Nn;
@@ -1486,6 +1554,7 @@ hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
                      0, stream, a, B);
         return hipGetLastError();
     }
+    if (!a.El) return hipErrorInvalidValue;     // only the slab form reads lhs itself
     // 4 wavefronts per workgroup: 32 rows i by 96 or 64 columns j
     a.tiles_x = (M + 31) / 32;
     a.tiles_y = (prefer_96(Nn) ? (Nn + 95) / 96 : (Nn + 63) / 64) * a.splits;
