@@ -536,7 +536,9 @@ __global__ __launch_bounds__(64 * kSlabWaves) void logmm_fwd_slab_kernel(const F
         const int i = min(rb * 16 + r, M - 1);
         const float *row = RAW ? a.lhs + (size_t)b * a.lsb + (size_t)i * a.lsm
                                : a.El + ((size_t)b * M + i) * Kp;
-        if (RAW) shift = finite_or_zero(a.lmax[(size_t)b * M + i]);
+        // (the loaded maximum is used as it is, and made finite only where it is
+        // applied: an operation on it here would wait for the load here)
+        if (RAW) shift = a.lmax[(size_t)b * M + i];
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             const int k = min(k0 + TQ * (half * CH + c) + 8 * g, Kp - 8);
@@ -549,8 +551,9 @@ __global__ __launch_bounds__(64 * kSlabWaves) void logmm_fwd_slab_kernel(const F
     // use them, one group of GB column blocks at a time (the scheduler is held to
     // that: left alone it hoists all reads of a half and spills); the other
     // wavefront of the SIMD covers the wait.
-    auto multiply = [&](int half, const v4f (&A)[2 * CH], float shift) {
+    auto multiply = [&](int half, const v4f (&A)[2 * CH], float row_max) {
         bf16x8 xp[3];
+        const float shift = finite_or_zero(row_max);
 #pragma unroll
         for (int item = 0; item < 2 * CH; ++item) {
             const int c = item >> 1, grp = item & 1;
@@ -1083,7 +1086,7 @@ __global__ __launch_bounds__(64 * kBwdWaves) void logmm_bwd_lhs_slab_kernel(cons
         }
         const float *erow = RAW ? a.own + (size_t)b * a.osb + (size_t)pl * a.osp
                                 : a.Eown + ((size_t)b * P + pl) * Kp;
-        const float own_shift = RAW ? finite_or_zero(a.own_max[(size_t)b * P + pl]) : 0.0f;
+        const float own_max = RAW ? a.own_max[(size_t)b * P + pl] : 0.0f;
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
             ev[kb] = *reinterpret_cast<const v4f *>(erow + min(k0 + kb * 16 + 4 * g, Kp - 4));
@@ -1095,6 +1098,7 @@ __global__ __launch_bounds__(64 * kBwdWaves) void logmm_bwd_lhs_slab_kernel(cons
                 const Split3 sp = split3(i < 4 ? cv[2 * ch][i] : cv[2 * ch + 1][i - 4]);
                 cp[ch][0][i] = sp.h, cp[ch][1][i] = sp.m, cp[ch][2][i] = sp.l;
             }
+        const float own_shift = finite_or_zero(own_max);
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) {
             v4f acc = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -1206,7 +1210,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int j = 0; j < 4; ++j) {
             const int q = chunk * TQ + 4 * tg + j;
             e[j] = *reinterpret_cast<const v4f *>(el_base + (size_t)min(q, q_last) * el_row);
-            if (RAW) shift[j] = finite_or_zero(shifts[min(q, q_last)]);
+            // (made finite in stash: an operation on it here would wait for the load here)
+            if (RAW) shift[j] = shifts[min(q, q_last)];
             cc[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
             if (has_c && q < Qb) cc[j] = *reinterpret_cast<const v4f *>(c_base + (size_t)q * a.cgq);
         }
@@ -1218,7 +1223,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             float x[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                x[j] = RAW ? exp2_hw((e[j][i] - shift[j]) * kLog2eF) : e[j][i];
+                x[j] = RAW ? exp2_hw((e[j][i] - finite_or_zero(shift[j])) * kLog2eF) : e[j][i];
             const Pair3 lo = split3_pair(x[0], x[1]), hi = split3_pair(x[2], x[3]);
             *reinterpret_cast<uint2 *>(&s_el[0][4 * k4 + i][4 * tg]) = make_uint2(lo.h, hi.h);
             *reinterpret_cast<uint2 *>(&s_el[1][4 * k4 + i][4 * tg]) = make_uint2(lo.m, hi.m);
