@@ -106,6 +106,7 @@ SimpleWorkspace carve_simple(void *base, int N, int T, int U) {
 struct PairWorkspace {
     float *factors;
     int *flags;
+    LogmmPairPlanes planes;   // null where they have no use
     size_t bytes;
 };
 
@@ -115,6 +116,13 @@ PairWorkspace carve_pairs(void *base, int B, int M, int Nn) {
     w.factors = reinterpret_cast<float *>(base);
     w.flags = reinterpret_cast<int *>(reinterpret_cast<uintptr_t>(base) + fb);
     w.bytes = fb + align256((size_t)B * M * sizeof(int));
+    const size_t pb = logmm_pair_planes_bytes(B, M, Nn), sb = logmm_pair_shifts_bytes(B, M, Nn);
+    w.planes = {nullptr, nullptr};
+    if (pb && sb) {
+        w.planes.planes = reinterpret_cast<unsigned short *>(reinterpret_cast<uintptr_t>(base) + w.bytes);
+        w.planes.shifts = reinterpret_cast<float *>(reinterpret_cast<uintptr_t>(base) + w.bytes + pb);
+        w.bytes += pb + sb;
+    }
     return w;
 }
 
@@ -784,7 +792,7 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
                                  const_cast<float *>(gexp)};
         if (T > 0) {
             int rc = done(launch_logmm_pair_factor(grad_den, den, fmax, gmax, grad_out, lx, ly,
-                                                   pw.factors, pw.flags, N, T, U1, st));
+                                                   pw.factors, pw.flags, pw.planes, N, T, U1, st));
             if (rc != WARPCTCT_OK) return rc;
         }
         if (dense_f) {
@@ -797,6 +805,7 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
             // gradient of rhs[b,k,j] = g[b,j,k] stored straight into the (N,U+1,V) layout
             const LogmmGrad gr = {dense_g, (long)U1 * V, 1L, (long)V};
             int rc = done(launch_logmm_bwd_rhs(lhs, rhs, sh, grad_den, den, pw.factors, pw.flags,
+                                               pw.planes,
                                                gr, N, T, V, U1, lx, ly, grad_out, st));
             if (rc != WARPCTCT_OK) return rc;
         }
@@ -866,7 +875,7 @@ int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, lo
         int rc = done(launch_logmm_shift_exp(l, r, w.sh, B, M, K, Nn, nullptr, nullptr, st));
         if (rc != WARPCTCT_OK) return rc;
         rc = done(launch_logmm_pair_factor(grad_out, res, w.sh.lmax, w.sh.rmax, nullptr, nullptr,
-                                           nullptr, w.pw.factors, w.pw.flags, B, M, Nn, st));
+                                           nullptr, w.pw.factors, w.pw.flags, w.pw.planes, B, M, Nn, st));
         if (rc != WARPCTCT_OK) return rc;
     }
     if (grad_lhs) {
@@ -877,7 +886,8 @@ int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, lo
     }
     if (grad_rhs) {
         const LogmmGrad g = {grad_rhs, grsb, grsk, grsn};
-        int rc = done(launch_logmm_bwd_rhs(l, r, w.sh, grad_out, res, w.pw.factors, w.pw.flags, g,
+        int rc = done(launch_logmm_bwd_rhs(l, r, w.sh, grad_out, res, w.pw.factors, w.pw.flags,
+                                           w.pw.planes, g,
                                            B, M, K, Nn, nullptr, nullptr, nullptr, st));
         if (rc != WARPCTCT_OK) return rc;
     }

@@ -219,13 +219,28 @@ hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
                             const LogmmShifted &sh, float *res, float *partial, int B, int M,
                             int K, int Nn, const int *row_len, const int *col_len,
                             hipStream_t stream);
+// The pair factors once more, laid out for the gradient of the operand with few
+// rows (see logmm_bwd_rhs_planes_kernel): transposed and split into three
+// bfloat16 planes (3, B, logmm_pair_row(Nn), logmm_pair_frames(M)), frames
+// contiguous, zeros beyond M; and per frame the shift of its row of lhs
+// (B, logmm_pair_frames(M)): the finite row maximum, +inf for padding.
+// Both null: not wanted.
+struct LogmmPairPlanes {
+    unsigned short *planes;
+    float *shifts;
+};
+inline int logmm_pair_frames(int M) { return (M + 31) / 32 * 32; }
+// bytes of the two buffers (each a multiple of 256), 0 where the planes have no use
+size_t logmm_pair_planes_bytes(int B, int M, int Nn);
+size_t logmm_pair_shifts_bytes(int B, int M, int Nn);
 // C (B,M,logmm_pair_row(Nn)) and flags (B,M): the pair factors go * exp(lmax + rmax - res) that
 // both gradients share, and per row whether a pair was left to the exact pass;
 // batch_scale (may be null) multiplies grad_out per batch.
 hipError_t launch_logmm_pair_factor(const float *go, const float *res, const float *lmax,
                                     const float *rmax, const float *batch_scale,
                                     const int *row_len, const int *col_len, float *C, int *flags,
-                                    int B, int M, int Nn, hipStream_t stream);
+                                    const LogmmPairPlanes &planes, int B, int M, int Nn,
+                                    hipStream_t stream);
 hipError_t launch_logmm_bwd_lhs(const LogmmOperand &lhs, const LogmmOperand &rhs,
                                 const LogmmShifted &sh, const float *go, const float *res,
                                 const float *C, const int *flags, const LogmmGrad &grad, int B,
@@ -233,8 +248,9 @@ hipError_t launch_logmm_bwd_lhs(const LogmmOperand &lhs, const LogmmOperand &rhs
                                 const float *batch_scale, hipStream_t stream);
 hipError_t launch_logmm_bwd_rhs(const LogmmOperand &lhs, const LogmmOperand &rhs,
                                 const LogmmShifted &sh, const float *go, const float *res,
-                                const float *C, const int *flags, const LogmmGrad &grad, int B,
-                                int M, int K, int Nn, const int *row_len, const int *col_len,
-                                const float *batch_scale, hipStream_t stream);
+                                const float *C, const int *flags, const LogmmPairPlanes &planes,
+                                const LogmmGrad &grad, int B, int M, int K, int Nn,
+                                const int *row_len, const int *col_len, const float *batch_scale,
+                                hipStream_t stream);
 
 }  // namespace wctct

@@ -417,6 +417,7 @@ __global__ __launch_bounds__(64 * WR * WC) void logmm_fwd_kernel(const FwdArgs a
 // v_mfma_f32_16x16x4_f32 do per 32 in fp32, in 96 instead of 256 cycles.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 struct Split3 {
     __bf16 h, m, l;
@@ -667,6 +668,66 @@ __global__ __launch_bounds__(256) void logmm_pair_factor_kernel(
     if (lane == 0) flags[(size_t)b * M + i] = unsafe;
 }
 
+// The same, 8 rows i per workgroup, which also writes the pair factors transposed
+// and split into three bfloat16 planes, planes[pl][b][j][i] with ct_frames =
+// logmm_pair_frames(M) entries per row (8 consecutive i of one j: one 16-byte
+// store per plane), zeros for i >= M, and shifts[b][i] = the finite maximum of
+// row i of lhs, +inf for rows that are padding (their exponentials are then 0).
+// Requires logmm_pair_row(Nn) <= 96.  grid (ct_frames / 8, B), 512 threads.
+__global__ __launch_bounds__(512) void logmm_pair_factor_planes_kernel(
+    const float *__restrict__ go, const float *__restrict__ res, const float *__restrict__ lmax,
+    const float *__restrict__ rmax, const float *__restrict__ batch_scale,
+    const int *__restrict__ row_len, const int *__restrict__ col_len, float *__restrict__ C,
+    int *__restrict__ flags, unsigned short *__restrict__ planes, float *__restrict__ shifts,
+    int B, int M, int Nn, int ct_frames) {
+    __shared__ float s_c[8][96];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int i = blockIdx.x * 8 + wave, b = blockIdx.y;
+    const int Mb = row_len ? min(max(row_len[b], 0), M) : M;
+    const int Nb = col_len ? min(max(col_len[b], 0) + 1, Nn) : Nn;
+    const float scale = batch_scale ? batch_scale[b] : 1.0f;
+    const int Cq = logmm_pair_row(Nn);
+    const bool in_rows = i < M;
+    const size_t row = ((size_t)b * M + min(i, M - 1)) * Nn;
+    float *crow = C + ((size_t)b * M + min(i, M - 1)) * Cq;
+    const float ml = in_rows ? lmax[(size_t)b * M + i] : neg_inf_f();
+    int unsafe = 0;
+    for (int j = lane; j < Cq; j += 64) {
+        float cv = 0.0f;
+        if (i < Mb && j < Nb) {
+            const float gv = go[row + j] * scale, rr = res[row + j];
+            if (gv != 0.0f && rr != neg_inf_f()) {
+                const float ex = (ml + rmax[(size_t)b * Nn + j] - rr) * kLog2eF;
+                if (ex <= kMaxShiftLog2)
+                    cv = gv * exp2_hw(ex);
+                else
+                    unsafe = 1;
+            }
+        }
+        if (in_rows) crow[j] = cv;
+        s_c[wave][j] = cv;
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) unsafe |= __shfl_xor(unsafe, off, 64);
+    if (lane == 0) {
+        if (in_rows) flags[(size_t)b * M + i] = unsafe;
+        shifts[(size_t)b * ct_frames + i] = (i < Mb) ? finite_or_zero(ml) : __builtin_huge_valf();
+    }
+    __syncthreads();
+    if (tid < Cq) {
+        float x[8];
+#pragma unroll
+        for (int w = 0; w < 8; ++w) x[w] = s_c[w][tid];
+        const Pair3 p0 = split3_pair(x[0], x[1]), p1 = split3_pair(x[2], x[3]);
+        const Pair3 p2 = split3_pair(x[4], x[5]), p3 = split3_pair(x[6], x[7]);
+        const size_t plane = (size_t)B * Cq * ct_frames;
+        unsigned short *at = planes + ((size_t)b * Cq + tid) * ct_frames + blockIdx.x * 8;
+        *reinterpret_cast<uint4 *>(at) = make_uint4(p0.h, p1.h, p2.h, p3.h);
+        *reinterpret_cast<uint4 *>(at + plane) = make_uint4(p0.m, p1.m, p2.m, p3.m);
+        *reinterpret_cast<uint4 *>(at + 2 * plane) = make_uint4(p0.l, p1.l, p2.l, p3.l);
+    }
+}
+
 // One kernel serves both operands.  "own" is the operand whose gradient is
 // produced, own[b, p, k] with p = i (lhs) or j (rhs); "oth" is the other one,
 // oth[b, q, k].  C / go / res are addressed as [b, p*gp + q*gq].
@@ -691,6 +752,11 @@ struct BwdArgs {
     int p_extra, q_extra;
     int flags_follow_p;        // rows i are p (lhs gradient) or q (rhs gradient)
     int B, tiles_x, tiles_y;   // batch entries, p tiles, k tiles (or groups of k tiles)
+    // logmm_bwd_rhs_planes_kernel only: C transposed and split (3, B, ct_rows, ct_frames)
+    // and the shifts of the rows of oth (B, ct_frames), see LogmmPairPlanes
+    const unsigned short *ct = nullptr;
+    const float *ct_shift = nullptr;
+    int ct_rows = 0, ct_frames = 0;
 };
 
 // E_own * sum; the sum is 0 where nothing was added: avoid 0 * inf or 0 * nan
@@ -1149,6 +1215,44 @@ __global__ __launch_bounds__(64 * kBwdWaves) void logmm_bwd_lhs_slab_kernel(cons
     }
 }
 
+// The end of the two kernels below: the sums of a wavefront (lane l holds
+// D[p = ub*16 + 4*(l/16) + q][k = kb*16 + l%16] in register q) times E_own, to
+// the gradient.  All of a lane's values of E_own are requested before the first
+// is used (one round trip to memory; asked for one by one, inside the
+// conditions, each load was waited for by itself: 48 round trips, 15 us).
+template <int UB>
+__device__ __forceinline__ void rhs_store_sums(const BwdArgs &a, int b, int k0, int wave, int c,
+                                               int g, const v4f (&acc)[2][UB], bool slow, int Pb,
+                                               int Qb) {
+    const int P = a.P, K = a.K, Kp = a.Kp;
+    float eo[2][UB][4];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+        const int k = min(k0 + (2 * wave + kk) * 16 + c, Kp - 1);
+#pragma unroll
+        for (int ub = 0; ub < UB; ++ub)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                eo[kk][ub][q] = a.Eown[((size_t)b * P + min(ub * 16 + 4 * g + q, P - 1)) * Kp + k];
+    }
+    float *db = a.grad + (size_t)b * a.dsb;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+        const int k = k0 + (2 * wave + kk) * 16 + c;
+        if (k >= K) continue;
+#pragma unroll
+        for (int ub = 0; ub < UB; ++ub)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int p = ub * 16 + 4 * g + q;
+                if (p >= P) continue;
+                float v = (p < Pb) ? scaled_sum(acc[kk][ub][q], eo[kk][ub][q]) : 0.0f;
+                if (slow && p < Pb) v += exact_pairs(a, b, p, k, Qb);
+                db[(size_t)p * a.dsp + (size_t)k * a.dsk] = v;
+            }
+    }
+}
+
 // The gradient of the operand with FEW rows and a LONG reduction (the g of a
 // joiner: P = labels + 1 <= 96, Q = frames, K = vocabulary):
 //   grad[b,p,k] = E_own[p,k] * sum_q C[q,p] * E_oth[q,k].
@@ -1176,7 +1280,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const TileId tile = xcd_tile(a.tiles_x, 1);
     const int b = tile.b, k0 = tile.x * kRhsSlab;
     if (b >= a.B) return;
-    const int P = a.P, Q = a.Q, K = a.K, Kp = a.Kp;
+    const int P = a.P, Q = a.Q, Kp = a.Kp;
     const int Pb = a.p_len ? min(max(a.p_len[b], 0) + a.p_extra, P) : P;
     const int Qb = a.q_len ? min(max(a.q_len[b], 0) + a.q_extra, Q) : Q;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -1275,27 +1379,159 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
     }
     __syncthreads();
-    const bool slow = s_unsafe != 0;
-    // lane l holds D[p = ub*16 + 4*(l/16) + q][k = kb*16 + l%16] in register q
-    float *db = a.grad + (size_t)b * a.dsb;
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-        const int k = k0 + (2 * wave + kk) * 16 + c;
-        if (k >= K) continue;
-#pragma unroll
-        for (int ub = 0; ub < UB; ++ub)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int p = ub * 16 + 4 * g + q;
-                if (p >= P) continue;
-                float v = 0.0f;
-                if (p < Pb) {
-                    v = scaled_sum(acc[kk][ub][q], a.Eown[((size_t)b * P + p) * Kp + k]);
-                    if (slow) v += exact_pairs(a, b, p, k, Qb);
-                }
-                db[(size_t)p * a.dsp + (size_t)k * a.dsk] = v;
-            }
+    rhs_store_sums<UB>(a, b, k0, wave, c, g, acc, s_unsafe != 0, Pb, Qb);
+}
+
+// The same product with nothing split or transposed for C on the way: the pair
+// factors arrive as bfloat16 planes with the frames contiguous (written once by
+// logmm_pair_factor_planes_kernel), and a lane takes its 8 frames of one column
+// k of the long operand straight from memory, one 4-byte load per frame (the 16
+// lanes of a column block read 64 contiguous bytes of a row), exponentiates
+// (RAW) and splits them in registers: they are its share of the matrix
+// instruction's second operand as they are.  Only the planes of C pass through
+// LDS (a plain copy, two buffers, one barrier per chunk of 32 frames); the long
+// operand never does, and no value is split more than once per workgroup.
+// Per chunk a lane issues ~150 vector instructions where the kernel above
+// issues ~350, for the same 72 matrix instructions.
+template <int UB, bool RAW>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void logmm_bwd_rhs_planes_kernel(const BwdArgs a) {
+    constexpr int NT = 256, DEPTH = 2;
+    constexpr int ROWS = 16 * UB;
+    constexpr int CV = 3 * ROWS * 4;               // 16-byte vectors of one chunk of the planes
+    constexpr int CPT = (CV + NT - 1) / NT;        // ... per thread (the last ones repeat)
+    __shared__ __attribute__((aligned(16))) __bf16 s_ct[2][3][ROWS][kRhsLd];
+    __shared__ int s_unsafe;
+    const TileId tile = xcd_tile(a.tiles_x, 1);
+    const int b = tile.b, k0 = tile.x * kRhsSlab;
+    if (b >= a.B) return;
+    const int P = a.P, Q = a.Q, Kp = a.Kp, Tp = a.ct_frames;
+    const int Pb = a.p_len ? min(max(a.p_len[b], 0) + a.p_extra, P) : P;
+    const int Qb = a.q_len ? min(max(a.q_len[b], 0) + a.q_extra, Q) : Q;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c = lane & 15, g = lane >> 4;
+    if (tid == 0) s_unsafe = 0;
+    __syncthreads();
+    {
+        const int *fl = a.flags + (size_t)b * Q;
+        int unsafe = 0;
+        for (int q = tid; q < Qb; q += NT) unsafe |= fl[q];
+        if (unsafe) s_unsafe = 1;
     }
+    const int n = (Qb + TQ - 1) / TQ, last_chunk = Tp / TQ - 1;
+    // the planes: vector e of a chunk is (plane, row u, 8 frames j)
+    const unsigned short *ct_src[CPT];
+    int ct_dst[CPT];
+#pragma unroll
+    for (int it = 0; it < CPT; ++it) {
+        const int e = min(tid + it * NT, CV - 1);
+        const int pl = e / (ROWS * 4), u = (e >> 2) % ROWS, j = e & 3;
+        ct_src[it] = a.ct + (((size_t)pl * a.B + b) * a.ct_rows + u) * Tp + 8 * j;
+        ct_dst[it] = (pl * ROWS + u) * kRhsLd + 8 * j;
+    }
+    auto ct_fetch = [&](int chunk, u32x4 (&v)[CPT]) {
+        const int t0 = min(chunk, last_chunk) * TQ;
+#pragma unroll
+        for (int it = 0; it < CPT; ++it) v[it] = *reinterpret_cast<const u32x4 *>(ct_src[it] + t0);
+    };
+    auto ct_put = [&](int buf, const u32x4 (&v)[CPT]) {
+        __bf16 *dst = &s_ct[buf][0][0][0];
+#pragma unroll
+        for (int it = 0; it < CPT; ++it) *reinterpret_cast<u32x4 *>(dst + ct_dst[it]) = v[it];
+    };
+    // the long operand: this lane's column of each of the wavefront's two blocks
+    // of 16 (a pair of blocks beyond the reduction repeats the last pair: its
+    // sums are dropped), frames 8g .. 8g+7 of the chunk; frames beyond the
+    // entry's length repeat its last one (C is 0 there, and RAW their shift +inf)
+    const int kc = min(k0 + 32 * wave, Kp - 32) + c;
+    const float *e_base = RAW ? a.oth + (size_t)b * a.tsb : a.Eoth + (size_t)b * Q * Kp;
+    const int e_row = RAW ? a.tsq : Kp;
+    const int q_last = RAW ? max(Qb - 1, 0) : Q - 1;
+    const float *shift_base = a.ct_shift + (size_t)b * Tp + 8 * g;
+    auto fetch = [&](int chunk, float (&x)[2][8], v4f (&sf)[2]) {
+        const int t0 = min(chunk, last_chunk) * TQ;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            // (offsets inside one batch entry fit 32 bits: the launcher checks)
+            const unsigned off = (unsigned)(min(t0 + 8 * g + i, q_last) * e_row + kc);
+            x[0][i] = e_base[off];
+            x[1][i] = e_base[off + 16];
+        }
+        if (RAW) {
+            sf[0] = *reinterpret_cast<const v4f *>(shift_base + t0);
+            sf[1] = *reinterpret_cast<const v4f *>(shift_base + t0 + 4);
+        }
+    };
+    v4f acc[2][UB];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int ub = 0; ub < UB; ++ub) acc[kk][ub] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    float e[DEPTH][2][8];
+    v4f sf[DEPTH][2];
+    u32x4 cr[CPT];
+    // (requested in the order of the loop: the compiler counts the loads in
+    // flight at the head of the loop along both ways into it)
+    static_assert(DEPTH == 2, "the order of the requests below is that of a loop two chunks deep");
+    ct_fetch(0, cr);
+    __builtin_amdgcn_sched_barrier(0);
+    ct_put(0, cr);
+    fetch(0, e[0], sf[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    ct_fetch(1, cr);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(1, e[1], sf[1]);
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    // one chunk: `cur` even works from buffer 0 and register set 0
+    auto half = [&](int cur, int buf, float (&ex)[2][8], v4f (&es)[2]) {
+        // the next chunk's planes into the buffer that the chunk before read
+        // (everyone has passed the barrier behind it), the one after it requested
+        ct_put(buf ^ 1, cr);
+        ct_fetch(cur + 2, cr);
+        // (held in this order: requested behind the loads of the long operand,
+        // the planes would be waited for with nothing else left in flight)
+        __builtin_amdgcn_sched_barrier(0);
+        bf16x8 bk[2][3];
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+            float x[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                x[i] = RAW ? exp2_hw((ex[kk][i] - es[i >> 2][i & 3]) * kLog2eF) : ex[kk][i];
+            const Pair3 p0 = split3_pair(x[0], x[1]), p1 = split3_pair(x[2], x[3]);
+            const Pair3 p2 = split3_pair(x[4], x[5]), p3 = split3_pair(x[6], x[7]);
+            const u32x4 h = {p0.h, p1.h, p2.h, p3.h};
+            const u32x4 m = {p0.m, p1.m, p2.m, p3.m};
+            const u32x4 l = {p0.l, p1.l, p2.l, p3.l};
+            bk[kk][0] = __builtin_bit_cast(bf16x8, h);
+            bk[kk][1] = __builtin_bit_cast(bf16x8, m);
+            bk[kk][2] = __builtin_bit_cast(bf16x8, l);
+        }
+        fetch(cur + DEPTH, ex, es);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ub = 0; ub < UB; ++ub) {
+            bf16x8 au[3];
+#pragma unroll
+            for (int pn = 0; pn < 3; ++pn)
+                au[pn] = *reinterpret_cast<const bf16x8 *>(&s_ct[buf][pn][ub * 16 + c][8 * g]);
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) acc[kk][ub] = mfma6(au, bk[kk], acc[kk][ub]);
+        }
+        __syncthreads();
+    };
+    // two chunks per trip and no way out of the loop between them: with one, the
+    // compiler would count the loads in flight along a path that skips the second
+    // chunk, and wait for loads that were only just issued
+    int chunk = 0;
+    for (; chunk + 1 < n; chunk += 2) {
+        half(chunk, 0, e[0], sf[0]);
+        half(chunk + 1, 1, e[1], sf[1]);
+    }
+    if (chunk < n) half(chunk, 0, e[0], sf[0]);
+    __syncthreads();
+    rhs_store_sums<UB>(a, b, k0, wave, c, g, acc, s_unsafe != 0, Pb, Qb);
 }
 
 // Tiles of 64 or 96 along an extent, whichever pads the tiled extent less.
@@ -1370,6 +1606,33 @@ hipError_t launch_bwd(const BwdArgs &args, int B, hipStream_t stream) {
         else
             LAUNCH_LHS_SLAB(3);
 #undef LAUNCH_LHS_SLAB
+        return hipGetLastError();
+    }
+    if (a.ct && a.ct_shift && a.cgp == 1 && a.P <= 96 && a.Kp >= 2 * kRhsSlab && a.Q >= 4 * TQ &&
+        a.Eown && (a.Eoth || (a.tsk == 1 && a.K == a.Kp)) &&
+        fits_int((long)(a.Q - 1) * (a.Eoth ? a.Kp : a.tsq) + a.Kp)) {
+        // the same shapes with C's planes at hand (the joiner's backward)
+        const int ub = (a.P + 15) / 16;
+        a.tiles_x = (a.Kp + kRhsSlab - 1) / kRhsSlab, a.tiles_y = 1;
+        if (!xcd_grid_fits(a.tiles_x, 1, B)) return hipErrorInvalidValue;
+        const dim3 grid(xcd_grid(a.tiles_x, 1, B));
+        const bool raw = a.Eoth == nullptr;
+#define RHS_PLANES(UBN)                                                                         \
+    do {                                                                                        \
+        if (raw)                                                                                \
+            TIMED_LAUNCH((logmm_bwd_rhs_planes_kernel<UBN, true>), grid, dim3(256), 0, stream, a); \
+        else                                                                                    \
+            TIMED_LAUNCH((logmm_bwd_rhs_planes_kernel<UBN, false>), grid, dim3(256), 0, stream, a); \
+    } while (0)
+        switch (ub) {
+            case 1: RHS_PLANES(1); break;
+            case 2: RHS_PLANES(2); break;
+            case 3: RHS_PLANES(3); break;
+            case 4: RHS_PLANES(4); break;
+            case 5: RHS_PLANES(5); break;
+            default: RHS_PLANES(6); break;
+        }
+#undef RHS_PLANES
         return hipGetLastError();
     }
     if (a.cgp == 1 && a.P <= 96 && a.Kp >= 2 * kRhsSlab && a.Q >= 4 * TQ) {
@@ -1577,11 +1840,32 @@ hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
     return hipGetLastError();
 }
 
+// The planes serve the gradient of the operand with few rows where it has at
+// most 96 of them and the other at least 128 (the shapes of launch_bwd's branch).
+static bool pair_planes_apply(int M, int Nn) { return Nn >= 1 && Nn <= 3 * TQ && M >= 4 * TQ; }
+size_t logmm_pair_planes_bytes(int B, int M, int Nn) {
+    if (!pair_planes_apply(M, Nn)) return 0;
+    const size_t bytes = (size_t)3 * B * logmm_pair_row(Nn) * logmm_pair_frames(M) * sizeof(unsigned short);
+    return (bytes + 255) / 256 * 256;
+}
+size_t logmm_pair_shifts_bytes(int B, int M, int Nn) {
+    if (!pair_planes_apply(M, Nn)) return 0;
+    return ((size_t)B * logmm_pair_frames(M) * sizeof(float) + 255) / 256 * 256;
+}
+
 hipError_t launch_logmm_pair_factor(const float *go, const float *res, const float *lmax,
                                     const float *rmax, const float *batch_scale,
                                     const int *row_len, const int *col_len, float *C, int *flags,
-                                    int B, int M, int Nn, hipStream_t stream) {
+                                    const LogmmPairPlanes &planes, int B, int M, int Nn,
+                                    hipStream_t stream) {
     if (B == 0 || M == 0) return hipSuccess;
+    if (planes.planes && planes.shifts && pair_planes_apply(M, Nn)) {
+        const int frames = logmm_pair_frames(M);
+        TIMED_LAUNCH(logmm_pair_factor_planes_kernel, dim3(frames / 8, B), dim3(512), 0, stream, go,
+                     res, lmax, rmax, batch_scale, row_len, col_len, C, flags, planes.planes,
+                     planes.shifts, B, M, Nn, frames);
+        return hipGetLastError();
+    }
     TIMED_LAUNCH(logmm_pair_factor_kernel, dim3((M + 3) / 4, B), dim3(256), 0, stream, go,
                        res, lmax, rmax, batch_scale, row_len, col_len, C, flags, M, Nn);
     return hipGetLastError();
@@ -1614,9 +1898,10 @@ hipError_t launch_logmm_bwd_lhs(const LogmmOperand &lhs, const LogmmOperand &rhs
 
 hipError_t launch_logmm_bwd_rhs(const LogmmOperand &lhs, const LogmmOperand &rhs,
                                 const LogmmShifted &sh, const float *go, const float *res,
-                                const float *C, const int *flags, const LogmmGrad &grad, int B,
-                                int M, int K, int Nn, const int *row_len, const int *col_len,
-                                const float *batch_scale, hipStream_t stream) {
+                                const float *C, const int *flags, const LogmmPairPlanes &planes,
+                                const LogmmGrad &grad, int B, int M, int K, int Nn,
+                                const int *row_len, const int *col_len, const float *batch_scale,
+                                hipStream_t stream) {
     if (B == 0 || Nn == 0 || K == 0) return hipSuccess;
     if (!stride_ok(lhs.s1) || !stride_ok(lhs.s2) || !stride_ok(rhs.s1) || !stride_ok(rhs.s2) ||
         !stride_ok(grad.s1) || !stride_ok(grad.s2))
@@ -1635,6 +1920,10 @@ hipError_t launch_logmm_bwd_rhs(const LogmmOperand &lhs, const LogmmOperand &rhs
     a.P = Nn, a.Q = M, a.K = K, a.Kp = logmm_padded_reduction(K);
     a.p_len = col_len, a.p_extra = 1, a.q_len = row_len, a.q_extra = 0;
     a.batch_scale = batch_scale;
+    if (planes.planes && planes.shifts && pair_planes_apply(M, Nn)) {
+        a.ct = planes.planes, a.ct_shift = planes.shifts;
+        a.ct_rows = logmm_pair_row(Nn), a.ct_frames = logmm_pair_frames(M);
+    }
     return launch_bwd(a, B, stream);
 }
 
