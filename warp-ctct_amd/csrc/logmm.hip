@@ -65,8 +65,7 @@ __global__ __launch_bounds__(256) void shift_exp_kernel(const float *__restrict_
     float *e = E + ((size_t)b * R + r) * Kp;
     const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
     if (r >= Rb) {
-        if (E)
-            for (int k = lane * 4; k < Kp; k += 256) *reinterpret_cast<v4f *>(e + k) = zero;
+        for (int k = lane * 4; k < Kp; k += 256) *reinterpret_cast<v4f *>(e + k) = zero;
         if (lane == 0) mx[(size_t)b * R + r] = neg_inf_f();
         return;
     }
@@ -85,7 +84,6 @@ __global__ __launch_bounds__(256) void shift_exp_kernel(const float *__restrict_
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
     if (lane == 0) mx[(size_t)b * R + r] = m;
-    if (!E) return;                                   // the maxima only
     const float shift = finite_or_zero(m);
     if (vec) {
         for (int k = lane * 4; k < Kp; k += 256) {
@@ -122,8 +120,7 @@ __global__ __launch_bounds__(256) void shift_exp_rows_kernel(const float *__rest
     float *e = E + ((size_t)b * R + r) * Kp;
     const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
     if (r >= Rb) {
-        if (E)
-            for (int k = lane * 4; k < Kp; k += 256) *reinterpret_cast<v4f *>(e + k) = zero;
+        for (int k = lane * 4; k < Kp; k += 256) *reinterpret_cast<v4f *>(e + k) = zero;
         if (lane == 0) mx[(size_t)b * R + r] = neg_inf_f();
         return;
     }
@@ -141,7 +138,6 @@ __global__ __launch_bounds__(256) void shift_exp_rows_kernel(const float *__rest
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
     if (lane == 0) mx[(size_t)b * R + r] = m;
-    if (!E) return;                                   // the maxima only
     const float shift = finite_or_zero(m);
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
@@ -275,6 +271,10 @@ struct FwdArgs {
     float *partial;
     int splits, chunks_per_split;
     int pM, pN;               // rows and row length of one partial sum (>= M, Nn)
+    // the slab kernel reading lhs itself: every slab shifts a row by the row's
+    // maximum inside the slab, slab_max (splits,B,pM), and the finish kernel
+    // brings the partial sums to the row's maximum, which it writes to lmax_out
+    float *slab_max = nullptr, *lmax_out = nullptr;
     int M, K, Kp, Nn;
     int B, tiles_x, tiles_y;  // batch entries, row tiles, column tiles * splits
     const int *row_len, *col_len;
@@ -532,14 +532,11 @@ __global__ __launch_bounds__(64 * kSlabWaves) void logmm_fwd_slab_kernel(const F
     // block is walked without a branch (the waits are then counted exactly).
     // Vectors past the reduction are clamped into it (they meet zeros of the
     // slab), row blocks past the last repeat it (and are dropped).
-    auto request = [&](int st, int half, v4f (&A)[2 * CH], float &shift) {
+    auto request = [&](int st, int half, v4f (&A)[2 * CH]) {
         const int rb = wave + NW * min(st, steps - 1);
         const int i = min(rb * 16 + r, M - 1);
         const float *row = RAW ? a.lhs + (size_t)b * a.lsb + (size_t)i * a.lsm
                                : a.El + ((size_t)b * M + i) * Kp;
-        // (the loaded maximum is used as it is, and made finite only where it is
-        // applied: an operation on it here would wait for the load here)
-        if (RAW) shift = a.lmax[(size_t)b * M + i];
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             const int k = min(k0 + TQ * (half * CH + c) + 8 * g, Kp - 8);
@@ -552,9 +549,8 @@ __global__ __launch_bounds__(64 * kSlabWaves) void logmm_fwd_slab_kernel(const F
     // use them, one group of GB column blocks at a time (the scheduler is held to
     // that: left alone it hoists all reads of a half and spills); the other
     // wavefront of the SIMD covers the wait.
-    auto multiply = [&](int half, const v4f (&A)[2 * CH], float row_max) {
+    auto multiply = [&](int half, const v4f (&A)[2 * CH], float shift) {
         bf16x8 xp[3];
-        const float shift = finite_or_zero(row_max);
 #pragma unroll
         for (int item = 0; item < 2 * CH; ++item) {
             const int c = item >> 1, grp = item & 1;
@@ -583,19 +579,36 @@ __global__ __launch_bounds__(64 * kSlabWaves) void logmm_fwd_slab_kernel(const F
         }
     };
     v4f A0[2 * CH], A1[2 * CH];
-    float shift0 = 0.0f, shift1 = 0.0f;
-    request(0, 0, A0, shift0);
+    request(0, 0, A0);
     // (the two halves in this order, as in the loop: the waits for a half are
     // counted from the loads issued after it)
     __builtin_amdgcn_sched_barrier(0);
-    request(0, 1, A1, shift1);
+    request(0, 1, A1);
     __builtin_amdgcn_sched_barrier(0);
+    float *slab_max = RAW ? a.slab_max + ((size_t)slab * a.B + b) * a.pM : nullptr;
     for (int st = 0; st < steps; ++st) {
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) acc[cb] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-        multiply(0, A0, shift0);
-        request(st + 1, 0, A0, shift0);
-        multiply(1, A1, shift1);
+        float shift = 0.0f;
+        if (RAW) {
+            // the row's maximum inside the slab: this lane's 64 values, then the
+            // 4 lanes of the row (vectors clamped into the reduction repeat
+            // values of the same row: the maximum may only come out larger than
+            // the slab's own, and any shift >= it serves)
+            float m = neg_inf_f();
+#pragma unroll
+            for (int v = 0; v < 2 * CH; ++v) {
+                m = fmaxf(fmaxf(m, fmaxf(A0[v][0], A0[v][1])), fmaxf(A0[v][2], A0[v][3]));
+                m = fmaxf(fmaxf(m, fmaxf(A1[v][0], A1[v][1])), fmaxf(A1[v][2], A1[v][3]));
+            }
+            m = fmaxf(m, __shfl_xor(m, 16, 64));
+            m = fmaxf(m, __shfl_xor(m, 32, 64));
+            if (g == 0) slab_max[(wave + NW * st) * 16 + r] = m;
+            shift = finite_or_zero(m);
+        }
+        multiply(0, A0, shift);
+        request(st + 1, 0, A0);
+        multiply(1, A1, shift);
         // lane l holds D[4*(l/16) + q][l%16] of each block in register q; the
         // stores come before the second request, so that at the head of the
         // loop nothing but the two halves is outstanding
@@ -606,7 +619,7 @@ __global__ __launch_bounds__(64 * kSlabWaves) void logmm_fwd_slab_kernel(const F
 #pragma unroll
             for (int q = 0; q < 4; ++q) at[(size_t)q * a.pN + cb * 16] = acc[cb][q];
         __builtin_amdgcn_sched_barrier(0);
-        request(st + 1, 1, A1, shift1);
+        request(st + 1, 1, A1);
     }
 }
 
@@ -618,10 +631,42 @@ __global__ __launch_bounds__(256) void logmm_fwd_finish_kernel(const FwdArgs a, 
     const int i = e / a.Nn, j = e - i * a.Nn;
     const int Mb = a.row_len ? min(max(a.row_len[b], 0), a.M) : a.M;
     const int Nb = a.col_len ? min(max(a.col_len[b], 0) + 1, a.Nn) : a.Nn;
-    if (i >= Mb || j >= Nb) return;
+    if (i >= Mb) {   // padding: its maximum is -inf, as shift_exp_kernel writes it
+        if (j == 0 && a.lmax_out) a.lmax_out[(size_t)b * a.M + i] = neg_inf_f();
+        return;
+    }
     const size_t per = (size_t)a.pM * a.pN;
     const float *p = a.partial + (size_t)b * per + (size_t)i * a.pN + j;
     float s = 0.0f;
+    if (a.slab_max) {
+        // every slab's sum was taken against the slab's own maximum of the row
+        // (at most 8 slabs; all loads first, one round trip to memory)
+        const float *sm = a.slab_max + (size_t)b * a.pM + i;
+        float pv[8], mv[8];
+#pragma unroll
+        for (int sp = 0; sp < 8; ++sp) {
+            const int spc = min(sp, a.splits - 1);
+            pv[sp] = p[(size_t)spc * B * per];
+            mv[sp] = sp < a.splits ? sm[(size_t)spc * B * a.pM] : neg_inf_f();
+        }
+        float m = neg_inf_f();
+#pragma unroll
+        for (int sp = 0; sp < 8; ++sp) m = fmaxf(m, mv[sp]);
+        if (j == 0) a.lmax_out[(size_t)b * a.M + i] = m;
+        if (j >= Nb) return;
+#pragma unroll
+        for (int sp = 0; sp < 8; ++sp)
+            if (mv[sp] != neg_inf_f()) s += pv[sp] * exp2_hw((mv[sp] - m) * kLog2eF);
+        if (s >= kTiny && s < __builtin_huge_valf()) {
+            a.res[(size_t)b * a.M * a.Nn + e] = m + a.rmax[(size_t)b * a.Nn + j] + log2_hw(s) * kLn2F;
+            return;
+        }
+        a.res[(size_t)b * a.M * a.Nn + e] =
+            exact_lse(a.lhs + (size_t)b * a.lsb + (size_t)i * a.lsm, a.lsk,
+                      a.rhs + (size_t)b * a.rsb + (size_t)j * a.rsn, a.rsk, a.K);
+        return;
+    }
+    if (j >= Nb) return;
     for (int sp = 0; sp < a.splits; ++sp) s += p[(size_t)sp * B * per];
     a.res[(size_t)b * a.M * a.Nn + e] = fwd_result(a, b, i, j, s);
 }
@@ -1745,7 +1790,9 @@ hipError_t launch_logmm_shift_exp(const LogmmOperand &lhs, const LogmmOperand &r
                                   const int *row_len, const int *col_len, hipStream_t stream) {
     const int Kp = logmm_padded_reduction(K);
     if (B == 0 || Kp == 0) return hipSuccess;
-    if (M > 0) {
+    // (an operand that the kernels read themselves has its maxima taken by the
+    // forward: launch_logmm_fwd must follow)
+    if (M > 0 && sh.El) {
         launch_shift_exp_rows(lhs.p, lhs.sb, lhs.s1, lhs.s2, B, M, K, Kp, row_len, 0, sh.lmax,
                               sh.El, stream);
         hipError_t e = hipGetLastError();
@@ -1761,8 +1808,10 @@ hipError_t launch_logmm_shift_exp(const LogmmOperand &lhs, const LogmmOperand &r
 
 size_t logmm_fwd_partial_floats(int B, int M, int Nn) {
     // up to 8 partial sums of whole row blocks (16) and column tiles (96 or 64)
+    // and of 8 slab maxima per row
     const int tn = prefer_96(Nn) ? 96 : 64;
-    return (size_t)8 * B * ((M + 15) / 16 * 16) * ((Nn + tn - 1) / tn * tn);
+    const size_t pM = (size_t)(M + 15) / 16 * 16;
+    return (size_t)8 * B * pM * ((Nn + tn - 1) / tn * tn) + (size_t)8 * B * pM;
 }
 
 int logmm_fwd_splits(int B, int M, int K, int Nn) {
@@ -1807,6 +1856,10 @@ hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
         const size_t lds = (size_t)3 * tn * kSlabLd * sizeof(__bf16);
         const bool raw = a.El == nullptr;
         if (raw && (a.lsk != 1 || a.K != a.Kp)) return hipErrorInvalidValue;
+        if (raw) {   // behind the partial sums
+            a.slab_max = partial + (size_t)slabs * B * a.pM * a.pN;
+            a.lmax_out = sh.lmax;
+        }
         if (wide && raw)
             TIMED_LAUNCH((logmm_fwd_slab_kernel<6, true>), grid, dim3(64 * kSlabWaves), lds, stream, a, slabs);
         else if (wide)
