@@ -416,6 +416,30 @@ def test_simple_loss_repeated_labels_weighted_and_backward_twice(case, normalize
     np.testing.assert_allclose(first[1].cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
 
 
+def test_simple_normalized_labels_crowded_into_few_columns():
+    """All 40 labels of one sample (with repeats) lie in columns 1..99 of a
+    512-column vocabulary, those of the other are spread out: the gradient through
+    the gathers lands on a few columns of the dense gradient wrt f, on top of the
+    gradient through the normaliser, in a shape that takes the matrix-core kernels
+    (T a multiple of 16 >= 128, V a multiple of 128 >= 512)."""
+    import warp_ctct
+    N, T, U, V = 2, 144, 40, 512
+    f, g, ys, lx, ly = make_simple_case(23, N, T, U, V, lx=[144, 130], ly=[40, 33], normalized=True)
+    rng = np.random.default_rng(23)
+    ys[0] = rng.integers(1, 100, U)
+    ys[0, 1::2] = ys[0, 0::2]
+    w = np.array([1.5, -0.5])
+    _, gf, gg, costs = O.ctct_simple_loss(f, g, ys, lx, ly, reduction="none", normalized=True,
+                                          grad_output=w)
+    tf, tg = dev(f).requires_grad_(True), dev(g).requires_grad_(True)
+    out = warp_ctct.ctct_simple_loss(tf, tg, dev(ys), dev(lx), dev(ly), reduction="none",
+                                     normalized=True)
+    np.testing.assert_allclose(out.detach().cpu().numpy(), costs, rtol=LOSS_RTOL)
+    (out * dev(w, torch.float32)).sum().backward()
+    np.testing.assert_allclose(tf.grad.cpu().numpy(), gf, atol=GRAD_ATOL, rtol=1e-5)
+    np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
+
+
 @pytest.mark.parametrize("normalized", [True, False])
 def test_simple_loss_edge_shapes(normalized):
     """No label dimension at all (g holds the one start context), samples

@@ -737,14 +737,25 @@ __global__ __launch_bounds__(512) void logmm_pair_factor_planes_kernel(
     float *crow = C + ((size_t)b * M + min(i, M - 1)) * Cq;
     const float ml = in_rows ? lmax[(size_t)b * M + i] : neg_inf_f();
     int unsafe = 0;
-    for (int j = lane; j < Cq; j += 64) {
+    // (a row has at most 96 entries: both of a lane's are requested before the
+    // first is used)
+    float gv[2], rr[2], rm[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const int j = min(lane + 64 * t, Nn - 1);
+        gv[t] = go[row + j], rr[t] = res[row + j], rm[t] = rmax[(size_t)b * Nn + j];
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const int j = lane + 64 * t;
+        if (j >= Cq) break;
         float cv = 0.0f;
         if (i < Mb && j < Nb) {
-            const float gv = go[row + j] * scale, rr = res[row + j];
-            if (gv != 0.0f && rr != neg_inf_f()) {
-                const float ex = (ml + rmax[(size_t)b * Nn + j] - rr) * kLog2eF;
+            const float gs = gv[t] * scale;
+            if (gs != 0.0f && rr[t] != neg_inf_f()) {
+                const float ex = (ml + rm[t] - rr[t]) * kLog2eF;
                 if (ex <= kMaxShiftLog2)
-                    cv = gv * exp2_hw(ex);
+                    cv = gs * exp2_hw(ex);
                 else
                     unsafe = 1;
             }
