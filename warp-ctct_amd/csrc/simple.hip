@@ -227,23 +227,30 @@ __global__ __launch_bounds__(kBlock) void simple_sum_partials_kernel(
 // dense_f[n,t,idx(u)] += w[n] * grad_f[n,t,u],  idx = [0, y0 .. y_{U-1}]: the
 // backward of f.gather (warp_ctct/__init__.py:205-208).  The same label may
 // occur at several u, so the adds are atomic.  Padding holds zeros: skipped.
-__global__ __launch_bounds__(kBlock) void simple_scatter_f_kernel(
-    const float *__restrict__ grad_f, const int *__restrict__ ys, const int *__restrict__ lx,
-    const int *__restrict__ ly, const float *__restrict__ grad_out, float *__restrict__ dense_f,
-    int T, int U, int V) {
+__device__ __forceinline__ void scatter_f_cell(
+    int cell, const float *__restrict__ grad_f, const int *__restrict__ ys,
+    const int *__restrict__ lx, const int *__restrict__ ly, const float *__restrict__ grad_out,
+    float *__restrict__ dense_f, int T, int U, int V) {
     const int U1 = U + 1;
     const int n = blockIdx.y;
-    const int cell = blockIdx.x * kBlock + threadIdx.x;
     if (cell >= T * U1) return;
     const int t = cell / U1, u = cell - t * U1;
     const int Tn = clampi(lx[n], 0, T), Un = clampi(ly[n], 0, U);
     if (t >= Tn || u > Un) return;
-    // cells that no complete alignment passes through hold exact zeros: no add
+    // (all three loads requested before the first is looked at)
     const float gv = grad_f[((size_t)n * T + t) * U1 + u];
-    if (gv == 0.0f) return;
     const float w = grad_out ? grad_out[n] : 1.0f;
-    const int col = (u == 0) ? 0 : clampi(ys[(size_t)n * U + u - 1], 0, V - 1);
-    atomicAdd(dense_f + ((size_t)n * T + t) * V + col, w * gv);
+    const int col = U > 0 ? clampi(ys[(size_t)n * U + max(u - 1, 0)], 0, V - 1) : 0;   // (no labels: ys may be null)
+    // cells that no complete alignment passes through hold exact zeros: no add
+    if (gv == 0.0f) return;
+    atomicAdd(dense_f + ((size_t)n * T + t) * V + (u == 0 ? 0 : col), w * gv);
+}
+
+__global__ __launch_bounds__(kBlock) void simple_scatter_f_kernel(
+    const float *__restrict__ grad_f, const int *__restrict__ ys, const int *__restrict__ lx,
+    const int *__restrict__ ly, const float *__restrict__ grad_out, float *__restrict__ dense_f,
+    int T, int U, int V) {
+    scatter_f_cell(blockIdx.x * kBlock + threadIdx.x, grad_f, ys, lx, ly, grad_out, dense_f, T, U, V);
 }
 
 // dense_f[n,t,:] as a whole row: zeros plus w[n] * grad_f[n,t,u] at idx(u), the
@@ -288,12 +295,12 @@ __global__ __launch_bounds__(kBlock) void simple_dense_f_rows_kernel(
 
 // dense_g[n,u,{0,y[u-1],y[u]}] += w[n] * grad_g[n,u,k]: backward of g.gather
 // (warp_ctct/__init__.py:211-215).  One thread per (n,u,k).
-__global__ __launch_bounds__(kBlock) void simple_scatter_g_kernel(
-    const float *__restrict__ grad_g, const int *__restrict__ ys, const int *__restrict__ ly,
-    const float *__restrict__ grad_out, float *__restrict__ dense_g, int U, int V) {
+__device__ __forceinline__ void scatter_g_entry(
+    int e, const float *__restrict__ grad_g, const int *__restrict__ ys,
+    const int *__restrict__ ly, const float *__restrict__ grad_out, float *__restrict__ dense_g,
+    int U, int V) {
     const int U1 = U + 1;
     const int n = blockIdx.y;
-    const int e = blockIdx.x * kBlock + threadIdx.x;
     if (e >= U1 * 3) return;
     const int u = e / 3, k = e - u * 3;
     const int Un = clampi(ly[n], 0, U);
@@ -303,6 +310,27 @@ __global__ __launch_bounds__(kBlock) void simple_scatter_g_kernel(
     if (k == 1) col = clampi(ys[(size_t)n * U + u - 1], 0, V - 1);
     if (k == 2) col = clampi(ys[(size_t)n * U + u], 0, V - 1);
     atomicAdd(dense_g + ((size_t)n * U1 + u) * V + col, w * grad_g[((size_t)n * U1 + u) * 3 + k]);
+}
+
+__global__ __launch_bounds__(kBlock) void simple_scatter_g_kernel(
+    const float *__restrict__ grad_g, const int *__restrict__ ys, const int *__restrict__ ly,
+    const float *__restrict__ grad_out, float *__restrict__ dense_g, int U, int V) {
+    scatter_g_entry(blockIdx.x * kBlock + threadIdx.x, grad_g, ys, ly, grad_out, dense_g, U, V);
+}
+
+// Both scatters in one launch: the first f_blocks workgroups of a sample take
+// the cells of f, the rest the entries of g.
+__global__ __launch_bounds__(kBlock) void simple_scatter_fg_kernel(
+    const float *__restrict__ grad_f, const float *__restrict__ grad_g,
+    const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
+    const float *__restrict__ grad_out, float *__restrict__ dense_f, float *__restrict__ dense_g,
+    int T, int U, int V, int f_blocks) {
+    if ((int)blockIdx.x < f_blocks)
+        scatter_f_cell(blockIdx.x * kBlock + threadIdx.x, grad_f, ys, lx, ly, grad_out, dense_f, T,
+                       U, V);
+    else
+        scatter_g_entry((blockIdx.x - f_blocks) * kBlock + threadIdx.x, grad_g, ys, ly, grad_out,
+                        dense_g, U, V);
 }
 
 inline dim3 cell_grid(int N, int T, int U) {
@@ -376,6 +404,13 @@ hipError_t launch_simple_scatter(const float *grad_f, const float *grad_g, const
                                  const int *lx, const int *ly, const float *grad_out,
                                  float *dense_f, float *dense_g, int N, int T, int U, int V,
                                  hipStream_t stream) {
+    if (dense_f && dense_g) {
+        const dim3 fg = cell_grid(N, T, U);
+        const unsigned g_blocks = ((U + 1) * 3 + kBlock - 1) / kBlock;
+        TIMED_LAUNCH(simple_scatter_fg_kernel, dim3(fg.x + g_blocks, N), dim3(kBlock), 0, stream,
+                     grad_f, grad_g, ys, lx, ly, grad_out, dense_f, dense_g, T, U, V, (int)fg.x);
+        return hipGetLastError();
+    }
     if (dense_f) {
         TIMED_LAUNCH(simple_scatter_f_kernel, cell_grid(N, T, U), dim3(kBlock), 0, stream,
                            grad_f, ys, lx, ly, grad_out, dense_f, T, U, V);
