@@ -331,9 +331,11 @@ size_t warpctct_simple_workspace_bytes(int N, int T, int U);
 /* 0 where the log-matmul kernels of the normalised path read f itself and form
  * exp(f - fmax) on the way (U+1 <= 96 contexts, 512 <= V <= 2048 in whole
  * multiples of 32, T >= 128, f aligned to 16 bytes): fexp is then neither
- * written by the forward nor read by the backward and may be NULL in both.
- * 1 otherwise.  No counterpart in the reference (which recomputes every
- * exponential in every kernel, csrc/logmatmul.cu:44-146). */
+ * written by the forward nor read by the backward and may be NULL in both,
+ * and fmax is written by the forward's last log-matmul kernel instead of a
+ * pass of its own over f.  1 otherwise.  No counterpart in the reference
+ * (which recomputes every exponential in every kernel,
+ * csrc/logmatmul.cu:44-146). */
 int warpctct_simple_needs_fexp(const float *f, int T, int U, int V);
 
 int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, const int *lx,
@@ -349,8 +351,10 @@ int warpctct_simple_forward_units_f32(const float *f_g, const float *g_g, const 
                                       int U, void *workspace, size_t workspace_bytes, float *costs,
                                       float *grad_f, float *grad_g, float *grad_den, void *stream);
 
-/* Bytes of workspace for warpctct_simple_backward_f32 (the factors
- * w*grad_den*exp(fmax+gmax-den) shared by both gradients of the den-path). */
+/* Bytes of workspace for warpctct_simple_backward_f32: the factors
+ * w*grad_den*exp(fmax+gmax-den) shared by both gradients of the den-path, and,
+ * for U+1 <= 96 and T >= 128, the same factors once more as transposed
+ * bfloat16 planes for the gradient wrt g. */
 size_t warpctct_simple_backward_workspace_bytes(int N, int T, int U);
 
 /* Dense gradients of ctct_simple_loss: dense_f (N,T,V), dense_g (N,U+1,V),

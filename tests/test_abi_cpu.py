@@ -130,3 +130,19 @@ def test_generic_dtype_and_logits_entry_points_check_their_arguments():
     w2 = lib.warpctct_logmm_workspace_bytes(2, 10, 65, 5)
     assert w2 - w1 == 4 * 32 * 2 * (10 + 5)
     assert lib.warpctct_simple_backward_workspace_bytes(N, T, U) >= 4 * N * T * (U + 1) + 4 * N * T
+    # the pair factors once more as three bfloat16 planes over frames padded to 32,
+    # and a float per padded frame, where the gradient wrt g uses them (U+1 <= 96, T >= 128)
+    small = lib.warpctct_simple_backward_workspace_bytes(2, 120, 80)
+    assert small < 2 * 120 * 96 * 4 + 2 * 120 * 4 + 1024
+    big = lib.warpctct_simple_backward_workspace_bytes(2, 400, 80)
+    assert big >= 2 * 400 * 96 * 4 + 2 * 400 * 4 + 3 * 2 * 96 * 416 * 2 + 2 * 416 * 4
+    # whether the joiner path stores exp(f - fmax): not for its production shapes
+    lib.warpctct_simple_needs_fexp.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+    aligned, odd = ctypes.c_void_p(4096), ctypes.c_void_p(4100)
+    assert lib.warpctct_simple_needs_fexp(aligned, 400, 80, 2048) == 0
+    assert lib.warpctct_simple_needs_fexp(aligned, 128, 0, 512) == 0
+    assert lib.warpctct_simple_needs_fexp(odd, 400, 80, 2048) == 1       # rows not 16-byte aligned
+    assert lib.warpctct_simple_needs_fexp(aligned, 400, 80, 2040) == 1   # not whole chunks of 32
+    assert lib.warpctct_simple_needs_fexp(aligned, 400, 80, 4096) == 1   # beyond the slab kernels
+    assert lib.warpctct_simple_needs_fexp(aligned, 100, 80, 2048) == 1   # too few frames
+    assert lib.warpctct_simple_needs_fexp(aligned, 400, 100, 2048) == 1  # too many contexts

@@ -267,6 +267,11 @@ SIMPLE_CASES = [
     # contexts (no resident slab), and a frame count that tiles better by 96
     ("wide_contexts", 5, 2, 130, 110, 40, [130, 125], [110, 100]),
     ("ninety_frames", 6, 3, 90, 20, 70, [90, 81, 66], [20, 17, 9]),
+    # shapes whose log-matmul kernels read f itself (at least 128 frames, at most 96
+    # contexts, a vocabulary of 512..2048 in whole chunks of 32): one block of 16
+    # contexts and four, a vocabulary that ends inside a slab, ragged lengths
+    ("reads_f_itself_few_contexts", 7, 2, 160, 5, 512, [160, 131], [5, 3]),
+    ("reads_f_itself_partial_slab", 8, 2, 130, 60, 800, [130, 128], [60, 33]),
 ]
 
 

@@ -1271,7 +1271,7 @@ __global__ __launch_bounds__(64 * kBwdWaves) void logmm_bwd_lhs_slab_kernel(cons
     }
 }
 
-// The end of the two kernels below: the sums of a wavefront (lane l holds
+// The end of the kernel below: the sums of a wavefront (lane l holds
 // D[p = ub*16 + 4*(l/16) + q][k = kb*16 + l%16] in register q) times E_own, to
 // the gradient.  All of a lane's values of E_own are requested before the first
 // is used (one round trip to memory; asked for one by one, inside the
@@ -1316,129 +1316,11 @@ __device__ __forceinline__ void rhs_store_sums(const BwdArgs &a, int b, int k0, 
 // workgroup of 4 wavefronts takes one batch entry and kRhsSlab columns k and
 // keeps its (16*UB x kRhsSlab) sums in registers (a wavefront: 32 columns).  The
 // reduction runs in chunks of 32 rows q.  Both operands have q as their ROW
-// index in memory, the matrix instruction wants 8 consecutive q per lane: a
-// thread loads 4 rows x 4 columns (16-byte vectors), splits the 16 values into
-// bfloat16 planes and writes them to LDS transposed, 4 consecutive q at a time
-// (8-byte stores; lanes run along q first, which keeps the stores free of bank
-// conflicts).  The next chunk is loaded while the present one is multiplied.
+// index in memory, the matrix instruction wants 8 consecutive q per lane.
 constexpr int kRhsSlab = 128;
-constexpr int kRhsLd = TQ + 8;       // bfloat16 per LDS row (80 bytes)
-constexpr int kRhsDepth = 3;          // chunks on their way while one is multiplied
+constexpr int kRhsLd = TQ + 8;       // bfloat16 per LDS row (80 bytes: rows 4 banks apart)
 
-// RAW: E_oth is not in memory; the kernel reads the long operand itself (k
-// contiguous, K a multiple of 32) and forms exp(oth - oth_max) before the split.
-template <int UB, bool RAW>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void logmm_bwd_rhs_slab_kernel(const BwdArgs a) {
-    constexpr int NT = 256, DEPTH = kRhsDepth;
-    __shared__ __attribute__((aligned(16))) __bf16 s_el[3][kRhsSlab][kRhsLd];   // E_oth^T planes
-    __shared__ __attribute__((aligned(16))) __bf16 s_ct[3][16 * UB][kRhsLd];    // C^T planes
-    __shared__ int s_unsafe;
-    const TileId tile = xcd_tile(a.tiles_x, 1);
-    const int b = tile.b, k0 = tile.x * kRhsSlab;
-    if (b >= a.B) return;
-    const int P = a.P, Q = a.Q, Kp = a.Kp;
-    const int Pb = a.p_len ? min(max(a.p_len[b], 0) + a.p_extra, P) : P;
-    const int Qb = a.q_len ? min(max(a.q_len[b], 0) + a.q_extra, Q) : Q;
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int c = lane & 15, g = lane >> 4;
-    // rows q flagged by the pair-factor kernel (pairs left to the exact pass)
-    if (tid == 0) s_unsafe = 0;
-    __syncthreads();
-    {
-        const int *fl = a.flags + (size_t)b * Q;
-        int unsafe = 0;
-        for (int q = tid; q < Qb; q += NT) unsafe |= fl[q];
-        if (unsafe) s_unsafe = 1;
-    }
-    // staging roles: 4 rows q (tg) x 4 columns (k4 of the slab / u4 of C)
-    const int tg = tid & 7, k4 = tid >> 3, u4 = tid >> 3;
-    const bool has_c = u4 < 4 * UB;
-    const float *el_base = (RAW ? a.oth + (size_t)b * a.tsb : a.Eoth + (size_t)b * Q * Kp) +
-                           min(k0 + 4 * k4, Kp - 4);
-    const size_t el_row = RAW ? (size_t)a.tsq : (size_t)Kp;
-    const float *shifts = a.oth_max + (size_t)b * Q;
-    const float *c_base = a.C + (size_t)b * a.csb + 4 * u4;
-    v4f el[DEPTH][4], cv[DEPTH][4];
-    float sh[DEPTH][4];
-    // rows beyond the reduction: E_oth clamped to a valid row, C = 0 (RAW: to a
-    // row within the entry's own length, whose values and maximum are real ones;
-    // what lies in the padding of the operand is never looked at)
-    const int q_last = RAW ? max(Qb - 1, 0) : Q - 1;
-    auto fetch = [&](int chunk, v4f (&e)[4], v4f (&cc)[4], float (&shift)[4]) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int q = chunk * TQ + 4 * tg + j;
-            e[j] = *reinterpret_cast<const v4f *>(el_base + (size_t)min(q, q_last) * el_row);
-            // (made finite in stash: an operation on it here would wait for the load here)
-            if (RAW) shift[j] = shifts[min(q, q_last)];
-            cc[j] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-            if (has_c && q < Qb) cc[j] = *reinterpret_cast<const v4f *>(c_base + (size_t)q * a.cgq);
-        }
-    };
-    // 4 rows x 4 columns -> per column the 4 rows as bfloat16 planes, 8 bytes each
-    auto stash = [&](const v4f (&e)[4], const v4f (&cc)[4], const float (&shift)[4]) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float x[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                x[j] = RAW ? exp2_hw((e[j][i] - finite_or_zero(shift[j])) * kLog2eF) : e[j][i];
-            const Pair3 lo = split3_pair(x[0], x[1]), hi = split3_pair(x[2], x[3]);
-            *reinterpret_cast<uint2 *>(&s_el[0][4 * k4 + i][4 * tg]) = make_uint2(lo.h, hi.h);
-            *reinterpret_cast<uint2 *>(&s_el[1][4 * k4 + i][4 * tg]) = make_uint2(lo.m, hi.m);
-            *reinterpret_cast<uint2 *>(&s_el[2][4 * k4 + i][4 * tg]) = make_uint2(lo.l, hi.l);
-        }
-        if (has_c) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const Pair3 lo = split3_pair(cc[0][i], cc[1][i]), hi = split3_pair(cc[2][i], cc[3][i]);
-                *reinterpret_cast<uint2 *>(&s_ct[0][4 * u4 + i][4 * tg]) = make_uint2(lo.h, hi.h);
-                *reinterpret_cast<uint2 *>(&s_ct[1][4 * u4 + i][4 * tg]) = make_uint2(lo.m, hi.m);
-                *reinterpret_cast<uint2 *>(&s_ct[2][4 * u4 + i][4 * tg]) = make_uint2(lo.l, hi.l);
-            }
-        }
-    };
-    v4f acc[2][UB];
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-        for (int ub = 0; ub < UB; ++ub) acc[kk][ub] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-    const int n = (Qb + TQ - 1) / TQ;
-    // DEPTH chunks are on their way while one is multiplied: a chunk's phases
-    // (split and store, multiply) take about a microsecond, a load takes longer
-#pragma unroll
-    for (int d = 0; d < DEPTH; ++d) fetch(d, el[d], cv[d], sh[d]);
-    for (int chunk = 0; chunk < n; chunk += DEPTH) {
-#pragma unroll
-        for (int d = 0; d < DEPTH; ++d) {
-            if (chunk + d >= n) break;
-            __syncthreads();                    // the chunk before is no longer read
-            stash(el[d], cv[d], sh[d]);
-            __syncthreads();
-            fetch(chunk + d + DEPTH, el[d], cv[d], sh[d]);
-            bf16x8 bk[2][3];
-#pragma unroll
-            for (int kk = 0; kk < 2; ++kk)
-#pragma unroll
-                for (int pn = 0; pn < 3; ++pn)
-                    bk[kk][pn] = *reinterpret_cast<const bf16x8 *>(&s_el[pn][(2 * wave + kk) * 16 + c][8 * g]);
-#pragma unroll
-            for (int ub = 0; ub < UB; ++ub) {
-                bf16x8 au[3];
-#pragma unroll
-                for (int pn = 0; pn < 3; ++pn)
-                    au[pn] = *reinterpret_cast<const bf16x8 *>(&s_ct[pn][ub * 16 + c][8 * g]);
-#pragma unroll
-                for (int kk = 0; kk < 2; ++kk) acc[kk][ub] = mfma6(au, bk[kk], acc[kk][ub]);
-            }
-        }
-    }
-    __syncthreads();
-    rhs_store_sums<UB>(a, b, k0, wave, c, g, acc, s_unsafe != 0, Pb, Qb);
-}
-
-// The same product with nothing split or transposed for C on the way: the pair
+// Nothing is split or transposed for C on the way: the pair
 // factors arrive as bfloat16 planes with the frames contiguous (written once by
 // logmm_pair_factor_planes_kernel), and a lane takes its 8 frames of one column
 // k of the long operand straight from memory, one 4-byte load per frame (the 16
@@ -1447,8 +1329,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // instruction's second operand as they are.  Only the planes of C pass through
 // LDS (a plain copy, two buffers, one barrier per chunk of 32 frames); the long
 // operand never does, and no value is split more than once per workgroup.
-// Per chunk a lane issues ~150 vector instructions where the kernel above
-// issues ~350, for the same 72 matrix instructions.
+// Per chunk a lane issues ~150 vector instructions and 72 matrix instructions.
+// (Before: both operands loaded row-wise as 16-byte vectors, split, and written
+// to LDS transposed, two barriers per chunk: ~350 vector instructions per chunk
+// and lane, 52 us where this kernel takes 39.)
 template <int UB, bool RAW>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void logmm_bwd_rhs_planes_kernel(const BwdArgs a) {
     constexpr int NT = 256, DEPTH = 2;
@@ -1689,34 +1573,6 @@ hipError_t launch_bwd(const BwdArgs &args, int B, hipStream_t stream) {
             default: RHS_PLANES(6); break;
         }
 #undef RHS_PLANES
-        return hipGetLastError();
-    }
-    if (a.cgp == 1 && a.P <= 96 && a.Kp >= 2 * kRhsSlab && a.Q >= 4 * TQ) {
-        // few rows, long reduction with the reduction index as the row index of C
-        // (the gradient of the operand with few rows): sums in registers, E_oth
-        // streamed once
-        const int ub = (a.P + 15) / 16;
-        a.tiles_x = (a.Kp + kRhsSlab - 1) / kRhsSlab, a.tiles_y = 1;
-        if (!xcd_grid_fits(a.tiles_x, 1, B)) return hipErrorInvalidValue;
-        const dim3 grid(xcd_grid(a.tiles_x, 1, B));
-        const bool raw = a.Eoth == nullptr;
-        if (!a.Eown || (raw && (a.tsk != 1 || a.K != a.Kp))) return hipErrorInvalidValue;
-#define RHS_SLAB(UBN)                                                                          \
-    do {                                                                                       \
-        if (raw)                                                                               \
-            TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<UBN, true>), grid, dim3(256), 0, stream, a); \
-        else                                                                                   \
-            TIMED_LAUNCH((logmm_bwd_rhs_slab_kernel<UBN, false>), grid, dim3(256), 0, stream, a); \
-    } while (0)
-        switch (ub) {
-            case 1: RHS_SLAB(1); break;
-            case 2: RHS_SLAB(2); break;
-            case 3: RHS_SLAB(3); break;
-            case 4: RHS_SLAB(4); break;
-            case 5: RHS_SLAB(5); break;
-            default: RHS_SLAB(6); break;
-        }
-#undef RHS_SLAB
         return hipGetLastError();
     }
     if (!a.Eown || !a.Eoth) return hipErrorInvalidValue;   // only the slab kernels read an operand itself
