@@ -35,7 +35,7 @@ MFMA_FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix, published
 # FETCH_SIZE 9 710.3 KiB x 2.0, the factors being what the same counters read
 # for a plain 1 GiB -> 1 GiB elementwise kernel (WRITE_SIZE 1 048 576,
 # FETCH_SIZE 524 300 KiB).
-LATTICE_FILL_TRAFFIC_BYTES = 1964748 * 1024 + int(9716.3 * 2 * 1024)
+LATTICE_FILL_TRAFFIC_BYTES = 1964748 * 1024 + int(9724.4 * 2 * 1024)
 
 
 def make_batch(torch, N, T, U, V, seed=2024):
