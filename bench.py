@@ -273,7 +273,9 @@ def summarise(name, facts, sec_per_step, kernels):
         tf = flops / (gemm_us * 1e-6) / 1e12 if gemm_us > 0 else 0.0
         out["algorithmic_flops_per_step"] = flops
         out["roofline"] = {"bound": "mfma", "kernel": "the three matrix products of the log-matmul "
-                           "(forward with its partial-sum pass, gradient wrt f, gradient wrt g): "
+                           "(forward, gradient wrt f, gradient wrt g; the forward's pass over its "
+                           "slabs' partial sums runs inside simple_gather_units_kernel<true>, which it "
+                           "lengthens by 4 us, not counted here): "
                            "fp32 operands split on the fly into three bfloat16 planes, six bf16 "
                            "matrix instructions per fp32 product, priced against the fp32 peak",
                            "achieved": tf, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",

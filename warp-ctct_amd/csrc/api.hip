@@ -648,8 +648,9 @@ int warpctct_simple_gather_units_f32(const float *f, const float *g, const float
     if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
     if (N == 0 || T == 0) return WARPCTCT_OK;
     if (!f || !g || !lx || !ly || !units_out || (U > 0 && !ys)) return WARPCTCT_EINVAL;
-    return done(launch_simple_gather_units(f, g, den, ys, lx, ly, units_out, N, T, U, V,
-                                           RelaySlots{}, as_stream(stream)));
+    return done(launch_simple_gather_units(f, g, const_cast<float *>(den), ys, lx, ly, units_out, N,
+                                           T, U, V, RelaySlots{}, LogmmDeferred{}, nullptr,
+                                           as_stream(stream)));
 }
 
 int warpctct_simple_reduce_f32(const float *unit_grads, float *grad_f, float *grad_g,
@@ -709,6 +710,7 @@ int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, c
     if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
     hipStream_t st = as_stream(stream);
     if (T > 0) {
+        LogmmDeferred deferred = {};
         if (normalized) {
             // den[n,t,u] = logsumexp_v(f[n,t,v] + g[n,u,v]):  lhs = f, rhs[b,k,j] = g[b,j,k]
             const LogmmOperand lhs = {f, (long)T * V, (long)V, 1L};
@@ -716,12 +718,15 @@ int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, c
             const LogmmShifted sh = {fmax, gmax, keeps_fexp ? fexp : nullptr, gexp};
             int rc = done(launch_logmm_shift_exp(lhs, rhs, sh, N, T, V, U + 1, lx, ly, st));
             if (rc != WARPCTCT_OK) return rc;
-            rc = done(launch_logmm_fwd(lhs, rhs, sh, den, w.partial, N, T, V, U + 1, lx, ly, st));
+            // (its last pass, where it is a pass of its own, is left to the gather)
+            rc = done(launch_logmm_fwd(lhs, rhs, sh, den, w.partial, N, T, V, U + 1, lx, ly,
+                                       &deferred, st));
             if (rc != WARPCTCT_OK) return rc;
         }
         int rc = done(launch_simple_gather_units(f, g, normalized ? den : nullptr, ys, lx, ly,
                                                  w.lattice.units, N, T, U, V,
-                                                 relay_slots_of(w.lattice.relay, N, T, U), st));
+                                                 relay_slots_of(w.lattice.relay, N, T, U), deferred,
+                                                 fmax, st));
         if (rc != WARPCTCT_OK) return rc;
     }
     if (want_grad && T == 0) {   // no frames: the only gradient with elements is all zeros
@@ -852,7 +857,7 @@ int warpctct_logmm_fwd_f32(const float *lhs, long lsb, long lsm, long lsk, const
                                          as_stream(stream)));
     if (rc != WARPCTCT_OK) return rc;
     return done(launch_logmm_fwd(l, r, w.sh, res, w.partial, B, M, K, Nn, nullptr, nullptr,
-                                 as_stream(stream)));
+                                 nullptr, as_stream(stream)));
 }
 
 int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, long lsm, long lsk,

@@ -147,9 +147,23 @@ hipError_t launch_logits_grad(const void *logits, int io_type, const float *lse,
                               int N, int T, int U, int V, hipStream_t stream);
 
 // ---- log-add joiner path -------------------------------------------------
-hipError_t launch_simple_gather_units(const float *f, const float *g, const float *den,
-                                      const int *ys, const int *lx, const int *ly, double *units,
-                                      int N, int T, int U, int V, const RelaySlots &relay,
+// The last pass of a log-matmul forward left to the kernel that reads the
+// product first: where launch_logmm_fwd fills this in (partial != null), res and
+// the row maxima of lhs have NOT been written yet; that kernel computes each
+// res[b,i,j] with logmm_finish_cell (logmm_finish.h), and writes res and the
+// maxima.
+struct LogmmDeferred {
+    const float *partial;    // (splits, B, pM, pN): the slabs' sums; null: nothing deferred
+    const float *slab_max;   // (splits, B, pM): maxima of the rows of lhs inside the slabs
+    const float *rmax;       // (B, Nn)
+    int splits, B, pM, pN, Nn;
+};
+// den (N,T,U+1): read, or, with `deferred.partial`, computed from the deferred
+// pass and written, together with fmax (N,T) (-inf for frames beyond lx).
+hipError_t launch_simple_gather_units(const float *f, const float *g, float *den, const int *ys,
+                                      const int *lx, const int *ly, double *units, int N, int T,
+                                      int U, int V, const RelaySlots &relay,
+                                      const LogmmDeferred &deferred, float *fmax,
                                       hipStream_t stream);
 // compact gradients of the joiner path straight from the lattices: grad_f
 // (N,T,U+1), grad_g (N,U+1,3), grad_den (N,T,U+1) or null; `partial` is scratch
@@ -215,10 +229,13 @@ int logmm_fwd_splits(int B, int M, int K, int Nn);
 __host__ __device__ inline int logmm_pair_row(int Nn) { return (Nn + 31) / 32 * 32; }
 // floats of `partial` that launch_logmm_fwd may use, whatever K is
 size_t logmm_fwd_partial_floats(int B, int M, int Nn);
+// `defer` (may be null): where the forward takes the form whose last pass can
+// be left to the next kernel, that pass is not launched and *defer describes it
+// (LogmmDeferred above); otherwise defer->partial is null afterwards.
 hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
                             const LogmmShifted &sh, float *res, float *partial, int B, int M,
                             int K, int Nn, const int *row_len, const int *col_len,
-                            hipStream_t stream);
+                            LogmmDeferred *defer, hipStream_t stream);
 // The pair factors once more, laid out for the gradient of the operand with few
 // rows (see logmm_bwd_rhs_planes_kernel): transposed and split into three
 // bfloat16 planes (3, B, logmm_pair_row(Nn), logmm_pair_frames(M)), frames

@@ -30,6 +30,7 @@
 
 #include "device_utils.h"
 #include "launch.h"
+#include "logmm_finish.h"
 
 namespace wctct {
 
@@ -640,30 +641,14 @@ __global__ __launch_bounds__(256) void logmm_fwd_finish_kernel(const FwdArgs a, 
     float s = 0.0f;
     if (a.slab_max) {
         // every slab's sum was taken against the slab's own maximum of the row
-        // (at most 8 slabs; all loads first, one round trip to memory)
-        const float *sm = a.slab_max + (size_t)b * a.pM + i;
-        float pv[8], mv[8];
-#pragma unroll
-        for (int sp = 0; sp < 8; ++sp) {
-            const int spc = min(sp, a.splits - 1);
-            pv[sp] = p[(size_t)spc * B * per];
-            mv[sp] = sp < a.splits ? sm[(size_t)spc * B * a.pM] : neg_inf_f();
-        }
-        float m = neg_inf_f();
-#pragma unroll
-        for (int sp = 0; sp < 8; ++sp) m = fmaxf(m, mv[sp]);
+        const LogmmDeferred d = {a.partial, a.slab_max, a.rmax, a.splits, B, a.pM, a.pN, a.Nn};
+        float m;
+        const float r = logmm_finish_cell(d, b, i, min(j, Nb - 1),
+                                          a.lhs + (size_t)b * a.lsb + (size_t)i * a.lsm, a.lsk,
+                                          a.rhs + (size_t)b * a.rsb + (size_t)min(j, Nb - 1) * a.rsn,
+                                          a.rsk, a.K, m);
         if (j == 0) a.lmax_out[(size_t)b * a.M + i] = m;
-        if (j >= Nb) return;
-#pragma unroll
-        for (int sp = 0; sp < 8; ++sp)
-            if (mv[sp] != neg_inf_f()) s += pv[sp] * exp2_hw((mv[sp] - m) * kLog2eF);
-        if (s >= kTiny && s < __builtin_huge_valf()) {
-            a.res[(size_t)b * a.M * a.Nn + e] = m + a.rmax[(size_t)b * a.Nn + j] + log2_hw(s) * kLn2F;
-            return;
-        }
-        a.res[(size_t)b * a.M * a.Nn + e] =
-            exact_lse(a.lhs + (size_t)b * a.lsb + (size_t)i * a.lsm, a.lsk,
-                      a.rhs + (size_t)b * a.rsb + (size_t)j * a.rsn, a.rsk, a.K);
+        if (j < Nb) a.res[(size_t)b * a.M * a.Nn + e] = r;
         return;
     }
     if (j >= Nb) return;
@@ -1694,7 +1679,8 @@ int logmm_fwd_splits(int B, int M, int K, int Nn) {
 hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
                             const LogmmShifted &sh, float *res, float *partial, int B, int M,
                             int K, int Nn, const int *row_len, const int *col_len,
-                            hipStream_t stream) {
+                            LogmmDeferred *defer, hipStream_t stream) {
+    if (defer) *defer = LogmmDeferred{};
     if (B == 0 || M == 0 || Nn == 0) return hipSuccess;
     FwdArgs a;
     a.splits = partial ? logmm_fwd_splits(B, M, K, Nn) : 1;
@@ -1737,6 +1723,10 @@ hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
             TIMED_LAUNCH((logmm_fwd_slab_kernel<4, false>), grid, dim3(64 * kSlabWaves), lds, stream, a, slabs);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
+        if (defer && raw) {   // the pass over the slabs' sums is the caller's next kernel's
+            *defer = LogmmDeferred{partial, a.slab_max, sh.rmax, slabs, B, a.pM, a.pN, Nn};
+            return hipSuccess;
+        }
         const long outs = (long)M * Nn;
         TIMED_LAUNCH(logmm_fwd_finish_kernel, dim3((unsigned)((outs + 255) / 256), B), dim3(256),
                      0, stream, a, B);

@@ -12,6 +12,7 @@
 //    (SimpleCTCTLoss.backward, warp_ctct/__init__.py:76-85).
 #include "device_utils.h"
 #include "launch.h"
+#include "logmm_finish.h"
 #include "unit_grad.h"
 
 namespace wctct {
@@ -27,10 +28,16 @@ __device__ __forceinline__ int clampi(int v, int lo, int hi) { return min(max(v,
 // f[t, y[u]] serves two cells, as the next label of (t,u) and as the current
 // label of (t,u+1): every lane reads it once and hands it to its neighbour
 // (one scattered read of f per cell instead of two).
+// DEFERRED: den is not there yet.  The log-matmul that produces it has left its
+// last pass (the sum over the slabs of the reduction, LogmmDeferred) to this
+// kernel: every cell u <= ly of a live frame computes its den[t,u], writes it
+// (the backward reads all of them), and context 0 writes the frame's fmax.
+template <bool DEFERRED>
 __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
-    const float *__restrict__ f, const float *__restrict__ g, const float *__restrict__ den,
+    const float *__restrict__ f, const float *__restrict__ g, float *__restrict__ den,
     const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
-    double *__restrict__ units, int T, int U, int V, int P, const RelaySlots relay) {
+    double *__restrict__ units, int T, int U, int V, int P, const RelaySlots relay,
+    const LogmmDeferred deferred, float *__restrict__ fmax) {
     relay_clear_share(relay);
     const int U1 = U + 1;
     const int n = blockIdx.y;
@@ -38,9 +45,24 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     const int lane = threadIdx.x & 63;
     const int t = cell / P, u = cell - t * P;      // t is the same for the whole wavefront
     const int Tn = clampi(lx[n], 0, T), Un = clampi(ly[n], 0, U);
-    if (t >= Tn) return;                           // (covers cell >= T * P)
-    const bool live = u <= Un && !outside_band(t, u, Tn, Un);
+    if (t >= Tn) {                                 // (covers cell >= T * P)
+        if (DEFERRED && t < T && u == 0) fmax[(size_t)n * T + t] = -__builtin_huge_valf();
+        return;
+    }
     const float *fr = f + ((size_t)n * T + t) * V;
+    float den_tu = 0.0f;
+    if (DEFERRED) {
+        if (u <= Un) {
+            float row_max;
+            den_tu = logmm_finish_cell(deferred, n, t, u, fr, 1, g + ((size_t)n * U1 + u) * V, 1, V,
+                                       row_max);
+            den[((size_t)n * T + t) * U1 + u] = den_tu;
+            if (u == 0) fmax[(size_t)n * T + t] = row_max;
+        }
+    } else if (den && u <= Un) {
+        den_tu = den[((size_t)n * T + t) * U1 + u];
+    }
+    const bool live = u <= Un && !outside_band(t, u, Tn, Un);
     const int *y = ys + (size_t)n * U;
     // the next label's column: wanted by this cell or by the cell of context u+1
     const bool has2 = u < Un;
@@ -60,7 +82,7 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
         return;
     }
     const float *gr = g + ((size_t)n * U1 + u) * V;
-    const double d = den ? (double)den[((size_t)n * T + t) * U1 + u] : 0.0;
+    const double d = (double)den_tu;
     const double b = (double)fr[0] + (double)gr[0] - d;
     double cur = b, nxt = neg_inf();
     if (u >= 1) cur = (double)f1 + (double)gr[c1] - d;
@@ -340,15 +362,24 @@ inline dim3 cell_grid(int N, int T, int U) {
 
 }  // namespace
 
-hipError_t launch_simple_gather_units(const float *f, const float *g, const float *den,
-                                      const int *ys, const int *lx, const int *ly, double *units,
-                                      int N, int T, int U, int V, const RelaySlots &relay,
+hipError_t launch_simple_gather_units(const float *f, const float *g, float *den, const int *ys,
+                                      const int *lx, const int *ly, double *units, int N, int T,
+                                      int U, int V, const RelaySlots &relay,
+                                      const LogmmDeferred &deferred, float *fmax,
                                       hipStream_t stream) {
     const int P = padded_contexts(U);
     const long cells = (long)T * P;
-    TIMED_LAUNCH(simple_gather_units_kernel,
-                       dim3((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N), dim3(kBlock),
-                       0, stream, f, g, den, ys, lx, ly, units, T, U, V, P, relay);
+    const dim3 grid((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N);
+    if (deferred.partial) {
+        if (!den || !fmax || deferred.splits < 1 || deferred.splits > 8 || deferred.B != N ||
+            deferred.Nn != U + 1)
+            return hipErrorInvalidValue;
+        TIMED_LAUNCH(simple_gather_units_kernel<true>, grid, dim3(kBlock), 0, stream, f, g, den, ys,
+                     lx, ly, units, T, U, V, P, relay, deferred, fmax);
+    } else {
+        TIMED_LAUNCH(simple_gather_units_kernel<false>, grid, dim3(kBlock), 0, stream, f, g, den, ys,
+                     lx, ly, units, T, U, V, P, relay, deferred, fmax);
+    }
     return hipGetLastError();
 }
 
