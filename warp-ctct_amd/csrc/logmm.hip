@@ -703,66 +703,82 @@ __global__ __launch_bounds__(256) void logmm_pair_factor_kernel(
 // logmm_pair_frames(M) entries per row (8 consecutive i of one j: one 16-byte
 // store per plane), zeros for i >= M, and shifts[b][i] = the finite maximum of
 // row i of lhs, +inf for rows that are padding (their exponentials are then 0).
-// Requires logmm_pair_row(Nn) <= 96.  grid (ct_frames / 8, B), 512 threads.
+// Requires logmm_pair_row(Nn) <= 96.  A workgroup of 8 wavefronts takes 32 rows
+// (the padded frame count is a multiple of 32), 4 per wavefront; grid
+// (ct_frames / 32, B), 512 threads.
+constexpr int kPairRowsPerWave = 4;
 __global__ __launch_bounds__(512) void logmm_pair_factor_planes_kernel(
     const float *__restrict__ go, const float *__restrict__ res, const float *__restrict__ lmax,
     const float *__restrict__ rmax, const float *__restrict__ batch_scale,
     const int *__restrict__ row_len, const int *__restrict__ col_len, float *__restrict__ C,
     int *__restrict__ flags, unsigned short *__restrict__ planes, float *__restrict__ shifts,
     int B, int M, int Nn, int ct_frames) {
-    __shared__ float s_c[8][96];
+    constexpr int R = kPairRowsPerWave;
+    __shared__ float s_c[8 * R][96];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int i = blockIdx.x * 8 + wave, b = blockIdx.y;
+    const int b = blockIdx.y, i0 = blockIdx.x * 8 * R;
     const int Mb = row_len ? min(max(row_len[b], 0), M) : M;
     const int Nb = col_len ? min(max(col_len[b], 0) + 1, Nn) : Nn;
     const float scale = batch_scale ? batch_scale[b] : 1.0f;
     const int Cq = logmm_pair_row(Nn);
-    const bool in_rows = i < M;
-    const size_t row = ((size_t)b * M + min(i, M - 1)) * Nn;
-    float *crow = C + ((size_t)b * M + min(i, M - 1)) * Cq;
-    const float ml = in_rows ? lmax[(size_t)b * M + i] : neg_inf_f();
-    int unsafe = 0;
-    // (a row has at most 96 entries: both of a lane's are requested before the
-    // first is used)
-    float gv[2], rr[2], rm[2];
+    // row r of this wavefront is local row 8*r + wave.  (A row has at most 96
+    // entries; all of a lane's loads are requested before the first is used.)
+    float gv[R][2], rr[R][2], rm[2], ml[R];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        const int j = min(lane + 64 * t, Nn - 1);
-        gv[t] = go[row + j], rr[t] = res[row + j], rm[t] = rmax[(size_t)b * Nn + j];
-    }
+    for (int t = 0; t < 2; ++t) rm[t] = rmax[(size_t)b * Nn + min(lane + 64 * t, Nn - 1)];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        const int j = lane + 64 * t;
-        if (j >= Cq) break;
-        float cv = 0.0f;
-        if (i < Mb && j < Nb) {
-            const float gs = gv[t] * scale;
-            if (gs != 0.0f && rr[t] != neg_inf_f()) {
-                const float ex = (ml + rm[t] - rr[t]) * kLog2eF;
-                if (ex <= kMaxShiftLog2)
-                    cv = gs * exp2_hw(ex);
-                else
-                    unsafe = 1;
-            }
+    for (int r = 0; r < R; ++r) {
+        const int i = min(i0 + 8 * r + wave, M - 1);
+        const size_t row = ((size_t)b * M + i) * Nn;
+        ml[r] = lmax[(size_t)b * M + i];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int j = min(lane + 64 * t, Nn - 1);
+            gv[r][t] = go[row + j], rr[r][t] = res[row + j];
         }
-        if (in_rows) crow[j] = cv;
-        s_c[wave][j] = cv;
     }
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) unsafe |= __shfl_xor(unsafe, off, 64);
-    if (lane == 0) {
-        if (in_rows) flags[(size_t)b * M + i] = unsafe;
-        shifts[(size_t)b * ct_frames + i] = (i < Mb) ? finite_or_zero(ml) : __builtin_huge_valf();
+    for (int r = 0; r < R; ++r) {
+        const int i = i0 + 8 * r + wave;
+        const bool in_rows = i < M;
+        float *crow = C + ((size_t)b * M + min(i, M - 1)) * Cq;
+        int unsafe = 0;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int j = lane + 64 * t;
+            if (j >= Cq) break;
+            float cv = 0.0f;
+            if (i < Mb && j < Nb) {
+                const float gs = gv[r][t] * scale;
+                if (gs != 0.0f && rr[r][t] != neg_inf_f()) {
+                    const float ex = (ml[r] + rm[t] - rr[r][t]) * kLog2eF;
+                    if (ex <= kMaxShiftLog2)
+                        cv = gs * exp2_hw(ex);
+                    else
+                        unsafe = 1;
+                }
+            }
+            if (in_rows) crow[j] = cv;
+            s_c[8 * r + wave][j] = cv;
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) unsafe |= __shfl_xor(unsafe, off, 64);
+        if (lane == 0) {
+            if (in_rows) flags[(size_t)b * M + i] = unsafe;
+            shifts[(size_t)b * ct_frames + i] = (i < Mb) ? finite_or_zero(ml[r]) : __builtin_huge_valf();
+        }
     }
     __syncthreads();
-    if (tid < Cq) {
+    // thread (group of 8 frames, row j of the planes)
+    for (int e = tid; e < R * Cq; e += 512) {
+        const int grp = e / Cq, j = e - grp * Cq;
         float x[8];
 #pragma unroll
-        for (int w = 0; w < 8; ++w) x[w] = s_c[w][tid];
+        for (int w = 0; w < 8; ++w) x[w] = s_c[8 * grp + w][j];
         const Pair3 p0 = split3_pair(x[0], x[1]), p1 = split3_pair(x[2], x[3]);
         const Pair3 p2 = split3_pair(x[4], x[5]), p3 = split3_pair(x[6], x[7]);
         const size_t plane = (size_t)B * Cq * ct_frames;
-        unsigned short *at = planes + ((size_t)b * Cq + tid) * ct_frames + blockIdx.x * 8;
+        unsigned short *at = planes + ((size_t)b * Cq + j) * ct_frames + i0 + 8 * grp;
         *reinterpret_cast<uint4 *>(at) = make_uint4(p0.h, p1.h, p2.h, p3.h);
         *reinterpret_cast<uint4 *>(at + plane) = make_uint4(p0.m, p1.m, p2.m, p3.m);
         *reinterpret_cast<uint4 *>(at + 2 * plane) = make_uint4(p0.l, p1.l, p2.l, p3.l);
@@ -1771,7 +1787,8 @@ hipError_t launch_logmm_pair_factor(const float *go, const float *res, const flo
     if (B == 0 || M == 0) return hipSuccess;
     if (planes.planes && planes.shifts && pair_planes_apply(M, Nn)) {
         const int frames = logmm_pair_frames(M);
-        TIMED_LAUNCH(logmm_pair_factor_planes_kernel, dim3(frames / 8, B), dim3(512), 0, stream, go,
+        TIMED_LAUNCH(logmm_pair_factor_planes_kernel, dim3(frames / (8 * kPairRowsPerWave), B),
+                     dim3(512), 0, stream, go,
                      res, lmax, rmax, batch_scale, row_len, col_len, C, flags, planes.planes,
                      planes.shifts, B, M, Nn, frames);
         return hipGetLastError();
