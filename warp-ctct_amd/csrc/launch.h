@@ -229,9 +229,9 @@ int logmm_fwd_splits(int B, int M, int K, int Nn);
 __host__ __device__ inline int logmm_pair_row(int Nn) { return (Nn + 31) / 32 * 32; }
 // floats of `partial` that launch_logmm_fwd may use, whatever K is
 size_t logmm_fwd_partial_floats(int B, int M, int Nn);
-// `defer` (may be null): where the forward takes the form whose last pass can
-// be left to the next kernel, that pass is not launched and *defer describes it
-// (LogmmDeferred above); otherwise defer->partial is null afterwards.
+// `defer` (null unless lhs is read itself, sh.El == nullptr, which requires it):
+// the forward's last pass is not launched and *defer describes it
+// (LogmmDeferred above); for a stored El, defer->partial is null afterwards.
 hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
                             const LogmmShifted &sh, float *res, float *partial, int B, int M,
                             int K, int Nn, const int *row_len, const int *col_len,

@@ -30,7 +30,6 @@
 
 #include "device_utils.h"
 #include "launch.h"
-#include "logmm_finish.h"
 
 namespace wctct {
 
@@ -273,9 +272,9 @@ struct FwdArgs {
     int splits, chunks_per_split;
     int pM, pN;               // rows and row length of one partial sum (>= M, Nn)
     // the slab kernel reading lhs itself: every slab shifts a row by the row's
-    // maximum inside the slab, slab_max (splits,B,pM), and the finish kernel
-    // brings the partial sums to the row's maximum, which it writes to lmax_out
-    float *slab_max = nullptr, *lmax_out = nullptr;
+    // maximum inside the slab, slab_max (splits,B,pM); the caller's next kernel
+    // brings the partial sums to the row's maximum (LogmmDeferred)
+    float *slab_max = nullptr;
     int M, K, Kp, Nn;
     int B, tiles_x, tiles_y;  // batch entries, row tiles, column tiles * splits
     const int *row_len, *col_len;
@@ -632,26 +631,10 @@ __global__ __launch_bounds__(256) void logmm_fwd_finish_kernel(const FwdArgs a, 
     const int i = e / a.Nn, j = e - i * a.Nn;
     const int Mb = a.row_len ? min(max(a.row_len[b], 0), a.M) : a.M;
     const int Nb = a.col_len ? min(max(a.col_len[b], 0) + 1, a.Nn) : a.Nn;
-    if (i >= Mb) {   // padding: its maximum is -inf, as shift_exp_kernel writes it
-        if (j == 0 && a.lmax_out) a.lmax_out[(size_t)b * a.M + i] = neg_inf_f();
-        return;
-    }
+    if (i >= Mb || j >= Nb) return;
     const size_t per = (size_t)a.pM * a.pN;
     const float *p = a.partial + (size_t)b * per + (size_t)i * a.pN + j;
     float s = 0.0f;
-    if (a.slab_max) {
-        // every slab's sum was taken against the slab's own maximum of the row
-        const LogmmDeferred d = {a.partial, a.slab_max, a.rmax, a.splits, B, a.pM, a.pN, a.Nn};
-        float m;
-        const float r = logmm_finish_cell(d, b, i, min(j, Nb - 1),
-                                          a.lhs + (size_t)b * a.lsb + (size_t)i * a.lsm, a.lsk,
-                                          a.rhs + (size_t)b * a.rsb + (size_t)min(j, Nb - 1) * a.rsn,
-                                          a.rsk, a.K, m);
-        if (j == 0) a.lmax_out[(size_t)b * a.M + i] = m;
-        if (j < Nb) a.res[(size_t)b * a.M * a.Nn + e] = r;
-        return;
-    }
-    if (j >= Nb) return;
     for (int sp = 0; sp < a.splits; ++sp) s += p[(size_t)sp * B * per];
     a.res[(size_t)b * a.M * a.Nn + e] = fwd_result(a, b, i, j, s);
 }
@@ -1725,9 +1708,11 @@ hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
         const size_t lds = (size_t)3 * tn * kSlabLd * sizeof(__bf16);
         const bool raw = a.El == nullptr;
         if (raw && (a.lsk != 1 || a.K != a.Kp)) return hipErrorInvalidValue;
-        if (raw) {   // behind the partial sums
-            a.slab_max = partial + (size_t)slabs * B * a.pM * a.pN;
-            a.lmax_out = sh.lmax;
+        if (raw) {
+            // the slabs' sums are taken against maxima of their own: only a caller
+            // that finishes them itself (logmm_finish_cell) can use this form
+            if (!defer) return hipErrorInvalidValue;
+            a.slab_max = partial + (size_t)slabs * B * a.pM * a.pN;   // behind the partial sums
         }
         if (wide && raw)
             TIMED_LAUNCH((logmm_fwd_slab_kernel<6, true>), grid, dim3(64 * kSlabWaves), lds, stream, a, slabs);
@@ -1739,7 +1724,7 @@ hipError_t launch_logmm_fwd(const LogmmOperand &lhs, const LogmmOperand &rhs,
             TIMED_LAUNCH((logmm_fwd_slab_kernel<4, false>), grid, dim3(64 * kSlabWaves), lds, stream, a, slabs);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
-        if (defer && raw) {   // the pass over the slabs' sums is the caller's next kernel's
+        if (raw) {   // the pass over the slabs' sums is the caller's next kernel's
             *defer = LogmmDeferred{partial, a.slab_max, sh.rmax, slabs, B, a.pM, a.pN, Nn};
             return hipSuccess;
         }
