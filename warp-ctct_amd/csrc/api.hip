@@ -800,18 +800,21 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
                                                    pw.factors, pw.flags, pw.planes, N, T, U1, st));
             if (rc != WARPCTCT_OK) return rc;
         }
-        if (dense_f) {
-            const LogmmGrad gl = {dense_f, (long)T * V, (long)V, 1L};
-            int rc = done(launch_logmm_bwd_lhs(lhs, rhs, sh, grad_den, den, pw.factors, pw.flags,
-                                               gl, N, T, V, U1, lx, ly, grad_out, st));
-            if (rc != WARPCTCT_OK) return rc;
-        }
+        // (the gradient wrt g first: it only reads f, which the gradient wrt f then
+        // finds in the memory-side cache, and whose own 4*N*T*V bytes of output are
+        // still there for the scatter that follows)
         if (dense_g) {
             // gradient of rhs[b,k,j] = g[b,j,k] stored straight into the (N,U+1,V) layout
             const LogmmGrad gr = {dense_g, (long)U1 * V, 1L, (long)V};
             int rc = done(launch_logmm_bwd_rhs(lhs, rhs, sh, grad_den, den, pw.factors, pw.flags,
                                                pw.planes,
                                                gr, N, T, V, U1, lx, ly, grad_out, st));
+            if (rc != WARPCTCT_OK) return rc;
+        }
+        if (dense_f) {
+            const LogmmGrad gl = {dense_f, (long)T * V, (long)V, 1L};
+            int rc = done(launch_logmm_bwd_lhs(lhs, rhs, sh, grad_den, den, pw.factors, pw.flags,
+                                               gl, N, T, V, U1, lx, ly, grad_out, st));
             if (rc != WARPCTCT_OK) return rc;
         }
     } else {
