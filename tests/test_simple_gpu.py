@@ -445,6 +445,48 @@ def test_simple_normalized_labels_crowded_into_few_columns():
     np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
 
 
+def test_simple_normalized_reads_f_itself_edge_values():
+    """Shapes whose log-matmul kernels read f itself (T >= 128, 512 <= V <= 2048 in
+    whole chunks of 32), at their edges: no label dimension at all (one context),
+    a sample whose lengths are zero beside a full one, vocabulary entries that are
+    -inf in f, in g, and in both (their exponentials are 0 in every kernel that
+    forms them), a whole 256-column slab of f at -inf, and a zero weight."""
+    import warp_ctct
+    rng = np.random.default_rng(31)
+    # U = 0
+    N, T, V = 2, 128, 512
+    f = np.log(rng.dirichlet(np.ones(V), (N, T))).astype(np.float32)
+    g = np.log(rng.dirichlet(np.ones(V), (N, 1))).astype(np.float32)
+    ys = np.zeros((N, 0), np.int32)
+    lx, ly = np.array([128, 77], np.int32), np.zeros(N, np.int32)
+    w = np.array([1.0, 0.0])
+    _, gf, gg, costs = O.ctct_simple_loss(f, g, ys, lx, ly, reduction="none", normalized=True,
+                                          grad_output=w)
+    tf, tg = dev(f).requires_grad_(True), dev(g).requires_grad_(True)
+    out = warp_ctct.ctct_simple_loss(tf, tg, dev(ys), dev(lx), dev(ly), reduction="none", normalized=True)
+    np.testing.assert_allclose(out.detach().cpu().numpy(), costs, rtol=LOSS_RTOL)
+    (out * dev(w, torch.float32)).sum().backward()
+    np.testing.assert_allclose(tf.grad.cpu().numpy(), gf, atol=GRAD_ATOL, rtol=1e-5)
+    np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
+    # -inf entries; labels avoid the masked columns, blank (0) stays finite
+    N, T, U, V = 2, 136, 6, 1024
+    f, g, ys, lx, ly = make_simple_case(32, N, T, U, V, lx=[136, 129], ly=[6, 4], normalized=True)
+    ys[:] = rng.integers(1, 200, ys.shape)
+    f[:, :, 300:400] = -np.inf          # in f only
+    g[:, :, 380:500] = -np.inf          # in g only, and 380..399 in both
+    f[0, 5:40, 512:768] = -np.inf       # a whole slab of the reduction for some frames
+    _, gf, gg, costs = O.ctct_simple_loss(f, g, ys, lx, ly, reduction="none", normalized=True,
+                                          grad_output=np.ones(N))
+    assert np.isfinite(costs).all()
+    tf, tg = dev(f).requires_grad_(True), dev(g).requires_grad_(True)
+    out = warp_ctct.ctct_simple_loss(tf, tg, dev(ys), dev(lx), dev(ly), reduction="none", normalized=True)
+    np.testing.assert_allclose(out.detach().cpu().numpy(), costs, rtol=LOSS_RTOL)
+    out.sum().backward()
+    assert torch.isfinite(tf.grad).all() and torch.isfinite(tg.grad).all()
+    np.testing.assert_allclose(tf.grad.cpu().numpy(), gf, atol=GRAD_ATOL, rtol=1e-5)
+    np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
+
+
 @pytest.mark.parametrize("normalized", [True, False])
 def test_simple_loss_edge_shapes(normalized):
     """No label dimension at all (g holds the one start context), samples
