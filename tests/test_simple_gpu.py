@@ -654,6 +654,58 @@ def test_full_size_log_add_joiner_against_the_float64_oracle():
         assert np.all(f.grad[n, t:].cpu().numpy() == 0) and np.all(g.grad[n, u + 1:].cpu().numpy() == 0)
 
 
+def test_full_size_normalized_joiner_invariants():
+    """N=32, T<=400, U<=80, V=2048, normalized: properties that hold at any size.
+    The normalised loss sees f and g only through log_softmax(f + g): adding a
+    constant to every vocabulary entry of a frame of f (of a context of g) changes
+    neither the costs nor the gradients; for the same reason the gradient wrt f
+    sums to zero over the vocabulary in every frame, and likewise that wrt g;
+    frames beyond lx and contexts beyond ly take no gradient; and the gradients
+    are linear in the weights of the samples."""
+    import warp_ctct
+    N, T, U, V = 32, 400, 80, 2048
+    rng = np.random.default_rng(515)
+    gen = torch.Generator(device="cuda").manual_seed(515)
+    f = torch.randn(N, T, V, device="cuda", generator=gen)
+    g = torch.randn(N, U + 1, V, device="cuda", generator=gen)
+    lx = rng.integers(300, 401, N).astype(np.int32)
+    ly = rng.integers(50, 81, N).astype(np.int32)
+    lx[3], ly[3] = 400, 80
+    ys = rng.integers(1, V, (N, U)).astype(np.int32)
+    d_ys, d_lx, d_ly = dev(ys), dev(lx), dev(ly)
+    w = torch.randn(N, device="cuda", generator=gen)
+
+    def run(ff, gg, weights):
+        ff = ff.clone().requires_grad_(True)
+        gg = gg.clone().requires_grad_(True)
+        costs = warp_ctct.ctct_simple_loss(ff, gg, d_ys, d_lx, d_ly, reduction="none", normalized=True)
+        (costs * weights).sum().backward()
+        return costs.detach(), ff.grad, gg.grad
+
+    c0, gf0, gg0 = run(f, g, w)
+    assert torch.isfinite(c0).all()
+    # shifts per frame and per context, of the size of the values themselves
+    sf = 3.0 * torch.randn(N, T, 1, device="cuda", generator=gen)
+    sg = 3.0 * torch.randn(N, U + 1, 1, device="cuda", generator=gen)
+    c1, gf1, gg1 = run(f + sf, g + sg, w)
+    torch.testing.assert_close(c1, c0, rtol=2e-5, atol=1e-3)
+    scale = float(w.abs().max())
+    torch.testing.assert_close(gf1, gf0, rtol=1e-4, atol=2 * GRAD_ATOL * scale)
+    torch.testing.assert_close(gg1, gg0, rtol=1e-4, atol=2 * GRAD_ATOL * scale)
+    # zero sum over the vocabulary (each row sums 2048 terms of either sign)
+    assert float(gf0.sum(-1).abs().max()) < 1e-3 * scale
+    assert float(gg0.double().sum(-1).abs().max()) < 2e-2 * scale    # entries reach the hundreds
+    # nothing beyond the lengths
+    t_idx = torch.arange(T, device="cuda")[None, :] >= d_lx[:, None]
+    u_idx = torch.arange(U + 1, device="cuda")[None, :] > d_ly[:, None]
+    assert float(gf0[t_idx].abs().max()) == 0.0 and float(gg0[u_idx].abs().max()) == 0.0
+    # linear in the weights
+    c2, gf2, gg2 = run(f, g, -2.0 * w)
+    torch.testing.assert_close(c2, c0, rtol=0, atol=0)
+    torch.testing.assert_close(gf2, -2.0 * gf0, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(gg2, -2.0 * gg0, rtol=1e-5, atol=1e-5)
+
+
 def test_deep_lattice_unnormalized():
     """The long-utterance shape (T<=1500, U<=300) at a vocabulary that lets the
     joint be materialised for the identity check."""
