@@ -332,8 +332,8 @@ size_t warpctct_simple_workspace_bytes(int N, int T, int U);
  * exp(f - fmax) on the way (U+1 <= 96 contexts, 512 <= V <= 2048 in whole
  * multiples of 32, T >= 128, f aligned to 16 bytes): fexp is then neither
  * written by the forward nor read by the backward and may be NULL in both,
- * and fmax is written by the forward's last log-matmul kernel instead of a
- * pass of its own over f.  1 otherwise.  No counterpart in the reference
+ * and fmax is written by the kernel that gathers the lattice's inputs (which
+ * also finishes den) instead of a pass of its own over f.  1 otherwise.  No counterpart in the reference
  * (which recomputes every exponential in every kernel,
  * csrc/logmatmul.cu:44-146). */
 int warpctct_simple_needs_fexp(const float *f, int T, int U, int V);
