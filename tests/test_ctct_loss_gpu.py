@@ -344,6 +344,9 @@ LOGITS_CASES = [
     ("two_wavefronts_f32", 43, 2, 90, 70, 24, [90, 80], [70, 66], 1.0, torch.float32),
     ("bf16", 44, 3, 20, 6, 64, range(10, 21), range(2, 7), 2.0, torch.bfloat16),
     ("f16_odd_vocab", 45, 2, 14, 4, 33, [14, 9], [4, 3], 2.0, torch.float16),
+    # a frame whose units do not fit the kernel's LDS staging (more than 2340
+    # contexts): results stored row by row
+    ("frame_wider_than_lds_f32", 47, 2, 36, 2400, 8, [36, 30], [24, 9], 1.5, torch.float32),
 ]
 
 
@@ -584,6 +587,64 @@ def test_forward_and_backward_replay_from_a_hip_graph():
         torch.cuda.synchronize()
         assert torch.equal(got_loss, loss), "replay %d: loss differs from eager" % replay
         assert torch.equal(got_grad, grad), "replay %d: gradient differs from eager" % replay
+
+
+@pytest.mark.parametrize("reduction", ["none", "sum", "mean"])
+def test_no_frames_at_all(reduction):
+    """A batch without a single frame (T = 0): no gather runs, the lattice
+    launch still reduces over the batch; a sample without labels costs 0, one
+    with labels is infeasible (+inf), as in the oracle."""
+    import warp_ctct
+    ys = np.array([[1, 2], [3, 4], [2, 2]], dtype=np.int32)
+    lx = np.zeros(3, dtype=np.int32)
+    for ly in ([0, 0, 0], [0, 1, 0]):
+        ly = np.array(ly, dtype=np.int32)
+        ref = O.ctct_loss(np.zeros((3, 0, 3, 5)), ys, lx, ly, reduction=reduction)[0]
+        x = torch.zeros(3, 0, 3, 5, device="cuda", requires_grad=True)
+        loss = warp_ctct.ctct_loss(x, dev(ys), dev(lx), dev(ly), reduction=reduction)
+        np.testing.assert_array_equal(loss.detach().cpu().numpy(), np.asarray(ref, dtype=np.float32))
+        if np.all(np.isfinite(ref)):
+            grad, = torch.autograd.grad(loss.sum(), x)
+            assert grad.shape == x.shape
+        logits = torch.zeros(3, 0, 3, 5, device="cuda")
+        fused = warp_ctct.ctct_loss_with_logits(logits, dev(ys), dev(lx), dev(ly), reduction=reduction)
+        np.testing.assert_array_equal(fused.cpu().numpy(), np.asarray(ref, dtype=np.float32))
+
+
+def test_kernel_timing_records_stay_out_of_a_graph_capture():
+    """The per-kernel timing of the library (warpctct_profile) brackets launches
+    with events on their stream; a stream under capture takes none, so a
+    capture made while the timing is on is as good as any other and leaves no
+    error behind for the next call."""
+    import warp_ctct
+    lib = hip_lib.lib()
+    joint, ys, lx, ly = make_joint_case(73, 3, 21, 6, 17, lx=range(12, 22), ly=range(2, 7))
+    d_ys, d_lx, d_ly = dev(ys), dev(lx), dev(ly)
+    static_in = dev(joint).requires_grad_(True)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                       # warm-up outside the capture
+        torch.autograd.grad(warp_ctct.ctct_loss(static_in, d_ys, d_lx, d_ly), static_in)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    assert lib.warpctct_profile(1) == 0
+    try:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_loss = warp_ctct.ctct_loss(static_in, d_ys, d_lx, d_ly)
+            static_grad, = torch.autograd.grad(static_loss, static_in)
+        assert lib.warpctct_profile_count() == 0, "launches into the capture were bracketed"
+        graph.replay()
+        torch.cuda.synchronize()
+        x = dev(joint).requires_grad_(True)
+        loss = warp_ctct.ctct_loss(x, d_ys, d_lx, d_ly)      # eager: bracketed
+        grad, = torch.autograd.grad(loss, x)
+        torch.cuda.synchronize()
+        assert lib.warpctct_profile_count() > 0
+    finally:
+        lib.warpctct_profile(0)
+    assert torch.equal(static_loss, loss)
+    assert torch.equal(static_grad, grad)
 
 
 def test_operator_surface_on_gathered_units():

@@ -272,6 +272,14 @@ SIMPLE_CASES = [
     # contexts and four, a vocabulary that ends inside a slab, ragged lengths
     ("reads_f_itself_few_contexts", 7, 2, 160, 5, 512, [160, 131], [5, 3]),
     ("reads_f_itself_partial_slab", 8, 2, 130, 60, 800, [130, 128], [60, 33]),
+    # the remaining instances of the joiner's gradient kernels: two and five
+    # blocks of 16 contexts, with f read itself and with a vocabulary too long
+    # for that (2049..4096 and 4097..8192 entries: the row kernels of the shifted
+    # exponentials for 16 and 32 vectors per lane)
+    ("reads_f_itself_five_blocks", 9, 2, 130, 70, 800, [130, 128], [70, 41]),
+    ("reads_f_itself_two_blocks", 11, 2, 128, 20, 512, [128, 128], [20, 9]),
+    ("long_vocabulary_two_blocks", 10, 2, 144, 20, 2304, [144, 129], [20, 11]),
+    ("long_vocabulary_five_blocks", 12, 2, 144, 66, 4352, [144, 140], [66, 50]),
 ]
 
 

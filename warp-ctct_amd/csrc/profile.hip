@@ -41,6 +41,15 @@ void profile_begin(const char *kernel, hipStream_t stream, int *slot) {
     std::lock_guard<std::mutex> lock(g_mutex);
     if ((int)g_records.size() >= kMaxRecords) return;
     if (g_filter[0] && !std::strstr(kernel, g_filter)) return;
+    // A stream under graph capture takes no timing events (recording one would
+    // become a node of the graph, or fail and leave its error for the caller's
+    // own check of the launch): launches into a capture are not bracketed.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capture) != hipSuccess) {
+        (void)hipGetLastError();
+        return;
+    }
+    if (capture != hipStreamCaptureStatusNone) return;
     Record r = {kernel, nullptr, nullptr, false};
     if (hipEventCreate(&r.begin) != hipSuccess) return;
     if (hipEventCreate(&r.end) != hipSuccess) {
