@@ -344,6 +344,11 @@ LOGITS_CASES = [
     ("two_wavefronts_f32", 43, 2, 90, 70, 24, [90, 80], [70, 66], 1.0, torch.float32),
     ("bf16", 44, 3, 20, 6, 64, range(10, 21), range(2, 7), 2.0, torch.bfloat16),
     ("f16_odd_vocab", 45, 2, 14, 4, 33, [14, 9], [4, 3], 2.0, torch.float16),
+    # rows of 2-byte elements read as 16-byte vectors: one vector, and more than
+    # one round of 1024 elements with a partial last round
+    ("f16_vector_rows", 48, 2, 14, 4, 8, [14, 9], [4, 3], 2.0, torch.float16),
+    ("f16_vector_rows_two_rounds", 49, 2, 9, 3, 1096, [9, 6], [3, 2], 2.0, torch.float16),
+    ("bf16_vector_rows_two_rounds", 50, 2, 9, 3, 1096, [9, 6], [3, 2], 2.0, torch.bfloat16),
     # a frame whose units do not fit the kernel's LDS staging (more than 2340
     # contexts): results stored row by row
     ("frame_wider_than_lds_f32", 47, 2, 36, 2400, 8, [36, 30], [24, 9], 1.5, torch.float32),

@@ -117,13 +117,14 @@ __device__ __forceinline__ void unpack(const float *, const raw16 &v, float (&x)
 #pragma unroll
     for (int i = 0; i < 4; ++i) x[i] = __uint_as_float(v[i]);
 }
+// (each half taken out of its word with integer operations: a cast of the word
+// to a vector of two halves read word 0 for every i once compiled)
 __device__ __forceinline__ void unpack(const __half *, const raw16 &v, float (&x)[8]) {
-    typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const v2h h = __builtin_bit_cast(v2h, v[i]);
-        x[2 * i] = (float)h[0];
-        x[2 * i + 1] = (float)h[1];
+        const unsigned word = v[i];
+        x[2 * i] = (float)__builtin_bit_cast(_Float16, (unsigned short)(word & 0xffffu));
+        x[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (unsigned short)(word >> 16));
     }
 }
 __device__ __forceinline__ void unpack(const __hip_bfloat16 *, const raw16 &v, float (&x)[8]) {
