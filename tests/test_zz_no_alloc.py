@@ -54,8 +54,10 @@ def forward_both(joint, ys, lx, ly):
 def test_static_scratch_forward_matches_the_workspace_forward():
     lib = hip_lib.lib()
     big = make_joint_case(101, 6, 120, 40, 50, lx=range(70, 121), ly=range(15, 41))
+    # lattices of two and three workgroups each: their hand-over slots lie in the array too
+    chains = make_joint_case(103, 3, 150, 140, 7, lx=range(145, 151), ly=range(70, 141))
     small = make_joint_case(102, 3, 31, 9, 17, lx=range(12, 32), ly=range(2, 10))
-    for joint, ys, lx, ly in (big, small):        # the second call is the smaller problem
+    for joint, ys, lx, ly in (big, chains, small):        # the last call is the smallest problem
         (c_ws, g_ws), (c_st, g_st) = forward_both(joint, ys, lx, ly)
         np.testing.assert_array_equal(c_st, c_ws)
         np.testing.assert_array_equal(g_st, g_ws)
