@@ -327,7 +327,9 @@ size_t warpctct_simple_workspace_bytes(int N, int T, int U);
  * fexp (N,T,Vp) = exp(f - fmax) (see warpctct_simple_needs_fexp) and
  * gexp (N,U+1,Vp) = exp(g - gmax) with
  * Vp = warpctct_logmm_padded_reduction(V), zero in the padding.
- * grad_f/grad_g/grad_den may all be NULL (no-grad mode). */
+ * grad_f/grad_g/grad_den may all be NULL (no-grad mode); without frames
+ * (T = 0) grad_f and grad_den have no elements and may be NULL beside a
+ * grad_g, which is then cleared. */
 /* 0 where the log-matmul kernels of the normalised path read f itself and form
  * exp(f - fmax) on the way (U+1 <= 96 contexts, 512 <= V <= 2048 in whole
  * multiples of 32, T >= 128, f aligned to 16 bytes): fexp is then neither

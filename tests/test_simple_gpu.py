@@ -335,6 +335,28 @@ def test_public_simple_loss_and_grads(case, normalized):
 
 
 @pytest.mark.parametrize("normalized", [True, False])
+def test_simple_loss_without_a_single_frame(normalized):
+    """T = 0: a sample without labels costs 0, one with labels is infeasible
+    (+inf); the gradients have the operands' shapes, that of g all zeros."""
+    import warp_ctct
+    ys = np.array([[1, 2], [3, 4], [2, 2]], dtype=np.int32)
+    lx = np.zeros(3, dtype=np.int32)
+    for ly in ([0, 0, 0], [0, 1, 0]):
+        ly = np.array(ly, dtype=np.int32)
+        _, _, _, costs = O.ctct_simple_loss(np.zeros((3, 0, 5)), np.zeros((3, 3, 5)), ys, lx, ly,
+                                            reduction="none", normalized=normalized)
+        tf = torch.zeros(3, 0, 5, device="cuda", requires_grad=True)
+        tg = torch.zeros(3, 3, 5, device="cuda", requires_grad=True)
+        out = warp_ctct.ctct_simple_loss(tf, tg, dev(ys), dev(lx), dev(ly), reduction="none",
+                                         normalized=normalized)
+        np.testing.assert_array_equal(out.detach().cpu().numpy(), costs.astype(np.float32))
+        if np.all(np.isfinite(costs)):
+            out.sum().backward()
+            assert tf.grad.shape == tf.shape and tg.grad.shape == tg.shape
+            assert np.all(tg.grad.cpu().numpy() == 0)
+
+
+@pytest.mark.parametrize("normalized", [True, False])
 def test_simple_loss_replays_from_a_hip_graph(normalized):
     """A captured ctct_simple_loss step (log-matmul, lattice, scatter) replays
     with the eager results of the same inputs; the scatter adds atomically, so

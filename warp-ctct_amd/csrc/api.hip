@@ -701,7 +701,9 @@ int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, c
     const bool want_grad = grad_f || grad_g || grad_den;
     if (!g || !lx || !ly || !costs || !workspace || (T > 0 && !f) || (U > 0 && !ys))
         return WARPCTCT_EINVAL;
-    if (want_grad && (!grad_f || !grad_g || (normalized && !grad_den))) return WARPCTCT_EINVAL;
+    // (without frames the gradients of f and den have no elements, and no address)
+    if (want_grad && (!grad_g || (T > 0 && (!grad_f || (normalized && !grad_den)))))
+        return WARPCTCT_EINVAL;
     // where the log-matmul kernels read f itself, exp(f - fmax) is not stored
     const bool keeps_fexp = warpctct_simple_needs_fexp(f, T, U, V) != 0;
     if (normalized && T > 0 && (!den || !fmax || !gmax || !gexp || (keeps_fexp && !fexp)))
@@ -746,7 +748,8 @@ int warpctct_simple_forward_units_f32(const float *f_g, const float *g_g, const 
     const bool want_grad = grad_f || grad_g || grad_den;
     if (!g_g || !lx || !ly || !costs || !workspace || (T > 0 && !f_g) || (U > 0 && !ys))
         return WARPCTCT_EINVAL;
-    if (want_grad && (!grad_f || !grad_g || (den && !grad_den))) return WARPCTCT_EINVAL;
+    if (want_grad && (!grad_g || (T > 0 && (!grad_f || (den && !grad_den)))))
+        return WARPCTCT_EINVAL;
     const SimpleWorkspace w = carve_simple(workspace, N, T, U);
     if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
     hipStream_t st = as_stream(stream);
