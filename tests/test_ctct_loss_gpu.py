@@ -594,6 +594,26 @@ def test_forward_and_backward_replay_from_a_hip_graph():
         assert torch.equal(got_grad, grad), "replay %d: gradient differs from eager" % replay
 
 
+def test_more_lattice_chains_than_the_gpu_holds_at_once():
+    """1200 lattices of two workgroups per direction: 4800 single-wavefront
+    workgroups that wait for one another, more than are resident at a time.
+    A consumer is never dispatched before its producer (workgroup index order),
+    so every wait ends: no NaN (the mark of a hand-over given up), and costs and
+    gradients as the oracle's."""
+    import warp_ctct
+    N, T, U, V = 1200, 100, 70, 5
+    joint, ys, lx, ly = make_joint_case(81, N, T, U, V, lx=range(96, 101), ly=range(64, 71))
+    assert ly.min() >= 64 and 2 * N * 2 > 4096
+    x = dev(joint).requires_grad_(True)
+    out = warp_ctct.ctct_loss(x, dev(ys), dev(lx), dev(ly), reduction="none")
+    out.sum().backward()
+    got = out.detach().cpu().numpy()
+    assert not np.any(np.isnan(got))
+    _, ref_grad, costs = O.ctct_loss(joint, ys, lx, ly, reduction="sum")
+    np.testing.assert_allclose(got, costs, rtol=LOSS_RTOL)
+    np.testing.assert_allclose(x.grad.cpu().numpy(), ref_grad, atol=GRAD_ATOL, rtol=0)
+
+
 @pytest.mark.parametrize("reduction", ["none", "sum", "mean"])
 def test_no_frames_at_all(reduction):
     """A batch without a single frame (T = 0): no gather runs, the lattice
