@@ -414,7 +414,8 @@ int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, lo
  * warpctct_profile_filter(text) limits the bracketing to kernels whose name
  * contains `text` (at most 63 characters; NULL or "": every kernel), so that
  * one kernel can be timed inside a timed region at the cost of two events.
- * Creating events allocates: keep it off in production and under graph capture. */
+ * Creating events allocates: keep it off in production.  Launches into a stream
+ * that is under graph capture are not bracketed and leave no record. */
 int warpctct_profile(int enable);
 int warpctct_profile_filter(const char *text);
 int warpctct_profile_count(void);
