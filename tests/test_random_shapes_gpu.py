@@ -131,7 +131,8 @@ def test_random_joiner_cases(seed):
 @pytest.mark.parametrize("seed", [31, 32])
 def test_random_log_matmul_cases(seed):
     """_C.log_matmul and log_matmul_backward: either operand the long one, the
-    right operand contiguous, a transposed view, or shared by the batch; rows
+    right operand contiguous, a transposed view, or shared by the batch, or both
+    operands views into wider tensors; rows
     and columns of -inf and maxima 300 apart in a quarter of the cases."""
     from warp_ctct import _C
     rng = np.random.default_rng(seed)
@@ -146,7 +147,7 @@ def test_random_log_matmul_cases(seed):
             M, Nn = Nn, M
         if B * M * K * Nn > 20e6:
             continue
-        layout = ["contiguous", "transposed", "shared"][int(rng.integers(0, 3))]
+        layout = ["contiguous", "transposed", "shared", "offset"][int(rng.integers(0, 4))]
         special = int(rng.integers(0, 4)) == 0
         case_seed = int(rng.integers(0, 1 << 30))
         print("case B=%d M=%d K=%d Nn=%d %s special=%s seed=%d"
@@ -167,6 +168,13 @@ def test_random_log_matmul_cases(seed):
         d_lhs = dev(lhs)
         if layout == "transposed":
             d_rhs = dev(np.ascontiguousarray(rhs.transpose(0, 2, 1))).transpose(1, 2)
+        elif layout == "offset":    # both operands inside wider tensors, rows not on 16-byte boundaries
+            wide_l = torch.zeros(B, M, K + 3, device="cuda")
+            wide_l[..., 1:K + 1] = d_lhs
+            d_lhs = wide_l[..., 1:K + 1]
+            wide_r = torch.zeros(B, K, Nn + 2, device="cuda")
+            wide_r[..., 1:Nn + 1] = dev(rhs)
+            d_rhs = wide_r[..., 1:Nn + 1]
         else:
             d_rhs = dev(rhs)
         out = _C.log_matmul(d_lhs, d_rhs)
