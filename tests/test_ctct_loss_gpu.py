@@ -352,6 +352,8 @@ LOGITS_CASES = [
     # a frame whose units do not fit the kernel's LDS staging (more than 2340
     # contexts): results stored row by row
     ("frame_wider_than_lds_f32", 47, 2, 36, 2400, 8, [36, 30], [24, 9], 1.5, torch.float32),
+    ("frame_wider_than_lds_f16", 51, 2, 36, 2400, 16, [36, 30], [24, 9], 1.5, torch.float16),
+    ("frame_wider_than_lds_bf16_odd_vocab", 52, 2, 36, 2400, 7, [36, 30], [24, 9], 1.5, torch.bfloat16),
 ]
 
 
