@@ -197,3 +197,53 @@ def test_random_log_matmul_cases(seed):
         np.testing.assert_allclose(out_r.cpu().numpy(), gr, atol=atol * Br if layout != "shared" else atol * B,
                                    rtol=1e-4)
         done += 1
+
+
+@pytest.mark.parametrize("seed", [41, 42])
+def test_random_cases_of_the_operators_on_gathered_inputs(seed):
+    """_C.ctct_loss_fwd and _C.ctct_loss_simple_fwd (the reference's own operator
+    surface): up to 601 contexts (chains of ten workgroups; beyond 512 the
+    joiner's reductions take their own kernels), with and without gradients."""
+    from warp_ctct import _C
+    rng = np.random.default_rng(seed)
+    Ts = [1, 2, 7, 8, 9, 12, 13, 24, 25, 37, 70, 140, 300]
+    Us = [0, 1, 2, 5, 62, 63, 64, 65, 127, 128, 129, 200, 511, 512, 513, 600]
+    done = 0
+    while done < 300:
+        N, T = int(rng.integers(1, 5)), int(rng.choice(Ts))
+        U, V = int(rng.choice(Us)), int(rng.choice([3, 5, 9, 33]))
+        if N * T * (U + 1) > 1.0e6:
+            continue
+        case_seed, want = int(rng.integers(0, 1 << 30)), bool(rng.integers(0, 4) > 0)
+        which = int(rng.integers(0, 3))
+        print("case op=%d N=%d T=%d U=%d V=%d requires_grad=%s seed=%d"
+              % (which, N, T, U, V, want, case_seed), flush=True)
+        if which == 0:
+            joint, ys, lx, ly = make_joint_case(case_seed, N, T, U, V)
+            lp3 = O.gather_units(joint, ys).astype(np.float32)
+            with np.errstate(all="ignore"):
+                costs_ref, grads_ref = O.ctct_loss_fwd(lp3, ys, lx, ly)
+            costs, grads = _C.ctct_loss_fwd(dev(lp3), dev(ys), dev(lx), dev(ly), want)
+            finite = same_costs(costs.cpu().numpy(), costs_ref)
+            if want and finite:
+                np.testing.assert_allclose(grads.cpu().numpy(), grads_ref, atol=GRAD_ATOL, rtol=0)
+            if not want:       # the reference returns the costs twice
+                np.testing.assert_array_equal(grads.cpu().numpy(), costs.cpu().numpy())
+        else:
+            normalized = which == 1
+            f, g, ys, lx, ly = make_simple_case(case_seed, N, T, U, V, normalized=normalized)
+            f_g, g_g = O.gather_separate(f, g, ys)
+            den = O.log_matmul(f, np.swapaxes(g, 1, 2)).astype(np.float32) if normalized else None
+            with np.errstate(all="ignore"):
+                costs_ref, gf, gg, gd = O.ctct_loss_simple_fwd(f_g, g_g, ys, den, lx, ly)
+            d_den = dev(den) if normalized else torch.empty(1)
+            out = _C.ctct_loss_simple_fwd(dev(f_g), dev(g_g), dev(ys), d_den, dev(lx), dev(ly), want)
+            finite = same_costs(out[0].cpu().numpy(), costs_ref)
+            if want and finite:
+                np.testing.assert_allclose(out[1].cpu().numpy(), gf, atol=GRAD_ATOL, rtol=0)
+                np.testing.assert_allclose(out[2].cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
+                if normalized:
+                    np.testing.assert_allclose(out[3].cpu().numpy(), gd, atol=GRAD_ATOL, rtol=0)
+            if not want:
+                assert out[1] is None and out[2] is None and out[3] is None
+        done += 1
