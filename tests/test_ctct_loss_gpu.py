@@ -934,3 +934,38 @@ def test_full_size(cfg):
     for n in range(N):
         np.testing.assert_allclose(mass[n, :lx[n]], -wn[n], rtol=1e-4, atol=1e-5)
         assert np.all(mass[n, lx[n]:] == 0)
+
+
+@pytest.mark.parametrize("dtype,logits", [(torch.float16, True), (torch.bfloat16, False)],
+                         ids=["float16_logits", "bfloat16_joint"])
+def test_full_size_typical_batch_in_half_precision(dtype, logits):
+    """The typical batch (N=32, T<=250, U<=60, V=1024) with 2-byte elements,
+    through the fused logits entry and through the joint, against the float64
+    oracle on the rounded inputs: loss within 1e-5 relative, every gradient
+    entry within 1e-4 of the sample weight (1/N) plus one unit in the last
+    place of the type."""
+    import warp_ctct
+    N, T, U, V = 32, 250, 60, 1024
+    rng = np.random.default_rng(5)
+    lx = rng.integers(150, T + 1, N).astype(np.int32)
+    ly = rng.integers(30, U + 1, N).astype(np.int32)
+    ys = rng.integers(1, V, (N, U)).astype(np.int32)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(N, T, U + 1, V, device="cuda", generator=gen) * 2
+    if not logits:
+        x = x.log_softmax(-1)
+    x = x.to(dtype).requires_grad_(True)
+    fn = warp_ctct.ctct_loss_with_logits if logits else warp_ctct.ctct_loss
+    loss = fn(x, dev(ys), dev(lx), dev(ly), reduction="mean")
+    loss.backward()
+    rounded = x.detach().double().cpu().numpy()
+    if logits:
+        ref_loss, ref_grad, _ = O.ctct_loss_with_logits(rounded, ys, lx, ly, "mean", False)
+    else:
+        ref_loss, ref_grad, _ = O.ctct_loss(rounded, ys, lx, ly, reduction="mean")
+    del rounded
+    np.testing.assert_allclose(loss.item(), ref_loss, rtol=LOSS_RTOL)
+    got = x.grad.double().cpu().numpy()
+    ulp = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+    assert np.all(np.abs(got - ref_grad) <= GRAD_ATOL / N + ulp * np.abs(ref_grad))
+    assert np.all(got[ref_grad == 0] == 0)
