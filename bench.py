@@ -138,9 +138,11 @@ OTHER = {
     # torch.log_softmax followed by ctct_loss (what a caller of the reference does)
     "c2_logits": ("logits", 32, 250, 60, 1024, 1.0),
     "c2_logits_bf16": ("logits", 32, 250, 60, 1024, 1.0),
+    "c2_logits_f16": ("logits", 32, 250, 60, 1024, 1.0),
     "c2_logits_unfused": ("logits_unfused", 32, 250, 60, 1024, 1.0),
 }
-IO_DTYPE = {"c2_bf16": "bfloat16", "c2_f16": "float16", "c2_logits_bf16": "bfloat16"}
+IO_DTYPE = {"c2_bf16": "bfloat16", "c2_f16": "float16", "c2_logits_bf16": "bfloat16",
+            "c2_logits_f16": "float16"}
 WORKLOAD = {
     "c1": "ctct_loss fp32, N=2, T=40, U=10, V=32, full lengths (the reference's CPU-sized case)",
     "c2": "ctct_loss fp32, typical ASR batch: N=32, lx in [150,250], ly in [30,60], V=1024",
