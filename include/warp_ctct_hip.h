@@ -29,6 +29,12 @@
 extern "C" {
 #endif
 
+/* The library is built with hidden symbol visibility; the entry points declared
+ * here are its whole exported surface. */
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
+
 enum {
     WARPCTCT_OK = 0,
     WARPCTCT_EINVAL = 1,     /* null pointer, negative size, or beyond N <= 65535,
@@ -42,7 +48,8 @@ enum {
 /* Human-readable text for a return code (static storage). */
 const char *warpctct_error_string(int code);
 
-/* Library version, "major.minor.patch". */
+/* Version of this C ABI, "major.minor.patch"; independent of the Python
+ * distribution's version, which follows the reference distribution. */
 const char *warpctct_version(void);
 
 /* Contexts per frame in the work buffers: the smallest multiple of 64 that is
@@ -101,7 +108,9 @@ int warpctct_simple_units_f32(const float *f_g, const float *g_g, const float *d
  * warpctct_lattice_wait_limit(spins): how often a waiting workgroup asks again
  * before it gives up (0: the first look decides; negative: back to the default,
  * about a second of polling); applies to launches made afterwards, returns the
- * previous limit.  It has no counterpart in the reference, whose spin lock
+ * previous limit.  The limit is one value for the whole process (every thread's
+ * later launches see it) and exists for tests; production code leaves it alone.
+ * It has no counterpart in the reference, whose spin lock
  * (csrc/gather.cu:88, :106, :171) is unbounded; tests use it to exercise the give-up
  * path with kernels that still run to their end. */
 size_t warpctct_lattice_relay_bytes(int N, int T, int U);
@@ -405,6 +414,30 @@ int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, lo
                            float *grad_lhs, long glsb, long glsm, long glsk, float *grad_rhs,
                            long grsb, long grsk, long grsn, void *stream);
 
+/* ---- status word ----------------------------------------------------------
+ * Kernels never synchronise with the host, so what the reference reports by
+ * raising (torch.gather on a label outside [0, V): warp_ctct/__init__.py:131)
+ * is recorded instead in a sticky word on the device, one per GPU:
+ *   WARPCTCT_STATUS_LABEL_RANGE    a label outside [0, V) was clamped into it
+ *                                  before it was used as a column index;
+ *   WARPCTCT_STATUS_NAN_INPUT      a gathered log-probability was NaN (the
+ *                                  lattice treats such a unit as -inf: the
+ *                                  hardware's maximum drops NaN operands);
+ *   WARPCTCT_STATUS_LOST_HAND_OVER a chain of workgroups gave up waiting for a
+ *                                  hand-over (see warpctct_lattice_f32): the NaN
+ *                                  costs / gradients of that call do not come
+ *                                  from the inputs.
+ * warpctct_status waits for the work queued on the current device
+ * (hipDeviceSynchronize: the one entry point that does), copies the word to
+ * *bits and, with clear != 0, sets it back to 0.  Bits set by launches that
+ * overlap the call may land before or after it. */
+enum {
+    WARPCTCT_STATUS_LABEL_RANGE = 1,
+    WARPCTCT_STATUS_NAN_INPUT = 2,
+    WARPCTCT_STATUS_LOST_HAND_OVER = 4
+};
+int warpctct_status(unsigned *bits, int clear);
+
 /* ---- measurement aid ------------------------------------------------------
  * No counterpart in the reference.  warpctct_profile(1) clears earlier records
  * and starts bracketing every kernel launch of the library with two HIP events
@@ -420,6 +453,10 @@ int warpctct_profile(int enable);
 int warpctct_profile_filter(const char *text);
 int warpctct_profile_count(void);
 int warpctct_profile_read(int index, const char **kernel, float *microseconds);
+
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
 
 #ifdef __cplusplus
 }

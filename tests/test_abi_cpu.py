@@ -14,6 +14,17 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), name
 
 
+def test_library_exports_nothing_but_the_declared_symbols():
+    """The shared object is linked with hidden visibility and a version script:
+    its dynamic symbol table holds the C ABI of include/warp_ctct_hip.h and no
+    C++ internals, helper functions or compiler-generated data."""
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", hip_lib.LIB_PATH], capture_output=True,
+                         text=True, check=True).stdout
+    exported = sorted(line.split()[-1] for line in out.splitlines() if line.strip())
+    assert exported == hip_lib.declared_symbols()
+
+
 def test_version_and_error_strings():
     lib = hip_lib.lib()
     assert lib.warpctct_version().decode().count(".") == 2

@@ -516,12 +516,15 @@ def test_lost_hand_over_never_yields_a_plausible_number():
         torch.cuda.synchronize()
         return c.detach().cpu().numpy(), x.grad.cpu().numpy()
 
+    warp_ctct.status(reset=True)
     default = lib.warpctct_lattice_wait_limit(0)
     try:
         assert default > 1000
         costs, grad = run()
     finally:
         assert lib.warpctct_lattice_wait_limit(-1) == 0
+    # the status word tells these NaN from NaN that came in with the inputs
+    assert warp_ctct.status() == warp_ctct.STATUS_LOST_HAND_OVER
     lost = np.isnan(costs)
     assert lost[[0, 1, 3, 4, 5]].any(), "no consumer ever caught up with its producer"
     assert not lost[2]                                   # 11 contexts: one wavefront, no hand-over
@@ -533,6 +536,7 @@ def test_lost_hand_over_never_yields_a_plausible_number():
             # (a finite cost with NaN in the gradient: only the alpha chain lost its input)
             np.testing.assert_allclose(grad[n], ref_dense[n], atol=GRAD_ATOL, rtol=0)
     costs, grad = run()
+    assert warp_ctct.status() == 0
     np.testing.assert_allclose(costs, ref_costs, rtol=LOSS_RTOL)
     np.testing.assert_allclose(grad, ref_dense, atol=GRAD_ATOL, rtol=0)
 
@@ -781,7 +785,29 @@ def test_label_range_check_is_opt_in():
     ys[0, 1] = 7                              # == V
     ys[1, 0] = -1
     x, d_ys, d_lx, d_ly = dev(joint), dev(ys), dev(lx), dev(ly)
+    warp_ctct.status(reset=True)
     assert torch.isfinite(warp_ctct.ctct_loss(x, d_ys, d_lx, d_ly, reduction="none")).all()
+    # without any synchronisation in the loss: the clamped labels are on record
+    assert warp_ctct.label_range_violated(reset=False)
+    assert warp_ctct.status(reset=True) & warp_ctct.STATUS_LABEL_RANGE
+    assert not warp_ctct.label_range_violated()
+    for bad, fn in ((7, warp_ctct.ctct_loss), (-1, warp_ctct.ctct_loss_with_logits)):
+        one = ys.copy()
+        one[0, 1], one[1, 0] = 1, 1
+        one[1, 2] = bad
+        fn(x, dev(one), d_lx, d_ly)
+        assert warp_ctct.label_range_violated(), (bad, fn.__name__)
+        assert not warp_ctct.label_range_violated()
+    one = ys.copy()
+    one[0, 1], one[1, 0] = 7, 1
+    warp_ctct.ctct_simple_loss(x[:, :, 0], x[:, 0], dev(one), d_lx, d_ly)
+    assert warp_ctct.label_range_violated()
+    # labels inside the range, also in the padding of short samples, leave no mark
+    one[0, 1] = 6
+    for fn in (warp_ctct.ctct_loss, warp_ctct.ctct_loss_with_logits):
+        fn(x, dev(one), d_lx, d_ly)
+    warp_ctct.ctct_simple_loss(x[:, :, 0], x[:, 0], dev(one), d_lx, d_ly)
+    assert warp_ctct.status() == 0
     warp_ctct.CHECK_LABEL_RANGE = True
     try:
         with pytest.raises(IndexError):
@@ -796,6 +822,33 @@ def test_label_range_check_is_opt_in():
         warp_ctct.CHECK_LABEL_RANGE = False
 
 
+def test_nan_input_is_reported_and_acts_as_log_zero():
+    """A NaN among the gathered log-probabilities: the unit counts as log 0
+    (the lattice's maximum drops NaN operands), so the cost is that of the same
+    joint with -inf in its place, and the status word says that it happened."""
+    import warp_ctct
+    joint, ys, lx, ly = make_joint_case(78, 2, 9, 4, 7)
+    t, u = 3, 2
+    col = int(ys[0, u - 1])
+    poisoned, masked = joint.copy(), joint.copy()
+    poisoned[0, t, u, col] = np.nan
+    masked[0, t, u, col] = -np.inf
+    warp_ctct.status(reset=True)
+    got = warp_ctct.ctct_loss(dev(poisoned), dev(ys), dev(lx), dev(ly), reduction="none")
+    ref = warp_ctct.ctct_loss(dev(masked), dev(ys), dev(lx), dev(ly), reduction="none")
+    assert warp_ctct.status(reset=False) & warp_ctct.STATUS_NAN_INPUT
+    assert warp_ctct.status() & warp_ctct.STATUS_NAN_INPUT and warp_ctct.status() == 0
+    np.testing.assert_array_equal(got.cpu().numpy(), ref.cpu().numpy())
+    _, _, want = O.ctct_loss(masked, ys, lx, ly, reduction="none")
+    np.testing.assert_allclose(got.cpu().numpy(), want, rtol=LOSS_RTOL)
+    # a NaN outside the gathered columns is never read
+    poisoned = joint.copy()
+    free = [v for v in range(1, 7) if v not in (int(ys[0, u - 1]), int(ys[0, u]))][0]
+    poisoned[0, t, u, free] = np.nan
+    warp_ctct.ctct_loss(dev(poisoned), dev(ys), dev(lx), dev(ly))
+    assert warp_ctct.status() == 0
+
+
 def test_infeasible_sample_has_infinite_cost():
     import warp_ctct
     joint, ys, lx, ly = make_joint_case(17, 2, 6, 3, 5, force_repeat=False)
@@ -806,6 +859,30 @@ def test_infeasible_sample_has_infinite_cost():
     _, _, ref = O.ctct_loss(joint, ys, lx, ly, reduction="none")
     assert np.isposinf(c[0]) and np.isposinf(ref[0])
     np.testing.assert_allclose(c[1], ref[1], rtol=LOSS_RTOL)
+    # Its gradient is NaN, as the reference's (csrc/gather.cu:339-340: the
+    # exponent holds -inf - (-inf) once the log-likelihood is -inf): at every
+    # gathered column of the cells that complete alignments could pass through,
+    # and nowhere else; the feasible sample beside it is not touched by that.
+    x = dev(joint).requires_grad_(True)
+    warp_ctct.ctct_loss(x, dev(ys), dev(lx), dev(ly), reduction="sum").backward()
+    got = x.grad.cpu().numpy()
+    _, ref_dense, _ = O.ctct_loss(joint, ys, lx, ly, reduction="sum")
+    np.testing.assert_allclose(got[1], ref_dense[1], atol=GRAD_ATOL, rtol=0)
+    expect_nan = np.zeros(got[0].shape, dtype=bool)
+    Tn, Un = int(lx[0]), int(ly[0])
+    for t in range(Tn):
+        for u in range(Un + 1):
+            if t < u or Tn - t < Un - u:          # outside the band: exactly zero
+                continue
+            expect_nan[t, u, 0] = True
+            if u >= 1:
+                expect_nan[t, u, ys[0, u - 1]] = True
+            if u < Un:
+                expect_nan[t, u, ys[0, u]] = True
+    assert expect_nan.any()
+    assert np.all(np.isnan(got[0][expect_nan])), "infeasible sample: gradient must be NaN"
+    assert np.all(got[0][~expect_nan] == 0)
+    assert np.all(np.isnan(ref_dense[0][expect_nan]))      # the float64 oracle agrees
 
 
 def test_committed_brute_force_vectors():

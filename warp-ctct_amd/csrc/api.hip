@@ -222,7 +222,7 @@ const char *warpctct_error_string(int code) {
     }
 }
 
-const char *warpctct_version(void) { return "0.1.0"; }
+const char *warpctct_version(void) { return "0.2.0"; }
 
 int warpctct_padded_contexts(int U) { return U < 0 ? 0 : padded_contexts(U); }
 

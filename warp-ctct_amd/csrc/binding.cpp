@@ -648,4 +648,13 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           pybind11::arg("grad_out"), pybind11::arg("lhs"), pybind11::arg("rhs"),
           pybind11::arg("res"), pybind11::arg("grad_masks"));
     m.def("library_version", []() { return std::string(warpctct_version()); });
+    m.def(
+        "status",
+        [](const bool clear) {
+            unsigned bits = 0;
+            check_rc(warpctct_status(&bits, clear ? 1 : 0), "status");
+            return static_cast<int64_t>(bits);
+        },
+        "Sticky status bits of the current device (synchronises with it).",
+        pybind11::arg("clear") = true);
 }

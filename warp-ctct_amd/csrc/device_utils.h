@@ -23,6 +23,20 @@ __device__ __forceinline__ void store_from_float(__hip_bfloat16 *p, float v) {
     *p = __float2bfloat16(v);
 }
 
+// A label as a column index: clamped into [0, V) so that a corrupt label cannot
+// make a kernel read outside its tensors.  `status` (may be null) is the
+// device's status word: a label that had to be clamped sets its label-range bit
+// there (the reference's torch.gather raises instead, warp_ctct/__init__.py:131).
+__device__ __forceinline__ int label_column(int y, int V, unsigned *status) {
+    const int c = min(max(y, 0), V - 1);
+    if (c != y && status) atomicOr(status, 1u);
+    return c;
+}
+// A gathered log-probability that is NaN is reported in the same word (bit 2).
+__device__ __forceinline__ void report_nan(float a, float b, float c, unsigned *status) {
+    if ((a != a || b != b || c != c) && status) atomicOr(status, 2u);
+}
+
 constexpr int kWave = 64;
 constexpr double kLog2e = 1.4426950408889634074;
 constexpr double kLn2 = 0.6931471805599453094;

@@ -242,7 +242,7 @@ static __device__ __forceinline__ unsigned slots_state(const unsigned long long 
 template <bool BETA, bool HAS_IN>
 static __device__ void sweep(const double *units_n, const int *y, int Tn, int Un, int T, int P, int wave,
                       double *lat_n, float *cost_n, const unsigned long long *slots_in,
-                      unsigned long long *slots_out, int max_spins) {
+                      unsigned long long *slots_out, int max_spins, unsigned *status) {
     const int lane = threadIdx.x & 63;
     const int u = wave * 64 + lane;
     double o_mask = 0.0;
@@ -374,6 +374,8 @@ static __device__ void sweep(const double *units_n, const int *y, int Tn, int Un
             // from them, and the cost if this is the end of the beta chain), and
             // the consumer, which has been waiting since, is told.
             f.e = f.o = __longlong_as_double(0x7ff8000000000000LL);
+            // (the device's status word tells this NaN from one that came in with the inputs)
+            if (status && lane == 0) atomicOr(status, kStatusLostHandOver);
             for (int s = lost_from; s < Tn; ++s)
                 front_store(out + (size_t)(BETA ? Tn - 1 - s : s + 1) * srow, f);
             if (slots_out && lane == edge_lane)
@@ -400,7 +402,8 @@ static __device__ __forceinline__ void lattice_block(const double *__restrict__ 
                                               float *__restrict__ costs,
                                               unsigned long long *__restrict__ relay, int N, int T,
                                               int U, int W, int dirs, int chains_pad,
-                                              const CostReduce &red, int max_spins) {
+                                              const CostReduce &red, int max_spins,
+                                              unsigned *status) {
     const int chain = blockIdx.x % chains_pad, link = blockIdx.x / chains_pad;
     if (chain >= N * dirs) return;
     const int n = chain / dirs;
@@ -425,15 +428,15 @@ static __device__ __forceinline__ void lattice_block(const double *__restrict__ 
     if (!beta) {
         const unsigned long long *in = wave > 0 ? slots_n + (size_t)(wave - 1) * TS : nullptr;
         unsigned long long *out = (wave + 1) * 64 <= Un ? slots_n + (size_t)wave * TS : nullptr;
-        if (in) sweep<false, true>(units_n, y, Tn, Un, T, P, wave, alphas + (size_t)n * lat, nullptr, in, out, max_spins);
-        else sweep<false, false>(units_n, y, Tn, Un, T, P, wave, alphas + (size_t)n * lat, nullptr, in, out, max_spins);
+        if (in) sweep<false, true>(units_n, y, Tn, Un, T, P, wave, alphas + (size_t)n * lat, nullptr, in, out, max_spins, status);
+        else sweep<false, false>(units_n, y, Tn, Un, T, P, wave, alphas + (size_t)n * lat, nullptr, in, out, max_spins, status);
         return;
     }
     {
         const unsigned long long *in = (wave + 1) * 64 <= Un ? slots_n + (size_t)wave * TS : nullptr;
         unsigned long long *out = wave > 0 ? slots_n + (size_t)(wave - 1) * TS : nullptr;
-        if (in) sweep<true, true>(units_n, y, Tn, Un, T, P, wave, betas + (size_t)n * lat, costs + n, in, out, max_spins);
-        else sweep<true, false>(units_n, y, Tn, Un, T, P, wave, betas + (size_t)n * lat, costs + n, in, out, max_spins);
+        if (in) sweep<true, true>(units_n, y, Tn, Un, T, P, wave, betas + (size_t)n * lat, costs + n, in, out, max_spins, status);
+        else sweep<true, false>(units_n, y, Tn, Un, T, P, wave, betas + (size_t)n * lat, costs + n, in, out, max_spins, status);
     }
     if (wave != 0) return;
     // thread 0 (context 0) has just written costs[n]
@@ -472,9 +475,10 @@ __global__ __launch_bounds__(64) void lattice_kernel(const double *__restrict__ 
                                                      float *__restrict__ costs,
                                                      unsigned long long *__restrict__ relay, int N,
                                                      int T, int U, int W, int dirs, int chains_pad,
-                                                     const CostReduce red, int max_spins) {
+                                                     const CostReduce red, int max_spins,
+                                                     unsigned *__restrict__ status) {
     Chunked<12>::lattice_block(units, ys, lx, ly, alphas, betas, costs, relay, N, T, U, W, dirs,
-                               chains_pad, red, max_spins);
+                               chains_pad, red, max_spins, status);
 }
 
 // The same sweeps with a memory clear riding along: workgroups of 256 threads,
@@ -487,8 +491,8 @@ __global__ __launch_bounds__(256) void lattice_fill_kernel(
     const double *__restrict__ units, const int *__restrict__ ys, const int *__restrict__ lx,
     const int *__restrict__ ly, double *__restrict__ alphas, double *__restrict__ betas,
     float *__restrict__ costs, unsigned long long *__restrict__ relay, int N, int T, int U, int W,
-    int dirs, int chains_pad, const CostReduce red, int max_spins, v4f_fill *__restrict__ fill,
-    size_t n4, unsigned lattice_blocks) {
+    int dirs, int chains_pad, const CostReduce red, int max_spins, unsigned *__restrict__ status,
+    v4f_fill *__restrict__ fill, size_t n4, unsigned lattice_blocks) {
     if (blockIdx.x >= lattice_blocks) {
         const size_t i = (size_t)(blockIdx.x - lattice_blocks) * 256 + threadIdx.x;
         if (i < n4) fill[i] = v4f_fill{0.0f, 0.0f, 0.0f, 0.0f};
@@ -496,7 +500,7 @@ __global__ __launch_bounds__(256) void lattice_fill_kernel(
     }
     if (threadIdx.x >= 64) return;
     Chunked<8>::lattice_block(units, ys, lx, ly, alphas, betas, costs, relay, N, T, U, W, dirs,
-                              chains_pad, red, max_spins);
+                              chains_pad, red, max_spins, status);
 }
 
 }  // namespace
@@ -533,6 +537,7 @@ hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream) {
         relay = nullptr;
     }
     const int max_spins = g_wait_limit.load(std::memory_order_relaxed);
+    unsigned *status = W > 1 ? device_status_word() : nullptr;   // only chains can lose a hand-over
     const int dirs = a.beta_only ? 1 : 2;
     const long chains = (long)a.N * dirs;
     const long chains_pad = (chains + 7) / 8 * 8;
@@ -542,13 +547,13 @@ hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream) {
         if (blocks > 0x7fffffffUL) return hipErrorInvalidValue;
         TIMED_LAUNCH(lattice_fill_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a.units,
                      a.ys, a.lx, a.ly, a.alphas, a.betas, a.costs, relay, a.N, a.T, a.U, W, dirs,
-                     (int)chains_pad, a.reduce, max_spins, static_cast<v4f_fill *>(a.fill.p), a.fill.n4,
+                     (int)chains_pad, a.reduce, max_spins, status, static_cast<v4f_fill *>(a.fill.p), a.fill.n4,
                      (unsigned)(chains_pad * W));
         return hipGetLastError();
     }
     TIMED_LAUNCH(lattice_kernel, dim3((unsigned)(chains_pad * W)), dim3(64), 0, stream, a.units,
                  a.ys, a.lx, a.ly, a.alphas, a.betas, a.costs, relay, a.N, a.T, a.U, W, dirs,
-                 (int)chains_pad, a.reduce, max_spins);
+                 (int)chains_pad, a.reduce, max_spins, status);
     return hipGetLastError();
 }
 

@@ -19,6 +19,14 @@ enum IoType { kIoF32 = 0, kIoF16 = 1, kIoBF16 = 2 };
 inline size_t io_size(int t) { return t == kIoF32 ? 4 : 2; }
 inline bool io_valid(int t) { return t == kIoF32 || t == kIoF16 || t == kIoBF16; }
 
+// Bits of the device's sticky status word (WARPCTCT_STATUS_* of the C ABI).
+constexpr unsigned kStatusLabelRange = 1u;     // a label outside [0, V) was clamped
+constexpr unsigned kStatusNanInput = 2u;       // a gathered log-probability was NaN
+constexpr unsigned kStatusLostHandOver = 4u;   // a chain of workgroups gave up waiting
+// The current device's status word, for kernels to set bits in (atomic OR), or
+// null when it cannot be found (kernels then report nothing).
+unsigned *device_status_word();
+
 // Reduction over the batch folded into the lattice kernel: the workgroup that
 // finishes last (counted in *counter, which must be 0 at launch) adds up the N
 // costs in a fixed order.  mode 0 = none, 1 = sum, 2 = mean.

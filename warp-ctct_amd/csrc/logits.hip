@@ -163,7 +163,7 @@ __global__ __launch_bounds__(64 * kRowsPerBlock)
     logits_units_kernel(const IO *__restrict__ logits, const int *__restrict__ ys,
                     const int *__restrict__ lx, const int *__restrict__ ly,
                     double *__restrict__ units, float *__restrict__ lse, int T, int U, int V, int P,
-                    unsigned *__restrict__ counter) {
+                    unsigned *__restrict__ counter, unsigned *__restrict__ status) {
     constexpr int EV = 16 / (int)sizeof(IO);    // elements per 16-byte vector
     constexpr int NV = 1024 / (64 * EV);        // vectors per lane and round of 1024 elements
     if (counter && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *counter = 0u;
@@ -203,6 +203,14 @@ __global__ __launch_bounds__(64 * kRowsPerBlock)
         if (lane != 0) return;
         const float l = M + log2_hw(S) * kLn2F;   // natural-log logsumexp of the row
         lse_out[u] = l;
+        // what the status word reports: a label that had to be clamped into [0, V)
+        // on its way to a column index, a NaN among the values that become units
+        if (status) {
+            const bool bad = (u >= 1 && (unsigned)y[u - 1] >= (unsigned)V) ||
+                             (u < Un && (unsigned)y[u] >= (unsigned)V);
+            if (bad) atomicOr(status, 1u);
+            report_nan(xb - l, u >= 1 ? x1 : 0.0f, u < Un ? x2 : 0.0f, status);
+        }
         double *o = frame_out + (size_t)u * 3;
         const double b = (double)xb - (double)l;
         double cur = b, nxt = neg_inf();
@@ -445,11 +453,11 @@ void launch_units_typed(const void *logits, const int *ys, const int *lx, const 
     if (staged <= 64 * 1024) {
         TIMED_LAUNCH((logits_units_kernel<IO, true>), dim3((unsigned)T, (unsigned)N),
                      dim3(64 * kRowsPerBlock), staged, stream, static_cast<const IO *>(logits), ys,
-                     lx, ly, units, lse, T, U, V, P, counter);
+                     lx, ly, units, lse, T, U, V, P, counter, device_status_word());
     } else {   // a frame too wide for LDS: results stored row by row
         TIMED_LAUNCH((logits_units_kernel<IO, false>), dim3((unsigned)T, (unsigned)N),
                      dim3(64 * kRowsPerBlock), 0, stream, static_cast<const IO *>(logits), ys, lx,
-                     ly, units, lse, T, U, V, P, counter);
+                     ly, units, lse, T, U, V, P, counter, device_status_word());
     }
 }
 

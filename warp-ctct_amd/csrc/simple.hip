@@ -37,7 +37,7 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     const float *__restrict__ f, const float *__restrict__ g, float *__restrict__ den,
     const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
     double *__restrict__ units, int T, int U, int V, int P, const RelaySlots relay,
-    const LogmmDeferred deferred, float *__restrict__ fmax) {
+    const LogmmDeferred deferred, float *__restrict__ fmax, unsigned *__restrict__ status) {
     relay_clear_share(relay);
     const int U1 = U + 1;
     const int n = blockIdx.y;
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     const int *y = ys + (size_t)n * U;
     // the next label's column: wanted by this cell or by the cell of context u+1
     const bool has2 = u < Un;
-    const int c2 = has2 ? clampi(y[u], 0, V - 1) : 0;
+    const int c2 = has2 ? label_column(y[u], V, status) : 0;
     const bool wanted = has2 && (live || !outside_band(t, u + 1, Tn, Un));
     const float f2 = wanted ? fr[c2] : 0.0f;
     float f1 = __shfl_up(f2, 1, 64);
@@ -87,6 +87,7 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     double cur = b, nxt = neg_inf();
     if (u >= 1) cur = (double)f1 + (double)gr[c1] - d;
     if (has2) nxt = ((double)f2 + (double)gr[c2] - d) * kLog2e;
+    report_nan((float)b, (float)cur, has2 ? (float)nxt : 0.0f, status);
     o[0] = b * kLog2e;
     o[1] = cur * kLog2e;
     o[2] = nxt;
@@ -375,10 +376,10 @@ hipError_t launch_simple_gather_units(const float *f, const float *g, float *den
             deferred.Nn != U + 1)
             return hipErrorInvalidValue;
         TIMED_LAUNCH(simple_gather_units_kernel<true>, grid, dim3(kBlock), 0, stream, f, g, den, ys,
-                     lx, ly, units, T, U, V, P, relay, deferred, fmax);
+                     lx, ly, units, T, U, V, P, relay, deferred, fmax, device_status_word());
     } else {
         TIMED_LAUNCH(simple_gather_units_kernel<false>, grid, dim3(kBlock), 0, stream, f, g, den, ys,
-                     lx, ly, units, T, U, V, P, relay, deferred, fmax);
+                     lx, ly, units, T, U, V, P, relay, deferred, fmax, device_status_word());
     }
     return hipGetLastError();
 }

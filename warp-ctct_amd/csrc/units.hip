@@ -89,7 +89,8 @@ template <bool BAND_ONLY, typename IO>
 __global__ __launch_bounds__(kCellBlock) void gather_units_kernel(
     const IO *__restrict__ joint, const JointStrides js, const int *__restrict__ ys,
     const int *__restrict__ lx, const int *__restrict__ ly, double *__restrict__ units, int T,
-    int U, int V, int P, unsigned *__restrict__ counter, const RelaySlots relay) {
+    int U, int V, int P, unsigned *__restrict__ counter, const RelaySlots relay,
+    unsigned *__restrict__ status) {
     if (counter && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *counter = 0u;
     relay_clear_share(relay);
     Cell c = locate_cell(lx, ly, T, U, P);
@@ -100,8 +101,9 @@ __global__ __launch_bounds__(kCellBlock) void gather_units_kernel(
     const float b = nt_load(row);
     float cur = b, nxt = b;   // the reference gathers index 0 where no label exists
     // labels are clamped into [0,V) so that a corrupt label cannot fault
-    if (c.u >= 1) cur = nt_load(row + (long)min(max(y[c.u - 1], 0), V - 1) * js.v);
-    if (c.u < c.Un) nxt = nt_load(row + (long)min(max(y[c.u], 0), V - 1) * js.v);
+    if (c.u >= 1) cur = nt_load(row + (long)label_column(y[c.u - 1], V, status) * js.v);
+    if (c.u < c.Un) nxt = nt_load(row + (long)label_column(y[c.u], V, status) * js.v);
+    report_nan(b, cur, nxt, status);
     store_units(units, c, T, P, b, cur, nxt);
 }
 
@@ -169,12 +171,13 @@ void launch_gather_typed(const void *joint, const JointStrides &js, const int *y
                          unsigned *counter, const RelaySlots &relay, hipStream_t stream) {
     const int P = padded_contexts(U);
     const IO *j = static_cast<const IO *>(joint);
+    unsigned *status = device_status_word();
     if (band_only) {
         TIMED_LAUNCH((gather_units_kernel<true, IO>), cell_grid(N, T, P), dim3(kCellBlock),
-                           0, stream, j, js, ys, lx, ly, units, T, U, V, P, counter, relay);
+                           0, stream, j, js, ys, lx, ly, units, T, U, V, P, counter, relay, status);
     } else {
         TIMED_LAUNCH((gather_units_kernel<false, IO>), cell_grid(N, T, P), dim3(kCellBlock),
-                           0, stream, j, js, ys, lx, ly, units, T, U, V, P, counter, relay);
+                           0, stream, j, js, ys, lx, ly, units, T, U, V, P, counter, relay, status);
     }
 }
 

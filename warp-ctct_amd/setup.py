@@ -16,6 +16,13 @@ from setuptools import setup
 from torch.utils.cpp_extension import BuildExtension, CppExtension
 
 HERE = os.path.dirname(os.path.abspath(__file__))
+
+# The distribution carries the version of the reference distribution whose API
+# it implements (setup.py:18 of the reference: 0.3.0), so that code gating on
+# warp_ctct.__version__ behaves the same; the kernel library's own ABI version
+# (warpctct_version()) is separate.
+with open(os.path.join(HERE, "warp_ctct", "_version.py")) as fh:
+    VERSION = fh.read().split('"')[1]
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 
@@ -38,7 +45,7 @@ ext = CppExtension(
 
 setup(
     name="warp_ctct",
-    version="0.1.0",
+    version=VERSION,
     description="MI355X (gfx950) CTC-Transducer loss with the warp_ctct API",
     packages=["warp_ctct"],
     # the HIP kernels + C ABI travel with the package, next to the binding that

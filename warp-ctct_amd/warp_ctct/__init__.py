@@ -22,18 +22,25 @@ except ImportError as exc:  # pragma: no cover - exercised only on a broken inst
         "(needs hipcc, --offload-arch=gfx950)"
     ) from exc
 
-__all__ = ["ctct_loss", "ctct_loss_compact", "ctct_loss_with_logits", "ctct_simple_loss"]
+# The reference exports exactly these two (warp_ctct/__init__.py:17), so that
+# `from warp_ctct import *` binds the same names.  ctct_loss_with_logits,
+# ctct_loss_compact and label_range_violated are additions of this build and are
+# reached by name (warp_ctct.ctct_loss_with_logits, ...).
+__all__ = ["ctct_loss", "ctct_simple_loss"]
 
 
 def _package_version():
     """Version of the installed distribution (the reference reads it the same
-    way, warp_ctct/__init__.py:14); the library's own version string when the
-    package is used from a source tree without distribution metadata."""
+    way, warp_ctct/__init__.py:14), which is the reference distribution's 0.3.0;
+    the same string from _version.py when the package is used from a source tree
+    without distribution metadata.  The kernel library has an ABI version of its
+    own: warp_ctct._C.library_version()."""
     try:
         from importlib.metadata import version
         return version("warp_ctct")
     except Exception:
-        return core.library_version()
+        from ._version import __version__ as source_version
+        return source_version
 
 
 __version__ = _package_version()
@@ -60,10 +67,43 @@ CLEAR_GRADIENT_IN_FORWARD = True
 
 # The kernels clamp labels into [0, V) before they use them as column indices,
 # so that a corrupt label cannot make the GPU fault; the reference's
-# torch.gather raises on such an index (warp_ctct/__init__.py:131).  Set this
-# to True to get that behaviour back while debugging a data pipeline: every
-# call then checks its labels on the host (one device-to-host synchronisation).
+# torch.gather raises on such an index (warp_ctct/__init__.py:131).  A clamped
+# label is recorded on the device and shows up in label_range_violated() /
+# status() without any synchronisation in the loss itself.  Set this to True to
+# get the reference's behaviour back while debugging a data pipeline: every call
+# then checks its labels on the host (one device-to-host synchronisation).
 CHECK_LABEL_RANGE = False
+
+
+STATUS_LABEL_RANGE, STATUS_NAN_INPUT, STATUS_LOST_HAND_OVER = 1, 2, 4
+
+
+def status(reset: bool = True, device=None) -> int:
+    """Sticky status bits of a GPU (the current one by default), set by the
+    kernels of every call since the last reset:
+
+    * ``STATUS_LABEL_RANGE``: a label outside [0, V) was met and clamped (the
+      reference raises for it, warp_ctct/__init__.py:131);
+    * ``STATUS_NAN_INPUT``: a gathered log-probability was NaN (the lattice
+      treats such a unit as log 0);
+    * ``STATUS_LOST_HAND_OVER``: a lattice was not swept to its end (its costs
+      and gradients are NaN by construction, not because of the inputs).
+
+    Nothing in ``ctct_loss`` / ``ctct_simple_loss`` synchronises with the host;
+    this call does (it waits for the device), so use it where a pipeline would
+    check anyway: once per epoch, or when a loss looks wrong."""
+    if device is None:
+        return int(core.status(bool(reset)))
+    with torch.cuda.device(device):
+        return int(core.status(bool(reset)))
+
+
+def label_range_violated(reset: bool = True, device=None) -> bool:
+    """True if any call since the last reset met a label outside [0, V)."""
+    bits = status(reset=False, device=device)
+    if reset and bits & STATUS_LABEL_RANGE:
+        status(reset=True, device=device)
+    return bool(bits & STATUS_LABEL_RANGE)
 
 
 def _check_labels(labels, vocabulary):
@@ -293,6 +333,15 @@ def ctct_loss(log_probs: torch.Tensor,
         labels_lengths: (N,) number of labels of each sample.
         reduction: 'none' | 'mean' | 'sum' (None behaves like 'none').
         average_frames: divide each sample's loss by its number of frames.
+
+    Memory: when ``log_probs`` requires a gradient, the forward allocates the
+    gradient's buffer (the shape and type of ``log_probs``: 2 GB for a
+    (32, 250, 61, 1024) float32 joint) and clears it beside the lattice sweeps;
+    the buffer lives until the backward has run or the graph is freed.  Code
+    that evaluates several losses before one backward holds one such buffer per
+    loss; ``warp_ctct.CLEAR_GRADIENT_IN_FORWARD = False`` allocates and clears
+    it in the backward instead, as the reference's autograd does (one more
+    launch per step).
     """
     assert average_frames is None or isinstance(average_frames, bool)
     assert reduction is None or reduction in ("none", "mean", "sum")
