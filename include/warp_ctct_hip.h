@@ -420,9 +420,12 @@ int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, lo
  * is recorded instead in a sticky word on the device, one per GPU:
  *   WARPCTCT_STATUS_LABEL_RANGE    a label outside [0, V) was clamped into it
  *                                  before it was used as a column index;
- *   WARPCTCT_STATUS_NAN_INPUT      a gathered log-probability was NaN (the
- *                                  lattice treats such a unit as -inf: the
- *                                  hardware's maximum drops NaN operands);
+ *   WARPCTCT_STATUS_NAN_INPUT      a gathered log-probability was NaN; it
+ *                                  entered the lattice as log 0 (-inf), so the
+ *                                  cost is that of the joint with that entry
+ *                                  masked, not NaN as in the reference, whose
+ *                                  logaddexpf_ (csrc/gather.cu:23-34) lets a
+ *                                  NaN through;
  *   WARPCTCT_STATUS_LOST_HAND_OVER a chain of workgroups gave up waiting for a
  *                                  hand-over (see warpctct_lattice_f32): the NaN
  *                                  costs / gradients of that call do not come

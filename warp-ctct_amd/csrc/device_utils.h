@@ -32,9 +32,13 @@ __device__ __forceinline__ int label_column(int y, int V, unsigned *status) {
     if (c != y && status) atomicOr(status, 1u);
     return c;
 }
-// A gathered log-probability that is NaN is reported in the same word (bit 2).
-__device__ __forceinline__ void report_nan(float a, float b, float c, unsigned *status) {
-    if ((a != a || b != b || c != c) && status) atomicOr(status, 2u);
+// A gathered log-probability that is NaN becomes log 0 (-inf) before it enters
+// the lattice, whose maximum would otherwise drop it in one place and let it
+// erase a state in another, and is reported in the same word (bit 2).
+__device__ __forceinline__ float unit_or_log_zero(float x, unsigned *status) {
+    if (x == x) return x;
+    if (status) atomicOr(status, 2u);
+    return -__builtin_huge_valf();
 }
 
 constexpr int kWave = 64;

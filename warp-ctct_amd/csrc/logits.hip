@@ -209,13 +209,21 @@ __global__ __launch_bounds__(64 * kRowsPerBlock)
             const bool bad = (u >= 1 && (unsigned)y[u - 1] >= (unsigned)V) ||
                              (u < Un && (unsigned)y[u] >= (unsigned)V);
             if (bad) atomicOr(status, 1u);
-            report_nan(xb - l, u >= 1 ? x1 : 0.0f, u < Un ? x2 : 0.0f, status);
         }
         double *o = frame_out + (size_t)u * 3;
         const double b = (double)xb - (double)l;
         double cur = b, nxt = neg_inf();
         if (u >= 1) cur = (double)x1 - (double)l;
         if (u < Un) nxt = ((double)x2 - (double)l) * kLog2e;
+        // a NaN unit (a NaN anywhere in the row makes its logsumexp NaN) enters the
+        // lattice as log 0 and is reported
+        if (b != b || cur != cur || nxt != nxt) {
+            if (status) atomicOr(status, kStatusNanInput);
+            o[0] = (b != b) ? neg_inf() : b * kLog2e;
+            o[1] = (cur != cur) ? neg_inf() : cur * kLog2e;
+            o[2] = (nxt != nxt) ? neg_inf() : nxt;
+            return;
+        }
         o[0] = b * kLog2e;
         o[1] = cur * kLog2e;
         o[2] = nxt;

@@ -87,7 +87,14 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     double cur = b, nxt = neg_inf();
     if (u >= 1) cur = (double)f1 + (double)gr[c1] - d;
     if (has2) nxt = ((double)f2 + (double)gr[c2] - d) * kLog2e;
-    report_nan((float)b, (float)cur, has2 ? (float)nxt : 0.0f, status);
+    // a NaN unit (NaN in f, g or den) enters the lattice as log 0 and is reported
+    if (b != b || cur != cur || nxt != nxt) {
+        if (status) atomicOr(status, kStatusNanInput);
+        o[0] = (b != b) ? neg_inf() : b * kLog2e;
+        o[1] = (cur != cur) ? neg_inf() : cur * kLog2e;
+        o[2] = (nxt != nxt) ? neg_inf() : nxt;
+        return;
+    }
     o[0] = b * kLog2e;
     o[1] = cur * kLog2e;
     o[2] = nxt;

@@ -103,8 +103,8 @@ __global__ __launch_bounds__(kCellBlock) void gather_units_kernel(
     // labels are clamped into [0,V) so that a corrupt label cannot fault
     if (c.u >= 1) cur = nt_load(row + (long)label_column(y[c.u - 1], V, status) * js.v);
     if (c.u < c.Un) nxt = nt_load(row + (long)label_column(y[c.u], V, status) * js.v);
-    report_nan(b, cur, nxt, status);
-    store_units(units, c, T, P, b, cur, nxt);
+    store_units(units, c, T, P, unit_or_log_zero(b, status), unit_or_log_zero(cur, status),
+                unit_or_log_zero(nxt, status));
 }
 
 __global__ __launch_bounds__(kCellBlock) void scale_units_kernel(
