@@ -35,7 +35,7 @@ MFMA_FP32_PEAK_TFLOPS = 157.3   # MI355X dense fp32 matrix, published
 # FETCH_SIZE 9 710.3 KiB x 2.0, the factors being what the same counters read
 # for a plain 1 GiB -> 1 GiB elementwise kernel (WRITE_SIZE 1 048 576,
 # FETCH_SIZE 524 300 KiB).
-LATTICE_FILL_TRAFFIC_BYTES = 1964748 * 1024 + int(9724.4 * 2 * 1024)
+LATTICE_FILL_TRAFFIC_BYTES = 1964748 * 1024 + int(9710.3 * 2 * 1024)
 
 
 def make_batch(torch, N, T, U, V, seed=2024):
@@ -140,6 +140,9 @@ OTHER = {
     "c2_logits_bf16": ("logits", 32, 250, 60, 1024, 1.0),
     "c2_logits_f16": ("logits", 32, 250, 60, 1024, 1.0),
     "c2_logits_unfused": ("logits_unfused", 32, 250, 60, 1024, 1.0),
+    # the typical batch handed over in compact form: costs and the (N,T,U+1,3) unit
+    # gradients of ctct_loss_compact, no dense gradient at all
+    "c2_compact": ("compact", 32, 250, 60, 1024, 1.0),
 }
 IO_DTYPE = {"c2_bf16": "bfloat16", "c2_f16": "float16", "c2_logits_bf16": "bfloat16",
             "c2_logits_f16": "float16"}
@@ -149,6 +152,10 @@ WORKLOAD = {
     "c3": "ctct_loss fp32, large vocabulary / long lattice: N=8, lx in [400,500], ly in [80,120], V=4096, N(0,2) logits",
     "c4": "ctct_simple_loss fp32 normalized (log-add joiner): N=32, lx in [300,400], ly in [50,80], V=2048",
     "c5": "ctct_simple_loss fp32 unnormalized, long-utterance stress: N=4, lx in [1200,1500], ly in [250,300], V=8192",
+    "c2_bf16": "ctct_loss on a bfloat16 joint (gradient written in bfloat16), typical ASR batch: N=32, lx in [150,250], ly in [30,60], V=1024",
+    "c2_logits": "ctct_loss_with_logits on fp32 logits (log_softmax and its backward inside), typical ASR batch: N=32, lx in [150,250], ly in [30,60], V=1024",
+    "c2_logits_bf16": "ctct_loss_with_logits on bfloat16 logits, typical ASR batch: N=32, lx in [150,250], ly in [30,60], V=1024",
+    "c2_compact": "ctct_loss_compact on the fp32 joint (costs + unit gradients (N,T,U+1,3), no dense gradient), typical ASR batch: N=32, lx in [150,250], ly in [30,60], V=1024",
 }
 
 
@@ -172,8 +179,11 @@ def build_config(name, torch, warp_ctct):
     ys[:, 3] = ys[:, 2]
     d_ys, d_lx, d_ly = (torch.as_tensor(a).cuda() for a in (ys, lx, ly))
     live = int(sum(int(a) * (int(b) + 1) for a, b in zip(lx, ly)))
+    # cells that a complete alignment can pass through: t >= u and lx - t >= ly - u
+    band = int(sum(sum(max(0, min(int(b), t) - max(0, int(b) - (int(a) - t)) + 1) for t in range(int(a)))
+                   for a, b in zip(lx, ly)))
     facts = {"kind": kind, "N": N, "T": T, "U": U, "V": V, "max_frames": int(lx.max()),
-             "live_cells": live}
+             "live_cells": live, "band_cells": band}
     if kind == "full":
         joint = torch.randn(N, T, U + 1, V, device="cuda", generator=gen).mul_(sigma).log_softmax(-1)
         t_idx = torch.arange(T, device="cuda")[None, :, None, None]
@@ -188,6 +198,15 @@ def build_config(name, torch, warp_ctct):
 
         def loss_fn():
             return warp_ctct.ctct_loss(joint, d_ys, d_lx, d_ly)
+    elif kind == "compact":
+        joint = torch.randn(N, T, U + 1, V, device="cuda", generator=gen).log_softmax(-1)
+        # algorithmic bytes: three gathered reads and three unit gradients per cell
+        facts["algorithmic_bytes_per_step"] = 12 * live + 12 * N * T * (U + 1) + 4 * N * (U + 3)
+
+        def step():
+            return warp_ctct.ctct_loss_compact(joint, d_ys, d_lx, d_ly)
+
+        return step, facts
     elif kind in ("logits", "logits_unfused"):
         io = getattr(torch, IO_DTYPE.get(name, "float32"))
         logits = torch.randn(N, T, U + 1, V, device="cuda", generator=gen).mul_(3.0).to(io)
@@ -195,6 +214,8 @@ def build_config(name, torch, warp_ctct):
         leaves = (logits,)
         # algorithmic bytes: live rows read twice (forward, backward), gradient written once
         facts["algorithmic_bytes_per_step"] = logits.element_size() * V * (2 * live + N * T * (U + 1))
+        # the backward's kernel: rows inside the band read, every row written
+        facts["logits_grad_bytes"] = logits.element_size() * V * (band + N * T * (U + 1))
 
         if kind == "logits":
             def loss_fn():
@@ -255,7 +276,15 @@ def summarise(name, facts, sec_per_step, kernels):
         out["lattice_kernel_us"] = lattice
         out["lattice_ns_per_frame"] = lattice * 1e3 / facts["max_frames"]
     fill = us.get("lattice_fill_kernel")
-    if name == "c1" or facts["kind"] == "simple_unnorm":
+    grad_us = sum(v for k, v in us.items() if k.startswith("logits_grad_kernel"))
+    if facts["kind"] == "logits" and grad_us > 0:
+        gbs = facts["logits_grad_bytes"] / (grad_us * 1e-6) / 1e9
+        out["roofline"] = {"bound": "hbm", "kernel": "logits_grad_kernel (rows inside the band of "
+                           "complete alignments read, every row of the gradient written)",
+                           "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": gbs / HBM_PEAK_GBS, "avg_launch_us": grad_us,
+                           "algorithmic_bytes_per_launch": facts["logits_grad_bytes"]}
+    elif name == "c1" or facts["kind"] in ("simple_unnorm", "compact"):
         out["roofline"] = {"bound": "latency", "kernel": "lattice_kernel",
                            "note": "serial recursion over max_frames dependent steps; reported as "
                                    "ns per frame, an HBM fraction would be structurally low",
@@ -436,7 +465,12 @@ def main():
         configs = {"c2": {"workload": WORKLOAD["c2"], "ms_per_step": ms_per_step,
                           "kernel_us_per_step": {k: round(v["us_per_step"], 2) for k, v in sorted(
                               kernels.items(), key=lambda kv: -kv[1]["us_per_step"])}}}
-        for name, steps in (("c1", 50), ("c3", 8), ("c4", 20), ("c5", 20)):
+        for name, steps in (("c1", 50), ("c3", 8), ("c4", 20), ("c5", 20), ("c2_bf16", 20),
+                            ("c2_logits", 10), ("c2_logits_bf16", 10), ("c2_compact", 30)):
+            # (this batch's tensors go before the next configuration's are made: c3 alone holds 16 GB)
+            if name == "c1":
+                del joint, loss, grad, step
+                torch.cuda.empty_cache()
             configs[name] = measure_config(name, torch, warp_ctct, steps)
         result["configs"] = configs
     print(json.dumps(result))

@@ -7,7 +7,8 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_SO = os.path.join(_HERE, "libctct_oracle.so")
+# (CTCT_ORACLE_LIB: another build of the same sources, e.g. with sanitizers)
+_SO = os.environ.get("CTCT_ORACLE_LIB") or os.path.join(_HERE, "libctct_oracle.so")
 _lib = None
 
 

@@ -5,7 +5,10 @@ import os
 import re
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LIB_PATH = os.path.join(ROOT, "warp-ctct_amd", "warp_ctct", "libwarpctct_hip.so")
+# (WARPCTCT_HIP_LIB: another build of the same library, e.g. one whose host code
+# is compiled with sanitizers: tests/run_host_sanitizers.sh)
+LIB_PATH = os.environ.get("WARPCTCT_HIP_LIB") or os.path.join(
+    ROOT, "warp-ctct_amd", "warp_ctct", "libwarpctct_hip.so")
 HEADER = os.path.join(ROOT, "include", "warp_ctct_hip.h")
 
 
