@@ -133,9 +133,11 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor> ctct_loss_joint_fwd(
 
     auto ws = make_workspace(joint, N, T, U);
     const auto f32 = joint.options().dtype(at::ScalarType::Float);
-    auto costs = torch::empty({N}, f32);
+    // the per-sample costs and the reduced scalar share one allocation
+    auto costs_and_sum = N > 0 ? torch::empty({N + 1}, f32) : torch::zeros({1}, f32);
+    auto costs = costs_and_sum.narrow(0, 0, N);
     torch::Tensor reduced;
-    if (reduction != 0) reduced = N > 0 ? torch::empty({}, f32) : torch::zeros({}, f32);
+    if (reduction != 0) reduced = costs_and_sum.select(0, N);
     const long strides[4] = {static_cast<long>(joint.stride(0)), static_cast<long>(joint.stride(1)),
                              static_cast<long>(joint.stride(2)), static_cast<long>(joint.stride(3))};
     // With clear_gradient the buffer of the dense gradient is allocated now and
@@ -253,9 +255,10 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_loss_logits_fwd(const torch::Tenso
     const DeviceGuard device_guard(device_of(logits));
     auto ws = make_bytes(logits, warpctct_logits_workspace_bytes(N, T, U));
     const auto f32 = logits.options().dtype(at::ScalarType::Float);
-    auto costs = torch::empty({N}, f32);
+    auto costs_and_sum = N > 0 ? torch::empty({N + 1}, f32) : torch::zeros({1}, f32);
+    auto costs = costs_and_sum.narrow(0, 0, N);
     torch::Tensor reduced;
-    if (reduction != 0) reduced = N > 0 ? torch::empty({}, f32) : torch::zeros({}, f32);
+    if (reduction != 0) reduced = costs_and_sum.select(0, N);
     check_rc(warpctct_logits_loss_lattice(logits.data_ptr(), dtype, ys.data_ptr<int>(),
                                           lx.data_ptr<int>(), ly.data_ptr<int>(), N, T, U, V,
                                           ws.data_ptr(), ws.numel(), costs.data_ptr<float>(),
@@ -592,9 +595,190 @@ std::tuple<torch::Tensor, torch::Tensor> log_matmul_backward(
     return std::make_tuple(grad_lhs, grad_rhs);
 }
 
+// ---- the public losses as autograd functions -------------------------------
+// One crossing from Python into this module per direction: the forward below
+// is what warp_ctct.ctct_loss calls, and autograd calls the backward here
+// without going through Python.  They are the counterpart of the reference's
+// gather + CTCTLoss + reduction (warp_ctct/__init__.py:124-147), of its
+// SimpleCTCTLoss / LogMMExp chain (:55-85, :36-52, :195-225) and of the caller's
+// log_softmax in front of ctct_loss.
+
+// labels and lengths as contiguous int32 (the reference casts with .int(),
+// warp_ctct/__init__.py:135-136); tensors that already are cost nothing
+torch::Tensor as_int32(const torch::Tensor &t) {
+    if (t.scalar_type() == at::ScalarType::Int && t.is_contiguous()) return t;
+    return t.to(at::ScalarType::Int).contiguous();
+}
+
+torch::Tensor upstream(const torch::Tensor &grad_output) {
+    return grad_output.reshape({-1}).to(at::ScalarType::Float).contiguous();
+}
+
+using torch::autograd::AutogradContext;
+using torch::autograd::tensor_list;
+
+class JointLoss : public torch::autograd::Function<JointLoss> {
+   public:
+    static torch::Tensor forward(AutogradContext *ctx, const torch::Tensor &joint,
+                                 const torch::Tensor &ys, const torch::Tensor &lx,
+                                 const torch::Tensor &ly, const bool requires_grad,
+                                 const int64_t reduction, const bool average_frames,
+                                 const bool clear_in_forward) {
+        auto out = ctct_loss_joint_fwd(joint, ys, lx, ly, requires_grad, reduction, average_frames,
+                                       requires_grad && clear_in_forward);
+        if (requires_grad) {
+            ctx->save_for_backward({std::get<1>(out), ys, lx, ly});
+            // the buffer of the dense gradient, cleared beside the lattices: it
+            // serves the first backward; a later one (retained graph) clears its own
+            ctx->saved_data["dense"] = std::get<2>(out);
+            ctx->saved_data["like"] = torch::empty({0}, joint.options());
+            ctx->saved_data["sizes"] = joint.sizes().vec();
+            ctx->saved_data["scale"] = reduction == 2 ? 1.0 / static_cast<double>(joint.size(0)) : 1.0;
+            ctx->saved_data["average_frames"] = average_frames;
+        }
+        return std::get<0>(out);
+    }
+
+    static tensor_list backward(AutogradContext *ctx, tensor_list grad_outputs) {
+        const auto saved = ctx->get_saved_variables();
+        const auto sizes = ctx->saved_data["sizes"].toIntVector();
+        torch::Tensor dense = ctx->saved_data["dense"].toTensor();
+        ctx->saved_data["dense"] = torch::empty({0}, dense.options());
+        if (dense.numel() == 0 && sizes[0] * sizes[1] * sizes[2] * sizes[3] > 0)
+            dense = dense_zero_fill(ctx->saved_data["like"].toTensor(), sizes[0], sizes[1], sizes[2],
+                                    sizes[3]);
+        else if (dense.numel() == 0)
+            dense = torch::empty(sizes, dense.options());
+        dense_patch_lattice(saved[0], saved[1], saved[2], saved[3], upstream(grad_outputs[0]),
+                            ctx->saved_data["scale"].toDouble(),
+                            ctx->saved_data["average_frames"].toBool(), dense);
+        return {dense, torch::Tensor(), torch::Tensor(), torch::Tensor(), torch::Tensor(),
+                torch::Tensor(), torch::Tensor(), torch::Tensor()};
+    }
+};
+
+torch::Tensor ctct_loss_op(const torch::Tensor &joint, const torch::Tensor &labels,
+                           const torch::Tensor &frames_lengths, const torch::Tensor &labels_lengths,
+                           const int64_t reduction, const bool average_frames,
+                           const bool clear_in_forward) {
+    const bool requires_grad = joint.requires_grad() && at::GradMode::is_enabled();
+    return JointLoss::apply(joint, as_int32(labels), as_int32(frames_lengths),
+                            as_int32(labels_lengths), requires_grad, reduction, average_frames,
+                            clear_in_forward);
+}
+
+class LogitsLoss : public torch::autograd::Function<LogitsLoss> {
+   public:
+    static torch::Tensor forward(AutogradContext *ctx, const torch::Tensor &logits,
+                                 const torch::Tensor &ys, const torch::Tensor &lx,
+                                 const torch::Tensor &ly, const bool requires_grad,
+                                 const int64_t reduction, const bool average_frames) {
+        auto out = ctct_loss_logits_fwd(logits, ys, lx, ly, requires_grad, reduction, average_frames);
+        if (requires_grad) {
+            ctx->save_for_backward({std::get<1>(out), logits, ys, lx, ly});
+            ctx->saved_data["scale"] = reduction == 2 ? 1.0 / static_cast<double>(logits.size(0)) : 1.0;
+            ctx->saved_data["average_frames"] = average_frames;
+        }
+        return std::get<0>(out);
+    }
+
+    static tensor_list backward(AutogradContext *ctx, tensor_list grad_outputs) {
+        const auto saved = ctx->get_saved_variables();
+        auto grad = ctct_loss_logits_bwd(saved[0], saved[1], saved[2], saved[3], saved[4],
+                                         upstream(grad_outputs[0]),
+                                         ctx->saved_data["scale"].toDouble(),
+                                         ctx->saved_data["average_frames"].toBool());
+        return {grad, torch::Tensor(), torch::Tensor(), torch::Tensor(), torch::Tensor(),
+                torch::Tensor(), torch::Tensor()};
+    }
+};
+
+torch::Tensor ctct_loss_with_logits_op(const torch::Tensor &logits, const torch::Tensor &labels,
+                                       const torch::Tensor &frames_lengths,
+                                       const torch::Tensor &labels_lengths, const int64_t reduction,
+                                       const bool average_frames) {
+    const bool requires_grad = logits.requires_grad() && at::GradMode::is_enabled();
+    return LogitsLoss::apply(logits.contiguous(), as_int32(labels), as_int32(frames_lengths),
+                             as_int32(labels_lengths), requires_grad, reduction, average_frames);
+}
+
+// ctct_simple_loss on the un-gathered f (N,T,V), g (N,U+1,V): per-sample costs.
+class JoinerLoss : public torch::autograd::Function<JoinerLoss> {
+   public:
+    static torch::Tensor forward(AutogradContext *ctx, const torch::Tensor &f,
+                                 const torch::Tensor &g, const torch::Tensor &ys,
+                                 const torch::Tensor &lx, const torch::Tensor &ly,
+                                 const bool normalized, const bool track_f, const bool track_g) {
+        const bool need_grad = track_f || track_g;
+        auto out = ctct_simple_fwd(f, g, ys, lx, ly, normalized, need_grad);
+        if (need_grad) {
+            // f, g, labels, lengths; the compact gradients; den and what the
+            // log-matmul keeps for its backward (normalised variant only)
+            tensor_list keep = {f, g, ys, lx, ly, std::get<3>(out), std::get<4>(out)};
+            if (normalized) {
+                keep.push_back(std::get<1>(out));
+                keep.push_back(std::get<5>(out));
+                for (const auto &t : std::get<2>(out)) keep.push_back(t);
+            }
+            ctx->save_for_backward(keep);
+            ctx->saved_data["normalized"] = normalized;
+            ctx->saved_data["track_f"] = track_f;
+            ctx->saved_data["track_g"] = track_g;
+        }
+        return std::get<0>(out);
+    }
+
+    static tensor_list backward(AutogradContext *ctx, tensor_list grad_outputs) {
+        const auto s = ctx->get_saved_variables();
+        const bool normalized = ctx->saved_data["normalized"].toBool();
+        c10::optional<torch::Tensor> den, grad_den;
+        std::vector<torch::Tensor> shifted;
+        if (normalized) {
+            den = s[7];
+            grad_den = s[8];
+            shifted.assign(s.begin() + 9, s.end());
+        }
+        auto dense = ctct_simple_bwd(s[0], s[1], den, shifted, s[5], s[6], grad_den, s[2], s[3], s[4],
+                                     upstream(grad_outputs[0]),
+                                     ctx->saved_data["track_f"].toBool(),
+                                     ctx->saved_data["track_g"].toBool());
+        return {std::get<0>(dense), std::get<1>(dense), torch::Tensor(), torch::Tensor(),
+                torch::Tensor(), torch::Tensor(), torch::Tensor(), torch::Tensor()};
+    }
+};
+
+torch::Tensor ctct_simple_loss_op(const torch::Tensor &f, const torch::Tensor &g,
+                                  const torch::Tensor &labels, const torch::Tensor &frames_lengths,
+                                  const torch::Tensor &labels_lengths, const bool normalized) {
+    const bool grad_mode = at::GradMode::is_enabled();
+    const bool track_f = f.requires_grad() && grad_mode, track_g = g.requires_grad() && grad_mode;
+    auto as_float = [](const torch::Tensor &t) {
+        return (t.scalar_type() == at::ScalarType::Float && t.is_contiguous())
+                   ? t
+                   : t.to(at::ScalarType::Float).contiguous();
+    };
+    return JoinerLoss::apply(as_float(f), as_float(g), as_int32(labels), as_int32(frames_lengths),
+                             as_int32(labels_lengths), normalized, track_f, track_g);
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+    m.def("ctct_loss", &ctct_loss_op,
+          "warp_ctct.ctct_loss: the un-gathered joint in, the reduced loss out, differentiable.",
+          pybind11::arg("log_probs"), pybind11::arg("labels"), pybind11::arg("frames_lengths"),
+          pybind11::arg("labels_lengths"), pybind11::arg("reduction"),
+          pybind11::arg("average_frames"), pybind11::arg("clear_in_forward"));
+    m.def("ctct_loss_with_logits", &ctct_loss_with_logits_op,
+          "ctct_loss(logits.log_softmax(-1), ...) in one pass over the logits, differentiable.",
+          pybind11::arg("logits"), pybind11::arg("labels"), pybind11::arg("frames_lengths"),
+          pybind11::arg("labels_lengths"), pybind11::arg("reduction"),
+          pybind11::arg("average_frames"));
+    m.def("ctct_simple_loss", &ctct_simple_loss_op,
+          "Per-sample costs of warp_ctct.ctct_simple_loss on un-gathered f and g, differentiable.",
+          pybind11::arg("f"), pybind11::arg("g"), pybind11::arg("labels"),
+          pybind11::arg("frames_lengths"), pybind11::arg("labels_lengths"),
+          pybind11::arg("normalized"));
     m.def("ctct_loss_fwd", &ctct_loss_fwd, "CTC-Transducer loss on gathered units (forward).",
           pybind11::arg("log_probs"), pybind11::arg("ys"), pybind11::arg("lx"),
           pybind11::arg("ly"), pybind11::arg("requires_grad"));

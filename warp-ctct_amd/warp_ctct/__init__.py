@@ -46,19 +46,6 @@ def _package_version():
 __version__ = _package_version()
 
 
-# Optional observer for profiling: called as observer(kernel_name, fn) and must
-# return fn().  bench.py uses it to bracket single kernels with HIP events on
-# the stream they are launched on; it is None in normal use.
-_kernel_observer = None
-
-
-def set_kernel_observer(observer):
-    """Install (or clear, with None) a callable ``observer(name, fn)`` that
-    runs ``fn()`` and returns its result; used to time individual kernels."""
-    global _kernel_observer
-    _kernel_observer = observer
-
-
 # ctct_loss allocates and clears the joint's gradient during the forward (in the
 # lattice kernel's launch, beside the sweeps) when the joint requires a gradient.  The
 # buffer then lives from the forward to the backward; set this to False to
@@ -114,12 +101,6 @@ def _check_labels(labels, vocabulary):
                              % (vocabulary, lo, hi))
 
 
-def _run(name, fn):
-    if _kernel_observer is None:
-        return fn()
-    return _kernel_observer(name, fn)
-
-
 def _no_autocast():
     return torch.autocast(device_type="cuda", enabled=False)
 
@@ -145,108 +126,37 @@ _REDUCTION_CODE = {None: 0, "none": 0, "sum": 1, "mean": 2}
 _NATIVE_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
 
 
-class _CTCTLoss(torch.autograd.Function):
-    """ctct_loss on the un-gathered joint, reduction included.
-
-    Counterpart of the reference's gather (warp_ctct/__init__.py:124-131), the
-    cast to float (:135), CTCTLoss (:20-33) and the reduction (:138-147).
-    Forward runs gather, both lattices and the batch reduction on the GPU and
-    keeps their workspace.  The dense gradient is all zeros but <= 3 entries
-    per live row, so its buffer is allocated in the forward and cleared, at
-    HBM write bandwidth, inside the launch of the lattice kernel (whose sweeps
-    are bound by latency and leave the memory system idle); backward then only
-    writes the non-zero entries, already weighted by the upstream gradient and by the
-    reduction's own factor (1/N, 1/lx[n]), so autograd launches nothing else.
-    A float16 or bfloat16 joint is read as it is and its gradient is written
-    in the same type (the lattice itself always runs in float32 / float64).
-
-    The cleared buffer serves one backward: a second backward through the same
-    graph (retain_graph=True) clears and fills a buffer of its own."""
-
-    @staticmethod
-    def forward(ctx, joint, labels, lx, ly, requires_grad, reduction, average_frames):
-        clear = bool(requires_grad and CLEAR_GRADIENT_IN_FORWARD)
-        loss, workspace, dense = _run("loss_forward", lambda: core.ctct_loss_joint_fwd(
-            joint, labels, lx, ly, requires_grad, _REDUCTION_CODE[reduction], average_frames,
-            clear))
-        if requires_grad:
-            ctx.save_for_backward(workspace, labels, lx, ly)
-            ctx.shape = tuple(joint.shape)
-            ctx.like = joint.new_empty(0)
-            ctx.dense = dense if clear else None
-            ctx.scale = 1.0 / joint.size(0) if reduction == "mean" else 1.0
-            ctx.average_frames = bool(average_frames)
-        return loss
-
-    @staticmethod
-    def backward(ctx, grad_outputs):
-        workspace, labels, lx, ly = ctx.saved_tensors
-        n, t, u1, v = ctx.shape
-        grad_outputs = grad_outputs.reshape(-1).float().contiguous()
-        dense, ctx.dense = ctx.dense, None
-        if dense is None:
-            dense = _run("dense_zero_fill", lambda: core.dense_zero_fill(ctx.like, n, t, u1, v))
-        _run("dense_patch", lambda: core.dense_patch_lattice(
-            workspace, labels, lx, ly, grad_outputs, ctx.scale, ctx.average_frames, dense))
-        return dense, None, None, None, None, None, None
-
-
-class _CTCTLossLogits(torch.autograd.Function):
-    """ctct_loss(logits.log_softmax(-1), ...) without the log-probability tensor.
-
-    Forward takes the row-wise logsumexp inside the gather and keeps it next
-    to the lattices; backward writes d(loss)/d(logits) = w * (G - softmax *
-    sum(G)) in one pass, G being the <= 3 non-zero gather-backward entries of
-    the row.  Rows of padding are never read."""
-
-    @staticmethod
-    def forward(ctx, logits, labels, lx, ly, requires_grad, reduction, average_frames):
-        loss, workspace = _run("logits_forward", lambda: core.ctct_loss_logits_fwd(
-            logits, labels, lx, ly, requires_grad, _REDUCTION_CODE[reduction], average_frames))
-        if requires_grad:
-            ctx.save_for_backward(workspace, logits, labels, lx, ly)
-            ctx.scale = 1.0 / logits.size(0) if reduction == "mean" else 1.0
-            ctx.average_frames = bool(average_frames)
-        return loss
-
-    @staticmethod
-    def backward(ctx, grad_outputs):
-        workspace, logits, labels, lx, ly = ctx.saved_tensors
-        grad_outputs = grad_outputs.reshape(-1).float().contiguous()
-        grad = _run("logits_backward", lambda: core.ctct_loss_logits_bwd(
-            workspace, logits, labels, lx, ly, grad_outputs, ctx.scale, ctx.average_frames))
-        return grad, None, None, None, None, None, None
-
-
-class _SimpleCTCTLoss(torch.autograd.Function):
-    """ctct_simple_loss on the un-gathered f (N,T,V) and g (N,U+1,V).
-
-    Counterpart of the reference's LogMMExp (warp_ctct/__init__.py:36-52), the
-    two gathers (:204-215) and SimpleCTCTLoss (:55-85).  Forward computes den
-    (if normalized), the lattice and the compact gradients wrt the gathered f,
-    g and den; backward expands them to dense gradients wrt f and g, including
-    the path through den, scaled by grad_output[n].  The forward's exp(f - max f)
-    and exp(g - max g) are kept for the backward (one more tensor of f's size)."""
-
-    @staticmethod
-    def forward(ctx, f, g, labels, lx, ly, normalized, track_f, track_g):
-        need_grad = track_f or track_g
-        costs, den, shifted, grad_f, grad_g, grad_den = _run(
-            "simple_forward", lambda: core.ctct_simple_fwd(f, g, labels, lx, ly, normalized,
-                                                           need_grad))
-        if need_grad:
-            ctx.save_for_backward(f, g, den, grad_f, grad_g, grad_den, labels, lx, ly, *shifted)
-            ctx.track = (track_f, track_g)
-        return costs
-
-    @staticmethod
-    def backward(ctx, grad_outputs):
-        f, g, den, grad_f, grad_g, grad_den, labels, lx, ly, *shifted = ctx.saved_tensors
-        grad_outputs = grad_outputs.reshape(-1).float().contiguous()
-        dense_f, dense_g = _run("simple_backward", lambda: core.ctct_simple_bwd(
-            f, g, den, list(shifted), grad_f, grad_g, grad_den, labels, lx, ly, grad_outputs,
-            ctx.track[0], ctx.track[1]))
-        return dense_f, dense_g, None, None, None, None, None, None
+# The fused losses are autograd functions of the binding (csrc/binding.cpp:
+# JointLoss, LogitsLoss, JoinerLoss): one crossing into C++ per call, and the
+# backward runs without Python.
+#
+# JointLoss (ctct_loss on the un-gathered joint, reduction included) is the
+# counterpart of the reference's gather (warp_ctct/__init__.py:124-131), the cast
+# to float (:135), CTCTLoss (:20-33) and the reduction (:138-147).  Its forward
+# runs gather, both lattices and the batch reduction on the GPU and keeps their
+# workspace.  The dense gradient is all zeros but <= 3 entries per live row, so
+# its buffer is allocated in the forward and cleared, at HBM write bandwidth,
+# inside the launch of the lattice kernel (whose sweeps are bound by latency and
+# leave the memory system idle); the backward then only writes the non-zero
+# entries, already weighted by the upstream gradient and by the reduction's own
+# factor (1/N, 1/lx[n]), so autograd launches nothing else.  A float16 or
+# bfloat16 joint is read as it is and its gradient is written in the same type
+# (the lattice itself always runs in float32 / float64).  The cleared buffer
+# serves one backward: a second backward through the same graph
+# (retain_graph=True) clears and fills a buffer of its own.
+#
+# LogitsLoss is ctct_loss(logits.log_softmax(-1), ...) without the
+# log-probability tensor: the forward takes the row-wise logsumexp inside the
+# gather and keeps it next to the lattices; the backward writes d(loss)/d(logits)
+# = w * (G - softmax * sum(G)) in one pass, G being the <= 3 non-zero
+# gather-backward entries of the row.  Rows of padding are never read.
+#
+# JoinerLoss (ctct_simple_loss on the un-gathered f (N,T,V) and g (N,U+1,V)) is
+# the counterpart of the reference's LogMMExp (warp_ctct/__init__.py:36-52), the
+# two gathers (:204-215) and SimpleCTCTLoss (:55-85): the forward computes den
+# (if normalized), the lattice and the compact gradients wrt the gathered f, g
+# and den; the backward expands them to dense gradients wrt f and g, including
+# the path through den, scaled by grad_output[n].
 
 
 class CTCTLoss(torch.autograd.Function):
@@ -355,14 +265,14 @@ def ctct_loss(log_probs: torch.Tensor,
         return _reduce(log_probs.float().sum(dim=(1, 2, 3)), frames_lengths, reduction,
                        average_frames)
     _check_labels(labels, log_probs.size(3))
-    enable_grad = log_probs.requires_grad and torch.is_grad_enabled()
     if log_probs.dtype not in _NATIVE_DTYPES:
         log_probs = log_probs.float()      # as the reference does for every dtype (:135)
-    with _no_autocast():
-        # a strided view is gathered through its strides, not copied
-        return _CTCTLoss.apply(log_probs, _as_int(labels), _as_int(frames_lengths),
-                               _as_int(labels_lengths), enable_grad, reduction,
-                               bool(average_frames))
+    # (the reference computes under autocast(enabled=False), :134; nothing in
+    # here is subject to autocast.)  A strided view is gathered through its
+    # strides, not copied.
+    return core.ctct_loss(log_probs, labels, frames_lengths, labels_lengths,
+                          _REDUCTION_CODE[reduction], bool(average_frames),
+                          bool(CLEAR_GRADIENT_IN_FORWARD))
 
 
 def ctct_loss_compact(log_probs: torch.Tensor,
@@ -426,13 +336,10 @@ def ctct_loss_with_logits(logits: torch.Tensor,
         return _reduce(logits.float().sum(dim=(1, 2, 3)), frames_lengths, reduction,
                        average_frames)
     _check_labels(labels, logits.size(3))
-    enable_grad = logits.requires_grad and torch.is_grad_enabled()
     if logits.dtype not in _NATIVE_DTYPES:
         logits = logits.float()
-    with _no_autocast():
-        return _CTCTLossLogits.apply(logits.contiguous(), _as_int(labels),
-                                     _as_int(frames_lengths), _as_int(labels_lengths),
-                                     enable_grad, reduction, bool(average_frames))
+    return core.ctct_loss_with_logits(logits, labels, frames_lengths, labels_lengths,
+                                      _REDUCTION_CODE[reduction], bool(average_frames))
 
 
 def ctct_simple_loss(f: torch.Tensor,
@@ -461,10 +368,5 @@ def ctct_simple_loss(f: torch.Tensor,
     assert f.size(0) == g.size(0) == labels.size(0) == frames_lengths.size(0) == labels_lengths.size(0)
 
     _check_labels(labels, f.size(-1))
-    track_f = f.requires_grad and torch.is_grad_enabled()
-    track_g = g.requires_grad and torch.is_grad_enabled()
-    with _no_autocast():
-        costs = _SimpleCTCTLoss.apply(f.float().contiguous(), g.float().contiguous(),
-                                      _as_int(labels), _as_int(frames_lengths),
-                                      _as_int(labels_lengths), bool(normalized), track_f, track_g)
+    costs = core.ctct_simple_loss(f, g, labels, frames_lengths, labels_lengths, bool(normalized))
     return _reduce(costs, frames_lengths, reduction, average_frames)
