@@ -10,17 +10,21 @@
 namespace wctct {
 
 bool profile_enabled();
-void profile_begin(const char *kernel, hipStream_t stream, int *slot);
-void profile_end(hipStream_t stream, int slot);
+// slot: index of the record that was opened (-1: none); generation: which run of
+// records it belongs to (warpctct_profile(1) starts a new one and drops the
+// old records: an end that arrives for an earlier generation is ignored)
+void profile_begin(const char *kernel, hipStream_t stream, int *slot, unsigned *generation);
+void profile_end(hipStream_t stream, int slot, unsigned generation);
 
 struct KernelTimer {
     hipStream_t stream;
     int slot;
-    KernelTimer(const char *kernel, hipStream_t s) : stream(s), slot(-1) {
-        if (profile_enabled()) profile_begin(kernel, s, &slot);
+    unsigned generation;
+    KernelTimer(const char *kernel, hipStream_t s) : stream(s), slot(-1), generation(0) {
+        if (profile_enabled()) profile_begin(kernel, s, &slot, &generation);
     }
     ~KernelTimer() {
-        if (slot >= 0) profile_end(stream, slot);
+        if (slot >= 0) profile_end(stream, slot, generation);
     }
     KernelTimer(const KernelTimer &) = delete;
     KernelTimer &operator=(const KernelTimer &) = delete;

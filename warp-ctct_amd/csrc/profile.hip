@@ -23,9 +23,11 @@ struct Record {
 std::atomic<bool> g_enabled{false};
 std::mutex g_mutex;
 std::vector<Record> g_records;
+unsigned g_generation = 0;   // bumped whenever the records are dropped
 char g_filter[64] = "";   // bracket only kernels whose name contains this
 
 void drop_records() {
+    ++g_generation;
     for (Record &r : g_records) {
         (void)hipEventDestroy(r.begin);
         (void)hipEventDestroy(r.end);
@@ -37,7 +39,7 @@ void drop_records() {
 
 bool profile_enabled() { return g_enabled.load(std::memory_order_relaxed); }
 
-void profile_begin(const char *kernel, hipStream_t stream, int *slot) {
+void profile_begin(const char *kernel, hipStream_t stream, int *slot, unsigned *generation) {
     std::lock_guard<std::mutex> lock(g_mutex);
     if ((int)g_records.size() >= kMaxRecords) return;
     if (g_filter[0] && !std::strstr(kernel, g_filter)) return;
@@ -63,10 +65,13 @@ void profile_begin(const char *kernel, hipStream_t stream, int *slot) {
     }
     g_records.push_back(r);
     *slot = (int)g_records.size() - 1;
+    *generation = g_generation;
 }
 
-void profile_end(hipStream_t stream, int slot) {
+void profile_end(hipStream_t stream, int slot, unsigned generation) {
     std::lock_guard<std::mutex> lock(g_mutex);
+    // (the records this launch belongs to were dropped by another thread in between)
+    if (generation != g_generation) return;
     if (slot < 0 || slot >= (int)g_records.size()) return;
     g_records[slot].complete = hipEventRecord(g_records[slot].end, stream) == hipSuccess;
 }
