@@ -157,3 +157,23 @@ def test_generic_dtype_and_logits_entry_points_check_their_arguments():
     assert lib.warpctct_simple_needs_fexp(aligned, 400, 80, 4096) == 1   # beyond the slab kernels
     assert lib.warpctct_simple_needs_fexp(aligned, 100, 80, 2048) == 1   # too few frames
     assert lib.warpctct_simple_needs_fexp(aligned, 400, 100, 2048) == 1  # too many contexts
+
+
+def test_status_word_entry_point_without_a_device():
+    """warpctct_status refuses a null pointer, and reports that there is no
+    usable device where there is none (it is the one entry point that talks to
+    the device on its own; the CPU suite runs where no GPU is visible)."""
+    lib = hip_lib.lib()
+    EINVAL, ENODEVICE = 1, 4
+    assert lib.warpctct_status(ctypes.c_void_p(0), 0) == EINVAL
+    bits = ctypes.c_uint(0xdead)
+    rc = lib.warpctct_status(ctypes.byref(bits), 1)
+    try:
+        import torch
+        has_gpu = torch.cuda.is_available()
+    except Exception:
+        has_gpu = False
+    if has_gpu:
+        assert rc == 0 and bits.value < 8
+    else:
+        assert rc == ENODEVICE and bits.value == 0xdead

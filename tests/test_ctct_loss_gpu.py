@@ -749,6 +749,39 @@ def test_autograd_plumbing_views_non_leaf_and_repeated_backward():
     np.testing.assert_allclose(quiet.item(), ref_costs.sum(), rtol=LOSS_RTOL)
 
 
+def test_losses_under_autocast_and_with_int64_lengths():
+    """The reference computes under autocast(enabled=False) after casting to
+    float (warp_ctct/__init__.py:134-136): inside an autocast region the losses
+    and their gradients are what they are outside it, for all three entry
+    points, and int64 labels / lengths are cast as the reference casts them."""
+    import warp_ctct
+    from ctct_cases import make_simple_case
+    joint, ys, lx, ly = make_joint_case(91, 3, 21, 6, 24, lx=[21, 13, 17], ly=[6, 2, 5])
+    f, g, sys_, slx, sly = make_simple_case(92, 3, 19, 5, 40, lx=[19, 12, 15], ly=[5, 3, 4])
+
+    def run(autocast, wide):
+        cast = (lambda a: dev(a).long()) if wide else dev
+        out = []
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+            x = dev(joint).requires_grad_(True)
+            warp_ctct.ctct_loss(x, cast(ys), cast(lx), cast(ly)).backward()
+            out.append(x.grad)
+            z = dev(joint).requires_grad_(True)
+            warp_ctct.ctct_loss_with_logits(z, cast(ys), cast(lx), cast(ly), reduction="sum").backward()
+            out.append(z.grad)
+            tf, tg = dev(f).requires_grad_(True), dev(g).requires_grad_(True)
+            loss = warp_ctct.ctct_simple_loss(tf, tg, cast(sys_), cast(slx), cast(sly))
+            assert loss.dtype == torch.float32
+            loss.backward()
+            out += [tf.grad, tg.grad]
+        return out
+
+    plain = run(False, False)
+    for autocast, wide in ((True, False), (False, True), (True, True)):
+        for a, b in zip(plain, run(autocast, wide)):
+            assert a.dtype == torch.float32 and torch.equal(a, b)
+
+
 def test_gradient_buffer_cleared_in_the_forward_or_in_the_backward():
     """ctct_loss clears the joint's gradient beside the lattices in the forward
     (warp_ctct.CLEAR_GRADIENT_IN_FORWARD) or, with the switch off, in the
