@@ -821,13 +821,11 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
             if (rc != WARPCTCT_OK) return rc;
         }
     } else {
-        if (dense_f && simple_dense_f_rows_fit(V)) {
-            // rows built in LDS and written once, instead of zero-fill + atomic adds
-            int rc = done(launch_simple_dense_f_rows(grad_f, ys, lx, ly, grad_out, dense_f, N, T,
-                                                     U, V, st));
-            if (rc != WARPCTCT_OK) return rc;
-            dense_f = nullptr;
-        }
+        if (simple_dense_rows_fit(V))
+            // whole rows of both gradients built and written once, instead of
+            // zero-fill + atomic adds
+            return done(launch_simple_dense_rows(grad_f, grad_g, ys, lx, ly, grad_out, dense_f,
+                                                 dense_g, N, T, U, V, st));
         if (dense_f) {
             int rc = done(launch_zero_fill(dense_f, (size_t)N * T * V, st));
             if (rc != WARPCTCT_OK) return rc;

@@ -183,12 +183,13 @@ hipError_t launch_simple_grads(const double *units, const int *ys, const int *lx
                                hipStream_t stream);
 hipError_t launch_simple_reduce(const float *unit_grads, float *grad_f, float *grad_g,
                                 float *grad_den, int N, int T, int U, hipStream_t stream);
-// dense_f of the unnormalised path in one pass (zeros + scattered compact
-// gradients, whole rows); only for rows that fit into LDS
-bool simple_dense_f_rows_fit(int V);
-hipError_t launch_simple_dense_f_rows(const float *grad_f, const int *ys, const int *lx,
-                                      const int *ly, const float *grad_out, float *dense_f, int N,
-                                      int T, int U, int V, hipStream_t stream);
+// dense_f and dense_g of the unnormalised path in one pass (zeros + scattered
+// compact gradients, whole rows); only for rows that fit into LDS
+bool simple_dense_rows_fit(int V);
+hipError_t launch_simple_dense_rows(const float *grad_f, const float *grad_g, const int *ys,
+                                    const int *lx, const int *ly, const float *grad_out,
+                                    float *dense_f, float *dense_g, int N, int T, int U, int V,
+                                    hipStream_t stream);
 hipError_t launch_simple_scatter(const float *grad_f, const float *grad_g, const int *ys,
                                  const int *lx, const int *ly, const float *grad_out,
                                  float *dense_f, float *dense_g, int N, int T, int U, int V,

@@ -288,20 +288,61 @@ __global__ __launch_bounds__(kBlock) void simple_scatter_f_kernel(
 // workgroup per frame builds the row in LDS (repeated labels add there) and
 // writes it out with full-width stores, so no element of the row is touched
 // twice in memory and no partially written line is left behind.
-__global__ __launch_bounds__(kBlock) void simple_dense_f_rows_kernel(
-    const float *__restrict__ grad_f, const int *__restrict__ ys, const int *__restrict__ lx,
-    const int *__restrict__ ly, const float *__restrict__ grad_out, float *__restrict__ dense_f,
-    int T, int U, int V) {
-    extern __shared__ __attribute__((aligned(16))) float row[];   // V floats
+// The rows of dense_g ride in the same launch (workgroups f_rows.. of a sample,
+// one per context): zeros plus w[n] * grad_g[n,u,k] at columns 0, y[u-1], y[u].
+// A row of dense_g has at most three non-zero elements, so every thread
+// decides for its own columns what to store and LDS is not used.
+__global__ __launch_bounds__(kBlock) void simple_dense_rows_kernel(
+    const float *__restrict__ grad_f, const float *__restrict__ grad_g,
+    const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
+    const float *__restrict__ grad_out, float *__restrict__ dense_f, float *__restrict__ dense_g,
+    int T, int U, int V, int f_rows) {
+    extern __shared__ __attribute__((aligned(16))) float row[];   // V floats (f rows only)
+    typedef float v4f __attribute__((ext_vector_type(4)));
     const int U1 = U + 1;
-    const int n = blockIdx.y, t = blockIdx.x;
-    const int Tn = clampi(lx[n], 0, T), Un = clampi(ly[n], 0, U);
+    const int n = blockIdx.y;
+    const int Un = clampi(ly[n], 0, U);
+    const float w = grad_out ? grad_out[n] : 1.0f;
+    if ((int)blockIdx.x >= f_rows) {
+        const int u = blockIdx.x - f_rows;
+        float *out = dense_g + ((size_t)n * U1 + u) * V;
+        // entry k of the row: column and value; a column of -1 takes no part
+        int col[3] = {-1, -1, -1};
+        float val[3] = {0.0f, 0.0f, 0.0f};
+        if (u <= Un) {
+            const float *gg = grad_g + ((size_t)n * U1 + u) * 3;
+            col[0] = 0, val[0] = w * gg[0];
+            if (u >= 1) col[1] = clampi(ys[(size_t)n * U + u - 1], 0, V - 1), val[1] = w * gg[1];
+            if (u < Un) col[2] = clampi(ys[(size_t)n * U + u], 0, V - 1), val[2] = w * gg[2];
+        }
+        if ((V & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15u) == 0) {
+            for (int k = threadIdx.x * 4; k < V; k += kBlock * 4) {
+                v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int e = 0; e < 3; ++e)
+                    if ((col[e] >> 2) == (k >> 2)) {   // (-1 >> 2 is -1: never a vector of the row)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) v[q] += ((col[e] & 3) == q) ? val[e] : 0.0f;
+                    }
+                __builtin_nontemporal_store(v, reinterpret_cast<v4f *>(out + k));
+            }
+        } else {
+            for (int k = threadIdx.x; k < V; k += kBlock) {
+                float v = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 3; ++e) v += (col[e] == k) ? val[e] : 0.0f;
+                out[k] = v;
+            }
+        }
+        return;
+    }
+    const int t = blockIdx.x;
+    const int Tn = clampi(lx[n], 0, T);
     float *out = dense_f + ((size_t)n * T + t) * V;
     const bool live = t < Tn;
     if (live) {
         for (int k = threadIdx.x; k < V; k += kBlock) row[k] = 0.0f;
         __syncthreads();
-        const float w = grad_out ? grad_out[n] : 1.0f;
         for (int u = threadIdx.x; u <= Un; u += kBlock) {
             const float gv = grad_f[((size_t)n * T + t) * U1 + u];
             if (gv == 0.0f) continue;
@@ -311,7 +352,6 @@ __global__ __launch_bounds__(kBlock) void simple_dense_f_rows_kernel(
         __syncthreads();
     }
     if ((V & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15u) == 0) {
-        typedef float v4f __attribute__((ext_vector_type(4)));
         const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
         for (int k = threadIdx.x * 4; k < V; k += kBlock * 4)
             // (non-temporal: nothing of this path reads the rows again, and their
@@ -427,15 +467,18 @@ hipError_t launch_simple_reduce(const float *unit_grads, float *grad_f, float *g
     return hipGetLastError();
 }
 
-bool simple_dense_f_rows_fit(int V) { return (size_t)V * sizeof(float) <= 64 * 1024; }
+bool simple_dense_rows_fit(int V) { return (size_t)V * sizeof(float) <= 64 * 1024; }
 
-hipError_t launch_simple_dense_f_rows(const float *grad_f, const int *ys, const int *lx,
-                                      const int *ly, const float *grad_out, float *dense_f, int N,
-                                      int T, int U, int V, hipStream_t stream) {
-    if (N == 0 || T == 0) return hipSuccess;
-    TIMED_LAUNCH(simple_dense_f_rows_kernel, dim3(T, N), dim3(kBlock),
-                       (size_t)V * sizeof(float), stream, grad_f, ys, lx, ly, grad_out, dense_f, T,
-                       U, V);
+// Either dense pointer may be null: its rows are then left out of the launch.
+hipError_t launch_simple_dense_rows(const float *grad_f, const float *grad_g, const int *ys,
+                                    const int *lx, const int *ly, const float *grad_out,
+                                    float *dense_f, float *dense_g, int N, int T, int U, int V,
+                                    hipStream_t stream) {
+    const int f_rows = dense_f ? T : 0, g_rows = dense_g ? U + 1 : 0;
+    if (N == 0 || f_rows + g_rows == 0) return hipSuccess;
+    TIMED_LAUNCH(simple_dense_rows_kernel, dim3(f_rows + g_rows, N), dim3(kBlock),
+                 f_rows ? (size_t)V * sizeof(float) : 0, stream, grad_f, grad_g, ys, lx, ly,
+                 grad_out, dense_f, dense_g, T, U, V, f_rows);
     return hipGetLastError();
 }
 
