@@ -355,6 +355,19 @@ int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, c
                                 float *gmax, float *fexp, float *gexp, float *costs,
                                 float *grad_f, float *grad_g, float *grad_den, void *stream);
 
+/* The same with the reduction over the batch that ctct_simple_loss applies to
+ * the costs (warp_ctct/__init__.py:138-147) folded into the lattice kernel, as
+ * in warpctct_loss_lattice: costs[n] is divided by lx[n] if average_frames, and
+ * for reduction 1 (sum) or 2 (mean) *reduced receives the sum or mean of the N
+ * costs, added in a fixed order (reduction 0: reduced may be NULL). */
+int warpctct_simple_forward_reduced_f32(const float *f, const float *g, const int *ys,
+                                        const int *lx, const int *ly, int N, int T, int U, int V,
+                                        int normalized, void *workspace, size_t workspace_bytes,
+                                        float *den, float *fmax, float *gmax, float *fexp,
+                                        float *gexp, float *costs, float *grad_f, float *grad_g,
+                                        float *grad_den, int reduction, int average_frames,
+                                        float *reduced, void *stream);
+
 /* _C.ctct_loss_simple_fwd proper: f_g (N,T,U+1), g_g (N,U+1,3) already
  * gathered, den (N,T,U+1) or NULL (unnormalised, csrc/simple_unnorm.cu). */
 int warpctct_simple_forward_units_f32(const float *f_g, const float *g_g, const float *den,
@@ -382,6 +395,23 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
                                  const float *grad_out, int N, int T, int U, int V,
                                  void *workspace, size_t workspace_bytes, float *dense_f,
                                  float *dense_g, void *stream);
+
+/* The same for a loss that went through warpctct_simple_forward_reduced_f32:
+ * sample n is weighted by grad_out[n * grad_out_stride] * scale (/ lx[n] if
+ * average_frames); stride 0 with scale 1/N is the backward of reduction 'mean'
+ * (warp_ctct/__init__.py:138-147, differentiated; grad_out NULL = ones).
+ * weights: N floats of scratch for the kernels that read a plain array of
+ * per-sample weights (may be NULL if grad_out already is one: stride 1,
+ * scale 1, no average_frames). */
+int warpctct_simple_backward_weighted_f32(const float *f, const float *g, const float *den,
+                                          const float *fmax, const float *gmax, const float *fexp,
+                                          const float *gexp, const float *grad_f,
+                                          const float *grad_g, const float *grad_den,
+                                          const int *ys, const int *lx, const int *ly,
+                                          const float *grad_out, int grad_out_stride, float scale,
+                                          int average_frames, float *weights, int N, int T, int U,
+                                          int V, void *workspace, size_t workspace_bytes,
+                                          float *dense_f, float *dense_g, void *stream);
 
 /* ---- log-semiring matmul -------------------------------------------------- */
 

@@ -420,6 +420,41 @@ def test_simple_loss_partial_tracking_and_reduction(track):
 
 
 @pytest.mark.parametrize("normalized", [True, False])
+@pytest.mark.parametrize("reduction", ["none", "sum", "mean"])
+@pytest.mark.parametrize("average_frames", [False, True])
+@pytest.mark.parametrize("shape", [(5, 24, 7, 19), (70, 9, 3, 6), (3, 136, 20, 512)],
+                         ids=["ragged", "batch_beyond_one_wavefront", "matrix_core_kernels"])
+def test_simple_loss_reduction_inside_the_kernels(shape, average_frames, reduction, normalized):
+    """reduction and average_frames of ctct_simple_loss (warp_ctct/__init__.py:138-147
+    of the reference) are applied by the lattice kernel in the forward and by the
+    per-sample weights of the backward: loss and both dense gradients against the
+    float64 oracle, with an upstream gradient other than one."""
+    import warp_ctct
+    N, T, U, V = shape
+    f, g, ys, lx, ly = make_simple_case(41 + N, N, T, U, V, lx=range(max(U + 2, T // 2), T + 1),
+                                        ly=range(1, U + 1), normalized=normalized)
+    rng = np.random.default_rng(N)
+    w = rng.uniform(-1.5, 2.0, size=N) if reduction == "none" else np.array(-0.75)
+    # the oracle takes the weight of every sample's cost in the differentiated scalar
+    per_sample = np.broadcast_to(w, (N,)).astype(np.float64)
+    if average_frames:
+        per_sample = per_sample / lx
+    if reduction == "mean":
+        per_sample = per_sample / N
+    loss, gf, gg, _ = O.ctct_simple_loss(f, g, ys, lx, ly, reduction=reduction,
+                                         average_frames=average_frames, normalized=normalized,
+                                         grad_output=per_sample)
+    tf, tg = dev(f).requires_grad_(True), dev(g).requires_grad_(True)
+    out = warp_ctct.ctct_simple_loss(tf, tg, dev(ys), dev(lx), dev(ly), reduction=reduction,
+                                     average_frames=average_frames, normalized=normalized)
+    assert out.shape == ((N,) if reduction == "none" else ())
+    np.testing.assert_allclose(out.detach().cpu().numpy(), loss, rtol=LOSS_RTOL)
+    (out * dev(w, torch.float32)).sum().backward()
+    np.testing.assert_allclose(tf.grad.cpu().numpy(), gf, atol=GRAD_ATOL, rtol=1e-5)
+    np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
+
+
+@pytest.mark.parametrize("normalized", [True, False])
 @pytest.mark.parametrize("case", [(3, 15, 5, 12, [15, 11, 8], [5, 3, 4]),
                                   (2, 140, 80, 9, [140, 125], [80, 70]),       # chains of two
                                   (2, 9, 4, 7, [9, 1], [4, 0])])

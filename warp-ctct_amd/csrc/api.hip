@@ -179,7 +179,8 @@ int static_scratch(void **out) {
 // lattice + unit gradients + reductions, shared by the two simple forwards
 int simple_from_units(const SimpleWorkspace &w, const int *ys, const int *lx, const int *ly, int N,
                       int T, int U, float *costs, float *grad_f, float *grad_g, float *grad_den,
-                      bool want_grad, bool relay_is_clear, hipStream_t stream) {
+                      bool want_grad, bool relay_is_clear, const CostReduce &reduce,
+                      hipStream_t stream) {
     // alpha is needed only for the gradients; those are reduced straight from the
     // lattices (the unit-gradient region of the workspace holds the partial sums)
     LatticeArgs a = {};
@@ -196,6 +197,7 @@ int simple_from_units(const SimpleWorkspace &w, const int *ys, const int *lx, co
     a.T = T;
     a.U = U;
     a.beta_only = !want_grad;
+    a.reduce = reduce;
     int rc = done(launch_lattice(a, stream));
     if (rc != WARPCTCT_OK || !want_grad) return rc;
     return done(launch_simple_grads(w.lattice.units, ys, lx, ly, w.lattice.alphas, w.lattice.betas,
@@ -649,7 +651,7 @@ int warpctct_simple_gather_units_f32(const float *f, const float *g, const float
     if (N == 0 || T == 0) return WARPCTCT_OK;
     if (!f || !g || !lx || !ly || !units_out || (U > 0 && !ys)) return WARPCTCT_EINVAL;
     return done(launch_simple_gather_units(f, g, const_cast<float *>(den), ys, lx, ly, units_out, N,
-                                           T, U, V, RelaySlots{}, LogmmDeferred{}, nullptr,
+                                           T, U, V, RelaySlots{}, LogmmDeferred{}, nullptr, nullptr,
                                            as_stream(stream)));
 }
 
@@ -696,7 +698,20 @@ int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, c
                                 void *workspace, size_t workspace_bytes, float *den, float *fmax,
                                 float *gmax, float *fexp, float *gexp, float *costs,
                                 float *grad_f, float *grad_g, float *grad_den, void *stream) {
-    if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
+    return warpctct_simple_forward_reduced_f32(f, g, ys, lx, ly, N, T, U, V, normalized, workspace,
+                                               workspace_bytes, den, fmax, gmax, fexp, gexp, costs,
+                                               grad_f, grad_g, grad_den, 0, 0, nullptr, stream);
+}
+
+int warpctct_simple_forward_reduced_f32(const float *f, const float *g, const int *ys,
+                                        const int *lx, const int *ly, int N, int T, int U, int V,
+                                        int normalized, void *workspace, size_t workspace_bytes,
+                                        float *den, float *fmax, float *gmax, float *fexp,
+                                        float *gexp, float *costs, float *grad_f, float *grad_g,
+                                        float *grad_den, int reduction, int average_frames,
+                                        float *reduced, void *stream) {
+    if (!dims_ok(N, T, U) || V < 1 || reduction < 0 || reduction > 2) return WARPCTCT_EINVAL;
+    if (reduction != 0 && !reduced) return WARPCTCT_EINVAL;
     if (N == 0) return WARPCTCT_OK;
     const bool want_grad = grad_f || grad_g || grad_den;
     if (!g || !lx || !ly || !costs || !workspace || (T > 0 && !f) || (U > 0 && !ys))
@@ -711,6 +726,17 @@ int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, c
     const SimpleWorkspace w = carve_simple(workspace, N, T, U);
     if (workspace_bytes < w.bytes) return WARPCTCT_EWORKSPACE;
     hipStream_t st = as_stream(stream);
+    // the batch reduction rides in the lattice kernel; its arrival counter is
+    // cleared by the gather (or, without frames, by a launch of its own)
+    CostReduce reduce = {};
+    reduce.reduced = reduction != 0 ? reduced : nullptr;
+    reduce.counter = reduction != 0 ? w.lattice.counter : nullptr;
+    reduce.mode = reduction;
+    reduce.average_frames = average_frames != 0;
+    if (T == 0 && reduce.counter) {
+        int rc = done(launch_clear_counter(reduce.counter, st));
+        if (rc != WARPCTCT_OK) return rc;
+    }
     if (T > 0) {
         LogmmDeferred deferred = {};
         if (normalized) {
@@ -728,7 +754,7 @@ int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, c
         int rc = done(launch_simple_gather_units(f, g, normalized ? den : nullptr, ys, lx, ly,
                                                  w.lattice.units, N, T, U, V,
                                                  relay_slots_of(w.lattice.relay, N, T, U), deferred,
-                                                 fmax, st));
+                                                 fmax, reduce.counter, st));
         if (rc != WARPCTCT_OK) return rc;
     }
     if (want_grad && T == 0) {   // no frames: the only gradient with elements is all zeros
@@ -736,7 +762,8 @@ int warpctct_simple_forward_f32(const float *f, const float *g, const int *ys, c
         if (rc != WARPCTCT_OK) return rc;
     }
     return simple_from_units(w, ys, lx, ly, N, T, U, costs, grad_f, grad_g,
-                             normalized ? grad_den : nullptr, want_grad && T > 0, T > 0, st);
+                             normalized ? grad_den : nullptr, want_grad && T > 0, T > 0, reduce,
+                             st);
 }
 
 int warpctct_simple_forward_units_f32(const float *f_g, const float *g_g, const float *den,
@@ -762,7 +789,7 @@ int warpctct_simple_forward_units_f32(const float *f_g, const float *g_g, const 
         if (rc != WARPCTCT_OK) return rc;
     }
     return simple_from_units(w, ys, lx, ly, N, T, U, costs, grad_f, grad_g,
-                             den ? grad_den : nullptr, want_grad && T > 0, false, st);
+                             den ? grad_den : nullptr, want_grad && T > 0, false, CostReduce{}, st);
 }
 
 size_t warpctct_simple_backward_workspace_bytes(int N, int T, int U) {
@@ -778,10 +805,29 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
                                  const float *grad_out, int N, int T, int U, int V,
                                  void *workspace, size_t workspace_bytes, float *dense_f,
                                  float *dense_g, void *stream) {
-    if (!dims_ok(N, T, U) || V < 1) return WARPCTCT_EINVAL;
+    return warpctct_simple_backward_weighted_f32(f, g, den, fmax, gmax, fexp, gexp, grad_f, grad_g,
+                                                 grad_den, ys, lx, ly, grad_out, 1, 1.0f, 0,
+                                                 nullptr, N, T, U, V, workspace, workspace_bytes,
+                                                 dense_f, dense_g, stream);
+}
+
+int warpctct_simple_backward_weighted_f32(const float *f, const float *g, const float *den,
+                                          const float *fmax, const float *gmax, const float *fexp,
+                                          const float *gexp, const float *grad_f,
+                                          const float *grad_g, const float *grad_den,
+                                          const int *ys, const int *lx, const int *ly,
+                                          const float *grad_out, int grad_out_stride, float scale,
+                                          int average_frames, float *weights, int N, int T, int U,
+                                          int V, void *workspace, size_t workspace_bytes,
+                                          float *dense_f, float *dense_g, void *stream) {
+    if (!dims_ok(N, T, U) || V < 1 || (grad_out_stride != 0 && grad_out_stride != 1))
+        return WARPCTCT_EINVAL;
     if (N == 0) return WARPCTCT_OK;
     if (!lx || !ly || (U > 0 && !ys) || (dense_f && !grad_f) || (dense_g && !grad_g))
         return WARPCTCT_EINVAL;
+    const Weight weight = {grad_out, grad_out_stride, scale, average_frames != 0};
+    // grad_out as it is serves as the array of per-sample weights
+    const bool plain = scale == 1.0f && !average_frames && (!grad_out || grad_out_stride == 1);
     const bool keeps_fexp = warpctct_simple_needs_fexp(f, T, U, V) != 0;
     if (den && (!f || !g || !grad_den || !fmax || !gmax || !gexp || !workspace ||
                 (keeps_fexp && !fexp)))
@@ -791,6 +837,18 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
     hipStream_t st = as_stream(stream);
     const int U1 = U + 1;
     if (T == 0) dense_f = nullptr;
+    if (!den && simple_dense_rows_fit(V))
+        // whole rows of both gradients built and written once, instead of
+        // zero-fill + atomic adds
+        return done(launch_simple_dense_rows(grad_f, grad_g, ys, lx, ly, weight, dense_f, dense_g,
+                                             N, T, U, V, st));
+    // the other kernels read an array of N weights
+    if (!plain) {
+        if (!weights) return WARPCTCT_EINVAL;
+        int rc = done(launch_sample_weights(weight, lx, weights, N, st));
+        if (rc != WARPCTCT_OK) return rc;
+        grad_out = weights;
+    }
     if (den) {
         const LogmmOperand lhs = {f, (long)T * V, (long)V, 1L};
         const LogmmOperand rhs = {g, (long)U1 * V, 1L, (long)V};
@@ -821,11 +879,6 @@ int warpctct_simple_backward_f32(const float *f, const float *g, const float *de
             if (rc != WARPCTCT_OK) return rc;
         }
     } else {
-        if (simple_dense_rows_fit(V))
-            // whole rows of both gradients built and written once, instead of
-            // zero-fill + atomic adds
-            return done(launch_simple_dense_rows(grad_f, grad_g, ys, lx, ly, grad_out, dense_f,
-                                                 dense_g, N, T, U, V, st));
         if (dense_f) {
             int rc = done(launch_zero_fill(dense_f, (size_t)N * T * V, st));
             if (rc != WARPCTCT_OK) return rc;

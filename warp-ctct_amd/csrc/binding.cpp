@@ -384,7 +384,9 @@ std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor> ctct_loss
 }
 
 // Fused entry for ctct_simple_loss: un-gathered f (N,T,V), g (N,U+1,V).
-// Returns (costs, den, shifted, grad_f_g, grad_g_g, grad_den).  When normalized,
+// Returns (loss, den, shifted, grad_f_g, grad_g_g, grad_den); loss is the (N,)
+// costs (divided by lx with average_frames) for reduction 0, their sum (1) or
+// mean (2) as a 0-dim tensor otherwise.  When normalized,
 // den is defined and shifted = [fmax (N,T), gmax (N,U+1), fexp (N,T,Vp),
 // gexp (N,U+1,Vp)], the row maxima of f and g and the operands shifted by them
 // and exponentiated, which the backward reuses; otherwise shifted is empty.
@@ -393,13 +395,14 @@ std::tuple<torch::Tensor, torch::Tensor, std::vector<torch::Tensor>, torch::Tens
            torch::Tensor>
 ctct_simple_fwd(const torch::Tensor &f, const torch::Tensor &g, const torch::Tensor &ys,
                 const torch::Tensor &lx, const torch::Tensor &ly, const bool normalized,
-                const bool requires_grad) {
+                const bool requires_grad, const int64_t reduction, const bool average_frames) {
     CHECK_CONTIGUOUS(f);
     CHECK_CONTIGUOUS(g);
     CHECK_FLOAT(f);
     CHECK_FLOAT(g);
     CHECK_DEVICE(f);
     CHECK_DEVICE(g);
+    TORCH_CHECK(reduction >= 0 && reduction <= 2, "reduction must be 0 (none), 1 (sum), 2 (mean)");
     TORCH_CHECK(f.dim() == 3, "f must have 3 dims.");
     TORCH_CHECK(g.dim() == 3, "g must have 3 dims.");
     TORCH_CHECK(f.size(2) == g.size(2), "f and g must share the vocabulary dim");
@@ -408,7 +411,11 @@ ctct_simple_fwd(const torch::Tensor &f, const torch::Tensor &g, const torch::Ten
     check_lengths(ys, lx, ly, N, U);
     const DeviceGuard device_guard(device_of(f));
     auto ws = make_bytes(f, warpctct_simple_workspace_bytes(N, T, U));
-    auto costs = torch::empty({N}, f.options());
+    // the per-sample costs and the reduced scalar share one allocation
+    auto costs_and_sum = N > 0 ? torch::empty({N + 1}, f.options()) : torch::zeros({1}, f.options());
+    auto costs = costs_and_sum.narrow(0, 0, N);
+    torch::Tensor reduced;
+    if (reduction != 0) reduced = costs_and_sum.select(0, N);
     torch::Tensor den, fmax, gmax, fexp, gexp, grad_f, grad_g, grad_den;
     std::vector<torch::Tensor> shifted;
     if (normalized) {
@@ -427,7 +434,7 @@ ctct_simple_fwd(const torch::Tensor &f, const torch::Tensor &g, const torch::Ten
         grad_g = torch::empty({N, U + 1, 3}, f.options());
         if (normalized) grad_den = torch::empty({N, T, U + 1}, f.options());
     }
-    check_rc(warpctct_simple_forward_f32(
+    check_rc(warpctct_simple_forward_reduced_f32(
                  f.data_ptr<float>(), g.data_ptr<float>(), ys.data_ptr<int>(), lx.data_ptr<int>(),
                  ly.data_ptr<int>(), N, T, U, V, normalized ? 1 : 0, ws.data_ptr(), ws.numel(),
                  normalized ? den.data_ptr<float>() : nullptr,
@@ -438,19 +445,23 @@ ctct_simple_fwd(const torch::Tensor &f, const torch::Tensor &g, const torch::Ten
                  requires_grad ? grad_f.data_ptr<float>() : nullptr,
                  requires_grad ? grad_g.data_ptr<float>() : nullptr,
                  (requires_grad && normalized) ? grad_den.data_ptr<float>() : nullptr,
-                 current_stream()),
+                 static_cast<int>(reduction), average_frames ? 1 : 0,
+                 reduction != 0 ? reduced.data_ptr<float>() : nullptr, current_stream()),
              "ctct_simple_fwd");
-    return std::make_tuple(costs, den, shifted, grad_f, grad_g, grad_den);
+    return std::make_tuple(reduction != 0 ? reduced : costs, den, shifted, grad_f, grad_g, grad_den);
 }
 
-// Dense gradients (N,T,V) and (N,U+1,V) of the fused entry, scaled by
-// grad_out[n]; den / grad_den undefined selects the unnormalised variant.
+// Dense gradients (N,T,V) and (N,U+1,V) of the fused entry; sample n is
+// weighted by grad_out ((N,), or one element that is broadcast) times `scale`,
+// divided by lx[n] with average_frames.  den / grad_den undefined selects the
+// unnormalised variant.
 std::tuple<torch::Tensor, torch::Tensor> ctct_simple_bwd(
     const torch::Tensor &f, const torch::Tensor &g, const c10::optional<torch::Tensor> &den,
     const std::vector<torch::Tensor> &shifted,
     const torch::Tensor &grad_f_g, const torch::Tensor &grad_g_g,
     const c10::optional<torch::Tensor> &grad_den, const torch::Tensor &ys, const torch::Tensor &lx,
-    const torch::Tensor &ly, const torch::Tensor &grad_out, const bool want_f, const bool want_g) {
+    const torch::Tensor &ly, const torch::Tensor &grad_out, const bool want_f, const bool want_g,
+    const double scale, const bool average_frames) {
     CHECK_CONTIGUOUS(f);
     CHECK_CONTIGUOUS(g);
     CHECK_FLOAT(f);
@@ -467,7 +478,9 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_simple_bwd(
     TORCH_CHECK(f.dim() == 3 && g.dim() == 3 && f.size(2) == g.size(2), "f (N,T,V), g (N,U+1,V)");
     const int N = f.size(0), T = f.size(1), U = g.size(1) - 1, V = f.size(2);
     check_lengths(ys, lx, ly, N, U);
-    TORCH_CHECK(grad_out.dim() == 1 && grad_out.size(0) == N, "grad_out must be (N,)");
+    TORCH_CHECK(grad_out.dim() == 1 && (grad_out.size(0) == N || grad_out.size(0) == 1),
+                "grad_out must be (N,) or one element");
+    const int grad_out_stride = grad_out.size(0) == N ? 1 : 0;
     TORCH_CHECK(grad_f_g.dim() == 3 && grad_f_g.size(0) == N && grad_f_g.size(1) == T &&
                     grad_f_g.size(2) == U + 1, "grad_f must be (N,T,U+1)");
     TORCH_CHECK(grad_g_g.dim() == 3 && grad_g_g.size(0) == N && grad_g_g.size(1) == U + 1 &&
@@ -502,7 +515,10 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_simple_bwd(
     if (want_f) dense_f = torch::empty_like(f);
     if (want_g) dense_g = torch::empty_like(g);
     auto ws = make_bytes(f, normalized ? warpctct_simple_backward_workspace_bytes(N, T, U) : 0);
-    check_rc(warpctct_simple_backward_f32(
+    // scratch for the per-sample weights, where grad_out is not yet that array
+    torch::Tensor weights;
+    if (grad_out_stride != 1 || scale != 1.0 || average_frames) weights = torch::empty({N}, f.options());
+    check_rc(warpctct_simple_backward_weighted_f32(
                  f.data_ptr<float>(), g.data_ptr<float>(),
                  normalized ? den->data_ptr<float>() : nullptr,
                  normalized ? shifted[0].data_ptr<float>() : nullptr,
@@ -511,7 +527,9 @@ std::tuple<torch::Tensor, torch::Tensor> ctct_simple_bwd(
                  normalized ? shifted[3].data_ptr<float>() : nullptr, grad_f_g.data_ptr<float>(),
                  grad_g_g.data_ptr<float>(), normalized ? grad_den->data_ptr<float>() : nullptr,
                  ys.data_ptr<int>(), lx.data_ptr<int>(), ly.data_ptr<int>(),
-                 grad_out.data_ptr<float>(), N, T, U, V, ws.data_ptr(), ws.numel(),
+                 grad_out.data_ptr<float>(), grad_out_stride, static_cast<float>(scale),
+                 average_frames ? 1 : 0, weights.defined() ? weights.data_ptr<float>() : nullptr, N,
+                 T, U, V, ws.data_ptr(), ws.numel(),
                  want_f ? dense_f.data_ptr<float>() : nullptr,
                  want_g ? dense_g.data_ptr<float>() : nullptr, current_stream()),
              "ctct_simple_bwd");
@@ -702,15 +720,16 @@ torch::Tensor ctct_loss_with_logits_op(const torch::Tensor &logits, const torch:
                              as_int32(labels_lengths), requires_grad, reduction, average_frames);
 }
 
-// ctct_simple_loss on the un-gathered f (N,T,V), g (N,U+1,V): per-sample costs.
+// ctct_simple_loss on the un-gathered f (N,T,V), g (N,U+1,V).
 class JoinerLoss : public torch::autograd::Function<JoinerLoss> {
    public:
     static torch::Tensor forward(AutogradContext *ctx, const torch::Tensor &f,
                                  const torch::Tensor &g, const torch::Tensor &ys,
                                  const torch::Tensor &lx, const torch::Tensor &ly,
-                                 const bool normalized, const bool track_f, const bool track_g) {
+                                 const bool normalized, const bool track_f, const bool track_g,
+                                 const int64_t reduction, const bool average_frames) {
         const bool need_grad = track_f || track_g;
-        auto out = ctct_simple_fwd(f, g, ys, lx, ly, normalized, need_grad);
+        auto out = ctct_simple_fwd(f, g, ys, lx, ly, normalized, need_grad, reduction, average_frames);
         if (need_grad) {
             // f, g, labels, lengths; the compact gradients; den and what the
             // log-matmul keeps for its backward (normalised variant only)
@@ -724,6 +743,8 @@ class JoinerLoss : public torch::autograd::Function<JoinerLoss> {
             ctx->saved_data["normalized"] = normalized;
             ctx->saved_data["track_f"] = track_f;
             ctx->saved_data["track_g"] = track_g;
+            ctx->saved_data["scale"] = reduction == 2 ? 1.0 / static_cast<double>(f.size(0)) : 1.0;
+            ctx->saved_data["average_frames"] = average_frames;
         }
         return std::get<0>(out);
     }
@@ -741,15 +762,19 @@ class JoinerLoss : public torch::autograd::Function<JoinerLoss> {
         auto dense = ctct_simple_bwd(s[0], s[1], den, shifted, s[5], s[6], grad_den, s[2], s[3], s[4],
                                      upstream(grad_outputs[0]),
                                      ctx->saved_data["track_f"].toBool(),
-                                     ctx->saved_data["track_g"].toBool());
+                                     ctx->saved_data["track_g"].toBool(),
+                                     ctx->saved_data["scale"].toDouble(),
+                                     ctx->saved_data["average_frames"].toBool());
         return {std::get<0>(dense), std::get<1>(dense), torch::Tensor(), torch::Tensor(),
-                torch::Tensor(), torch::Tensor(), torch::Tensor(), torch::Tensor()};
+                torch::Tensor(), torch::Tensor(), torch::Tensor(), torch::Tensor(),
+                torch::Tensor(), torch::Tensor()};
     }
 };
 
 torch::Tensor ctct_simple_loss_op(const torch::Tensor &f, const torch::Tensor &g,
                                   const torch::Tensor &labels, const torch::Tensor &frames_lengths,
-                                  const torch::Tensor &labels_lengths, const bool normalized) {
+                                  const torch::Tensor &labels_lengths, const bool normalized,
+                                  const int64_t reduction, const bool average_frames) {
     const bool grad_mode = at::GradMode::is_enabled();
     const bool track_f = f.requires_grad() && grad_mode, track_g = g.requires_grad() && grad_mode;
     auto as_float = [](const torch::Tensor &t) {
@@ -758,7 +783,8 @@ torch::Tensor ctct_simple_loss_op(const torch::Tensor &f, const torch::Tensor &g
                    : t.to(at::ScalarType::Float).contiguous();
     };
     return JoinerLoss::apply(as_float(f), as_float(g), as_int32(labels), as_int32(frames_lengths),
-                             as_int32(labels_lengths), normalized, track_f, track_g);
+                             as_int32(labels_lengths), normalized, track_f, track_g, reduction,
+                             average_frames);
 }
 
 }  // namespace
@@ -775,10 +801,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           pybind11::arg("labels_lengths"), pybind11::arg("reduction"),
           pybind11::arg("average_frames"));
     m.def("ctct_simple_loss", &ctct_simple_loss_op,
-          "Per-sample costs of warp_ctct.ctct_simple_loss on un-gathered f and g, differentiable.",
+          "warp_ctct.ctct_simple_loss on un-gathered f and g: the reduced loss, differentiable.",
           pybind11::arg("f"), pybind11::arg("g"), pybind11::arg("labels"),
           pybind11::arg("frames_lengths"), pybind11::arg("labels_lengths"),
-          pybind11::arg("normalized"));
+          pybind11::arg("normalized"), pybind11::arg("reduction") = 0,
+          pybind11::arg("average_frames") = false);
     m.def("ctct_loss_fwd", &ctct_loss_fwd, "CTC-Transducer loss on gathered units (forward).",
           pybind11::arg("log_probs"), pybind11::arg("ys"), pybind11::arg("lx"),
           pybind11::arg("ly"), pybind11::arg("requires_grad"));
@@ -819,13 +846,15 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("ctct_simple_fwd", &ctct_simple_fwd,
           "CTC-Transducer loss with the log-add joiner on un-gathered f, g (forward).",
           pybind11::arg("f"), pybind11::arg("g"), pybind11::arg("ys"), pybind11::arg("lx"),
-          pybind11::arg("ly"), pybind11::arg("normalized"), pybind11::arg("requires_grad"));
+          pybind11::arg("ly"), pybind11::arg("normalized"), pybind11::arg("requires_grad"),
+          pybind11::arg("reduction") = 0, pybind11::arg("average_frames") = false);
     m.def("ctct_simple_bwd", &ctct_simple_bwd, "Dense gradients wrt f and g.", pybind11::arg("f"),
           pybind11::arg("g"), pybind11::arg("den"), pybind11::arg("shifted"),
           pybind11::arg("grad_f"),
           pybind11::arg("grad_g"), pybind11::arg("grad_den"), pybind11::arg("ys"),
           pybind11::arg("lx"), pybind11::arg("ly"), pybind11::arg("grad_out"),
-          pybind11::arg("want_f"), pybind11::arg("want_g"));
+          pybind11::arg("want_f"), pybind11::arg("want_g"), pybind11::arg("scale") = 1.0,
+          pybind11::arg("average_frames") = false);
     m.def("log_matmul", &log_matmul, "Log matrix multiplication", pybind11::arg("lhs"),
           pybind11::arg("rhs"));
     m.def("log_matmul_backward", &log_matmul_backward, "Log matrix multiplication backward",

@@ -27,6 +27,17 @@ constexpr unsigned kStatusLostHandOver = 4u;   // a chain of workgroups gave up 
 // null when it cannot be found (kernels then report nothing).
 unsigned *device_status_word();
 
+// Per-sample weight of the upstream gradient: grad_out[n * stride] (stride 0
+// broadcasts a scalar), times `scale` (1/N for reduction='mean'), divided by
+// lx[n] when the loss was averaged over frames (warp_ctct/__init__.py:138-147
+// of the reference, differentiated).
+struct Weight {
+    const float *grad_out;   // null = ones
+    int stride;
+    float scale;
+    int average_frames;
+};
+
 // Reduction over the batch folded into the lattice kernel: the workgroup that
 // finishes last (counted in *counter, which must be 0 at launch) adds up the N
 // costs in a fixed order.  mode 0 = none, 1 = sum, 2 = mean.
@@ -172,7 +183,7 @@ hipError_t launch_simple_gather_units(const float *f, const float *g, float *den
                                       const int *lx, const int *ly, double *units, int N, int T,
                                       int U, int V, const RelaySlots &relay,
                                       const LogmmDeferred &deferred, float *fmax,
-                                      hipStream_t stream);
+                                      unsigned *counter, hipStream_t stream);
 // compact gradients of the joiner path straight from the lattices: grad_f
 // (N,T,U+1), grad_g (N,U+1,3), grad_den (N,T,U+1) or null; `partial` is scratch
 // of N * T * (U+1) * 3 floats (partial sums over blocks of 8 frames, or, for
@@ -187,9 +198,12 @@ hipError_t launch_simple_reduce(const float *unit_grads, float *grad_f, float *g
 // compact gradients, whole rows); only for rows that fit into LDS
 bool simple_dense_rows_fit(int V);
 hipError_t launch_simple_dense_rows(const float *grad_f, const float *grad_g, const int *ys,
-                                    const int *lx, const int *ly, const float *grad_out,
+                                    const int *lx, const int *ly, const Weight &weight,
                                     float *dense_f, float *dense_g, int N, int T, int U, int V,
                                     hipStream_t stream);
+// weights[n] = grad_out[n * stride] * scale (/ lx[n] with average_frames), see Weight
+hipError_t launch_sample_weights(const Weight &weight, const int *lx, float *weights, int N,
+                                 hipStream_t stream);
 hipError_t launch_simple_scatter(const float *grad_f, const float *grad_g, const int *ys,
                                  const int *lx, const int *ly, const float *grad_out,
                                  float *dense_f, float *dense_g, int N, int T, int U, int V,

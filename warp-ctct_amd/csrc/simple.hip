@@ -37,8 +37,11 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     const float *__restrict__ f, const float *__restrict__ g, float *__restrict__ den,
     const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
     double *__restrict__ units, int T, int U, int V, int P, const RelaySlots relay,
-    const LogmmDeferred deferred, float *__restrict__ fmax, unsigned *__restrict__ status) {
+    const LogmmDeferred deferred, float *__restrict__ fmax, unsigned *__restrict__ counter,
+    unsigned *__restrict__ status) {
     relay_clear_share(relay);
+    // (the arrival counter of the lattice kernel's cost reduction, if there is one)
+    if (counter && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *counter = 0u;
     const int U1 = U + 1;
     const int n = blockIdx.y;
     const int cell = blockIdx.x * kBlock + threadIdx.x;
@@ -295,14 +298,14 @@ __global__ __launch_bounds__(kBlock) void simple_scatter_f_kernel(
 __global__ __launch_bounds__(kBlock) void simple_dense_rows_kernel(
     const float *__restrict__ grad_f, const float *__restrict__ grad_g,
     const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
-    const float *__restrict__ grad_out, float *__restrict__ dense_f, float *__restrict__ dense_g,
+    const Weight weight, float *__restrict__ dense_f, float *__restrict__ dense_g,
     int T, int U, int V, int f_rows) {
     extern __shared__ __attribute__((aligned(16))) float row[];   // V floats (f rows only)
     typedef float v4f __attribute__((ext_vector_type(4)));
     const int U1 = U + 1;
     const int n = blockIdx.y;
     const int Un = clampi(ly[n], 0, U);
-    const float w = grad_out ? grad_out[n] : 1.0f;
+    const float w = sample_weight(weight, n, lx[n]);
     if ((int)blockIdx.x >= f_rows) {
         const int u = blockIdx.x - f_rows;
         float *out = dense_g + ((size_t)n * U1 + u) * V;
@@ -403,6 +406,15 @@ __global__ __launch_bounds__(kBlock) void simple_scatter_fg_kernel(
                         dense_g, U, V);
 }
 
+// weights[n] = grad_out[n * stride] * scale (/ lx[n]): what the kernels that take a
+// plain array of per-sample weights read after a reduction over the batch
+__global__ __launch_bounds__(kBlock) void sample_weights_kernel(const Weight weight,
+                                                                const int *__restrict__ lx,
+                                                                float *__restrict__ weights, int N) {
+    const int n = blockIdx.x * kBlock + threadIdx.x;
+    if (n < N) weights[n] = sample_weight(weight, n, lx[n]);
+}
+
 inline dim3 cell_grid(int N, int T, int U) {
     const long cells = (long)T * (U + 1);
     return dim3((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N);
@@ -414,7 +426,7 @@ hipError_t launch_simple_gather_units(const float *f, const float *g, float *den
                                       const int *lx, const int *ly, double *units, int N, int T,
                                       int U, int V, const RelaySlots &relay,
                                       const LogmmDeferred &deferred, float *fmax,
-                                      hipStream_t stream) {
+                                      unsigned *counter, hipStream_t stream) {
     const int P = padded_contexts(U);
     const long cells = (long)T * P;
     const dim3 grid((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N);
@@ -423,10 +435,10 @@ hipError_t launch_simple_gather_units(const float *f, const float *g, float *den
             deferred.Nn != U + 1)
             return hipErrorInvalidValue;
         TIMED_LAUNCH(simple_gather_units_kernel<true>, grid, dim3(kBlock), 0, stream, f, g, den, ys,
-                     lx, ly, units, T, U, V, P, relay, deferred, fmax, device_status_word());
+                     lx, ly, units, T, U, V, P, relay, deferred, fmax, counter, device_status_word());
     } else {
         TIMED_LAUNCH(simple_gather_units_kernel<false>, grid, dim3(kBlock), 0, stream, f, g, den, ys,
-                     lx, ly, units, T, U, V, P, relay, deferred, fmax, device_status_word());
+                     lx, ly, units, T, U, V, P, relay, deferred, fmax, counter, device_status_word());
     }
     return hipGetLastError();
 }
@@ -471,14 +483,22 @@ bool simple_dense_rows_fit(int V) { return (size_t)V * sizeof(float) <= 64 * 102
 
 // Either dense pointer may be null: its rows are then left out of the launch.
 hipError_t launch_simple_dense_rows(const float *grad_f, const float *grad_g, const int *ys,
-                                    const int *lx, const int *ly, const float *grad_out,
+                                    const int *lx, const int *ly, const Weight &weight,
                                     float *dense_f, float *dense_g, int N, int T, int U, int V,
                                     hipStream_t stream) {
     const int f_rows = dense_f ? T : 0, g_rows = dense_g ? U + 1 : 0;
     if (N == 0 || f_rows + g_rows == 0) return hipSuccess;
     TIMED_LAUNCH(simple_dense_rows_kernel, dim3(f_rows + g_rows, N), dim3(kBlock),
                  f_rows ? (size_t)V * sizeof(float) : 0, stream, grad_f, grad_g, ys, lx, ly,
-                 grad_out, dense_f, dense_g, T, U, V, f_rows);
+                 weight, dense_f, dense_g, T, U, V, f_rows);
+    return hipGetLastError();
+}
+
+hipError_t launch_sample_weights(const Weight &weight, const int *lx, float *weights, int N,
+                                 hipStream_t stream) {
+    if (N == 0) return hipSuccess;
+    TIMED_LAUNCH(sample_weights_kernel, dim3((N + kBlock - 1) / kBlock), dim3(kBlock), 0, stream,
+                 weight, lx, weights, N);
     return hipGetLastError();
 }
 

@@ -4,6 +4,7 @@
 #pragma once
 
 #include "device_utils.h"
+#include "launch.h"
 
 namespace wctct {
 
@@ -18,17 +19,7 @@ __device__ __forceinline__ bool outside_band(int t, int u, int Tn, int Un) {
     return t < u || Tn - t < Un - u;
 }
 
-// Per-sample weight of the upstream gradient: grad_out[n * stride] (stride 0
-// broadcasts a scalar), times `scale` (1/N for reduction='mean'), divided by
-// lx[n] when the loss was averaged over frames (warp_ctct/__init__.py:138-147
-// of the reference, differentiated).
-struct Weight {
-    const float *grad_out;   // null = ones
-    int stride;
-    float scale;
-    int average_frames;
-};
-
+// The weight of sample n (see Weight in launch.h); lxn = lx[n].
 __device__ __forceinline__ float sample_weight(const Weight &w, int n, int lxn) {
     float v = w.grad_out ? w.grad_out[(size_t)n * w.stride] : 1.0f;
     v *= w.scale;

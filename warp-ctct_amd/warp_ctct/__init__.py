@@ -368,5 +368,5 @@ def ctct_simple_loss(f: torch.Tensor,
     assert f.size(0) == g.size(0) == labels.size(0) == frames_lengths.size(0) == labels_lengths.size(0)
 
     _check_labels(labels, f.size(-1))
-    costs = core.ctct_simple_loss(f, g, labels, frames_lengths, labels_lengths, bool(normalized))
-    return _reduce(costs, frames_lengths, reduction, average_frames)
+    return core.ctct_simple_loss(f, g, labels, frames_lengths, labels_lengths, bool(normalized),
+                                 _REDUCTION_CODE[reduction], bool(average_frames))
