@@ -842,9 +842,10 @@ int warpctct_simple_backward_weighted_f32(const float *f, const float *g, const 
         // zero-fill + atomic adds
         return done(launch_simple_dense_rows(grad_f, grad_g, ys, lx, ly, weight, dense_f, dense_g,
                                              N, T, U, V, st));
-    // the other kernels read an array of N weights
-    if (!plain) {
-        if (!weights) return WARPCTCT_EINVAL;
+    // the other kernels read an array of N weights: the first kernel of the
+    // normalised path leaves it behind, otherwise a launch of its own does
+    if (!plain && !weights) return WARPCTCT_EINVAL;
+    if (!plain && !(den && T > 0)) {
         int rc = done(launch_sample_weights(weight, lx, weights, N, st));
         if (rc != WARPCTCT_OK) return rc;
         grad_out = weights;
@@ -857,10 +858,12 @@ int warpctct_simple_backward_weighted_f32(const float *f, const float *g, const 
                                  keeps_fexp ? const_cast<float *>(fexp) : nullptr,
                                  const_cast<float *>(gexp)};
         if (T > 0) {
-            int rc = done(launch_logmm_pair_factor(grad_den, den, fmax, gmax, grad_out, lx, ly,
-                                                   pw.factors, pw.flags, pw.planes, N, T, U1, st));
+            int rc = done(launch_logmm_pair_factor(grad_den, den, fmax, gmax, weight,
+                                                   plain ? nullptr : weights, lx, ly, pw.factors,
+                                                   pw.flags, pw.planes, N, T, U1, st));
             if (rc != WARPCTCT_OK) return rc;
         }
+        if (!plain) grad_out = weights;
         // (the gradient wrt g first: it only reads f, which the gradient wrt f then
         // finds in the memory-side cache, and whose own 4*N*T*V bytes of output are
         // still there for the scatter that follows)
@@ -936,7 +939,8 @@ int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, lo
     {
         int rc = done(launch_logmm_shift_exp(l, r, w.sh, B, M, K, Nn, nullptr, nullptr, st));
         if (rc != WARPCTCT_OK) return rc;
-        rc = done(launch_logmm_pair_factor(grad_out, res, w.sh.lmax, w.sh.rmax, nullptr, nullptr,
+        rc = done(launch_logmm_pair_factor(grad_out, res, w.sh.lmax, w.sh.rmax,
+                                           Weight{nullptr, 1, 1.0f, 0}, nullptr, nullptr,
                                            nullptr, w.pw.factors, w.pw.flags, w.pw.planes, B, M, Nn, st));
         if (rc != WARPCTCT_OK) return rc;
     }

@@ -275,9 +275,10 @@ size_t logmm_pair_planes_bytes(int B, int M, int Nn);
 size_t logmm_pair_shifts_bytes(int B, int M, int Nn);
 // C (B,M,logmm_pair_row(Nn)) and flags (B,M): the pair factors go * exp(lmax + rmax - res) that
 // both gradients share, and per row whether a pair was left to the exact pass;
-// batch_scale (may be null) multiplies grad_out per batch.
+// `weight` (with row_len as the frame counts) multiplies grad_out per batch
+// entry, and is left in weights_out[b] (may be null) for the kernels that follow.
 hipError_t launch_logmm_pair_factor(const float *go, const float *res, const float *lmax,
-                                    const float *rmax, const float *batch_scale,
+                                    const float *rmax, const Weight &weight, float *weights_out,
                                     const int *row_len, const int *col_len, float *C, int *flags,
                                     const LogmmPairPlanes &planes, int B, int M, int Nn,
                                     hipStream_t stream);

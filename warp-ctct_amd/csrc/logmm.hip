@@ -30,6 +30,7 @@
 
 #include "device_utils.h"
 #include "launch.h"
+#include "unit_grad.h"
 
 namespace wctct {
 
@@ -641,14 +642,16 @@ __global__ __launch_bounds__(256) void logmm_fwd_finish_kernel(const FwdArgs a, 
 
 // ---- backward ----------------------------------------------------------------
 // C[b,i,j] = scale[b] * go[b,i,j] * exp(ml[i] + mr[j] - res[b,i,j]), the factor
-// that a pair (i,j) contributes to both gradients; 0 for padding, for a zero
+// that a pair (i,j) contributes to both gradients; scale[b] is the sample's
+// weight (Weight, with row_len as the frame counts), which the kernel also
+// leaves in weights_out[b] (if not null) for the kernels that follow; 0 for padding, for a zero
 // grad_out and for an all -inf row (no gradient).  A pair whose exponent
 // exceeds 2^60 is stored as 0 and its row is flagged: flags[b,i] = 1 makes the
 // gradient kernels add such pairs term by term.  Rows of C are logmm_pair_row(Nn)
 // floats long, zeros in the padding.  One wavefront per row i.
 __global__ __launch_bounds__(256) void logmm_pair_factor_kernel(
     const float *__restrict__ go, const float *__restrict__ res, const float *__restrict__ lmax,
-    const float *__restrict__ rmax, const float *__restrict__ batch_scale,
+    const float *__restrict__ rmax, const Weight weight, float *__restrict__ weights_out,
     const int *__restrict__ row_len, const int *__restrict__ col_len, float *__restrict__ C,
     int *__restrict__ flags, int M, int Nn) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -656,7 +659,8 @@ __global__ __launch_bounds__(256) void logmm_pair_factor_kernel(
     if (i >= M) return;
     const int Mb = row_len ? min(max(row_len[b], 0), M) : M;
     const int Nb = col_len ? min(max(col_len[b], 0) + 1, Nn) : Nn;
-    const float scale = batch_scale ? batch_scale[b] : 1.0f;
+    const float scale = sample_weight(weight, b, row_len ? row_len[b] : 1);
+    if (weights_out && blockIdx.x == 0 && threadIdx.x == 0) weights_out[b] = scale;
     const size_t row = ((size_t)b * M + i) * Nn;
     const int Cq = logmm_pair_row(Nn);
     float *crow = C + ((size_t)b * M + i) * Cq;
@@ -692,7 +696,7 @@ __global__ __launch_bounds__(256) void logmm_pair_factor_kernel(
 constexpr int kPairRowsPerWave = 4;
 __global__ __launch_bounds__(512) void logmm_pair_factor_planes_kernel(
     const float *__restrict__ go, const float *__restrict__ res, const float *__restrict__ lmax,
-    const float *__restrict__ rmax, const float *__restrict__ batch_scale,
+    const float *__restrict__ rmax, const Weight weight, float *__restrict__ weights_out,
     const int *__restrict__ row_len, const int *__restrict__ col_len, float *__restrict__ C,
     int *__restrict__ flags, unsigned short *__restrict__ planes, float *__restrict__ shifts,
     int B, int M, int Nn, int ct_frames) {
@@ -702,7 +706,8 @@ __global__ __launch_bounds__(512) void logmm_pair_factor_planes_kernel(
     const int b = blockIdx.y, i0 = blockIdx.x * 8 * R;
     const int Mb = row_len ? min(max(row_len[b], 0), M) : M;
     const int Nb = col_len ? min(max(col_len[b], 0) + 1, Nn) : Nn;
-    const float scale = batch_scale ? batch_scale[b] : 1.0f;
+    const float scale = sample_weight(weight, b, row_len ? row_len[b] : 1);
+    if (weights_out && blockIdx.x == 0 && threadIdx.x == 0) weights_out[b] = scale;
     const int Cq = logmm_pair_row(Nn);
     // row r of this wavefront is local row 8*r + wave.  (A row has at most 96
     // entries; all of a lane's loads are requested before the first is used.)
@@ -1765,7 +1770,7 @@ size_t logmm_pair_shifts_bytes(int B, int M, int Nn) {
 }
 
 hipError_t launch_logmm_pair_factor(const float *go, const float *res, const float *lmax,
-                                    const float *rmax, const float *batch_scale,
+                                    const float *rmax, const Weight &weight, float *weights_out,
                                     const int *row_len, const int *col_len, float *C, int *flags,
                                     const LogmmPairPlanes &planes, int B, int M, int Nn,
                                     hipStream_t stream) {
@@ -1774,12 +1779,12 @@ hipError_t launch_logmm_pair_factor(const float *go, const float *res, const flo
         const int frames = logmm_pair_frames(M);
         TIMED_LAUNCH(logmm_pair_factor_planes_kernel, dim3(frames / (8 * kPairRowsPerWave), B),
                      dim3(512), 0, stream, go,
-                     res, lmax, rmax, batch_scale, row_len, col_len, C, flags, planes.planes,
+                     res, lmax, rmax, weight, weights_out, row_len, col_len, C, flags, planes.planes,
                      planes.shifts, B, M, Nn, frames);
         return hipGetLastError();
     }
     TIMED_LAUNCH(logmm_pair_factor_kernel, dim3((M + 3) / 4, B), dim3(256), 0, stream, go,
-                       res, lmax, rmax, batch_scale, row_len, col_len, C, flags, M, Nn);
+                       res, lmax, rmax, weight, weights_out, row_len, col_len, C, flags, M, Nn);
     return hipGetLastError();
 }
 
