@@ -112,15 +112,26 @@ def test_random_joiner_cases(seed):
             f[:, :, cols[: len(cols) // 2]] = -np.inf
             g[:, :, cols[len(cols) // 2:]] = -np.inf
             f[0, T // 2] -= 300.0
-        w = rng.standard_normal(N)
+        # the reduction over the batch and the division by the frame counts are
+        # part of the kernels: drawn at random too, with an upstream gradient
+        # per sample (no reduction) or one for the reduced scalar
+        reduction = ["none", "sum", "mean"][int(rng.integers(0, 3))]
+        average_frames = bool(rng.integers(0, 2))
+        w = rng.standard_normal(N) if reduction == "none" else rng.standard_normal(1)
+        per_sample = np.broadcast_to(w, (N,)).astype(np.float64)
+        if average_frames:
+            per_sample = per_sample / lx
+        if reduction == "mean":
+            per_sample = per_sample / N
         with np.errstate(all="ignore"):
-            _, gf, gg, costs = O.ctct_simple_loss(f, g, ys, lx, ly, reduction="none",
-                                                  normalized=normalized, grad_output=w)
+            loss, gf, gg, costs = O.ctct_simple_loss(f, g, ys, lx, ly, reduction=reduction,
+                                                     average_frames=average_frames,
+                                                     normalized=normalized, grad_output=per_sample)
         tf, tg = dev(f).requires_grad_(True), dev(g).requires_grad_(True)
-        out = warp_ctct.ctct_simple_loss(tf, tg, dev(ys), dev(lx), dev(ly), reduction="none",
-                                         normalized=normalized)
+        out = warp_ctct.ctct_simple_loss(tf, tg, dev(ys), dev(lx), dev(ly), reduction=reduction,
+                                         average_frames=average_frames, normalized=normalized)
         (out * dev(w, torch.float32)).sum().backward()
-        if same_costs(out.detach().cpu().numpy(), costs):
+        if same_costs(np.atleast_1d(out.detach().cpu().numpy()), np.atleast_1d(loss)):
             scale = max(1.0, float(np.abs(w).max()))
             # dense gradients sum up to T (resp. U+1) unit gradients per entry
             np.testing.assert_allclose(tf.grad.cpu().numpy(), gf, atol=GRAD_ATOL * scale, rtol=1e-5)
