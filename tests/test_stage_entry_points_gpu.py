@@ -347,6 +347,98 @@ def test_log_add_joiner_stages(case):
                                atol=2e-6, rtol=1e-5)
 
 
+FUSED_JOINER_CASES = [
+    # name, seed, N, T, U, V, lx, ly, normalized
+    ("normalized", 231, 3, 23, 7, 29, [23, 12, 17], [7, 3, 5], True),
+    ("unnormalized", 232, 3, 23, 7, 29, [23, 12, 17], [7, 3, 5], False),
+    ("matrix_core_kernels", 233, 2, 136, 20, 512, [136, 129], [20, 11], True),
+    ("chain_of_workgroups", 234, 2, 90, 70, 40, [90, 77], [70, 64], False),
+]
+
+
+@pytest.mark.parametrize("case", FUSED_JOINER_CASES, ids=[c[0] for c in FUSED_JOINER_CASES])
+@pytest.mark.parametrize("reduction,average_frames", [(0, 0), (1, 1), (2, 0), (2, 1)])
+def test_fused_joiner_entry_points_with_reduction(case, reduction, average_frames):
+    """warpctct_simple_forward_reduced_f32 and warpctct_simple_backward_weighted_f32 called
+    directly: un-gathered f and g in, costs / reduced loss out, dense gradients
+    for an upstream gradient that is one scalar (sum, mean) or one value per
+    sample (no reduction), against the float64 oracle."""
+    lib = hip_lib.lib()
+    _, seed, N, T, U, V, lx, ly, normalized = case
+    f, g, ys, lx, ly = make_simple_case(seed, N, T, U, V, lx=lx, ly=ly, normalized=normalized)
+    U1 = U + 1
+    p, s = hip_lib.ptr, hip_lib.stream_ptr()
+    for fn in ("warpctct_simple_workspace_bytes", "warpctct_simple_backward_workspace_bytes"):
+        getattr(lib, fn).restype = ctypes.c_size_t
+    Vp = lib.warpctct_logmm_padded_reduction(V)
+    d_f, d_g, d_ys, d_lx, d_ly = dev(f), dev(g), dev(ys), dev(lx), dev(ly)
+    ws = torch.empty(lib.warpctct_simple_workspace_bytes(N, T, U), dtype=torch.uint8, device="cuda")
+    den = nan_like(N, T, U1) if normalized else None
+    fmax = nan_like(N, T) if normalized else None
+    gmax = nan_like(N, U1) if normalized else None
+    keeps = lib.warpctct_simple_needs_fexp(p(d_f), T, U, V) != 0
+    fexp = nan_like(N, T, Vp) if normalized and keeps else None
+    gexp = nan_like(N, U1, Vp) if normalized else None
+    costs, reduced = nan_like(N), nan_like(1)
+    grad_f, grad_g = nan_like(N, T, U1), nan_like(N, U1, 3)
+    grad_den = nan_like(N, T, U1) if normalized else None
+    hip_lib.check(lib.warpctct_simple_forward_reduced_f32(
+        p(d_f), p(d_g), p(d_ys), p(d_lx), p(d_ly), N, T, U, V, int(normalized), p(ws),
+        ctypes.c_size_t(ws.numel()), p(den), p(fmax), p(gmax), p(fexp), p(gexp), p(costs),
+        p(grad_f), p(grad_g), p(grad_den), reduction, average_frames,
+        p(reduced) if reduction else p(None), s))
+    torch.cuda.synchronize()
+
+    rng = np.random.default_rng(seed)
+    up = rng.uniform(-1.5, 2.0, size=N if reduction == 0 else 1).astype(np.float32)
+    per_sample = np.broadcast_to(up, (N,)).astype(np.float64)
+    if average_frames:
+        per_sample = per_sample / lx
+    if reduction == 2:
+        per_sample = per_sample / N
+    name = {0: "none", 1: "sum", 2: "mean"}[reduction]
+    loss, gf, gg, costs_ref = O.ctct_simple_loss(f, g, ys, lx, ly, reduction=name,
+                                                 average_frames=bool(average_frames),
+                                                 normalized=normalized, grad_output=per_sample)
+    per_cost = costs_ref / lx if average_frames else costs_ref
+    np.testing.assert_allclose(costs.cpu().numpy(), per_cost, rtol=LOSS_RTOL)
+    if reduction:
+        np.testing.assert_allclose(float(reduced.cpu()), loss, rtol=LOSS_RTOL)
+    else:
+        assert np.isnan(float(reduced.cpu()))   # untouched
+
+    bws = torch.empty(max(lib.warpctct_simple_backward_workspace_bytes(N, T, U), 8),
+                      dtype=torch.uint8, device="cuda")
+    dense_f, dense_g = nan_like(N, T, V), nan_like(N, U1, V)
+    weights = nan_like(N)
+    d_up = dev(up)
+    scale = ctypes.c_float(1.0 / N if reduction == 2 else 1.0)
+
+    def backward(grad_out, stride, scale_arg, avg, weights_arg):
+        return lib.warpctct_simple_backward_weighted_f32(
+            p(d_f), p(d_g), p(den), p(fmax), p(gmax), p(fexp), p(gexp), p(grad_f), p(grad_g),
+            p(grad_den), p(d_ys), p(d_lx), p(d_ly), p(grad_out), stride, scale_arg, avg,
+            p(weights_arg), N, T, U, V, p(bws), ctypes.c_size_t(bws.numel()), p(dense_f), p(dense_g), s)
+
+    hip_lib.check(backward(d_up, 1 if reduction == 0 else 0, scale, average_frames, weights))
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(dense_f.cpu().numpy(), gf, atol=GRAD_ATOL, rtol=1e-5)
+    np.testing.assert_allclose(dense_g.cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
+    # arguments (1 = WARPCTCT_EINVAL): a stride other than 0 or 1, no scratch where the
+    # weights need one, a reduction that does not exist, a reduction without its output
+    assert backward(d_up, 2, scale, average_frames, weights) == 1
+    if normalized and (reduction != 0 or average_frames):
+        assert backward(d_up, 1 if reduction == 0 else 0, scale, average_frames, None) == 1
+    assert lib.warpctct_simple_forward_reduced_f32(
+        p(d_f), p(d_g), p(d_ys), p(d_lx), p(d_ly), N, T, U, V, int(normalized), p(ws),
+        ctypes.c_size_t(ws.numel()), p(den), p(fmax), p(gmax), p(fexp), p(gexp), p(costs),
+        p(grad_f), p(grad_g), p(grad_den), 3, 0, p(reduced), s) == 1
+    assert lib.warpctct_simple_forward_reduced_f32(
+        p(d_f), p(d_g), p(d_ys), p(d_lx), p(d_ly), N, T, U, V, int(normalized), p(ws),
+        ctypes.c_size_t(ws.numel()), p(den), p(fmax), p(gmax), p(fexp), p(gexp), p(costs),
+        p(grad_f), p(grad_g), p(grad_den), 1, 0, p(None), s) == 1
+
+
 def _scatter_g(gg, gi, ly, w, U1, V):
     N = gg.shape[0]
     out = np.zeros((N, U1, V))
