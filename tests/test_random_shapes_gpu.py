@@ -2,7 +2,12 @@
 (chains of workgroups per lattice, hand-over chunks, 16-byte vector rows, the
 shapes of the log-matmul kernels), against the float64 oracle through the
 public API.  Every case prints its parameters before it runs, so a failure or
-a fault names its case."""
+a fault names its case.
+
+WARPCTCT_RANDOM_CASES_SCALE=k in the environment runs k times as many cases per
+test (the same seeds, longer streams) for an occasional long run."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -13,6 +18,7 @@ from oracle import ctct_oracle as O
 
 pytestmark = pytest.mark.gpu
 
+SCALE = max(1, int(os.environ.get("WARPCTCT_RANDOM_CASES_SCALE", "1")))
 LOSS_RTOL = 1e-5     # loss: relative
 GRAD_ATOL = 1e-4     # gradients: absolute
 
@@ -40,7 +46,7 @@ def test_random_joint_and_logits_cases(seed):
     Vs = [2, 3, 4, 5, 8, 31, 32, 33, 64, 100]
     dts = [torch.float32, torch.float32, torch.bfloat16, torch.float16]
     done = 0
-    while done < 600:
+    while done < 600 * SCALE:
         N, T = int(rng.integers(1, 5)), int(rng.choice(Ts))
         U, V = int(rng.choice(Us)), int(rng.choice(Vs))
         if N * T * (U + 1) * V > 3e6:
@@ -97,7 +103,7 @@ def test_random_joiner_cases(seed):
     Us = [0, 1, 15, 16, 31, 32, 47, 48, 63, 64, 79, 80, 95, 96, 97, 130]
     Vs = [3, 33, 256, 480, 511, 512, 544, 800, 1000, 1024, 1056, 2016, 2047, 2048, 2049, 2080, 2304]
     done = 0
-    while done < 150:
+    while done < 150 * SCALE:
         N, T = int(rng.integers(1, 4)), int(rng.choice(Ts))
         U, V = int(rng.choice(Us)), int(rng.choice(Vs))
         if T * (U + 1) * V * N > 40e6:
@@ -151,7 +157,7 @@ def test_random_log_matmul_cases(seed):
     Ks = [1, 2, 31, 32, 33, 64, 255, 256, 257, 300, 511, 512, 544, 800, 1024, 2047, 2048, 2049, 2304]
     Ns = [1, 2, 15, 16, 17, 32, 33, 48, 64, 80, 96, 97, 130, 200]
     done = 0
-    while done < 400:
+    while done < 400 * SCALE:
         B, M = int(rng.integers(1, 4)), int(rng.choice(Ms))
         K, Nn = int(rng.choice(Ks)), int(rng.choice(Ns))
         if rng.integers(0, 2):
@@ -220,7 +226,7 @@ def test_random_cases_of_the_operators_on_gathered_inputs(seed):
     Ts = [1, 2, 7, 8, 9, 12, 13, 24, 25, 37, 70, 140, 300]
     Us = [0, 1, 2, 5, 62, 63, 64, 65, 127, 128, 129, 200, 511, 512, 513, 600]
     done = 0
-    while done < 300:
+    while done < 300 * SCALE:
         N, T = int(rng.integers(1, 5)), int(rng.choice(Ts))
         U, V = int(rng.choice(Us)), int(rng.choice([3, 5, 9, 33]))
         if N * T * (U + 1) > 1.0e6:
