@@ -460,6 +460,12 @@ int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, lo
  *                                  hand-over (see warpctct_lattice_f32): the NaN
  *                                  costs / gradients of that call do not come
  *                                  from the inputs.
+ *   WARPCTCT_STATUS_LINEAR_FELL_BACK  the fused joiner forward swept a batch's
+ *                                  lattices in the linear domain, its check
+ *                                  refused the result, and the log-domain
+ *                                  kernels computed the batch again (the
+ *                                  results are those; see
+ *                                  warpctct_joiner_linear_lattice).
  * warpctct_status waits for the work queued on the current device
  * (hipDeviceSynchronize: the one entry point that does), copies the word to
  * *bits and, with clear != 0, sets it back to 0.  Bits set by launches that
@@ -467,9 +473,31 @@ int warpctct_logmm_bwd_f32(const float *grad_out, const float *lhs, long lsb, lo
 enum {
     WARPCTCT_STATUS_LABEL_RANGE = 1,
     WARPCTCT_STATUS_NAN_INPUT = 2,
-    WARPCTCT_STATUS_LOST_HAND_OVER = 4
+    WARPCTCT_STATUS_LOST_HAND_OVER = 4,
+    WARPCTCT_STATUS_LINEAR_FELL_BACK = 8
 };
 int warpctct_status(unsigned *bits, int clear);
+
+/* The fused joiner forward (warpctct_simple_forward_f32 / _reduced_f32 with
+ * gradients, U + 1 <= 512, long inputs) sweeps its lattices in the LINEAR domain first: path
+ * masses relative to one power of two per 64 contexts and 12 frames, two
+ * multiplications and three additions per frame where the log domain needs two
+ * semiring sums per state (less than half the time per frame; the frames of a
+ * lattice are strictly serial, so that is the latency of the whole call).  The
+ * linear form drops states that lie ~2^-1000 below the largest of their 64
+ * contexts.  The kernel that forms the gradients therefore checks that the
+ * posteriors of every frame add up to 1 within 2e-5, that every gathered unit
+ * lies in [2^-80, 2^80] or is 0, and that everything is finite; if not, the
+ * log-domain kernels, launched behind it in the same stream, compute the batch
+ * again (they return at once otherwise), and
+ * WARPCTCT_STATUS_LINEAR_FELL_BACK is set.  No counterpart in the reference
+ * (csrc/simple.cu sweeps in the log domain).  The linear sweeps save 25-50 ns
+ * per frame and cost ~14 us per call (the launches that return at once, a
+ * slower gather and gradient kernel), so they are used from T = 1024 frames on.
+ * warpctct_joiner_linear_lattice(n) moves that limit for later calls of the
+ * process (0: never; 1: always; negative: the default) and returns the
+ * previous one. */
+int warpctct_joiner_linear_lattice(int from_frames);
 
 /* ---- measurement aid ------------------------------------------------------
  * No counterpart in the reference.  warpctct_profile(1) clears earlier records

@@ -12,6 +12,7 @@ import numpy as np
 import pytest
 import torch
 
+import hip_lib
 from ctct_cases import make_joint_case, make_simple_case
 from oracle import c_oracle as C
 from oracle import ctct_oracle as O
@@ -109,9 +110,13 @@ def test_random_joiner_cases(seed):
         if T * (U + 1) * V * N > 40e6:
             continue
         normalized, mask = bool(rng.integers(0, 2)), int(rng.integers(0, 4)) == 0
+        # the lattices swept in the linear domain (with their check and the log
+        # domain as fall-back) in half of the cases, whatever the number of frames
+        linear = int(rng.integers(0, 2))
         case_seed = int(rng.integers(0, 1 << 30))
-        print("case N=%d T=%d U=%d V=%d normalized=%s mask=%s seed=%d"
-              % (N, T, U, V, normalized, mask, case_seed), flush=True)
+        print("case N=%d T=%d U=%d V=%d normalized=%s mask=%s linear=%d seed=%d"
+              % (N, T, U, V, normalized, mask, linear, case_seed), flush=True)
+        hip_lib.lib().warpctct_joiner_linear_lattice(linear)
         f, g, ys, lx, ly = make_simple_case(case_seed, N, T, U, V, normalized=normalized)
         if mask:
             cols = rng.integers(1, V, size=max(2, V // 7))
@@ -143,6 +148,7 @@ def test_random_joiner_cases(seed):
             np.testing.assert_allclose(tf.grad.cpu().numpy(), gf, atol=GRAD_ATOL * scale, rtol=1e-5)
             np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=GRAD_ATOL * scale, rtol=1e-5)
         done += 1
+    hip_lib.lib().warpctct_joiner_linear_lattice(-1)
 
 
 @pytest.mark.parametrize("seed", [31, 32])

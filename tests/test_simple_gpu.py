@@ -11,10 +11,23 @@ from ctct_cases import make_joint_case, make_simple_case
 from oracle import c_oracle as C
 from oracle import ctct_oracle as O
 
+import hip_lib
+
 pytestmark = pytest.mark.gpu
 
 LOSS_RTOL = 1e-5
 GRAD_ATOL = 1e-4
+
+
+@pytest.fixture(autouse=True, params=["log_lattices", "linear_lattices"])
+def lattice_domain(request):
+    """Every test of this file runs twice: with the joiner's lattices swept in the
+    log domain only, and with the linear sweeps (checked, with the log domain as
+    their fall-back) used for every input, not just from 1024 frames on."""
+    lib = hip_lib.lib()
+    before = lib.warpctct_joiner_linear_lattice(1 if request.param == "linear_lattices" else 0)
+    yield request.param
+    lib.warpctct_joiner_linear_lattice(before)
 
 
 def dev(a, dtype=None):
@@ -819,3 +832,103 @@ def test_full_size_unnormalized_stress_against_c_oracle():
     exp_g = torch.zeros_like(g.grad, dtype=torch.float64)
     exp_g.scatter_add_(-1, gi, torch.as_tensor(gg_ref).cuda())
     np.testing.assert_allclose(g.grad.cpu().numpy(), exp_g.cpu().numpy(), atol=GRAD_ATOL, rtol=1e-5)
+
+
+# ------------------------------------------------- lattices in the linear domain
+def _launched_kernels(run):
+    """Names of the library's kernels that `run` launches (its timing hook)."""
+    import ctypes
+    lib = hip_lib.lib()
+    torch.cuda.synchronize()
+    assert lib.warpctct_profile(1) == 0
+    try:
+        run()
+        torch.cuda.synchronize()
+    finally:
+        lib.warpctct_profile(0)
+    name, us = ctypes.c_char_p(), ctypes.c_float()
+    names = []
+    for i in range(lib.warpctct_profile_count()):
+        if lib.warpctct_profile_read(i, ctypes.byref(name), ctypes.byref(us)) == 0:
+            names.append(name.value.decode())
+    return names
+
+
+def _loss_and_grads(f, g, ys, lx, ly, normalized, reduction="none", w=None):
+    import warp_ctct
+    tf, tg = dev(f).requires_grad_(True), dev(g).requires_grad_(True)
+    out = warp_ctct.ctct_simple_loss(tf, tg, dev(ys), dev(lx), dev(ly), reduction=reduction,
+                                     normalized=normalized)
+    (out * dev(w, torch.float32)).sum().backward() if w is not None else out.sum().backward()
+    return out.detach(), tf.grad, tg.grad
+
+
+@pytest.mark.parametrize("normalized", [True, False])
+def test_linear_lattices_are_used_from_1024_frames_and_hold_on_ordinary_input(normalized, lattice_domain):
+    """With the default setting the fused forward sweeps in the linear domain from
+    1024 frames on (lattice_lin_kernel is launched, the log-domain kernels behind it
+    return at once: the fall-back bit stays clear), and below that in the log
+    domain; both agree with the oracle.  A chain of two workgroups per lattice."""
+    import warp_ctct
+    lib = hip_lib.lib()
+    lib.warpctct_joiner_linear_lattice(-1)
+    for T, linear in ((1030, True), (1000, False)):
+        N, U, V = 2, 70, 24
+        f, g, ys, lx, ly = make_simple_case(60 + T, N, T, U, V, lx=[T, T - 37], ly=[U, 41],
+                                            normalized=normalized)
+        w = np.array([0.7, -1.3])
+        _, gf, gg, costs = O.ctct_simple_loss(f, g, ys, lx, ly, reduction="none", normalized=normalized,
+                                              grad_output=w)
+        warp_ctct.status(reset=True)
+        got = {}
+        names = _launched_kernels(lambda: got.update(r=_loss_and_grads(f, g, ys, lx, ly, normalized, w=w)))
+        assert any("lattice_lin_kernel" in k for k in names) == linear, names
+        assert not (warp_ctct.status(reset=True) & warp_ctct.STATUS_LINEAR_FELL_BACK)
+        out, df, dg = got["r"]
+        np.testing.assert_allclose(out.cpu().numpy(), costs, rtol=LOSS_RTOL)
+        np.testing.assert_allclose(df.cpu().numpy(), gf, atol=GRAD_ATOL * 1.3, rtol=1e-5)
+        np.testing.assert_allclose(dg.cpu().numpy(), gg, atol=GRAD_ATOL * 1.3, rtol=1e-5)
+
+
+@pytest.mark.parametrize("what", ["unit_out_of_range", "infeasible_sample", "mass_beyond_the_range"])
+def test_linear_lattices_fall_back_to_the_log_domain(what, lattice_domain):
+    """Input that the linear sweeps cannot take is computed again in the log
+    domain, in the same call: the results are bit for bit those of a call with the
+    linear sweeps switched off, and the status word says so.
+    - a gathered unit below 2^-80 (a frame whose label scores are ~-200);
+    - a sample with fewer frames than its labels need (cost +inf, NaN gradients);
+    - all units in range, but the mass that counts far below the largest state of
+      its 64 contexts: the one label can only be emitted in the first three frames
+      (log 0 afterwards), and the blank behind it scores -50 per frame, while the
+      blank before it scores 0 and keeps context 0 at mass 1: context 1 falls by
+      2^-72 per frame, is gone from the linear sweep after 15 frames, and the
+      total mass comes out as 0, which the check refuses."""
+    import warp_ctct
+    lib = hip_lib.lib()
+    N, T, U, V = 2, 64, 6, 11
+    f, g, ys, lx, ly = make_simple_case(77, N, T, U, V, lx=[T, T - 9], ly=[U, 4], normalized=False)
+    if what == "unit_out_of_range":
+        f[0, 20, :] = -200.0
+    elif what == "infeasible_sample":
+        lx[1] = 3
+    else:
+        N, T, U, V = 1, 400, 1, 4
+        f = np.zeros((N, T, V), np.float32)
+        g = np.zeros((N, U + 1, V), np.float32)
+        ys = np.array([[2]], np.int32)
+        lx, ly = np.array([T], np.int32), np.array([U], np.int32)
+        f[0, 3:, 2] = -np.inf
+        g[0, 1, 0] = -50.0
+    results = []
+    for frames in (0, 1):
+        lib.warpctct_joiner_linear_lattice(frames)
+        warp_ctct.status(reset=True)
+        results.append(_loss_and_grads(f, g, ys, lx, ly, False))
+        bits = warp_ctct.status(reset=True)
+        assert bool(bits & warp_ctct.STATUS_LINEAR_FELL_BACK) == (frames == 1), (what, bits)
+    for a, b in zip(*results):
+        assert torch.equal(torch.nan_to_num(a, nan=7.0), torch.nan_to_num(b, nan=7.0)), what
+    _, gf, gg, costs = O.ctct_simple_loss(f, g, ys, lx, ly, reduction="none", normalized=False)
+    if what != "infeasible_sample":
+        np.testing.assert_allclose(results[1][0].cpu().numpy(), costs, rtol=LOSS_RTOL)
+        np.testing.assert_allclose(results[1][1].cpu().numpy(), gf, atol=GRAD_ATOL, rtol=1e-5)

@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "launch.h"
@@ -84,10 +85,24 @@ int forward_from_units(const Workspace &w, const int *ys, const int *lx, const i
                                   stream));
 }
 
+// from how many frames on the fused joiner forward sweeps its lattices in the
+// linear domain first (warpctct_joiner_linear_lattice; 0: never).  The linear
+// sweeps save 25-50 ns per frame (less with many lattices in flight, whose
+// sweeps are slowed by the memory system, more for a few long ones) and cost
+// ~14 us per call (three launches that return at once, a slower gather and
+// gradient kernel): from 1024 frames on they never lose.
+constexpr int kLinearFromFrames = 1024;
+std::atomic<int> g_linear_from{kLinearFromFrames};
+
 struct SimpleWorkspace {
     Workspace lattice;
     float *unit_grads;   // (N,T,U+1,3)
     float *partial;      // logmm_fwd_partial_floats: partial sums of a split log-matmul reduction
+    // for the lattices in the linear domain (launch_lattice_lin): relay slots,
+    // scales, and the flag that sends the batch through the log-domain kernels
+    void *lin_relay;
+    int *lin_scales;
+    unsigned *lin_flag;
     size_t bytes;
 };
 
@@ -98,7 +113,13 @@ SimpleWorkspace carve_simple(void *base, int N, int T, int U) {
     const size_t ug_b = align256((size_t)N * T * (U + 1) * 3 * sizeof(float));
     w.unit_grads = reinterpret_cast<float *>(p);
     w.partial = reinterpret_cast<float *>(p + ug_b);
-    w.bytes = w.lattice.bytes + ug_b + align256(logmm_fwd_partial_floats(N, T, U + 1) * sizeof(float));
+    const size_t partial_b = align256(logmm_fwd_partial_floats(N, T, U + 1) * sizeof(float));
+    const size_t relay_b = align256(lattice_lin_relay_slots(N, T, U) * sizeof(unsigned long long));
+    const size_t scales_b = align256(lattice_lin_scales(N, T, U) * sizeof(int));
+    w.lin_relay = relay_b ? reinterpret_cast<void *>(p + ug_b + partial_b) : nullptr;
+    w.lin_scales = reinterpret_cast<int *>(p + ug_b + partial_b + relay_b);
+    w.lin_flag = reinterpret_cast<unsigned *>(p + ug_b + partial_b + relay_b + scales_b);
+    w.bytes = w.lattice.bytes + ug_b + partial_b + relay_b + scales_b + 256;
     return w;
 }
 
@@ -180,7 +201,7 @@ int static_scratch(void **out) {
 int simple_from_units(const SimpleWorkspace &w, const int *ys, const int *lx, const int *ly, int N,
                       int T, int U, float *costs, float *grad_f, float *grad_g, float *grad_den,
                       bool want_grad, bool relay_is_clear, const CostReduce &reduce,
-                      hipStream_t stream) {
+                      hipStream_t stream, const unsigned *only_if = nullptr) {
     // alpha is needed only for the gradients; those are reduced straight from the
     // lattices (the unit-gradient region of the workspace holds the partial sums)
     LatticeArgs a = {};
@@ -198,10 +219,11 @@ int simple_from_units(const SimpleWorkspace &w, const int *ys, const int *lx, co
     a.U = U;
     a.beta_only = !want_grad;
     a.reduce = reduce;
-    int rc = done(launch_lattice(a, stream));
+    // only_if: the run behind the lattices in the linear domain (see the caller)
+    int rc = done(launch_lattice(a, stream, only_if));
     if (rc != WARPCTCT_OK || !want_grad) return rc;
     return done(launch_simple_grads(w.lattice.units, ys, lx, ly, w.lattice.alphas, w.lattice.betas,
-                                    w.unit_grads, grad_f, grad_g, grad_den, N, T, U, stream));
+                                    w.unit_grads, grad_f, grad_g, grad_den, N, T, U, stream, only_if));
 }
 
 }  // namespace
@@ -261,6 +283,11 @@ int warpctct_simple_units_f32(const float *f_g, const float *g_g, const float *d
 }
 
 int warpctct_lattice_wait_limit(int spins) { return lattice_wait_limit(spins); }
+
+int warpctct_joiner_linear_lattice(int from_frames) {
+    return g_linear_from.exchange(from_frames < 0 ? kLinearFromFrames : from_frames,
+                                  std::memory_order_relaxed);
+}
 
 size_t warpctct_lattice_relay_bytes(int N, int T, int U) {
     if (N < 0 || T < 0 || U < 0) return 0;
@@ -750,6 +777,42 @@ int warpctct_simple_forward_reduced_f32(const float *f, const float *g, const in
             rc = done(launch_logmm_fwd(lhs, rhs, sh, den, w.partial, N, T, V, U + 1, lx, ly,
                                        &deferred, st));
             if (rc != WARPCTCT_OK) return rc;
+        }
+        const int linear_from = g_linear_from.load(std::memory_order_relaxed);
+        if (want_grad && linear_from > 0 && T >= linear_from && simple_grads_lin_applies(T, U)) {
+            // The lattices in the linear domain (less than half the time per frame),
+            // checked by the kernel that forms the gradients from them; the
+            // log-domain kernels follow and return at once unless that check, or
+            // anything else on the way, has raised the flag.
+            RelaySlots lin_slots;
+            lin_slots.n = w.lin_relay ? lattice_lin_relay_slots(N, T, U) : 0;
+            lin_slots.p = lin_slots.n ? static_cast<unsigned long long *>(w.lin_relay) : nullptr;
+            int rc = done(launch_simple_gather_units(f, g, normalized ? den : nullptr, ys, lx, ly,
+                                                     w.lattice.units, N, T, U, V, lin_slots, deferred,
+                                                     fmax, reduce.counter, st, w.lin_flag));
+            if (rc != WARPCTCT_OK) return rc;
+            LatticeArgs a = {};
+            a.units = w.lattice.units;
+            a.ys = ys, a.lx = lx, a.ly = ly;
+            a.alphas = w.lattice.alphas, a.betas = w.lattice.betas;
+            a.relay = w.lin_relay, a.relay_is_clear = true;
+            a.costs = costs;
+            a.N = N, a.T = T, a.U = U;
+            a.reduce = reduce;
+            rc = done(launch_lattice_lin(a, w.lin_scales, w.lin_flag, st));
+            if (rc != WARPCTCT_OK) return rc;
+            rc = done(launch_simple_grads_lin(w.lattice.units, ys, lx, ly, w.lattice.alphas,
+                                              w.lattice.betas, w.lin_scales, w.unit_grads, grad_f,
+                                              normalized ? grad_den : nullptr, N, T, U, w.lin_flag, st));
+            if (rc != WARPCTCT_OK) return rc;
+            rc = done(launch_simple_gather_units(f, g, normalized ? den : nullptr, ys, lx, ly,
+                                                 w.lattice.units, N, T, U, V,
+                                                 relay_slots_of(w.lattice.relay, N, T, U), deferred,
+                                                 fmax, reduce.counter, st, nullptr, w.lin_flag));
+            if (rc != WARPCTCT_OK) return rc;
+            return simple_from_units(w, ys, lx, ly, N, T, U, costs, grad_f, grad_g,
+                                     normalized ? grad_den : nullptr, true, true, reduce, st,
+                                     w.lin_flag);
         }
         int rc = done(launch_simple_gather_units(f, g, normalized ? den : nullptr, ys, lx, ly,
                                                  w.lattice.units, N, T, U, V,

@@ -38,6 +38,7 @@
 // (csrc/gather.cu:36-291) and their global-memory spin-lock row pipeline.
 #include <atomic>
 
+#include "cost_reduce.h"
 #include "device_utils.h"
 #include "launch.h"
 
@@ -440,28 +441,7 @@ static __device__ __forceinline__ void lattice_block(const double *__restrict__ 
     }
     if (wave != 0) return;
     // thread 0 (context 0) has just written costs[n]
-    const int lane = threadIdx.x;
-    if (red.average_frames && lane == 0) costs[n] /= (float)lx[n];
-    if (red.reduced == nullptr) return;
-    // Reduction over the batch (warp_ctct/__init__.py:142-147 of the reference)
-    // by the workgroup that finishes last: every workgroup publishes its cost
-    // (release fence), then counts itself; the one that sees N-1 earlier
-    // arrivals reads all N costs (acquire fence) and adds them in a fixed
-    // order, so the result does not depend on the order of arrival.
-    int last = 0;
-    if (lane == 0) {
-        __threadfence();
-        last = (atomicAdd(red.counter, 1u) == (unsigned)(N - 1)) ? 1 : 0;
-    }
-    last = __shfl(last, 0, 64);
-    if (!last) return;
-    __threadfence();
-    float s = 0.0f;
-    for (int i = lane; i < N; i += 64)
-        s += __hip_atomic_load(costs + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) s += __shfl_xor(s, off, 64);
-    if (lane == 0) *red.reduced = (red.mode == 2) ? s / (float)N : s;
+    cost_reduce_tail(red, costs, lx, n, N, threadIdx.x);
 }
 
 };
@@ -476,7 +456,13 @@ __global__ __launch_bounds__(64) void lattice_kernel(const double *__restrict__ 
                                                      unsigned long long *__restrict__ relay, int N,
                                                      int T, int U, int W, int dirs, int chains_pad,
                                                      const CostReduce red, int max_spins,
-                                                     unsigned *__restrict__ status) {
+                                                     unsigned *__restrict__ status,
+                                                     const unsigned *__restrict__ only_if) {
+    if (only_if) {
+        // the fall-back of the linear lattices: nothing to do while their flag is down
+        if (*only_if == 0u) return;
+        if (blockIdx.x == 0 && threadIdx.x == 0 && status) atomicOr(status, kStatusLinearFellBack);
+    }
     Chunked<12>::lattice_block(units, ys, lx, ly, alphas, betas, costs, relay, N, T, U, W, dirs,
                                chains_pad, red, max_spins, status);
 }
@@ -509,6 +495,8 @@ namespace {
 std::atomic<int> g_wait_limit{kMaxSpins};
 }
 
+int lattice_wait_limit_now() { return g_wait_limit.load(std::memory_order_relaxed); }
+
 int lattice_wait_limit(int spins) {
     return g_wait_limit.exchange(spins < 0 ? kMaxSpins : spins, std::memory_order_relaxed);
 }
@@ -518,7 +506,7 @@ size_t lattice_relay_slots(int N, int T, int U) {
     return (size_t)N * 2 * (size_t)(W - 1) * ((size_t)T + kRelayPad);
 }
 
-hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream) {
+hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream, const unsigned *only_if) {
     if (a.N == 0) return hipSuccess;
     const int W = (a.U + 1 + 63) / 64;
     const size_t slots = lattice_relay_slots(a.N, a.T, a.U);
@@ -537,12 +525,14 @@ hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream) {
         relay = nullptr;
     }
     const int max_spins = g_wait_limit.load(std::memory_order_relaxed);
-    unsigned *status = W > 1 ? device_status_word() : nullptr;   // only chains can lose a hand-over
+    // (only chains can lose a hand-over; a fall-back reports itself)
+    unsigned *status = (W > 1 || only_if) ? device_status_word() : nullptr;
     const int dirs = a.beta_only ? 1 : 2;
     const long chains = (long)a.N * dirs;
     const long chains_pad = (chains + 7) / 8 * 8;
     if (chains_pad * W > 0x7fffffffL) return hipErrorInvalidValue;
     if (a.fill.n4 > 0) {
+        if (only_if) return hipErrorInvalidValue;
         const size_t blocks = (size_t)(chains_pad * W) + (a.fill.n4 + 255) / 256;
         if (blocks > 0x7fffffffUL) return hipErrorInvalidValue;
         TIMED_LAUNCH(lattice_fill_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a.units,
@@ -553,7 +543,7 @@ hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream) {
     }
     TIMED_LAUNCH(lattice_kernel, dim3((unsigned)(chains_pad * W)), dim3(64), 0, stream, a.units,
                  a.ys, a.lx, a.ly, a.alphas, a.betas, a.costs, relay, a.N, a.T, a.U, W, dirs,
-                 (int)chains_pad, a.reduce, max_spins, status);
+                 (int)chains_pad, a.reduce, max_spins, status, only_if);
     return hipGetLastError();
 }
 

@@ -23,6 +23,7 @@ inline bool io_valid(int t) { return t == kIoF32 || t == kIoF16 || t == kIoBF16;
 constexpr unsigned kStatusLabelRange = 1u;     // a label outside [0, V) was clamped
 constexpr unsigned kStatusNanInput = 2u;       // a gathered log-probability was NaN
 constexpr unsigned kStatusLostHandOver = 4u;   // a chain of workgroups gave up waiting
+constexpr unsigned kStatusLinearFellBack = 8u; // the joiner's linear lattices were computed again in the log domain
 // The current device's status word, for kernels to set bits in (atomic OR), or
 // null when it cannot be found (kernels then report nothing).
 unsigned *device_status_word();
@@ -108,7 +109,28 @@ __device__ __forceinline__ void relay_clear_share(const RelaySlots &r) {
 // default, about a second).  Applies to launches made afterwards; returns the
 // previous limit.
 int lattice_wait_limit(int spins);
-hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream);
+int lattice_wait_limit_now();   // the limit in force
+// only_if (may be null): the kernel returns at once while *only_if is 0 (see
+// launch_lattice_lin: the log-domain lattices as the fall-back of the linear ones)
+hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream, const unsigned *only_if = nullptr);
+
+// ---- the joiner's lattices in the linear domain (lattice_lin.hip) -------------
+// Sweeps on path masses relative to a power of two per wavefront and chunk of
+// kLinChunk frames; alphas / betas then hold (N,T+1,P,2) pairs {o, e} of masses,
+// `scales` lattice_lin_scales(N,T,U) exponents: entry
+//   ((n*2 + d)*W + w)*(lin_chunks(T) + 1) + i,   d = 0: beta, 1: alpha,
+// with i = 0 for the initial row (alpha: frame 0, beta: frame Tn) and
+// i = 1 + step / kLinChunk for the row stored by that step (alpha: step = frame - 1,
+// beta: step = Tn - 1 - frame).  units are linear too (2^(log2 unit), neutral
+// {1, 1, 0}).  a.relay needs lattice_lin_relay_slots 64-bit words, cleared to
+// kRelayEmpty (a.relay_is_clear); *flag is raised where a hand-over was lost.
+// The results are only meaningful together with the check of the kernel that
+// reads them (launch_simple_grads_lin).
+constexpr int kLinChunk = 12;
+__host__ __device__ inline int lin_chunks(int T) { return (T + kLinChunk - 1) / kLinChunk; }
+size_t lattice_lin_relay_slots(int N, int T, int U);
+size_t lattice_lin_scales(int N, int T, int U);
+hipError_t launch_lattice_lin(const LatticeArgs &a, int *scales, unsigned *flag, hipStream_t stream);
 
 // Element strides of a joint tensor (N,T,U+1,V); dense row-major is
 // {T*(U+1)*V, (U+1)*V, V, 1}.
@@ -179,11 +201,16 @@ struct LogmmDeferred {
 };
 // den (N,T,U+1): read, or, with `deferred.partial`, computed from the deferred
 // pass and written, together with fmax (N,T) (-inf for frames beyond lx).
+// linear_flag (may be null): the units are stored in the linear domain, for
+// launch_lattice_lin, and *linear_flag is lowered; only_if (may be null): the
+// kernel returns at once while *only_if is 0.
 hipError_t launch_simple_gather_units(const float *f, const float *g, float *den, const int *ys,
                                       const int *lx, const int *ly, double *units, int N, int T,
                                       int U, int V, const RelaySlots &relay,
                                       const LogmmDeferred &deferred, float *fmax,
-                                      unsigned *counter, hipStream_t stream);
+                                      unsigned *counter, hipStream_t stream,
+                                      unsigned *linear_flag = nullptr,
+                                      const unsigned *only_if = nullptr);
 // compact gradients of the joiner path straight from the lattices: grad_f
 // (N,T,U+1), grad_g (N,U+1,3), grad_den (N,T,U+1) or null; `partial` is scratch
 // of N * T * (U+1) * 3 floats (partial sums over blocks of 8 frames, or, for
@@ -191,7 +218,17 @@ hipError_t launch_simple_gather_units(const float *f, const float *g, float *den
 hipError_t launch_simple_grads(const double *units, const int *ys, const int *lx, const int *ly,
                                const double *alphas, const double *betas, float *partial,
                                float *grad_f, float *grad_g, float *grad_den, int N, int T, int U,
-                               hipStream_t stream);
+                               hipStream_t stream, const unsigned *only_if = nullptr);
+// The same from lattices in the linear domain, without the last sum over the
+// blocks of frames (launch_simple_grads with only_if behind it does that sum
+// whether it recomputes or not); raises *flag where the linear lattices cannot
+// be trusted (posteriors of a frame not adding up to 1, a unit out of range,
+// anything not finite).  Needs simple_grads_lin_applies(T, U).
+bool simple_grads_lin_applies(int T, int U);
+hipError_t launch_simple_grads_lin(const double *units, const int *ys, const int *lx, const int *ly,
+                                   const double *alphas, const double *betas, const int *scales,
+                                   float *partial, float *grad_f, float *grad_den, int N, int T,
+                                   int U, unsigned *flag, hipStream_t stream);
 hipError_t launch_simple_reduce(const float *unit_grads, float *grad_f, float *grad_g,
                                 float *grad_den, int N, int T, int U, hipStream_t stream);
 // dense_f and dense_g of the unnormalised path in one pass (zeros + scattered

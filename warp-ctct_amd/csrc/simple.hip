@@ -32,16 +32,35 @@ __device__ __forceinline__ int clampi(int v, int lo, int hi) { return min(max(v,
 // last pass (the sum over the slabs of the reduction, LogmmDeferred) to this
 // kernel: every cell u <= ly of a live frame computes its den[t,u], writes it
 // (the backward reads all of them), and context 0 writes the frame's fmax.
-template <bool DEFERRED>
+// LINEAR: the units are stored as 2^(log2 unit), for the lattices in the linear
+// domain (lattice_lin.hip): neutral units are {1, 1, 0}, log 0 is 0.  That
+// variant also lowers `flag`, which the kernels behind it raise.
+// only_if (may be null): return at once while *only_if is 0 (the fall-back run
+// of the log-domain variant behind the linear lattices).
+template <bool LINEAR>
+__device__ __forceinline__ double unit_out(double log2_unit) {
+    if (!LINEAR) return log2_unit;
+    if (log2_unit == neg_inf()) return 0.0;
+    // 2^x = 2^floor(x) * 2^frac, the second factor on the fp32 transcendental unit
+    // (relative error ~1e-7 per unit, without bias: a product of a thousand
+    // units is off by a few 1e-6, the cost by as much in absolute terms)
+    const double fl = __builtin_floor(log2_unit);
+    const double clamped = __builtin_fmin(__builtin_fmax(fl, -2000.0), 2000.0);
+    return __builtin_amdgcn_ldexp((double)exp2_hw((float)(log2_unit - fl)), (int)clamped);
+}
+
+template <bool DEFERRED, bool LINEAR>
 __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     const float *__restrict__ f, const float *__restrict__ g, float *__restrict__ den,
     const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
     double *__restrict__ units, int T, int U, int V, int P, const RelaySlots relay,
     const LogmmDeferred deferred, float *__restrict__ fmax, unsigned *__restrict__ counter,
-    unsigned *__restrict__ status) {
+    unsigned *__restrict__ status, unsigned *__restrict__ flag, const unsigned *__restrict__ only_if) {
+    if (only_if && *only_if == 0u) return;
     relay_clear_share(relay);
     // (the arrival counter of the lattice kernel's cost reduction, if there is one)
     if (counter && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *counter = 0u;
+    if (LINEAR && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *flag = 0u;
     const int U1 = U + 1;
     const int n = blockIdx.y;
     const int cell = blockIdx.x * kBlock + threadIdx.x;
@@ -79,9 +98,9 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     // padding context of a live frame, or a cell outside the band of complete
     // alignments (its units cannot influence costs or gradients): neutral units
     if (!live) {
-        o[0] = 0.0;
-        o[1] = 0.0;
-        o[2] = neg_inf();
+        o[0] = LINEAR ? 1.0 : 0.0;
+        o[1] = LINEAR ? 1.0 : 0.0;
+        o[2] = LINEAR ? 0.0 : neg_inf();
         return;
     }
     const float *gr = g + ((size_t)n * U1 + u) * V;
@@ -93,14 +112,14 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     // a NaN unit (NaN in f, g or den) enters the lattice as log 0 and is reported
     if (b != b || cur != cur || nxt != nxt) {
         if (status) atomicOr(status, kStatusNanInput);
-        o[0] = (b != b) ? neg_inf() : b * kLog2e;
-        o[1] = (cur != cur) ? neg_inf() : cur * kLog2e;
-        o[2] = (nxt != nxt) ? neg_inf() : nxt;
+        o[0] = unit_out<LINEAR>((b != b) ? neg_inf() : b * kLog2e);
+        o[1] = unit_out<LINEAR>((cur != cur) ? neg_inf() : cur * kLog2e);
+        o[2] = unit_out<LINEAR>((nxt != nxt) ? neg_inf() : nxt);
         return;
     }
-    o[0] = b * kLog2e;
-    o[1] = cur * kLog2e;
-    o[2] = nxt;
+    o[0] = unit_out<LINEAR>(b * kLog2e);
+    o[1] = unit_out<LINEAR>(cur * kLog2e);
+    o[2] = unit_out<LINEAR>(nxt);
 }
 
 // Per frame: grad_den[t,u] = -(g0+g1+g2), grad_f[t,u>=1] = g1[t,u] + g2[t,u-1],
@@ -166,15 +185,29 @@ __global__ __launch_bounds__(kBlock) void simple_reduce_contexts_kernel(
 //   partial[n,block,u,k] = sum over the block's frames of g_k[t,u]
 // and simple_sum_partials_kernel adds the blocks up in a fixed order.
 constexpr int kFramesPerBlock = 8;
+// how far the posteriors of a frame may be from adding up to 1 before the
+// linear lattices are given up (their own rounding stays below 1e-6)
+constexpr float kPosteriorSlack = 2e-5f;
 
+// LIN: the lattices are those of lattice_lin.hip (linear domain; `scales` as
+// launch_lattice_lin describes them), and the kernel checks what it hands out:
+// the posteriors of a frame add up to 1 (every alignment consumes exactly one
+// unit per frame), every number is finite, and no unit lies outside the range
+// the linear sweeps can take.  Where a check fails it raises *flag, and the
+// log-domain kernels launched behind it (only_if) compute the batch again.
+// only_if (may be null): return at once while *only_if is 0.
+template <bool LIN>
 __global__ __launch_bounds__(512) void simple_grads_kernel(
     const double *__restrict__ units, const int *__restrict__ ys, const int *__restrict__ lx,
     const int *__restrict__ ly, const double *__restrict__ alphas,
     const double *__restrict__ betas, float *__restrict__ grad_f, float *__restrict__ grad_den,
-    float *__restrict__ partial, int T, int U, int P) {
+    float *__restrict__ partial, int T, int U, int P, const int *__restrict__ scales,
+    unsigned *__restrict__ flag, const unsigned *__restrict__ only_if) {
+    if (only_if && *only_if == 0u) return;
     constexpr int F = kFramesPerBlock;
     __shared__ float s_g2[F][512];
     __shared__ float s_blank[F][8];
+    __shared__ float s_all[F][8];
     const int U1 = U + 1;
     const int n = blockIdx.y, u = threadIdx.x;
     const int lane = u & 63, wave = u >> 6, waves = P >> 6;
@@ -184,16 +217,45 @@ __global__ __launch_bounds__(512) void simple_grads_kernel(
     const double *alpha_n = alphas + (size_t)n * lat, *beta_n = betas + (size_t)n * lat;
     const int *y = ys + (size_t)n * U;
     const int t_begin = blockIdx.x * F;
+    // LIN: the scales of this context's 64 and of the next context's (the same
+    // but for lane 63), and the lattice's total mass: beta(0, state 0)
+    const int chunks1 = lin_chunks(T) + 1;
+    const int *sc_beta = nullptr, *sc_beta_next = nullptr, *sc_alpha = nullptr;
+    double inv_ll = 0.0;
+    int s_ll = 0;
+    if (LIN) {
+        const int w_next = min((u + 1) >> 6, waves - 1);
+        sc_beta = scales + (((size_t)n * 2 + 0) * waves + wave) * chunks1;
+        sc_beta_next = scales + (((size_t)n * 2 + 0) * waves + w_next) * chunks1;
+        sc_alpha = scales + (((size_t)n * 2 + 1) * waves + wave) * chunks1;
+        const double ll = beta_n[1];
+        const int ex = (ll > 0.0 && ll < __builtin_huge_val()) ? __builtin_amdgcn_frexp_exp(ll) : 0;
+        inv_ll = 1.0 / __builtin_amdgcn_ldexp(ll, -ex);   // (0 or inf: NaN below, caught by the check)
+        // row 0 of beta was stored by step Tn - 1 of context 0's wavefront
+        s_ll = ex + scales[(((size_t)n * 2 + 0) * waves + 0) * chunks1 + (Tn > 0 ? 1 + (Tn - 1) / kLinChunk : 0)];
+    }
     // all frames of the block first (their loads are independent), then one exchange
     UnitGrad g[F];
     float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f;
+    bool bad_unit = false;
 #pragma unroll
     for (int f = 0; f < F; ++f) {
         const int t = t_begin + f;
         g[f] = UnitGrad{0.0f, 0.0f, 0.0f};
         // padding and cells outside the band of complete alignments: exactly zero
-        if (t < Tn && u <= Un && !outside_band(t, u, Tn, Un))
-            g[f] = unit_grad_cell(units_n, alpha_n, beta_n, y, t, u, Un, P);
+        if (t < Tn && u <= Un && !outside_band(t, u, Tn, Un)) {
+            if (LIN) {
+                // row t of alpha: step t - 1; row t + 1 of beta: step Tn - 2 - t
+                const int ia = t > 0 ? 1 + (t - 1) / kLinChunk : 0;
+                const int ib = t + 1 < Tn ? 1 + (Tn - 2 - t) / kLinChunk : 0;
+                bool bad;
+                g[f] = unit_grad_cell_lin(units_n, alpha_n, beta_n, y, t, u, Un, P, sc_alpha[ia],
+                                          sc_beta[ib], sc_beta_next[ib], inv_ll, s_ll, bad);
+                bad_unit = bad_unit || bad;
+            } else {
+                g[f] = unit_grad_cell(units_n, alpha_n, beta_n, y, t, u, Un, P);
+            }
+        }
         a0 += g[f].g0;
         a1 += g[f].g1;
         a2 += g[f].g2;
@@ -205,8 +267,28 @@ __global__ __launch_bounds__(512) void simple_grads_kernel(
         for (int off = 32; off >= 1; off >>= 1) blank += __shfl_xor(blank, off, 64);
         s_g2[f][u] = g[f].g2;
         if (lane == 0) s_blank[f][wave] = blank;
+        // The check: mass that the linear sweeps have lost is missing from every
+        // later frame's posteriors (alpha) or shows in them as a surplus (beta:
+        // the total they are divided by came out too small), so the first frame
+        // of each block and the sample's last frame are enough to look at.
+        if (LIN && (f == 0 || t_begin + f == Tn - 1)) {
+            float all = g[f].g0 + g[f].g1 + g[f].g2;
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) all += __shfl_xor(all, off, 64);
+            if (lane == 0) s_all[f][wave] = all;
+        }
     }
     __syncthreads();
+    if (LIN) {
+        if (u < F && (u == 0 || t_begin + u == Tn - 1)) {
+            const int t = t_begin + u;
+            float all = 0.0f;
+            for (int w = 0; w < waves; ++w) all += s_all[u][w];
+            // (a NaN fails the comparison too)
+            if (t < Tn && !(__builtin_fabsf(all + 1.0f) <= kPosteriorSlack)) atomicOr(flag, 1u);
+        }
+        if (__ballot(bad_unit) != 0ULL && lane == 0) atomicOr(flag, 1u);
+    }
     if (u >= U1) return;
 #pragma unroll
     for (int f = 0; f < F; ++f) {
@@ -426,29 +508,52 @@ hipError_t launch_simple_gather_units(const float *f, const float *g, float *den
                                       const int *lx, const int *ly, double *units, int N, int T,
                                       int U, int V, const RelaySlots &relay,
                                       const LogmmDeferred &deferred, float *fmax,
-                                      unsigned *counter, hipStream_t stream) {
+                                      unsigned *counter, hipStream_t stream, unsigned *linear_flag,
+                                      const unsigned *only_if) {
     const int P = padded_contexts(U);
     const long cells = (long)T * P;
     const dim3 grid((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N);
+    if (deferred.partial && (!den || !fmax || deferred.splits < 1 || deferred.splits > 8 ||
+                             deferred.B != N || deferred.Nn != U + 1))
+        return hipErrorInvalidValue;
+    unsigned *status = device_status_word();
+#define GATHER(DEF, LIN)                                                                            \
+    TIMED_LAUNCH((simple_gather_units_kernel<DEF, LIN>), grid, dim3(kBlock), 0, stream, f, g, den,  \
+                 ys, lx, ly, units, T, U, V, P, relay, deferred, fmax, counter, status,             \
+                 linear_flag, only_if)
     if (deferred.partial) {
-        if (!den || !fmax || deferred.splits < 1 || deferred.splits > 8 || deferred.B != N ||
-            deferred.Nn != U + 1)
-            return hipErrorInvalidValue;
-        TIMED_LAUNCH(simple_gather_units_kernel<true>, grid, dim3(kBlock), 0, stream, f, g, den, ys,
-                     lx, ly, units, T, U, V, P, relay, deferred, fmax, counter, device_status_word());
+        if (linear_flag) GATHER(true, true); else GATHER(true, false);
     } else {
-        TIMED_LAUNCH(simple_gather_units_kernel<false>, grid, dim3(kBlock), 0, stream, f, g, den, ys,
-                     lx, ly, units, T, U, V, P, relay, deferred, fmax, counter, device_status_word());
+        if (linear_flag) GATHER(false, true); else GATHER(false, false);
     }
+#undef GATHER
+    return hipGetLastError();
+}
+
+// The first half of launch_simple_grads for lattices in the linear domain (see
+// simple_grads_kernel<true>): grad_f, grad_den and the partial sums of grad_g;
+// the caller adds those up with launch_simple_grads' second half afterwards.
+bool simple_grads_lin_applies(int T, int U) { return T > 0 && padded_contexts(U) <= 512; }
+
+hipError_t launch_simple_grads_lin(const double *units, const int *ys, const int *lx, const int *ly,
+                                   const double *alphas, const double *betas, const int *scales,
+                                   float *partial, float *grad_f, float *grad_den, int N, int T,
+                                   int U, unsigned *flag, hipStream_t stream) {
+    if (!simple_grads_lin_applies(T, U) || !scales || !flag) return hipErrorInvalidValue;
+    const int P = padded_contexts(U);
+    const int blocks = (T + kFramesPerBlock - 1) / kFramesPerBlock;
+    TIMED_LAUNCH(simple_grads_kernel<true>, dim3(blocks, N), dim3(P), 0, stream, units, ys, lx, ly,
+                 alphas, betas, grad_f, grad_den, partial, T, U, P, scales, flag, nullptr);
     return hipGetLastError();
 }
 
 hipError_t launch_simple_grads(const double *units, const int *ys, const int *lx, const int *ly,
                                const double *alphas, const double *betas, float *partial,
                                float *grad_f, float *grad_g, float *grad_den, int N, int T, int U,
-                               hipStream_t stream) {
+                               hipStream_t stream, const unsigned *only_if) {
     const int P = padded_contexts(U);
     if (P > 512) {
+        if (only_if) return hipErrorInvalidValue;
         // more contexts than one workgroup of the fused kernel holds: unit
         // gradients into `partial` (it has room for all of them), then the two
         // reductions over them
@@ -458,8 +563,9 @@ hipError_t launch_simple_grads(const double *units, const int *ys, const int *lx
     }
     const int blocks = (T + kFramesPerBlock - 1) / kFramesPerBlock;
     if (T > 0) {
-        TIMED_LAUNCH(simple_grads_kernel, dim3(blocks, N), dim3(P), 0, stream, units, ys, lx,
-                           ly, alphas, betas, grad_f, grad_den, partial, T, U, P);
+        TIMED_LAUNCH(simple_grads_kernel<false>, dim3(blocks, N), dim3(P), 0, stream, units, ys, lx,
+                           ly, alphas, betas, grad_f, grad_den, partial, T, U, P, nullptr, nullptr,
+                           only_if);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }

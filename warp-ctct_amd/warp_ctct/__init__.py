@@ -62,7 +62,7 @@ CLEAR_GRADIENT_IN_FORWARD = True
 CHECK_LABEL_RANGE = False
 
 
-STATUS_LABEL_RANGE, STATUS_NAN_INPUT, STATUS_LOST_HAND_OVER = 1, 2, 4
+STATUS_LABEL_RANGE, STATUS_NAN_INPUT, STATUS_LOST_HAND_OVER, STATUS_LINEAR_FELL_BACK = 1, 2, 4, 8
 
 
 def status(reset: bool = True, device=None) -> int:
