@@ -271,7 +271,13 @@ def summarise(name, facts, sec_per_step, kernels):
                                             / HBM_PEAK_GBS)
     # (lattice_fill_kernel, the sweeps with the clear of the dense gradient in
     # the same launch, is as long as the clear: no figure per frame from it)
+    # (with the sweeps done in the linear domain, lattice_lin_kernel does the
+    # work and lattice_kernel, launched behind it as the fall-back, returns at
+    # once: the figure per frame is the sweeping kernel's)
     lattice = sum(v for k, v in us.items() if k.startswith("lattice_kernel"))
+    lattice_name = "lattice_kernel"
+    if us.get("lattice_lin_kernel", 0.0) > lattice:
+        lattice, lattice_name = us["lattice_lin_kernel"], "lattice_lin_kernel"
     if lattice > 0:
         out["lattice_kernel_us"] = lattice
         out["lattice_ns_per_frame"] = lattice * 1e3 / facts["max_frames"]
@@ -285,7 +291,7 @@ def summarise(name, facts, sec_per_step, kernels):
                            "frac": gbs / HBM_PEAK_GBS, "avg_launch_us": grad_us,
                            "algorithmic_bytes_per_launch": facts["logits_grad_bytes"]}
     elif name == "c1" or facts["kind"] in ("simple_unnorm", "compact"):
-        out["roofline"] = {"bound": "latency", "kernel": "lattice_kernel",
+        out["roofline"] = {"bound": "latency", "kernel": lattice_name,
                            "note": "serial recursion over max_frames dependent steps; reported as "
                                    "ns per frame, an HBM fraction would be structurally low",
                            "max_frames": facts["max_frames"]}
