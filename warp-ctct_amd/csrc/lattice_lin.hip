@@ -25,9 +25,10 @@
 // batch again.
 //
 // Chains of workgroups hand the boundary value over as in lattice.hip (one
-// 64-bit slot per boundary and frame, empty / lost patterns, bounded polls);
-// the producer's S of a chunk travels in a slot of its own, and the consumer
-// rescales what comes in by 2^(S_producer - S_own).  A wavefront that holds no
+// 64-bit slot per boundary and frame, empty / lost patterns, bounded polls),
+// here with the slots of a chunk in one line of 128 bytes: R values, then the
+// producer's S of the chunk.  The consumer fetches the line with one load (lane
+// r holds step r's value) and rescales it by 2^(S_producer - S_own) at once.  A wavefront that holds no
 // mass yet takes over the producer's S, so that the first mass to arrive is not
 // rounded against a scale that means nothing.
 //
@@ -43,16 +44,18 @@ namespace wctct {
 namespace {
 
 constexpr int R = kLinChunk;
-constexpr int kRelayPad = 16;   // slots behind a boundary's T, as in lattice.hip
+constexpr int kLine = 16;       // slots of a chunk's line: R values, the scale, spare ones
+constexpr int kLinesAhead = 4;  // lines behind a boundary's last chunk that a request may touch
+static_assert(R < kLine, "a chunk's values and its scale share a line");
 constexpr unsigned long long kEmptyBits = kRelayEmpty;
 constexpr unsigned long long kLostBits = kEmptyBits ^ (1ULL << 32);
-constexpr int kNoMass = -(1 << 30);   // "exponent" of a wavefront whose states are all 0
 
 struct ChunkL {
     double lp[R][3];
 };
 
 typedef unsigned v4u_lin __attribute__((ext_vector_type(4)));
+typedef unsigned v2u_lin __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ void pair_store(double *dst, double o, double e) {
     *reinterpret_cast<double2 *>(dst) = make_double2(o, e);
@@ -63,13 +66,13 @@ __device__ __forceinline__ void slot_put_lin(unsigned long long *slot, double v)
                        __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// The largest of v over the wavefront, in every lane: four rotations inside the
-// rows of 16 lanes (DPP row_ror), then the four rows through scalar registers.
-__device__ __forceinline__ int wave_max_int(int v) {
-    v = max(v, __builtin_amdgcn_update_dpp(v, v, 0x128 /* row_ror:8 */, 0xf, 0xf, false));
-    v = max(v, __builtin_amdgcn_update_dpp(v, v, 0x124 /* row_ror:4 */, 0xf, 0xf, false));
-    v = max(v, __builtin_amdgcn_update_dpp(v, v, 0x122 /* row_ror:2 */, 0xf, 0xf, false));
-    v = max(v, __builtin_amdgcn_update_dpp(v, v, 0x121 /* row_ror:1 */, 0xf, 0xf, false));
+// The largest of v >= 0 over the wavefront, as a scalar: four rotations inside
+// the rows of 16 lanes (DPP row_ror), then the four rows through scalar registers.
+__device__ __forceinline__ int wave_max_nonneg(int v) {
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x128 /* row_ror:8 */, 0xf, 0xf, true));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x124 /* row_ror:4 */, 0xf, 0xf, true));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x122 /* row_ror:2 */, 0xf, 0xf, true));
+    v = max(v, __builtin_amdgcn_update_dpp(0, v, 0x121 /* row_ror:1 */, 0xf, 0xf, true));
     const int a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
     const int c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
     return max(max(a, b), max(c, d));
@@ -87,19 +90,21 @@ static __device__ __forceinline__ void chunk_load_lin(ChunkL &c, const double *u
     }
 }
 
-// The units of R frames that all exist, through a pointer that walks from row to
-// row (two scalar additions per frame instead of a clamp and a 64-bit product):
-// `frame` points at the row of the chunk's first frame, the same for all lanes.
+// The units of R frames that all exist, through a buffer descriptor over the
+// sample's units and a scalar offset that walks from row to row (one scalar
+// addition per frame; the lane's part of the address is a constant register):
+// `at` is the byte offset of the row of the chunk's first frame.
 template <bool DOWN>
-static __device__ __forceinline__ void chunk_load_walk_lin(ChunkL &c, const char *&frame,
-                                                           unsigned lane_bytes, unsigned step) {
+static __device__ __forceinline__ void chunk_load_walk_lin(ChunkL &c, __amdgpu_buffer_rsrc_t units,
+                                                           unsigned &at, unsigned lane_bytes, unsigned step) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const double *p = reinterpret_cast<const double *>(frame + lane_bytes);
-        c.lp[r][0] = p[0];
-        c.lp[r][1] = p[1];
-        c.lp[r][2] = p[2];
-        frame = DOWN ? frame - step : frame + step;
+        const v4u_lin w = __builtin_amdgcn_raw_buffer_load_b128(units, lane_bytes, at, 0);
+        const v2u_lin x = __builtin_amdgcn_raw_buffer_load_b64(units, lane_bytes + 16u, at, 0);
+        c.lp[r][0] = __hiloint2double((int)w[1], (int)w[0]);
+        c.lp[r][1] = __hiloint2double((int)w[3], (int)w[2]);
+        c.lp[r][2] = __hiloint2double((int)x[1], (int)x[0]);
+        at = DOWN ? at - step : at + step;
     }
 }
 
@@ -116,39 +121,51 @@ __device__ __forceinline__ double wave_shift_down_zero(double x) {
     return __hiloint2double(hi, lo);
 }
 
-static __device__ __forceinline__ void slots_request_lin(const unsigned long long *slots, int s0,
-                                                         unsigned long long (&bits)[R]) {
-    const unsigned long long *p = slots + s0;
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-        bits[r] = __hip_atomic_load(p + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// What a chunk needs from the boundary it reads, in one load: lane r < R asks
+// for the value of the chunk's step r, lane R for the producer's S of the chunk
+// (the lanes behind repeat lane R).  `lines` is a descriptor over the boundary's
+// lines, lane_bytes = 8 * min(lane, R).
+static __device__ __forceinline__ unsigned long long chunk_request_lin(__amdgpu_buffer_rsrc_t lines, int k,
+                                                                       unsigned lane_bytes) {
+    const v2u_lin w = __builtin_amdgcn_raw_buffer_load_b64(lines, lane_bytes, (unsigned)k * (kLine * 8u),
+                                                           16 /* sc1: at agent scope */);
+    return ((unsigned long long)w[1] << 32) | w[0];
 }
 
-// 0: a slot is still empty; 1: none is empty and one says "lost"; else values.
-static __device__ __forceinline__ unsigned slots_state_lin(const unsigned long long (&bits)[R], int cnt,
-                                                           unsigned long long scale_bits) {
+// 0: one of the chunk's cnt values or its scale is still empty; 1: none is
+// empty and one says "lost"; else all are there.
+static __device__ __forceinline__ unsigned chunk_state_lin(unsigned long long bits, int cnt) {
     constexpr unsigned kEmptyHigh = (unsigned)(kEmptyBits >> 32);
-    unsigned least = (unsigned)(scale_bits >> 32) ^ kEmptyHigh;
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const unsigned d = (unsigned)(bits[r] >> 32) ^ kEmptyHigh;
-        least = min(least, r < cnt ? d : 0xffffffffu);
-    }
-    return (unsigned)__builtin_amdgcn_readfirstlane((int)least);
+    constexpr unsigned kLostHigh = (unsigned)(kLostBits >> 32);
+    const unsigned hi = (unsigned)(bits >> 32);
+    const unsigned long long need = ((1ULL << cnt) - 1ULL) | (1ULL << R);
+    if (__ballot(hi == kEmptyHigh) & need) return 0u;
+    if (__ballot(hi == kLostHigh) & need) return 1u;
+    return 2u;
+}
+
+// The double that lane `from` holds, as a scalar.
+template <int from>
+static __device__ __forceinline__ double lane_value(double x) {
+    return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(x), from),
+                            __builtin_amdgcn_readlane(__double2loint(x), from));
+}
+static __device__ __forceinline__ double mail_at(double x, int r) {   // r: constant once unrolled
+    return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(x), r),
+                            __builtin_amdgcn_readlane(__double2loint(x), r));
 }
 
 // One direction of the 64 contexts [64*wave, 64*wave + 64) of one lattice.
 // Step s handles frame t = s (alpha) or Tn-1-s (beta) and stores the front of
 // frame t+1 (alpha) or t (beta), as in lattice.hip.  scales[0] belongs to the
 // initial row, scales[1 + k] to the rows that chunk k stores.
-// slots_in / scale_in, slots_out / scale_out: the boundary this wavefront reads
-// and the one it writes (values per step, the producer's S per chunk), or null.
+// lines_in, lines_out: the lines (one per chunk) of the boundary this wavefront
+// reads and of the one it writes, or null.
 template <bool BETA, bool HAS_IN>
 static __device__ void sweep_lin(const double *units_n, const int *y, int Tn, int Un, int T, int P, int wave,
-                                 double *lat_n, int *scales, float *cost_n,
-                                 const unsigned long long *slots_in, const unsigned long long *scale_in,
-                                 unsigned long long *slots_out, unsigned long long *scale_out,
-                                 int max_spins, unsigned *flag, unsigned *status) {
+                                 double *lat_n, int *scales, float *cost_n, const unsigned long long *lines_in,
+                                 unsigned long long *lines_out, int max_spins, unsigned *flag,
+                                 unsigned *status) {
     const int lane = threadIdx.x & 63;
     const int u = wave * 64 + lane;
     double omask = 1.0, skipf, e, o;
@@ -178,64 +195,54 @@ static __device__ void sweep_lin(const double *units_n, const int *y, int Tn, in
         const int dir = BETA ? -1 : 1;
         const int t_start = BETA ? Tn - 1 : 0;
         chunk_load_lin(a, in, urow, Tn, t_start, dir);
-        // The relay slots of a chunk are requested kAhead chunks before they are
-        // used: a chunk of this sweep takes ~0.6 us, a slot's way from the
+        // What a chunk needs from the boundary is requested three chunks before
+        // it is used: a chunk of this sweep takes ~0.6 us, a slot's way from the
         // producer through the L2 and back longer than that, and a wavefront that
-        // looks too early pays a whole round trip for asking again.  Four register
-        // sets in rotation (set index = chunk index mod 4): the one chunk k reads
-        // was requested at the start of chunk k-3, and the set that chunk k-1 has
-        // read takes the request for chunk k+3.
-        unsigned long long q0[R], q1[R], q2[R], q3[R];
-        unsigned long long sq0 = kEmptyBits, sq1 = kEmptyBits, sq2 = kEmptyBits, sq3 = kEmptyBits;
-#pragma unroll
-        for (int r = 0; r < R; ++r) q0[r] = q1[r] = q2[r] = q3[r] = kEmptyBits;
-        auto request = [&](int k, unsigned long long (&set)[R], unsigned long long &sc) {
-            slots_request_lin(slots_in, min(k * R, T), set);
-            sc = __hip_atomic_load(scale_in + min(k, lin_chunks(T)), __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-        };
+        // looks too early pays a whole round trip for asking again.  Four registers
+        // in rotation (index = chunk index mod 4): the one chunk k reads was
+        // requested at the start of chunk k-3, and the one that chunk k-1 has read
+        // takes the request for chunk k+3.
+        unsigned long long q0 = kEmptyBits, q1 = kEmptyBits, q2 = kEmptyBits, q3 = kEmptyBits;
+        const __amdgpu_buffer_rsrc_t lines = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<unsigned long long *>(lines_in), 0, 0xffffffffu, 0x00020000);
+        const unsigned line_lane = 8u * (unsigned)min(lane, R);
+        // (a request past the last chunk reads one of the kLinesAhead spare lines)
+        auto request = [&](int k) { return chunk_request_lin(lines, k, line_lane); };
         if (HAS_IN) {
-            request(0, q0, sq0);
-            request(1, q1, sq1);
-            request(2, q2, sq2);
+            q0 = request(0);
+            q1 = request(1);
+            q2 = request(2);
         }
+        // 1 in the lane whose context borders on the producer's, 0 elsewhere
+        const double in_lane = (lane == (BETA ? 63 : 0)) ? 1.0 : 0.0;
         bool lost = false;
-        auto run_chunk = [&](const ChunkL &c, unsigned long long (&have)[R], unsigned long long &sc_have,
-                             unsigned long long (&next)[R], unsigned long long &sc_next, int s0,
-                             int cnt, bool full) {
-            const int k = s0 / R;
-            double mail[R], mine[R];
-#pragma unroll
-            for (int r = 0; r < R; ++r) mail[r] = 0.0;
+        auto run_chunk = [&](const ChunkL &c, unsigned long long &have, unsigned long long &next, int k,
+                             int cnt, bool full, bool last) {
+            double mine[R];
+            double mail = 0.0;   // lane r: what flows in at step r of this chunk, in this wavefront's scale
             if (HAS_IN) {
-                request(k + 3, next, sc_next);
-                unsigned state = slots_state_lin(have, cnt, sc_have);
+                next = request(k + 3);
+                unsigned state = chunk_state_lin(have, cnt);
                 if (state == 0 && max_spins > 0 && !lost) {
                     int spins = 0;
                     do {
                         __builtin_amdgcn_s_sleep(2);
-                        slots_request_lin(slots_in, s0, have);
-                        sc_have = __hip_atomic_load(scale_in + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        state = slots_state_lin(have, cnt, sc_have);
+                        have = request(k);
+                        state = chunk_state_lin(have, cnt);
                     } while (state == 0 && ++spins < max_spins);
                 }
                 if (state <= 1) lost = true;
                 if (!lost) {
-                    const int S_in = (int)__longlong_as_double((long long)sc_have);
+                    const double got = __longlong_as_double((long long)have);
+                    const int S_in = (int)lane_value<R>(got);
                     // no mass here yet: what flows in sets the scale
                     const bool any = __ballot(e != 0.0 || o != 0.0) != 0ULL;
                     if (!any) S = S_in;
-                    // the value belongs to the lane at the boundary; all other lanes
-                    // scale theirs down to 0 (every lane has loaded the same slot), so
-                    // that it can simply be added to what the DPP move brings
-                    const int shift = (lane == (BETA ? 63 : 0)) ? S_in - S : -5000;
-#pragma unroll
-                    for (int r = 0; r < R; ++r)
-                        if (full || r < cnt)
-                            mail[r] = __builtin_amdgcn_ldexp(__longlong_as_double((long long)have[r]), shift);
+                    mail = __builtin_amdgcn_ldexp(got, S_in - S);
                 }
             }
-            if (scale_out && !lost && lane == edge_lane) slot_put_lin(scale_out + k, (double)S);
+            unsigned long long *line_out = lines_out + (size_t)k * kLine;
+            if (lines_out && !lost && lane == edge_lane) slot_put_lin(line_out + R, (double)S);
             const int rows_here = full ? R : cnt;
             const __amdgpu_buffer_rsrc_t rows = __builtin_amdgcn_make_buffer_rsrc(
                 BETA ? out_row - (size_t)(rows_here - 1) * out_step : out_row, 0, 0xffffffffu, 0x00020000);
@@ -248,7 +255,8 @@ static __device__ void sweep_lin(const double *units_n, const int *y, int Tn, in
                         // beta(t,2u)   = beta(t+1,2u) lp0 + beta(t+1,2u+1) lp2
                         // beta(t,2u-1) = beta(t+1,2u-1) lp1 + beta(t+1,2u) lp0 + [skip] beta(t+1,2u+1) lp2
                         mine[r] = o;
-                        const double nb = HAS_IN ? wave_shift_down_zero(o) + mail[r] : wave_shift_down_zero(o);
+                        const double nb = HAS_IN ? __builtin_fma(mail_at(mail, r), in_lane, wave_shift_down_zero(o))
+                                                 : wave_shift_down_zero(o);
                         const double nxt = nb * c.lp[r][2];
                         const double stay_e = e * c.lp[r][0];
                         const double sel = __builtin_fma(skipf, nxt, stay_e);
@@ -260,7 +268,8 @@ static __device__ void sweep_lin(const double *units_n, const int *y, int Tn, in
                         // sends: ([skip] alpha(t,2u-1) + alpha(t,2u)) lp2
                         const double sum = e + o;
                         mine[r] = __builtin_fma(o, skipf, e) * c.lp[r][2];
-                        const double recv = HAS_IN ? wave_shift_up_zero(mine[r]) + mail[r] : wave_shift_up_zero(mine[r]);
+                        const double recv = HAS_IN ? __builtin_fma(mail_at(mail, r), in_lane, wave_shift_up_zero(mine[r]))
+                                                   : wave_shift_up_zero(mine[r]);
                         o = __builtin_fma(o, c.lp[r][1], recv);
                         e = sum * c.lp[r][0];
                     }
@@ -272,19 +281,22 @@ static __device__ void sweep_lin(const double *units_n, const int *y, int Tn, in
                 }
             }
             out_row = BETA ? out_row - (size_t)rows_here * out_step : out_row + (size_t)rows_here * out_step;
-            if (slots_out && !lost && lane == edge_lane) {
+            if (lines_out && !lost && lane == edge_lane) {
 #pragma unroll
                 for (int r = 0; r < R; ++r)
-                    if (full || r < cnt) slot_put_lin(slots_out + s0 + r, mine[r]);
+                    if (full || r < cnt) slot_put_lin(line_out + r, mine[r]);
             }
             if (lane == 0) scales[1 + k] = S;
             // the largest state back into [0.5, 1) (not after the last chunk: the
-            // cost below is taken from the rows as they were stored)
-            if (s0 + cnt < Tn) {
-                const double m = __builtin_fmax(e, o);
-                int ex = (m > 0.0 && m < __builtin_huge_val()) ? __builtin_amdgcn_frexp_exp(m) : kNoMass;
-                ex = wave_max_int(ex);
-                if (ex != kNoMass) {
+            // cost below is taken from the rows as they were stored).  The states
+            // are not negative, so the largest one has the largest high word, whose
+            // bits 20.. are its exponent + 1023: scalar arithmetic from there on.
+            // All states 0 (or below the normal range): nothing to scale; a state
+            // that is not finite: the check behind the sweeps will say so.
+            if (!last) {
+                const int top = wave_max_nonneg(max(__double2hiint(e), __double2hiint(o))) >> 20;
+                if (top > 0 && top < 0x7ff) {
+                    const int ex = top - 1022;
                     e = __builtin_amdgcn_ldexp(e, -ex);
                     o = __builtin_amdgcn_ldexp(o, -ex);
                     S += ex;
@@ -292,34 +304,35 @@ static __device__ void sweep_lin(const double *units_n, const int *y, int Tn, in
             }
         };
         int s0 = 0;
-        const unsigned in_lane = (unsigned)u * 3u * (unsigned)sizeof(double);
-        const unsigned in_step = (unsigned)(urow * sizeof(double));
-        // four chunks per turn (the slot sets come round); while the chunk after
+        // four chunks per turn (the requests come round); while the chunk after
         // the turn lies inside the sample, the rows of units need no clamp
         if (5 * R <= Tn) {
-            const char *frame = reinterpret_cast<const char *>(units_n) +
-                                (size_t)(t_start + dir * R) * urow * sizeof(double);
+            const __amdgpu_buffer_rsrc_t rows_in = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<double *>(units_n), 0, 0xffffffffu, 0x00020000);
+            const unsigned in_bytes = (unsigned)u * 3u * (unsigned)sizeof(double);
+            const unsigned in_step = (unsigned)(urow * sizeof(double));
+            unsigned at = (unsigned)(t_start + dir * R) * in_step;
+            int k = 0;
             do {
-                chunk_load_walk_lin<BETA>(b, frame, in_lane, in_step);
-                run_chunk(a, q0, sq0, q3, sq3, s0, R, true);
-                chunk_load_walk_lin<BETA>(a, frame, in_lane, in_step);
-                run_chunk(b, q1, sq1, q0, sq0, s0 + R, R, true);
-                chunk_load_walk_lin<BETA>(b, frame, in_lane, in_step);
-                run_chunk(a, q2, sq2, q1, sq1, s0 + 2 * R, R, true);
-                chunk_load_walk_lin<BETA>(a, frame, in_lane, in_step);
-                run_chunk(b, q3, sq3, q2, sq2, s0 + 3 * R, R, true);
+                chunk_load_walk_lin<BETA>(b, rows_in, at, in_bytes, in_step);
+                run_chunk(a, q0, q3, k, R, true, false);
+                chunk_load_walk_lin<BETA>(a, rows_in, at, in_bytes, in_step);
+                run_chunk(b, q1, q0, k + 1, R, true, false);
+                chunk_load_walk_lin<BETA>(b, rows_in, at, in_bytes, in_step);
+                run_chunk(a, q2, q1, k + 2, R, true, false);
+                chunk_load_walk_lin<BETA>(a, rows_in, at, in_bytes, in_step);
+                run_chunk(b, q3, q2, k + 3, R, true, false);
+                k += 4;
                 s0 += 4 * R;
             } while (s0 + 5 * R <= Tn);
         }
-        // the rest (fewer than five chunks), one chunk per turn: the sets move up
-        // by copies instead
+        // the rest (fewer than five chunks), one chunk per turn: the requests move
+        // up by copies instead
         while (s0 < Tn) {
             chunk_load_lin(b, in, urow, Tn, t_start + dir * (s0 + R), dir);
-            run_chunk(a, q0, sq0, q3, sq3, s0, min(Tn - s0, R), false);
+            run_chunk(a, q0, q3, s0 / R, min(Tn - s0, R), false, s0 + R >= Tn);
             a = b;
-#pragma unroll
-            for (int r = 0; r < R; ++r) q0[r] = q1[r], q1[r] = q2[r], q2[r] = q3[r];
-            sq0 = sq1, sq1 = sq2, sq2 = sq3;
+            q0 = q1, q1 = q2, q2 = q3;
             s0 += R;
         }
         if (lost) {
@@ -328,11 +341,11 @@ static __device__ void sweep_lin(const double *units_n, const int *y, int Tn, in
                 atomicOr(flag, 1u);
                 if (status) atomicOr(status, kStatusLostHandOver);
             }
-            if (slots_out && lane == edge_lane) {
-                for (int s = 0; s < Tn; ++s)
-                    __hip_atomic_store(slots_out + s, kLostBits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (lines_out && lane == edge_lane) {
                 for (int k = 0; k * R < Tn; ++k)
-                    __hip_atomic_store(scale_out + k, kLostBits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    for (int r = 0; r <= R; ++r)
+                        __hip_atomic_store(lines_out + (size_t)k * kLine + r, kLostBits, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
             }
         }
     }
@@ -370,35 +383,30 @@ __global__ __launch_bounds__(64) void lattice_lin_kernel(
     const size_t lat = (size_t)(T + 1) * P * 2;
     const int chunks = lin_chunks(T);
     int *sc = scales + (((size_t)n * 2 + (beta ? 0 : 1)) * W + wave) * (size_t)(chunks + 1);
-    // slots of one boundary and direction: T + kRelayPad values, then chunks + 1 scales
-    const size_t TS = (size_t)T + kRelayPad + (size_t)chunks + 1;
-    unsigned long long *slots_n =
+    // one boundary and direction: a line per chunk and the spare lines behind
+    const size_t TS = (size_t)(chunks + kLinesAhead) * kLine;
+    unsigned long long *lines_n =
         relay ? relay + ((size_t)n * 2 + (beta ? 0 : 1)) * (size_t)(W - 1) * TS : nullptr;
-    const size_t to_scales = (size_t)T + kRelayPad;
     if (!beta) {
-        const unsigned long long *in = wave > 0 ? slots_n + (size_t)(wave - 1) * TS : nullptr;
-        unsigned long long *out = (wave + 1) * 64 <= Un ? slots_n + (size_t)wave * TS : nullptr;
+        const unsigned long long *in = wave > 0 ? lines_n + (size_t)(wave - 1) * TS : nullptr;
+        unsigned long long *out = (wave + 1) * 64 <= Un ? lines_n + (size_t)wave * TS : nullptr;
         if (in)
             sweep_lin<false, true>(units_n, y, Tn, Un, T, P, wave, alphas + (size_t)n * lat, sc, nullptr, in,
-                                   in + to_scales, out, out ? out + to_scales : nullptr, max_spins, flag,
-                                   status);
+                                   out, max_spins, flag, status);
         else
             sweep_lin<false, false>(units_n, y, Tn, Un, T, P, wave, alphas + (size_t)n * lat, sc, nullptr,
-                                    nullptr, nullptr, out, out ? out + to_scales : nullptr, max_spins, flag,
-                                    status);
+                                    nullptr, out, max_spins, flag, status);
         return;
     }
     {
-        const unsigned long long *in = (wave + 1) * 64 <= Un ? slots_n + (size_t)wave * TS : nullptr;
-        unsigned long long *out = wave > 0 ? slots_n + (size_t)(wave - 1) * TS : nullptr;
+        const unsigned long long *in = (wave + 1) * 64 <= Un ? lines_n + (size_t)wave * TS : nullptr;
+        unsigned long long *out = wave > 0 ? lines_n + (size_t)(wave - 1) * TS : nullptr;
         if (in)
             sweep_lin<true, true>(units_n, y, Tn, Un, T, P, wave, betas + (size_t)n * lat, sc, costs + n, in,
-                                  in + to_scales, out, out ? out + to_scales : nullptr, max_spins, flag,
-                                  status);
+                                  out, max_spins, flag, status);
         else
             sweep_lin<true, false>(units_n, y, Tn, Un, T, P, wave, betas + (size_t)n * lat, sc, costs + n,
-                                   nullptr, nullptr, out, out ? out + to_scales : nullptr, max_spins, flag,
-                                   status);
+                                   nullptr, out, max_spins, flag, status);
     }
     if (wave != 0) return;
     cost_reduce_tail(red, costs, lx, n, N, threadIdx.x);
@@ -408,7 +416,7 @@ __global__ __launch_bounds__(64) void lattice_lin_kernel(
 
 size_t lattice_lin_relay_slots(int N, int T, int U) {
     const int W = (U + 1 + 63) / 64;
-    return (size_t)N * 2 * (size_t)(W - 1) * ((size_t)T + kRelayPad + (size_t)lin_chunks(T) + 1);
+    return (size_t)N * 2 * (size_t)(W - 1) * (size_t)(lin_chunks(T) + kLinesAhead) * kLine;
 }
 
 size_t lattice_lin_scales(int N, int T, int U) {
@@ -425,6 +433,8 @@ hipError_t launch_lattice_lin(const LatticeArgs &a, int *scales, unsigned *flag,
     if (slots > 0 && (!relay || !a.relay_is_clear)) return hipErrorInvalidValue;
     const long chains_pad = ((long)a.N * 2 + 7) / 8 * 8;
     if (chains_pad * W > 0x7fffffffL) return hipErrorInvalidValue;
+    // a sample's units are addressed through 32-bit byte offsets
+    if ((size_t)a.T * 64 * W * 3 * sizeof(double) >= (1ULL << 31)) return hipErrorInvalidValue;
     const int max_spins = lattice_wait_limit_now();
     TIMED_LAUNCH(lattice_lin_kernel, dim3((unsigned)(chains_pad * W)), dim3(64), 0, stream, a.units, a.ys,
                  a.lx, a.ly, a.alphas, a.betas, scales, a.costs, relay, a.N, a.T, a.U, W, (int)chains_pad,

@@ -533,7 +533,10 @@ hipError_t launch_simple_gather_units(const float *f, const float *g, float *den
 // The first half of launch_simple_grads for lattices in the linear domain (see
 // simple_grads_kernel<true>): grad_f, grad_den and the partial sums of grad_g;
 // the caller adds those up with launch_simple_grads' second half afterwards.
-bool simple_grads_lin_applies(int T, int U) { return T > 0 && padded_contexts(U) <= 512; }
+bool simple_grads_lin_applies(int T, int U) {
+    // (the linear sweeps address a sample's units through 32-bit byte offsets)
+    return T > 0 && padded_contexts(U) <= 512 && (size_t)T * padded_contexts(U) * 3 * sizeof(double) < (1ULL << 31);
+}
 
 hipError_t launch_simple_grads_lin(const double *units, const int *ys, const int *lx, const int *ly,
                                    const double *alphas, const double *betas, const int *scales,
