@@ -491,9 +491,9 @@ int warpctct_status(unsigned *bits, int clear);
  * log-domain kernels, launched behind it in the same stream, compute the batch
  * again (they return at once otherwise), and
  * WARPCTCT_STATUS_LINEAR_FELL_BACK is set.  No counterpart in the reference
- * (csrc/simple.cu sweeps in the log domain).  The linear sweeps save 25-50 ns
+ * (csrc/simple.cu sweeps in the log domain).  The linear sweeps save 30-40 ns
  * per frame and cost ~14 us per call (the launches that return at once, a
- * slower gather and gradient kernel), so they are used from T = 1024 frames on.
+ * slower gather and gradient kernel), so they are used from T = 768 frames on.
  * warpctct_joiner_linear_lattice(n) moves that limit for later calls of the
  * process (0: never; 1: always; negative: the default) and returns the
  * previous one. */

@@ -23,7 +23,7 @@ GRAD_ATOL = 1e-4
 def lattice_domain(request):
     """Every test of this file runs twice: with the joiner's lattices swept in the
     log domain only, and with the linear sweeps (checked, with the log domain as
-    their fall-back) used for every input, not just from 1024 frames on."""
+    their fall-back) used for every input, not just from 768 frames on."""
     lib = hip_lib.lib()
     before = lib.warpctct_joiner_linear_lattice(1 if request.param == "linear_lattices" else 0)
     yield request.param
@@ -864,15 +864,15 @@ def _loss_and_grads(f, g, ys, lx, ly, normalized, reduction="none", w=None):
 
 
 @pytest.mark.parametrize("normalized", [True, False])
-def test_linear_lattices_are_used_from_1024_frames_and_hold_on_ordinary_input(normalized, lattice_domain):
+def test_linear_lattices_are_used_from_768_frames_and_hold_on_ordinary_input(normalized, lattice_domain):
     """With the default setting the fused forward sweeps in the linear domain from
-    1024 frames on (lattice_lin_kernel is launched, the log-domain kernels behind it
+    768 frames on (lattice_lin_kernel is launched, the log-domain kernels behind it
     return at once: the fall-back bit stays clear), and below that in the log
     domain; both agree with the oracle.  A chain of two workgroups per lattice."""
     import warp_ctct
     lib = hip_lib.lib()
     lib.warpctct_joiner_linear_lattice(-1)
-    for T, linear in ((1030, True), (1000, False)):
+    for T, linear in ((780, True), (760, False)):
         N, U, V = 2, 70, 24
         f, g, ys, lx, ly = make_simple_case(60 + T, N, T, U, V, lx=[T, T - 37], ly=[U, 41],
                                             normalized=normalized)

@@ -87,11 +87,10 @@ int forward_from_units(const Workspace &w, const int *ys, const int *lx, const i
 
 // from how many frames on the fused joiner forward sweeps its lattices in the
 // linear domain first (warpctct_joiner_linear_lattice; 0: never).  The linear
-// sweeps save 25-50 ns per frame (less with many lattices in flight, whose
-// sweeps are slowed by the memory system, more for a few long ones) and cost
-// ~14 us per call (three launches that return at once, a slower gather and
-// gradient kernel): from 1024 frames on they never lose.
-constexpr int kLinearFromFrames = 1024;
+// sweeps save 30-40 ns per frame and cost ~14 us per call (three launches that
+// return at once, a slower gather and gradient kernel): measured, they gain from
+// about 600 frames on, more for chains of workgroups than for lone ones.
+constexpr int kLinearFromFrames = 768;
 std::atomic<int> g_linear_from{kLinearFromFrames};
 
 struct SimpleWorkspace {
