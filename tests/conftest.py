@@ -12,6 +12,8 @@ for p in (ROOT, PKG_ROOT, os.path.dirname(os.path.abspath(__file__))):
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: test needs a real MI355X (run with -m gpu)")
+    config.addinivalue_line("markers", "may_fall_back: the test's input is meant to (or may) send the joiner's "
+                                       "linear lattices back to the log domain")
 
 
 def _have_gpu():

@@ -24,10 +24,18 @@ def lattice_domain(request):
     """Every test of this file runs twice: with the joiner's lattices swept in the
     log domain only, and with the linear sweeps (checked, with the log domain as
     their fall-back) used for every input, not just from 768 frames on."""
+    import warp_ctct
     lib = hip_lib.lib()
     before = lib.warpctct_joiner_linear_lattice(1 if request.param == "linear_lattices" else 0)
+    warp_ctct.status(reset=True)
     yield request.param
     lib.warpctct_joiner_linear_lattice(before)
+    # the linear sweeps must hold on their own: a test whose input is meant to
+    # send them back to the log domain says so (the fall-back would hide a
+    # mistake in them from every comparison with the oracle)
+    fell_back = warp_ctct.status(reset=True) & warp_ctct.STATUS_LINEAR_FELL_BACK
+    if request.node.get_closest_marker("may_fall_back") is None:
+        assert not fell_back, "the linear lattices were given up on input that they should take"
 
 
 def dev(a, dtype=None):

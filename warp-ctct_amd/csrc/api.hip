@@ -97,28 +97,40 @@ struct SimpleWorkspace {
     Workspace lattice;
     float *unit_grads;   // (N,T,U+1,3)
     float *partial;      // logmm_fwd_partial_floats: partial sums of a split log-matmul reduction
-    // for the lattices in the linear domain (launch_lattice_lin): relay slots,
-    // scales, and the flag that sends the batch through the log-domain kernels
-    void *lin_relay;
+    // For the lattices in the linear domain (launch_lattice_lin): units and
+    // lattices in that form's layout, in the memory of the log-domain ones (which
+    // are written only if the linear ones are given up, and from scratch then);
+    // scales, the flag that sends the batch through the log-domain kernels, and
+    // an arrival counter of its own for the batch reduction (the log-domain one
+    // lies in memory that the linear buffers may cover).
+    double *lin_units, *lin_alphas, *lin_betas;
     int *lin_scales;
-    unsigned *lin_flag;
+    unsigned *lin_flag, *lin_counter;
     size_t bytes;
 };
 
 SimpleWorkspace carve_simple(void *base, int N, int T, int U) {
     SimpleWorkspace w;
     w.lattice = carve(base, N, T, U);
-    const uintptr_t p = reinterpret_cast<uintptr_t>(base) + w.lattice.bytes;
+    const bool lin = simple_grads_lin_applies(T, U);
+    const size_t Pl = (size_t)lin_padded(U);
+    const size_t lin_units_b = lin ? align256((size_t)N * T * Pl * kLinUnit * sizeof(double)) : 0;
+    const size_t lin_lat_b = lin ? align256((size_t)N * (T + 1) * Pl * 2 * sizeof(double)) : 0;
+    const uintptr_t b = reinterpret_cast<uintptr_t>(base);
+    w.lin_units = reinterpret_cast<double *>(b);
+    w.lin_alphas = reinterpret_cast<double *>(b + lin_units_b);
+    w.lin_betas = reinterpret_cast<double *>(b + lin_units_b + lin_lat_b);
+    const size_t lattice_b = std::max(w.lattice.bytes, lin_units_b + 2 * lin_lat_b);
+    const uintptr_t p = b + lattice_b;
     const size_t ug_b = align256((size_t)N * T * (U + 1) * 3 * sizeof(float));
     w.unit_grads = reinterpret_cast<float *>(p);
     w.partial = reinterpret_cast<float *>(p + ug_b);
     const size_t partial_b = align256(logmm_fwd_partial_floats(N, T, U + 1) * sizeof(float));
-    const size_t relay_b = align256(lattice_lin_relay_slots(N, T, U) * sizeof(unsigned long long));
-    const size_t scales_b = align256(lattice_lin_scales(N, T, U) * sizeof(int));
-    w.lin_relay = relay_b ? reinterpret_cast<void *>(p + ug_b + partial_b) : nullptr;
-    w.lin_scales = reinterpret_cast<int *>(p + ug_b + partial_b + relay_b);
-    w.lin_flag = reinterpret_cast<unsigned *>(p + ug_b + partial_b + relay_b + scales_b);
-    w.bytes = w.lattice.bytes + ug_b + partial_b + relay_b + scales_b + 256;
+    const size_t scales_b = lin ? align256(lattice_lin_scales(N, T, U) * sizeof(int)) : 0;
+    w.lin_scales = reinterpret_cast<int *>(p + ug_b + partial_b);
+    w.lin_flag = reinterpret_cast<unsigned *>(p + ug_b + partial_b + scales_b);
+    w.lin_counter = w.lin_flag + 32;
+    w.bytes = lattice_b + ug_b + partial_b + scales_b + 256;
     return w;
 }
 
@@ -783,35 +795,34 @@ int warpctct_simple_forward_reduced_f32(const float *f, const float *g, const in
             // checked by the kernel that forms the gradients from them; the
             // log-domain kernels follow and return at once unless that check, or
             // anything else on the way, has raised the flag.
-            RelaySlots lin_slots;
-            lin_slots.n = w.lin_relay ? lattice_lin_relay_slots(N, T, U) : 0;
-            lin_slots.p = lin_slots.n ? static_cast<unsigned long long *>(w.lin_relay) : nullptr;
-            int rc = done(launch_simple_gather_units(f, g, normalized ? den : nullptr, ys, lx, ly,
-                                                     w.lattice.units, N, T, U, V, lin_slots, deferred,
-                                                     fmax, reduce.counter, st, w.lin_flag));
+            CostReduce lin_reduce = reduce;
+            if (lin_reduce.counter) lin_reduce.counter = w.lin_counter;
+            int rc = done(launch_simple_gather_units_lin(f, g, normalized ? den : nullptr, ys, lx, ly,
+                                                         w.lin_units, N, T, U, V, deferred, fmax,
+                                                         lin_reduce.counter, w.lin_flag, st));
             if (rc != WARPCTCT_OK) return rc;
             LatticeArgs a = {};
-            a.units = w.lattice.units;
+            a.units = w.lin_units;
             a.ys = ys, a.lx = lx, a.ly = ly;
-            a.alphas = w.lattice.alphas, a.betas = w.lattice.betas;
-            a.relay = w.lin_relay, a.relay_is_clear = true;
+            a.alphas = w.lin_alphas, a.betas = w.lin_betas;
             a.costs = costs;
             a.N = N, a.T = T, a.U = U;
-            a.reduce = reduce;
+            a.reduce = lin_reduce;
             rc = done(launch_lattice_lin(a, w.lin_scales, w.lin_flag, st));
             if (rc != WARPCTCT_OK) return rc;
-            rc = done(launch_simple_grads_lin(w.lattice.units, ys, lx, ly, w.lattice.alphas,
-                                              w.lattice.betas, w.lin_scales, w.unit_grads, grad_f,
+            rc = done(launch_simple_grads_lin(w.lin_units, ys, lx, ly, w.lin_alphas, w.lin_betas,
+                                              w.lin_scales, w.unit_grads, grad_f,
                                               normalized ? grad_den : nullptr, N, T, U, w.lin_flag, st));
             if (rc != WARPCTCT_OK) return rc;
+            const unsigned *guard = w.lin_flag;
             rc = done(launch_simple_gather_units(f, g, normalized ? den : nullptr, ys, lx, ly,
                                                  w.lattice.units, N, T, U, V,
                                                  relay_slots_of(w.lattice.relay, N, T, U), deferred,
-                                                 fmax, reduce.counter, st, nullptr, w.lin_flag));
+                                                 fmax, reduce.counter, st, guard));
             if (rc != WARPCTCT_OK) return rc;
             return simple_from_units(w, ys, lx, ly, N, T, U, costs, grad_f, grad_g,
                                      normalized ? grad_den : nullptr, true, true, reduce, st,
-                                     w.lin_flag);
+                                     guard);
         }
         int rc = done(launch_simple_gather_units(f, g, normalized ? den : nullptr, ys, lx, ly,
                                                  w.lattice.units, N, T, U, V,

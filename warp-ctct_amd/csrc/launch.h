@@ -116,20 +116,32 @@ hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream, const unsign
 
 // ---- the joiner's lattices in the linear domain (lattice_lin.hip) -------------
 // Sweeps on path masses relative to a power of two per wavefront and chunk of
-// kLinChunk frames; alphas / betas then hold (N,T+1,P,2) pairs {o, e} of masses,
-// `scales` lattice_lin_scales(N,T,U) exponents: entry
-//   ((n*2 + d)*W + w)*(lin_chunks(T) + 1) + i,   d = 0: beta, 1: alpha,
-// with i = 0 for the initial row (alpha: frame 0, beta: frame Tn) and
-// i = 1 + step / kLinChunk for the row stored by that step (alpha: step = frame - 1,
-// beta: step = Tn - 1 - frame).  units are linear too (2^(log2 unit), neutral
-// {1, 1, 0}).  a.relay needs lattice_lin_relay_slots 64-bit words, cleared to
-// kRelayEmpty (a.relay_is_clear); *flag is raised where a hand-over was lost.
-// The results are only meaningful together with the check of the kernel that
-// reads them (launch_simple_grads_lin).
+// kLinChunk frames.  A wavefront holds kLinReal contexts in its lanes 1..62;
+// lane 0 / lane 63 stand for the context below / above, whose wavefront hands
+// its boundary value over THROUGH THE UNITS: context u lives in column
+// lin_column(u) of the lin_padded(U) columns that units, alphas and betas have
+// here, and the columns in between belong to those two lanes.
+//   units  (N,T,Pl,kLinUnit): {blank, label, next label, next label of the
+//          context below} as linear factors (neutral {1,1,0,0}); written by
+//          launch_simple_gather_units_lin, which also sets up the columns in
+//          between; the sweeps write what they hand over into them
+//   alphas, betas (N,T+1,Pl,2): pairs {o, e} of masses
+//   scales: lattice_lin_scales(N,T,U) exponents, entry
+//          ((n*2 + d)*W + w)*(lin_chunks(T) + 1) + i,   d = 0: beta, 1: alpha,
+//          W = lin_waves(U), i = 0 for the initial row (alpha: frame 0, beta:
+//          frame Tn) and i = 1 + step / kLinChunk for the row stored by that
+//          step (alpha: step = frame - 1, beta: step = Tn - 1 - frame)
+// *flag is raised where a hand-over was lost.  The results are only meaningful
+// together with the check of the kernel that reads them (launch_simple_grads_lin).
 constexpr int kLinChunk = 12;
+constexpr int kLinReal = 62;
+constexpr int kLinUnit = 4;
 __host__ __device__ inline int lin_chunks(int T) { return (T + kLinChunk - 1) / kLinChunk; }
-size_t lattice_lin_relay_slots(int N, int T, int U);
+__host__ __device__ inline int lin_waves(int U) { return (U + kLinReal) / kLinReal; }   // U + 1 contexts
+__host__ __device__ inline int lin_padded(int U) { return 64 * lin_waves(U); }
+__host__ __device__ inline int lin_column(int u) { return u + 2 * (u / kLinReal) + 1; }
 size_t lattice_lin_scales(int N, int T, int U);
+// a.units, a.alphas, a.betas: the buffers described above; a.relay is not used
 hipError_t launch_lattice_lin(const LatticeArgs &a, int *scales, unsigned *flag, hipStream_t stream);
 
 // Element strides of a joint tensor (N,T,U+1,V); dense row-major is
@@ -201,16 +213,19 @@ struct LogmmDeferred {
 };
 // den (N,T,U+1): read, or, with `deferred.partial`, computed from the deferred
 // pass and written, together with fmax (N,T) (-inf for frames beyond lx).
-// linear_flag (may be null): the units are stored in the linear domain, for
-// launch_lattice_lin, and *linear_flag is lowered; only_if (may be null): the
-// kernel returns at once while *only_if is 0.
+// only_if (may be null): the kernel returns at once while *only_if is 0.
 hipError_t launch_simple_gather_units(const float *f, const float *g, float *den, const int *ys,
                                       const int *lx, const int *ly, double *units, int N, int T,
                                       int U, int V, const RelaySlots &relay,
                                       const LogmmDeferred &deferred, float *fmax,
                                       unsigned *counter, hipStream_t stream,
-                                      unsigned *linear_flag = nullptr,
                                       const unsigned *only_if = nullptr);
+// The same for the sweeps in the linear domain: units as launch_lattice_lin
+// wants them (see there); *flag is lowered.
+hipError_t launch_simple_gather_units_lin(const float *f, const float *g, float *den, const int *ys,
+                                          const int *lx, const int *ly, double *units, int N, int T,
+                                          int U, int V, const LogmmDeferred &deferred, float *fmax,
+                                          unsigned *counter, unsigned *flag, hipStream_t stream);
 // compact gradients of the joiner path straight from the lattices: grad_f
 // (N,T,U+1), grad_g (N,U+1,3), grad_den (N,T,U+1) or null; `partial` is scratch
 // of N * T * (U+1) * 3 floats (partial sums over blocks of 8 frames, or, for
@@ -223,7 +238,8 @@ hipError_t launch_simple_grads(const double *units, const int *ys, const int *lx
 // blocks of frames (launch_simple_grads with only_if behind it does that sum
 // whether it recomputes or not); raises *flag where the linear lattices cannot
 // be trusted (posteriors of a frame not adding up to 1, a unit out of range,
-// anything not finite).  Needs simple_grads_lin_applies(T, U).
+// anything not finite).  units, alphas, betas, scales: as launch_lattice_lin
+// describes them.  Needs simple_grads_lin_applies(T, U).
 bool simple_grads_lin_applies(int T, int U);
 hipError_t launch_simple_grads_lin(const double *units, const int *ys, const int *lx, const int *ly,
                                    const double *alphas, const double *betas, const int *scales,

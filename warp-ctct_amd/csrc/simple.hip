@@ -32,14 +32,11 @@ __device__ __forceinline__ int clampi(int v, int lo, int hi) { return min(max(v,
 // last pass (the sum over the slabs of the reduction, LogmmDeferred) to this
 // kernel: every cell u <= ly of a live frame computes its den[t,u], writes it
 // (the backward reads all of them), and context 0 writes the frame's fmax.
-// LINEAR: the units are stored as 2^(log2 unit), for the lattices in the linear
-// domain (lattice_lin.hip): neutral units are {1, 1, 0}, log 0 is 0.  That
-// variant also lowers `flag`, which the kernels behind it raise.
 // only_if (may be null): return at once while *only_if is 0 (the fall-back run
-// of the log-domain variant behind the linear lattices).
-template <bool LINEAR>
-__device__ __forceinline__ double unit_out(double log2_unit) {
-    if (!LINEAR) return log2_unit;
+// behind the lattices in the linear domain).
+
+// 2^(log2 unit): a unit as the linear sweeps take it; log 0 is 0.
+__device__ __forceinline__ double unit_lin(double log2_unit) {
     if (log2_unit == neg_inf()) return 0.0;
     // 2^x = 2^floor(x) * 2^frac, the second factor on the fp32 transcendental unit
     // (relative error ~1e-7 per unit, without bias: a product of a thousand
@@ -49,18 +46,17 @@ __device__ __forceinline__ double unit_out(double log2_unit) {
     return __builtin_amdgcn_ldexp((double)exp2_hw((float)(log2_unit - fl)), (int)clamped);
 }
 
-template <bool DEFERRED, bool LINEAR>
+template <bool DEFERRED>
 __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     const float *__restrict__ f, const float *__restrict__ g, float *__restrict__ den,
     const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
     double *__restrict__ units, int T, int U, int V, int P, const RelaySlots relay,
     const LogmmDeferred deferred, float *__restrict__ fmax, unsigned *__restrict__ counter,
-    unsigned *__restrict__ status, unsigned *__restrict__ flag, const unsigned *__restrict__ only_if) {
+    unsigned *__restrict__ status, const unsigned *__restrict__ only_if) {
     if (only_if && *only_if == 0u) return;
     relay_clear_share(relay);
     // (the arrival counter of the lattice kernel's cost reduction, if there is one)
     if (counter && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *counter = 0u;
-    if (LINEAR && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) *flag = 0u;
     const int U1 = U + 1;
     const int n = blockIdx.y;
     const int cell = blockIdx.x * kBlock + threadIdx.x;
@@ -98,9 +94,9 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     // padding context of a live frame, or a cell outside the band of complete
     // alignments (its units cannot influence costs or gradients): neutral units
     if (!live) {
-        o[0] = LINEAR ? 1.0 : 0.0;
-        o[1] = LINEAR ? 1.0 : 0.0;
-        o[2] = LINEAR ? 0.0 : neg_inf();
+        o[0] = 0.0;
+        o[1] = 0.0;
+        o[2] = neg_inf();
         return;
     }
     const float *gr = g + ((size_t)n * U1 + u) * V;
@@ -112,14 +108,123 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
     // a NaN unit (NaN in f, g or den) enters the lattice as log 0 and is reported
     if (b != b || cur != cur || nxt != nxt) {
         if (status) atomicOr(status, kStatusNanInput);
-        o[0] = unit_out<LINEAR>((b != b) ? neg_inf() : b * kLog2e);
-        o[1] = unit_out<LINEAR>((cur != cur) ? neg_inf() : cur * kLog2e);
-        o[2] = unit_out<LINEAR>((nxt != nxt) ? neg_inf() : nxt);
+        o[0] = (b != b) ? neg_inf() : b * kLog2e;
+        o[1] = (cur != cur) ? neg_inf() : cur * kLog2e;
+        o[2] = (nxt != nxt) ? neg_inf() : nxt;
         return;
     }
-    o[0] = unit_out<LINEAR>(b * kLog2e);
-    o[1] = unit_out<LINEAR>(cur * kLog2e);
-    o[2] = unit_out<LINEAR>(nxt);
+    o[0] = b * kLog2e;
+    o[1] = cur * kLog2e;
+    o[2] = nxt;
+}
+
+// The units for the sweeps in the linear domain (lattice_lin.hip): one thread per
+// (frame, column); lanes 1..62 of a wavefront are the contexts 62 w .. 62 w + 61,
+// lane 0 and lane 63 the columns through which the wavefronts below / above hand
+// their boundary values over.  A context's cell holds {blank, label, next label,
+// next label of the context below} as linear factors (neutral {1, 1, 0, 0}); the
+// last one lets the beta sweep send what it hands down already multiplied.
+// Cells of the columns in between: lane 0 {1, 0, E, 0}, lane 63 {0, 1, 0, E},
+// E = "nothing there yet" where a wavefront will write, 0 where none does; the
+// zeros beside it take the sender's scale.  den, fmax, counter, status: as in
+// simple_gather_units_kernel; *flag is lowered.
+template <bool DEFERRED>
+__global__ __launch_bounds__(kBlock) void simple_gather_units_lin_kernel(
+    const float *__restrict__ f, const float *__restrict__ g, float *__restrict__ den,
+    const int *__restrict__ ys, const int *__restrict__ lx, const int *__restrict__ ly,
+    double *__restrict__ units, int T, int U, int V, int Pl, const LogmmDeferred deferred,
+    float *__restrict__ fmax, unsigned *__restrict__ counter, unsigned *__restrict__ status,
+    unsigned *__restrict__ flag) {
+    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+        if (counter) *counter = 0u;
+        *flag = 0u;
+    }
+    const int U1 = U + 1;
+    const int n = blockIdx.y;
+    const int cell = blockIdx.x * kBlock + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int t = cell / Pl, col = cell - t * Pl;   // t is the same for the whole wavefront
+    const int w = col >> 6;
+    const int u = w * kLinReal + lane - 1;
+    const int Tn = clampi(lx[n], 0, T), Un = clampi(ly[n], 0, U);
+    if (t >= Tn) {                                  // (covers cell >= T * Pl)
+        if (DEFERRED && t < T && col == 0) fmax[(size_t)n * T + t] = -__builtin_huge_valf();
+        return;
+    }
+    const float *fr = f + ((size_t)n * T + t) * V;
+    const bool real = lane >= 1 && lane <= kLinReal;
+    const bool in = real && u <= Un;
+    float den_tu = 0.0f;
+    if (DEFERRED) {
+        if (in) {
+            float row_max;
+            den_tu = logmm_finish_cell(deferred, n, t, u, fr, 1, g + ((size_t)n * U1 + u) * V, 1, V,
+                                       row_max);
+            den[((size_t)n * T + t) * U1 + u] = den_tu;
+            if (u == 0) fmax[(size_t)n * T + t] = row_max;
+        }
+    } else if (den && in) {
+        den_tu = den[((size_t)n * T + t) * U1 + u];
+    }
+    const bool live = in && !outside_band(t, u, Tn, Un);
+    const int *y = ys + (size_t)n * U;
+    // the next label's column: wanted by this cell or by the cell of context u+1
+    const bool has2 = real && u < Un;
+    const int c2 = has2 ? label_column(y[u], V, status) : 0;
+    const bool wanted = has2 && (live || !outside_band(t, u + 1, Tn, Un));
+    const float f2 = wanted ? fr[c2] : 0.0f;
+    float f1 = __shfl_up(f2, 1, 64);
+    const int c1 = (in && u >= 1) ? clampi(y[u - 1], 0, V - 1) : 0;
+    // (lane 1's neighbour is in another wavefront; its unit is wanted for the
+    // fourth factor even where this cell itself is outside the band)
+    const bool below_live = in && u >= 1 && !outside_band(t, u - 1, Tn, Un);
+    if (lane == 1 && (live || below_live) && u >= 1) f1 = fr[c1];
+    double v0 = 1.0, v1 = 1.0, v2 = 0.0;
+    if (live) {
+        const float *gr = g + ((size_t)n * U1 + u) * V;
+        const double d = (double)den_tu;
+        const double b = (double)fr[0] + (double)gr[0] - d;
+        double cur = b, nxt = neg_inf();
+        if (u >= 1) cur = (double)f1 + (double)gr[c1] - d;
+        if (has2) nxt = ((double)f2 + (double)gr[c2] - d) * kLog2e;
+        // a NaN unit (NaN in f, g or den) enters the lattice as log 0 and is reported
+        if (b != b || cur != cur || nxt != nxt) {
+            if (status) atomicOr(status, kStatusNanInput);
+        }
+        v0 = unit_lin((b != b) ? neg_inf() : b * kLog2e);
+        v1 = unit_lin((cur != cur) ? neg_inf() : cur * kLog2e);
+        v2 = unit_lin((nxt != nxt) ? neg_inf() : nxt);
+    }
+    // what the context below stores as its next-label unit (0 where it stores
+    // none), whether this cell itself is inside the band or not: the step from
+    // (t, u-1) to (t+1, u) may be part of an alignment that cell (t, u) is not
+    double v3 = __hiloint2double(__shfl_up(__double2hiint(v2), 1, 64), __shfl_up(__double2loint(v2), 1, 64));
+    if (lane == 1) {
+        v3 = 0.0;
+        if (below_live) {
+            float den_b = 0.0f;
+            const float *gb = g + ((size_t)n * U1 + u - 1) * V;
+            if (DEFERRED) {
+                float row_max;
+                den_b = logmm_finish_cell(deferred, n, t, u - 1, fr, 1, gb, 1, V, row_max);
+            } else if (den) {
+                den_b = den[((size_t)n * T + t) * U1 + u - 1];
+            }
+            const double below = ((double)f1 + (double)gb[c1] - (double)den_b) * kLog2e;
+            v3 = unit_lin((below != below) ? neg_inf() : below);
+        }
+    }
+    const double empty = __longlong_as_double((long long)kRelayEmpty);
+    if (lane == 0) {
+        v0 = 1.0, v1 = 0.0, v3 = 0.0;
+        v2 = (w >= 1 && w * kLinReal <= Un) ? empty : 0.0;
+    } else if (lane == 63) {
+        v0 = 0.0, v1 = 1.0, v2 = 0.0;
+        v3 = ((w + 1) * kLinReal <= Un) ? empty : 0.0;
+    }
+    double *o = units + (((size_t)n * T + t) * Pl + col) * kLinUnit;
+    *reinterpret_cast<double2 *>(o) = make_double2(v0, v1);
+    *reinterpret_cast<double2 *>(o + 2) = make_double2(v2, v3);
 }
 
 // Per frame: grad_den[t,u] = -(g0+g1+g2), grad_f[t,u>=1] = g1[t,u] + g2[t,u-1],
@@ -212,27 +317,30 @@ __global__ __launch_bounds__(512) void simple_grads_kernel(
     const int n = blockIdx.y, u = threadIdx.x;
     const int lane = u & 63, wave = u >> 6, waves = P >> 6;
     const int Tn = clampi(lx[n], 0, T), Un = clampi(ly[n], 0, U);
-    const size_t lat = (size_t)(T + 1) * P * 2;
-    const double *units_n = units + (size_t)n * T * P * 3;
+    // columns per row of the work buffers (LIN: those of the linear sweeps)
+    const int Pw = LIN ? lin_padded(U) : P;
+    const size_t lat = (size_t)(T + 1) * Pw * 2;
+    const double *units_n = units + (size_t)n * T * Pw * (LIN ? kLinUnit : 3);
     const double *alpha_n = alphas + (size_t)n * lat, *beta_n = betas + (size_t)n * lat;
     const int *y = ys + (size_t)n * U;
     const int t_begin = blockIdx.x * F;
-    // LIN: the scales of this context's 64 and of the next context's (the same
-    // but for lane 63), and the lattice's total mass: beta(0, state 0)
+    // LIN: the scales of this context's wavefront (of the sweeps) and of the next
+    // context's, and the lattice's total mass: beta(0, state 0)
     const int chunks1 = lin_chunks(T) + 1;
     const int *sc_beta = nullptr, *sc_beta_next = nullptr, *sc_alpha = nullptr;
     double inv_ll = 0.0;
     int s_ll = 0;
     if (LIN) {
-        const int w_next = min((u + 1) >> 6, waves - 1);
-        sc_beta = scales + (((size_t)n * 2 + 0) * waves + wave) * chunks1;
-        sc_beta_next = scales + (((size_t)n * 2 + 0) * waves + w_next) * chunks1;
-        sc_alpha = scales + (((size_t)n * 2 + 1) * waves + wave) * chunks1;
-        const double ll = beta_n[1];
+        const int lw = lin_waves(U);
+        const int w_own = min(u / kLinReal, lw - 1), w_next = min((u + 1) / kLinReal, lw - 1);
+        sc_beta = scales + (((size_t)n * 2 + 0) * lw + w_own) * chunks1;
+        sc_beta_next = scales + (((size_t)n * 2 + 0) * lw + w_next) * chunks1;
+        sc_alpha = scales + (((size_t)n * 2 + 1) * lw + w_own) * chunks1;
+        const double ll = beta_n[lin_column(0) * 2 + 1];
         const int ex = (ll > 0.0 && ll < __builtin_huge_val()) ? __builtin_amdgcn_frexp_exp(ll) : 0;
         inv_ll = 1.0 / __builtin_amdgcn_ldexp(ll, -ex);   // (0 or inf: NaN below, caught by the check)
         // row 0 of beta was stored by step Tn - 1 of context 0's wavefront
-        s_ll = ex + scales[(((size_t)n * 2 + 0) * waves + 0) * chunks1 + (Tn > 0 ? 1 + (Tn - 1) / kLinChunk : 0)];
+        s_ll = ex + scales[(((size_t)n * 2 + 0) * lw + 0) * chunks1 + (Tn > 0 ? 1 + (Tn - 1) / kLinChunk : 0)];
     }
     // all frames of the block first (their loads are independent), then one exchange
     UnitGrad g[F];
@@ -249,7 +357,7 @@ __global__ __launch_bounds__(512) void simple_grads_kernel(
                 const int ia = t > 0 ? 1 + (t - 1) / kLinChunk : 0;
                 const int ib = t + 1 < Tn ? 1 + (Tn - 2 - t) / kLinChunk : 0;
                 bool bad;
-                g[f] = unit_grad_cell_lin(units_n, alpha_n, beta_n, y, t, u, Un, P, sc_alpha[ia],
+                g[f] = unit_grad_cell_lin(units_n, alpha_n, beta_n, y, t, u, Un, Pw, sc_alpha[ia],
                                           sc_beta[ib], sc_beta_next[ib], inv_ll, s_ll, bad);
                 bad_unit = bad_unit || bad;
             } else {
@@ -508,7 +616,7 @@ hipError_t launch_simple_gather_units(const float *f, const float *g, float *den
                                       const int *lx, const int *ly, double *units, int N, int T,
                                       int U, int V, const RelaySlots &relay,
                                       const LogmmDeferred &deferred, float *fmax,
-                                      unsigned *counter, hipStream_t stream, unsigned *linear_flag,
+                                      unsigned *counter, hipStream_t stream,
                                       const unsigned *only_if) {
     const int P = padded_contexts(U);
     const long cells = (long)T * P;
@@ -517,16 +625,33 @@ hipError_t launch_simple_gather_units(const float *f, const float *g, float *den
                              deferred.B != N || deferred.Nn != U + 1))
         return hipErrorInvalidValue;
     unsigned *status = device_status_word();
-#define GATHER(DEF, LIN)                                                                            \
-    TIMED_LAUNCH((simple_gather_units_kernel<DEF, LIN>), grid, dim3(kBlock), 0, stream, f, g, den,  \
-                 ys, lx, ly, units, T, U, V, P, relay, deferred, fmax, counter, status,             \
-                 linear_flag, only_if)
-    if (deferred.partial) {
-        if (linear_flag) GATHER(true, true); else GATHER(true, false);
-    } else {
-        if (linear_flag) GATHER(false, true); else GATHER(false, false);
-    }
-#undef GATHER
+    if (deferred.partial)
+        TIMED_LAUNCH(simple_gather_units_kernel<true>, grid, dim3(kBlock), 0, stream, f, g, den, ys, lx,
+                     ly, units, T, U, V, P, relay, deferred, fmax, counter, status, only_if);
+    else
+        TIMED_LAUNCH(simple_gather_units_kernel<false>, grid, dim3(kBlock), 0, stream, f, g, den, ys, lx,
+                     ly, units, T, U, V, P, relay, deferred, fmax, counter, status, only_if);
+    return hipGetLastError();
+}
+
+hipError_t launch_simple_gather_units_lin(const float *f, const float *g, float *den, const int *ys,
+                                          const int *lx, const int *ly, double *units, int N, int T,
+                                          int U, int V, const LogmmDeferred &deferred, float *fmax,
+                                          unsigned *counter, unsigned *flag, hipStream_t stream) {
+    if (!simple_grads_lin_applies(T, U) || !flag) return hipErrorInvalidValue;
+    const int Pl = lin_padded(U);
+    const long cells = (long)T * Pl;
+    const dim3 grid((unsigned)((cells + kBlock - 1) / kBlock), (unsigned)N);
+    if (deferred.partial && (!den || !fmax || deferred.splits < 1 || deferred.splits > 8 ||
+                             deferred.B != N || deferred.Nn != U + 1))
+        return hipErrorInvalidValue;
+    unsigned *status = device_status_word();
+    if (deferred.partial)
+        TIMED_LAUNCH(simple_gather_units_lin_kernel<true>, grid, dim3(kBlock), 0, stream, f, g, den, ys,
+                     lx, ly, units, T, U, V, Pl, deferred, fmax, counter, status, flag);
+    else
+        TIMED_LAUNCH(simple_gather_units_lin_kernel<false>, grid, dim3(kBlock), 0, stream, f, g, den, ys,
+                     lx, ly, units, T, U, V, Pl, deferred, fmax, counter, status, flag);
     return hipGetLastError();
 }
 
@@ -535,7 +660,8 @@ hipError_t launch_simple_gather_units(const float *f, const float *g, float *den
 // the caller adds those up with launch_simple_grads' second half afterwards.
 bool simple_grads_lin_applies(int T, int U) {
     // (the linear sweeps address a sample's units through 32-bit byte offsets)
-    return T > 0 && padded_contexts(U) <= 512 && (size_t)T * padded_contexts(U) * 3 * sizeof(double) < (1ULL << 31);
+    return T > 0 && padded_contexts(U) <= 512 &&
+           (size_t)T * lin_padded(U) * kLinUnit * sizeof(double) < (1ULL << 31);
 }
 
 hipError_t launch_simple_grads_lin(const double *units, const int *ys, const int *lx, const int *ly,

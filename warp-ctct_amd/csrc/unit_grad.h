@@ -62,19 +62,22 @@ __device__ __forceinline__ UnitGrad unit_grad_cell(const double *units_n, const 
 }
 
 // The same from lattices in the linear domain (lattice_lin.hip): alpha / beta
-// rows are masses relative to 2^scale, one scale per (direction, 64 contexts,
-// chunk of frames); units are linear.  sa / sb / sb_next: the scales of row t of
+// rows are masses relative to 2^scale, one scale per (direction, wavefront of
+// kLinReal contexts, chunk of frames); units are linear; Pl columns per row,
+// context u in column lin_column(u).  sa / sb / sb_next: the scales of row t of
 // alpha, and of row t+1 of beta for context u and for context u+1; inv_ll and
 // s_ll: 1 / mantissa and exponent of the lattice's total mass beta(0, state 0).
 __device__ __forceinline__ UnitGrad unit_grad_cell_lin(const double *units_n, const double *alpha_n,
                                                        const double *beta_n, const int *y, int t,
-                                                       int u, int Un, int P, int sa, int sb,
+                                                       int u, int Un, int Pl, int sa, int sb,
                                                        int sb_next, double inv_ll, int s_ll,
                                                        bool &out_of_range) {
-    const double2 a = *reinterpret_cast<const double2 *>(alpha_n + ((size_t)t * P + u) * 2);
-    const double2 b = *reinterpret_cast<const double2 *>(beta_n + ((size_t)(t + 1) * P + u) * 2);
-    const double *lp = units_n + ((size_t)t * P + u) * 3;
-    const double lp0 = lp[0], lp1 = lp[1];
+    const int col = lin_column(u);
+    const double2 a = *reinterpret_cast<const double2 *>(alpha_n + ((size_t)t * Pl + col) * 2);
+    const double2 b = *reinterpret_cast<const double2 *>(beta_n + ((size_t)(t + 1) * Pl + col) * 2);
+    const double *lp = units_n + ((size_t)t * Pl + col) * kLinUnit;
+    const double2 lp01 = *reinterpret_cast<const double2 *>(lp);
+    const double lp0 = lp01.x, lp1 = lp01.y;
     // a unit outside [2^-80, 2^80] (other than 0) may overflow a chunk of frames,
     // or push a state out of range on its own: such a batch is not for this form
     auto bad = [](double x) { return x > 0x1p80 || (x != 0.0 && x < 0x1p-80); };
@@ -87,7 +90,7 @@ __device__ __forceinline__ UnitGrad unit_grad_cell_lin(const double *units_n, co
     if (u < Un) {
         const double lp2 = lp[2];
         out_of_range = out_of_range || bad(lp2);
-        const double bo_next = beta_n[((size_t)(t + 1) * P + u + 1) * 2];
+        const double bo_next = beta_n[((size_t)(t + 1) * Pl + lin_column(u + 1)) * 2];
         const double from = (u >= 1 && y[u - 1] != y[u]) ? a.y + a.x : a.y;
         r.g2 = -(float)((from * lp2) * bo_next * __builtin_amdgcn_ldexp(inv_ll, sa + sb_next - s_ll));
     }
