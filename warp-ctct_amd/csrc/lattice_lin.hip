@@ -134,16 +134,16 @@ static __device__ __forceinline__ void chunk_load_lin(ChunkL &c, __amdgpu_buffer
     }
 }
 
-// The units of R frames that all exist, the row offset walking by one scalar
-// addition per frame: `at` is the byte offset of the row of the chunk's first frame.
+// The units of R frames that all exist: `lowest` is the address of the chunk's
+// row with the lowest frame index, off[r] the byte offset of step r's row from
+// it (the same for every chunk, so no address arithmetic per frame).
 template <bool BETA, bool COHERENT>
-static __device__ __forceinline__ void chunk_load_walk_lin(ChunkL &c, __amdgpu_buffer_rsrc_t units,
-                                                           unsigned &at, unsigned lane_bytes, unsigned step) {
+static __device__ __forceinline__ void chunk_load_whole_lin(ChunkL &c, const char *lowest,
+                                                            const unsigned (&off)[R], unsigned lane_bytes) {
+    const __amdgpu_buffer_rsrc_t rows =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(lowest), 0, 0xffffffffu, 0x00020000);
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        row_load_lin<BETA, COHERENT>(c.lp[r], units, lane_bytes, at);
-        at = BETA ? at - step : at + step;
-    }
+    for (int r = 0; r < R; ++r) row_load_lin<BETA, COHERENT>(c.lp[r], rows, lane_bytes, off[r]);
 }
 
 // Only the fields another wavefront fills (the third factor of every frame and
@@ -241,11 +241,21 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
         // the column this wavefront fills for the next one: its lane kGhost's
         const unsigned send_bytes = (unsigned)((BETA ? wave - 1 : wave + 1) * 64 + kGhost) * kCellBytes;
         chunk_load_lin<BETA, false>(a, rows_in, in_bytes, in_step, Tn, t_start);
+        // byte offsets of a whole chunk's rows from its lowest one, in the units
+        // and in the lattice: step r's row is the r-th from the bottom (alpha) or
+        // from the top (beta)
+        unsigned in_off[R], out_off[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            in_off[r] = (unsigned)(BETA ? R - 1 - r : r) * in_step;
+            out_off[r] = (unsigned)(BETA ? R - 1 - r : r) * out_step;
+        }
         bool lost = false;     // the hand-over did not arrive in time, or its sender says so
         // whether a chunk has to find out that its hand-over was complete (not
         // once it is lost, or holds NaNs of the sender's own)
         bool watch = HAS_IN;
-        auto run_chunk = [&](ChunkL &c, int k, int cnt, bool full, bool last) {
+        // lowest: the address of the chunk's lowest row of units (whole chunks only)
+        auto run_chunk = [&](ChunkL &c, int k, int cnt, bool full, bool last, const char *lowest) {
             const int t_first = t_start + dir * k * R;
             const double e_kept = e, o_kept = o;
             const int S_kept = S;
@@ -296,7 +306,7 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
                         v4u_lin w;
                         w[0] = __double2loint(o), w[1] = __double2hiint(o);
                         w[2] = __double2loint(e), w[3] = __double2hiint(e);
-                        __builtin_amdgcn_raw_buffer_store_b128(w, rows, out_lane, at, 0);
+                        __builtin_amdgcn_raw_buffer_store_b128(w, rows, out_lane, full ? out_off[r] : at, 0);
                         at = BETA ? at - out_step : at + out_step;
                     }
                 }
@@ -335,14 +345,18 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
             out_row = BETA ? out_row - (size_t)(full ? R : cnt) * out_step
                            : out_row + (size_t)(full ? R : cnt) * out_step;
             if (has_out && !lost && lane == kEdge) {
+                const __amdgpu_buffer_rsrc_t to = full ? __builtin_amdgcn_make_buffer_rsrc(
+                                                             const_cast<char *>(lowest), 0, 0xffffffffu, 0x00020000)
+                                                       : rows_in;
                 unsigned at = (unsigned)t_first * in_step;
-                __builtin_amdgcn_raw_buffer_store_b64(as_words((double)S + kScaleBias), rows_in,
-                                                      send_bytes + scale_field<BETA>(), at, kAgentScope);
+                __builtin_amdgcn_raw_buffer_store_b64(as_words((double)S + kScaleBias), to,
+                                                      send_bytes + scale_field<BETA>(), full ? in_off[0] : at,
+                                                      kAgentScope);
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     if (full || r < cnt)
-                        __builtin_amdgcn_raw_buffer_store_b64(as_words(mine[r]), rows_in,
-                                                              send_bytes + third_field<BETA>(), at, kAgentScope);
+                        __builtin_amdgcn_raw_buffer_store_b64(as_words(mine[r]), to, send_bytes + third_field<BETA>(),
+                                                              full ? in_off[r] : at, kAgentScope);
                     at = BETA ? at - in_step : at + in_step;
                 }
             }
@@ -365,17 +379,21 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
         // four chunks per turn; while the chunk after the turn lies inside the
         // sample, the rows of units need no clamp
         if (5 * R <= Tn) {
-            unsigned at = (unsigned)(t_start + dir * R) * in_step;
+            // the lowest row of chunk 0, and from one chunk to the next
+            const char *lowest = reinterpret_cast<const char *>(units_n) +
+                                 (size_t)(BETA ? t_start - (R - 1) : 0) * in_step;
+            const ptrdiff_t onward = (ptrdiff_t)dir * R * (ptrdiff_t)in_step;
             int k = 0;
             do {
-                chunk_load_walk_lin<BETA, false>(b, rows_in, at, in_bytes, in_step);
-                run_chunk(a, k, R, true, false);
-                chunk_load_walk_lin<BETA, false>(a, rows_in, at, in_bytes, in_step);
-                run_chunk(b, k + 1, R, true, false);
-                chunk_load_walk_lin<BETA, false>(b, rows_in, at, in_bytes, in_step);
-                run_chunk(a, k + 2, R, true, false);
-                chunk_load_walk_lin<BETA, false>(a, rows_in, at, in_bytes, in_step);
-                run_chunk(b, k + 3, R, true, false);
+                chunk_load_whole_lin<BETA, false>(b, lowest + onward, in_off, in_bytes);
+                run_chunk(a, k, R, true, false, lowest);
+                chunk_load_whole_lin<BETA, false>(a, lowest + 2 * onward, in_off, in_bytes);
+                run_chunk(b, k + 1, R, true, false, lowest + onward);
+                chunk_load_whole_lin<BETA, false>(b, lowest + 3 * onward, in_off, in_bytes);
+                run_chunk(a, k + 2, R, true, false, lowest + 2 * onward);
+                chunk_load_whole_lin<BETA, false>(a, lowest + 4 * onward, in_off, in_bytes);
+                run_chunk(b, k + 3, R, true, false, lowest + 3 * onward);
+                lowest += 4 * onward;
                 k += 4;
                 s0 += 4 * R;
             } while (s0 + 5 * R <= Tn);
@@ -383,7 +401,7 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
         // the rest (fewer than five chunks), one chunk per turn
         while (s0 < Tn) {
             chunk_load_lin<BETA, false>(b, rows_in, in_bytes, in_step, Tn, t_start + dir * (s0 + R));
-            run_chunk(a, s0 / R, min(Tn - s0, R), false, s0 + R >= Tn);
+            run_chunk(a, s0 / R, min(Tn - s0, R), false, s0 + R >= Tn, nullptr);
             a = b;
             s0 += R;
         }
