@@ -479,24 +479,25 @@ enum {
 int warpctct_status(unsigned *bits, int clear);
 
 /* The fused joiner forward (warpctct_simple_forward_f32 / _reduced_f32 with
- * gradients, U + 1 <= 512, long inputs) sweeps its lattices in the LINEAR domain first: path
- * masses relative to one power of two per 64 contexts and 12 frames, two
- * multiplications and three additions per frame where the log domain needs two
- * semiring sums per state (less than half the time per frame; the frames of a
- * lattice are strictly serial, so that is the latency of the whole call).  The
- * linear form drops states that lie ~2^-1000 below the largest of their 64
- * contexts.  The kernel that forms the gradients therefore checks that the
- * posteriors of every frame add up to 1 within 2e-5, that every gathered unit
- * lies in [2^-80, 2^80] or is 0, and that everything is finite; if not, the
- * log-domain kernels, launched behind it in the same stream, compute the batch
- * again (they return at once otherwise), and
+ * gradients, U + 1 <= 512, long inputs) sweeps its lattices in the LINEAR domain
+ * first: path masses relative to one power of two per wavefront (62 contexts)
+ * and 12 frames, three multiplications and three additions per frame where the
+ * log domain needs two semiring sums per state (half the time per frame; the
+ * frames of a lattice are strictly serial, so that is the latency of the whole
+ * call).  The linear form drops states that lie ~2^-1000 below the largest of
+ * their wavefront.  The kernel that forms the gradients therefore checks that
+ * the posteriors of every frame add up to 1 within 2e-5, that every gathered
+ * unit lies in [2^-80, 2^80] or is 0, and that everything is finite; if not,
+ * the log-domain kernels, launched behind it in the same stream, compute the
+ * batch again (they return at once otherwise), and
  * WARPCTCT_STATUS_LINEAR_FELL_BACK is set.  No counterpart in the reference
- * (csrc/simple.cu sweeps in the log domain).  The linear sweeps save 30-40 ns
+ * (csrc/simple.cu sweeps in the log domain).  The linear sweeps save 35-45 ns
  * per frame and cost ~14 us per call (the launches that return at once, a
- * slower gather and gradient kernel), so they are used from T = 768 frames on.
- * warpctct_joiner_linear_lattice(n) moves that limit for later calls of the
- * process (0: never; 1: always; negative: the default) and returns the
- * previous one. */
+ * slower gather and gradient kernel), so they are used from T = 512 frames on,
+ * with normalisation from T = 1024 on.
+ * warpctct_joiner_linear_lattice(n) sets one limit for both for later calls of
+ * the process (0: never; 1: always; negative: back to those defaults) and
+ * returns the previous setting (negative: the defaults). */
 int warpctct_joiner_linear_lattice(int from_frames);
 
 /* ---- measurement aid ------------------------------------------------------

@@ -23,7 +23,7 @@ GRAD_ATOL = 1e-4
 def lattice_domain(request):
     """Every test of this file runs twice: with the joiner's lattices swept in the
     log domain only, and with the linear sweeps (checked, with the log domain as
-    their fall-back) used for every input, not just from 768 frames on."""
+    their fall-back) used for every input, not just for long ones."""
     import warp_ctct
     lib = hip_lib.lib()
     before = lib.warpctct_joiner_linear_lattice(1 if request.param == "linear_lattices" else 0)
@@ -872,15 +872,16 @@ def _loss_and_grads(f, g, ys, lx, ly, normalized, reduction="none", w=None):
 
 
 @pytest.mark.parametrize("normalized", [True, False])
-def test_linear_lattices_are_used_from_768_frames_and_hold_on_ordinary_input(normalized, lattice_domain):
+def test_linear_lattices_are_used_for_long_inputs_and_hold_on_ordinary_input(normalized, lattice_domain):
     """With the default setting the fused forward sweeps in the linear domain from
-    768 frames on (lattice_lin_kernel is launched, the log-domain kernels behind it
-    return at once: the fall-back bit stays clear), and below that in the log
-    domain; both agree with the oracle.  A chain of two workgroups per lattice."""
+    512 frames on, from 1024 with normalisation (lattice_lin_kernel is launched, the
+    log-domain kernels behind it return at once: the fall-back bit stays clear),
+    and below that in the log domain; both agree with the oracle.  A chain of two
+    workgroups per lattice."""
     import warp_ctct
     lib = hip_lib.lib()
     lib.warpctct_joiner_linear_lattice(-1)
-    for T, linear in ((780, True), (760, False)):
+    for T, linear in (((1030, True), (1000, False)) if normalized else ((520, True), (500, False))):
         N, U, V = 2, 70, 24
         f, g, ys, lx, ly = make_simple_case(60 + T, N, T, U, V, lx=[T, T - 37], ly=[U, 41],
                                             normalized=normalized)
@@ -940,3 +941,37 @@ def test_linear_lattices_fall_back_to_the_log_domain(what, lattice_domain):
     if what != "infeasible_sample":
         np.testing.assert_allclose(results[1][0].cpu().numpy(), costs, rtol=LOSS_RTOL)
         np.testing.assert_allclose(results[1][1].cpu().numpy(), gf, atol=GRAD_ATOL, rtol=1e-5)
+
+
+@pytest.mark.may_fall_back
+def test_linear_lattices_give_up_a_hand_over_that_does_not_arrive(lattice_domain):
+    """The bounded wait of the linear sweeps, forced from the host: with a wait
+    limit of 0 a wavefront that finds its neighbour's values missing declares them
+    lost at its first look (no kernel waits, every one of them exits), the status
+    word says so and that the batch went to the log-domain kernels, whose own
+    chains lose their hand-overs the same way.  The call after that, with the
+    limit back, is right again: nothing of the lost call is left in the buffers."""
+    import warp_ctct
+    lib = hip_lib.lib()
+    N, T, U, V = 3, 180, 150, 40                    # chains of three workgroups; sample 2 has one
+    f, g, ys, lx, ly = make_simple_case(91, N, T, U, V, lx=[T, 160, 40], ly=[U, 120, 30], normalized=False)
+    _, gf, gg, costs = O.ctct_simple_loss(f, g, ys, lx, ly, reduction="none", normalized=False)
+    assert np.all(np.isfinite(costs))               # (every sample has alignments)
+    lib.warpctct_joiner_linear_lattice(1)
+    warp_ctct.status(reset=True)
+    default = lib.warpctct_lattice_wait_limit(0)
+    try:
+        got = _loss_and_grads(f, g, ys, lx, ly, False)
+    finally:
+        assert lib.warpctct_lattice_wait_limit(-1) == 0
+    bits = warp_ctct.status(reset=True)
+    assert default > 1000
+    assert bits & warp_ctct.STATUS_LOST_HAND_OVER and bits & warp_ctct.STATUS_LINEAR_FELL_BACK, bits
+    # (the lone wavefront of sample 2 needs no hand-over, in either domain)
+    np.testing.assert_allclose(got[0].cpu().numpy()[2], costs[2], rtol=LOSS_RTOL)
+    got = _loss_and_grads(f, g, ys, lx, ly, False)
+    assert warp_ctct.status(reset=True) == 0
+    np.testing.assert_allclose(got[0].cpu().numpy(), costs, rtol=LOSS_RTOL)
+    np.testing.assert_allclose(got[1].cpu().numpy(), gf, atol=GRAD_ATOL, rtol=1e-5)
+    np.testing.assert_allclose(got[2].cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
+

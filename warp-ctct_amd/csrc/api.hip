@@ -86,12 +86,14 @@ int forward_from_units(const Workspace &w, const int *ys, const int *lx, const i
 }
 
 // from how many frames on the fused joiner forward sweeps its lattices in the
-// linear domain first (warpctct_joiner_linear_lattice; 0: never).  The linear
-// sweeps save 30-40 ns per frame and cost ~14 us per call (three launches that
-// return at once, a slower gather and gradient kernel): measured, they gain from
-// about 600 frames on, more for chains of workgroups than for lone ones.
-constexpr int kLinearFromFrames = 768;
-std::atomic<int> g_linear_from{kLinearFromFrames};
+// linear domain first (warpctct_joiner_linear_lattice; 0: never; negative: the
+// defaults below).  The linear sweeps save 35-45 ns per frame and cost ~14 us
+// per call (three launches that return at once, a slower gather and gradient
+// kernel; the gather more so where it also finishes the denominators):
+// measured, they gain from about 450 frames on without, and from about 800 with
+// the normalisation.
+constexpr int kLinearFromFrames = 512, kLinearFromFramesNormalized = 1024;
+std::atomic<int> g_linear_from{-1};
 
 struct SimpleWorkspace {
     Workspace lattice;
@@ -296,8 +298,7 @@ int warpctct_simple_units_f32(const float *f_g, const float *g_g, const float *d
 int warpctct_lattice_wait_limit(int spins) { return lattice_wait_limit(spins); }
 
 int warpctct_joiner_linear_lattice(int from_frames) {
-    return g_linear_from.exchange(from_frames < 0 ? kLinearFromFrames : from_frames,
-                                  std::memory_order_relaxed);
+    return g_linear_from.exchange(from_frames < 0 ? -1 : from_frames, std::memory_order_relaxed);
 }
 
 size_t warpctct_lattice_relay_bytes(int N, int T, int U) {
@@ -789,7 +790,8 @@ int warpctct_simple_forward_reduced_f32(const float *f, const float *g, const in
                                        &deferred, st));
             if (rc != WARPCTCT_OK) return rc;
         }
-        const int linear_from = g_linear_from.load(std::memory_order_relaxed);
+        int linear_from = g_linear_from.load(std::memory_order_relaxed);
+        if (linear_from < 0) linear_from = normalized ? kLinearFromFramesNormalized : kLinearFromFrames;
         if (want_grad && linear_from > 0 && T >= linear_from && simple_grads_lin_applies(T, U)) {
             // The lattices in the linear domain (less than half the time per frame),
             // checked by the kernel that forms the gradients from them; the

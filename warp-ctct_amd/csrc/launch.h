@@ -122,7 +122,9 @@ hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream, const unsign
 // lin_column(u) of the lin_padded(U) columns that units, alphas and betas have
 // here, and the columns in between belong to those two lanes.
 //   units  (N,T,Pl,kLinUnit): {blank, label, next label, next label of the
-//          context below} as linear factors (neutral {1,1,0,0}); written by
+//          context below} as linear factors ({0,0,0,.} in padding and outside the
+//          band of complete alignments: mass that gets there is gone, instead of
+//          sitting there undiminished and dictating the wavefront's scale); written by
 //          launch_simple_gather_units_lin, which also sets up the columns in
 //          between; the sweeps write what they hand over into them
 //   alphas, betas (N,T+1,Pl,2): pairs {o, e} of masses

@@ -122,7 +122,7 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
 // (frame, column); lanes 1..62 of a wavefront are the contexts 62 w .. 62 w + 61,
 // lane 0 and lane 63 the columns through which the wavefronts below / above hand
 // their boundary values over.  A context's cell holds {blank, label, next label,
-// next label of the context below} as linear factors (neutral {1, 1, 0, 0}); the
+// next label of the context below} as linear factors; the
 // last one lets the beta sweep send what it hands down already multiplied.
 // Cells of the columns in between: lane 0 {1, 0, E, 0}, lane 63 {0, 1, 0, E},
 // E = "nothing there yet" where a wavefront will write, 0 where none does; the
@@ -179,7 +179,12 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_lin_kernel(
     // fourth factor even where this cell itself is outside the band)
     const bool below_live = in && u >= 1 && !outside_band(t, u - 1, Tn, Un);
     if (lane == 1 && (live || below_live) && u >= 1) f1 = fr[c1];
-    double v0 = 1.0, v1 = 1.0, v2 = 0.0;
+    // Padding, and cells outside the band of complete alignments (their units
+    // cannot influence costs or gradients): all 0.  The mass of alignments that
+    // cannot be completed is then gone where it leaves the band; with factors of
+    // 1 it would stay there undiminished while the mass that counts shrinks with
+    // every frame, and the scale of its wavefront would follow it.
+    double v0 = 0.0, v1 = 0.0, v2 = 0.0;
     if (live) {
         const float *gr = g + ((size_t)n * U1 + u) * V;
         const double d = (double)den_tu;
