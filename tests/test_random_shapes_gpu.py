@@ -96,12 +96,15 @@ def test_random_joint_and_logits_cases(seed):
 def test_random_joiner_cases(seed):
     """ctct_simple_loss, normalized and not: sizes around 128 frames, 16..96
     contexts and vocabularies of 512..2048 in chunks of 32, where the
-    log-matmul kernels change; -inf vocabulary entries and a frame far below
-    the others in a quarter of the cases."""
+    log-matmul kernels change, and some long inputs with up to 261 contexts;
+    -inf vocabulary entries and a frame far below the others in a quarter of
+    the cases; the lattices swept in the linear domain in half of them."""
     import warp_ctct
     rng = np.random.default_rng(seed)
-    Ts = [1, 17, 96, 127, 128, 129, 143, 144, 160]
-    Us = [0, 1, 15, 16, 31, 32, 47, 48, 63, 64, 79, 80, 95, 96, 97, 130]
+    # (the long ones for the sweeps in the linear domain: whole turns of their
+    # chunks, and chains of up to five workgroups that run into one another)
+    Ts = [1, 17, 96, 127, 128, 129, 143, 144, 160, 333, 700]
+    Us = [0, 1, 15, 16, 31, 32, 47, 48, 61, 62, 63, 64, 79, 80, 95, 96, 97, 123, 124, 130, 260]
     Vs = [3, 33, 256, 480, 511, 512, 544, 800, 1000, 1024, 1056, 2016, 2047, 2048, 2049, 2080, 2304]
     done = 0
     while done < 150 * SCALE:
