@@ -28,11 +28,11 @@ def dev(a, dtype=None):
     return torch.as_tensor(np.ascontiguousarray(a), device="cuda", dtype=dtype)
 
 
-def same_costs(got, ref):
+def same_costs(got, ref, atol=1e-5):
     got, ref = np.asarray(got, dtype=np.float64), np.asarray(ref, dtype=np.float64)
     fin = np.isfinite(ref)
     assert np.array_equal(np.isfinite(got), fin)
-    np.testing.assert_allclose(got[fin], ref[fin], rtol=LOSS_RTOL, atol=1e-5)
+    np.testing.assert_allclose(got[fin], ref[fin], rtol=LOSS_RTOL, atol=atol)
     return bool(np.all(fin))
 
 
@@ -146,7 +146,10 @@ def test_random_joiner_cases(seed):
         out = warp_ctct.ctct_simple_loss(tf, tg, dev(ys), dev(lx), dev(ly), reduction=reduction,
                                          average_frames=average_frames, normalized=normalized)
         (out * dev(w, torch.float32)).sum().backward()
-        if same_costs(np.atleast_1d(out.detach().cpu().numpy()), np.atleast_1d(loss)):
+        # (a frame 300 below the others cancels against its own normaliser: a cost
+        # near 0 then carries the rounding of float32 numbers of size 300, 3e-5 each)
+        if same_costs(np.atleast_1d(out.detach().cpu().numpy()), np.atleast_1d(loss),
+                      atol=1e-4 if (mask and normalized) else 1e-5):
             scale = max(1.0, float(np.abs(w).max()))
             # dense gradients sum up to T (resp. U+1) unit gradients per entry
             np.testing.assert_allclose(tf.grad.cpu().numpy(), gf, atol=GRAD_ATOL * scale, rtol=1e-5)
