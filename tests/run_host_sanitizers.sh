@@ -18,7 +18,7 @@ SAN="-fsanitize=address,undefined -fno-omit-frame-pointer -fno-sanitize-recover=
 "$LLVM/clang" -O1 -g -fPIC -fopenmp -fno-fast-math -Wall -Wextra $SAN -shared-libasan -shared \
     -o "$OUT/libctct_oracle.so" "$ROOT/oracle/ctct_oracle.c" -lm
 
-SRCS="api lattice units dense_grad simple logmm logits profile status"
+SRCS="api lattice lattice_lin units dense_grad simple logmm logits profile status"
 OBJS=""
 for s in $SRCS; do
     /opt/rocm/bin/hipcc -O1 -g -std=c++17 -fPIC --offload-arch=gfx950 \
