@@ -486,8 +486,8 @@ int warpctct_status(unsigned *bits, int clear);
  * frames of a lattice are strictly serial, so that is the latency of the whole
  * call).  The linear form drops states that lie ~2^-1000 below the largest of
  * their wavefront.  The kernel that forms the gradients therefore checks that
- * the posteriors of every frame add up to 1 within 2e-5, that every gathered
- * unit lies in [2^-80, 2^80] or is 0, and that everything is finite; if not,
+ * the posteriors of every frame add up to 1 within 2e-5 (lost mass shows there,
+ * and so does anything not finite) and that no gathered unit exceeds 2^80; if not,
  * the log-domain kernels, launched behind it in the same stream, compute the
  * batch again (they return at once otherwise), and
  * WARPCTCT_STATUS_LINEAR_FELL_BACK is set.  No counterpart in the reference

@@ -904,7 +904,8 @@ def test_linear_lattices_fall_back_to_the_log_domain(what, lattice_domain):
     """Input that the linear sweeps cannot take is computed again in the log
     domain, in the same call: the results are bit for bit those of a call with the
     linear sweeps switched off, and the status word says so.
-    - a gathered unit below 2^-80 (a frame whose label scores are ~-200);
+    - a gathered unit above 2^80 (a frame whose scores are ~+60: twelve such frames
+      in a row would leave the range of a double);
     - a sample with fewer frames than its labels need (cost +inf, NaN gradients);
     - all units in range, but the mass that counts far below the largest state of
       its 64 contexts: the one label can only be emitted in the first three frames
@@ -917,7 +918,7 @@ def test_linear_lattices_fall_back_to_the_log_domain(what, lattice_domain):
     N, T, U, V = 2, 64, 6, 11
     f, g, ys, lx, ly = make_simple_case(77, N, T, U, V, lx=[T, T - 9], ly=[U, 4], normalized=False)
     if what == "unit_out_of_range":
-        f[0, 20, :] = -200.0
+        f[0, 20, :] = 60.0
     elif what == "infeasible_sample":
         lx[1] = 3
     else:
@@ -975,3 +976,35 @@ def test_linear_lattices_give_up_a_hand_over_that_does_not_arrive(lattice_domain
     np.testing.assert_allclose(got[1].cpu().numpy(), gf, atol=GRAD_ATOL, rtol=1e-5)
     np.testing.assert_allclose(got[2].cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
 
+
+
+@pytest.mark.parametrize("normalized", [False, True])
+def test_linear_lattices_hold_on_peaked_scores(normalized, lattice_domain):
+    """What a trained model hands in: at every frame one entry of the vocabulary far
+    above the others (the label due there, or blank), the others 40-150 below, so
+    that most units are between 2^-60 and 2^-220 and the mass of nearly every
+    alignment vanishes against the best one's.  The linear sweeps lose such states,
+    which is harmless: their check must pass, and costs and gradients are the
+    oracle's.  Chains of three workgroups, 300 frames."""
+    import warp_ctct
+    N, T, U, V = 2, 300, 130, 40
+    rng = np.random.default_rng(5)
+    f = (-40.0 - 110.0 * rng.random((N, T, V))).astype(np.float32)
+    g = (0.1 * rng.standard_normal((N, U + 1, V))).astype(np.float32)
+    ys = rng.integers(1, V, size=(N, U)).astype(np.int32)
+    lx, ly = np.array([T, T - 23], np.int32), np.array([U, 101], np.int32)
+    for n in range(N):
+        # the labels spread evenly over the frames, blank between them
+        at = np.linspace(2, lx[n] - 3, ly[n]).astype(int)
+        f[n, :, 0] = 0.0
+        f[n, at, 0] = -60.0
+        f[n, at, ys[n, :ly[n]]] = 0.0
+    _, gf, gg, costs = O.ctct_simple_loss(f, g, ys, lx, ly, reduction="none", normalized=normalized)
+    assert np.all(np.isfinite(costs))
+    warp_ctct.status(reset=True)
+    got = _loss_and_grads(f, g, ys, lx, ly, normalized)
+    assert not (warp_ctct.status() & warp_ctct.STATUS_LINEAR_FELL_BACK)
+    # (normalised, the best alignment has probability 1 within float32: a cost of 0)
+    np.testing.assert_allclose(got[0].cpu().numpy(), costs, rtol=LOSS_RTOL, atol=1e-5 if normalized else 0)
+    np.testing.assert_allclose(got[1].cpu().numpy(), gf, atol=GRAD_ATOL, rtol=1e-5)
+    np.testing.assert_allclose(got[2].cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)

@@ -17,9 +17,8 @@
 // unless the alignments that carry the posterior mass pass through such a
 // state.  The kernel that forms the gradients from these lattices therefore
 // checks, per frame, that the posteriors it hands out add up to 1 (every
-// alignment consumes exactly one unit per frame), and that no unit lies outside
-// the range in which R frames can neither overflow nor lose a state on their
-// own; if any check fails (or a value is not finite, or a hand-over was lost)
+// alignment consumes exactly one unit per frame), and that no unit is so large
+// that R frames could overflow; if any check fails (or a value is not finite, or a hand-over was lost)
 // it raises a flag, and the log-domain kernels of lattice.hip, which follow
 // in the same stream and return at once while the flag is down, compute the
 // batch again.

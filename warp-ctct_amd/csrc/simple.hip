@@ -301,9 +301,9 @@ constexpr float kPosteriorSlack = 2e-5f;
 
 // LIN: the lattices are those of lattice_lin.hip (linear domain; `scales` as
 // launch_lattice_lin describes them), and the kernel checks what it hands out:
-// the posteriors of a frame add up to 1 (every alignment consumes exactly one
-// unit per frame), every number is finite, and no unit lies outside the range
-// the linear sweeps can take.  Where a check fails it raises *flag, and the
+// the posteriors of every frame add up to 1 (every alignment consumes exactly
+// one unit per frame; lost mass and anything not finite fail that), and no unit
+// is so large that a chunk of frames could overflow.  Where a check fails it raises *flag, and the
 // log-domain kernels launched behind it (only_if) compute the batch again.
 // only_if (may be null): return at once while *only_if is 0.
 template <bool LIN>
@@ -380,11 +380,12 @@ __global__ __launch_bounds__(512) void simple_grads_kernel(
         for (int off = 32; off >= 1; off >>= 1) blank += __shfl_xor(blank, off, 64);
         s_g2[f][u] = g[f].g2;
         if (lane == 0) s_blank[f][wave] = blank;
-        // The check: mass that the linear sweeps have lost is missing from every
-        // later frame's posteriors (alpha) or shows in them as a surplus (beta:
-        // the total they are divided by came out too small), so the first frame
-        // of each block and the sample's last frame are enough to look at.
-        if (LIN && (f == 0 || t_begin + f == Tn - 1)) {
+        // The check, on every frame: mass that the linear sweeps have lost is
+        // missing from every later frame's posteriors (alpha) or shows in them as a
+        // surplus (beta: the total they are divided by came out too small); a
+        // product that left the range of a double on the way to one posterior
+        // shows in that frame only.
+        if (LIN) {
             float all = g[f].g0 + g[f].g1 + g[f].g2;
 #pragma unroll
             for (int off = 32; off >= 1; off >>= 1) all += __shfl_xor(all, off, 64);
@@ -393,7 +394,7 @@ __global__ __launch_bounds__(512) void simple_grads_kernel(
     }
     __syncthreads();
     if (LIN) {
-        if (u < F && (u == 0 || t_begin + u == Tn - 1)) {
+        if (u < F) {
             const int t = t_begin + u;
             float all = 0.0f;
             for (int w = 0; w < waves; ++w) all += s_all[u][w];

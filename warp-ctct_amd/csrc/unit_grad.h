@@ -78,21 +78,26 @@ __device__ __forceinline__ UnitGrad unit_grad_cell_lin(const double *units_n, co
     const double *lp = units_n + ((size_t)t * Pl + col) * kLinUnit;
     const double2 lp01 = *reinterpret_cast<const double2 *>(lp);
     const double lp0 = lp01.x, lp1 = lp01.y;
-    // a unit outside [2^-80, 2^80] (other than 0) may overflow a chunk of frames,
-    // or push a state out of range on its own: such a batch is not for this form
-    auto bad = [](double x) { return x > 0x1p80 || (x != 0.0 && x < 0x1p-80); };
-    out_of_range = bad(lp0) || (u >= 1 && bad(lp1));
-    const double k = __builtin_amdgcn_ldexp(inv_ll, sa + sb - s_ll);
+    // a unit above 2^80 may overflow a chunk of frames (small ones can only lose
+    // mass, which the sums of the posteriors show): such a batch is not for this form
+    out_of_range = lp0 > 0x1p80 || (u >= 1 && lp1 > 0x1p80);
+    // posterior = (alpha * unit) * beta * 2^(sa + sb - s_ll) / mantissa of the total;
+    // half of the power of two goes to each factor first, so that a product of two
+    // small numbers does not leave the range on its way to a posterior that is in it
+    const int k = sa + sb - s_ll, ka = k / 2;
+    const double2 as = make_double2(__builtin_amdgcn_ldexp(a.x, ka), __builtin_amdgcn_ldexp(a.y, ka));
+    const double bo = __builtin_amdgcn_ldexp(b.x, k - ka) * inv_ll, be = __builtin_amdgcn_ldexp(b.y, k - ka) * inv_ll;
     UnitGrad r;
-    r.g0 = -(float)(((a.y + a.x) * lp0) * b.y * k);
-    r.g1 = (u >= 1) ? -(float)((a.x * lp1) * b.x * k) : 0.0f;
+    r.g0 = -(float)(((as.y + as.x) * lp0) * be);
+    r.g1 = (u >= 1) ? -(float)((as.x * lp1) * bo) : 0.0f;
     r.g2 = 0.0f;
     if (u < Un) {
         const double lp2 = lp[2];
-        out_of_range = out_of_range || bad(lp2);
-        const double bo_next = beta_n[((size_t)(t + 1) * Pl + lin_column(u + 1)) * 2];
-        const double from = (u >= 1 && y[u - 1] != y[u]) ? a.y + a.x : a.y;
-        r.g2 = -(float)((from * lp2) * bo_next * __builtin_amdgcn_ldexp(inv_ll, sa + sb_next - s_ll));
+        out_of_range = out_of_range || lp2 > 0x1p80;
+        const int k2 = sa + sb_next - s_ll;
+        const double bo_next = __builtin_amdgcn_ldexp(beta_n[((size_t)(t + 1) * Pl + lin_column(u + 1)) * 2], k2 - ka) * inv_ll;
+        const double from = (u >= 1 && y[u - 1] != y[u]) ? as.y + as.x : as.y;
+        r.g2 = -(float)((from * lp2) * bo_next);
     }
     return r;
 }
