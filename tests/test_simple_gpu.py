@@ -954,8 +954,11 @@ def test_linear_lattices_give_up_a_hand_over_that_does_not_arrive(lattice_domain
     limit back, is right again: nothing of the lost call is left in the buffers."""
     import warp_ctct
     lib = hip_lib.lib()
-    N, T, U, V = 3, 180, 150, 40                    # chains of three workgroups; sample 2 has one
-    f, g, ys, lx, ly = make_simple_case(91, N, T, U, V, lx=[T, 160, 40], ly=[U, 120, 30], normalized=False)
+    # chains of three workgroups, 24 wavefronts that receive (any one of them finding
+    # its first values missing is enough); sample 2 has a lone wavefront
+    N, T, U, V = 7, 180, 150, 40
+    f, g, ys, lx, ly = make_simple_case(91, N, T, U, V, lx=[T, 160, 40, T, 170, T, 175],
+                                        ly=[U, 130, 30, 140, 128, U, 135], normalized=False)
     _, gf, gg, costs = O.ctct_simple_loss(f, g, ys, lx, ly, reduction="none", normalized=False)
     assert np.all(np.isfinite(costs))               # (every sample has alignments)
     lib.warpctct_joiner_linear_lattice(1)
