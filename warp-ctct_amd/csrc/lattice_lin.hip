@@ -40,7 +40,11 @@
 // chunk's fields (bounded, as in lattice.hip), fetches them again and repeats
 // the chunk from the states it had kept.  A NaN moves one lane per frame, so
 // what the wavefront itself hands over from the other end of its lanes was not
-// touched by it.
+// touched by it.  The first fetch of a field is an ordinary load, with the rest
+// of its row: if it finds an older copy of the line in a cache, that copy holds
+// the NaN pattern, never an older value, because a field changes once per launch
+// (the kernel that gathers the units writes the pattern, the sender the value);
+// the repeated fetch and the sender's stores go past the caches.
 //
 // Math restated from ref_ctct.py:6-74 of the reference, as in lattice.hip.
 #include <algorithm>
@@ -110,39 +114,38 @@ template <bool BETA>
 constexpr unsigned scale_field() { return BETA ? 0u : 8u; }
 
 // One row of units for this lane: `at` is the row's byte offset in the sample's units.
-template <bool BETA, bool COHERENT>
+template <bool BETA>
 static __device__ __forceinline__ void row_load_lin(double (&lp)[3], __amdgpu_buffer_rsrc_t units,
                                                     unsigned lane_bytes, unsigned at) {
-    const v4u_lin w = __builtin_amdgcn_raw_buffer_load_b128(units, lane_bytes, at, COHERENT ? kAgentScope : 0);
-    const v2u_lin x = __builtin_amdgcn_raw_buffer_load_b64(units, lane_bytes + third_field<BETA>(), at,
-                                                           COHERENT ? kAgentScope : 0);
+    const v4u_lin w = __builtin_amdgcn_raw_buffer_load_b128(units, lane_bytes, at, 0);
+    const v2u_lin x = __builtin_amdgcn_raw_buffer_load_b64(units, lane_bytes + third_field<BETA>(), at, 0);
     lp[0] = __hiloint2double((int)w[1], (int)w[0]);
     lp[1] = __hiloint2double((int)w[3], (int)w[2]);
     lp[2] = as_double(x);
 }
 
 // The units of R frames from t_first on in sweep direction, frames clamped to the sample.
-template <bool BETA, bool COHERENT>
+template <bool BETA>
 static __device__ __forceinline__ void chunk_load_lin(ChunkL &c, __amdgpu_buffer_rsrc_t units,
                                                       unsigned lane_bytes, unsigned step, int Tn,
                                                       int t_first) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int t = min(max(t_first + (BETA ? -r : r), 0), Tn - 1);
-        row_load_lin<BETA, COHERENT>(c.lp[r], units, lane_bytes, (unsigned)t * step);
+        row_load_lin<BETA>(c.lp[r], units, lane_bytes, (unsigned)t * step);
     }
 }
 
 // The units of R frames that all exist: `lowest` is the address of the chunk's
 // row with the lowest frame index, off[r] the byte offset of step r's row from
 // it (the same for every chunk, so no address arithmetic per frame).
-template <bool BETA, bool COHERENT>
+template <bool BETA>
 static __device__ __forceinline__ void chunk_load_whole_lin(ChunkL &c, const char *lowest,
                                                             const unsigned (&off)[R], unsigned lane_bytes) {
     const __amdgpu_buffer_rsrc_t rows =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(lowest), 0, 0xffffffffu, 0x00020000);
 #pragma unroll
-    for (int r = 0; r < R; ++r) row_load_lin<BETA, COHERENT>(c.lp[r], rows, lane_bytes, off[r]);
+    for (int r = 0; r < R; ++r) row_load_lin<BETA>(c.lp[r], rows, lane_bytes, off[r]);
 }
 
 // Only the fields another wavefront fills (the third factor of every frame and
@@ -239,7 +242,7 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
         const unsigned in_step = (unsigned)Pl * kCellBytes;
         // the column this wavefront fills for the next one: its lane kGhost's
         const unsigned send_bytes = (unsigned)((BETA ? wave - 1 : wave + 1) * 64 + kGhost) * kCellBytes;
-        chunk_load_lin<BETA, false>(a, rows_in, in_bytes, in_step, Tn, t_start);
+        chunk_load_lin<BETA>(a, rows_in, in_bytes, in_step, Tn, t_start);
         // byte offsets of a whole chunk's rows from its lowest one, in the units
         // and in the lattice: step r's row is the r-th from the bottom (alpha) or
         // from the top (beta)
@@ -384,13 +387,13 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
             const ptrdiff_t onward = (ptrdiff_t)dir * R * (ptrdiff_t)in_step;
             int k = 0;
             do {
-                chunk_load_whole_lin<BETA, false>(b, lowest + onward, in_off, in_bytes);
+                chunk_load_whole_lin<BETA>(b, lowest + onward, in_off, in_bytes);
                 run_chunk(a, k, R, true, false, lowest);
-                chunk_load_whole_lin<BETA, false>(a, lowest + 2 * onward, in_off, in_bytes);
+                chunk_load_whole_lin<BETA>(a, lowest + 2 * onward, in_off, in_bytes);
                 run_chunk(b, k + 1, R, true, false, lowest + onward);
-                chunk_load_whole_lin<BETA, false>(b, lowest + 3 * onward, in_off, in_bytes);
+                chunk_load_whole_lin<BETA>(b, lowest + 3 * onward, in_off, in_bytes);
                 run_chunk(a, k + 2, R, true, false, lowest + 2 * onward);
-                chunk_load_whole_lin<BETA, false>(a, lowest + 4 * onward, in_off, in_bytes);
+                chunk_load_whole_lin<BETA>(a, lowest + 4 * onward, in_off, in_bytes);
                 run_chunk(b, k + 3, R, true, false, lowest + 3 * onward);
                 lowest += 4 * onward;
                 k += 4;
@@ -399,7 +402,7 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
         }
         // the rest (fewer than five chunks), one chunk per turn
         while (s0 < Tn) {
-            chunk_load_lin<BETA, false>(b, rows_in, in_bytes, in_step, Tn, t_start + dir * (s0 + R));
+            chunk_load_lin<BETA>(b, rows_in, in_bytes, in_step, Tn, t_start + dir * (s0 + R));
             run_chunk(a, s0 / R, min(Tn - s0, R), false, s0 + R >= Tn, nullptr);
             a = b;
             s0 += R;
