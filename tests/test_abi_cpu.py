@@ -130,6 +130,14 @@ def test_generic_dtype_and_logits_entry_points_check_their_arguments():
     default = lib.warpctct_lattice_wait_limit(5)
     assert default > 1000 and lib.warpctct_lattice_wait_limit(-1) == 5
     assert lib.warpctct_lattice_wait_limit(-1) == default
+    # from how many frames on the joiner sweeps in the linear domain: the same
+    # kind of setting (negative: the defaults), also through the Python package
+    assert lib.warpctct_joiner_linear_lattice(0) < 0
+    assert lib.warpctct_joiner_linear_lattice(700) == 0
+    assert lib.warpctct_joiner_linear_lattice(-5) == 700
+    import warp_ctct
+    assert warp_ctct.joiner_linear_lattice(1) < 0 and warp_ctct.joiner_linear_lattice(-1) == 1
+    assert lib.warpctct_joiner_linear_lattice(-1) < 0
     # workspace sizes: logits = lattice + one float per row; log-matmul grows with K
     N, T, U = 4, 50, 20
     lat = lib.warpctct_workspace_bytes(N, T, U)

@@ -862,6 +862,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           pybind11::arg("res"), pybind11::arg("grad_masks"));
     m.def("library_version", []() { return std::string(warpctct_version()); });
     m.def(
+        "joiner_linear_lattice", [](const int from_frames) { return warpctct_joiner_linear_lattice(from_frames); },
+        "From how many frames on the fused joiner forward sweeps in the linear domain (0: never, 1: always, "
+        "negative: the defaults); returns the previous setting.",
+        pybind11::arg("from_frames"));
+    m.def(
         "status",
         [](const bool clear) {
             unsigned bits = 0;

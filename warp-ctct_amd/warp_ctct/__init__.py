@@ -74,7 +74,11 @@ def status(reset: bool = True, device=None) -> int:
     * ``STATUS_NAN_INPUT``: a gathered log-probability was NaN (the lattice
       treats such a unit as log 0);
     * ``STATUS_LOST_HAND_OVER``: a lattice was not swept to its end (its costs
-      and gradients are NaN by construction, not because of the inputs).
+      and gradients are NaN by construction, not because of the inputs);
+    * ``STATUS_LINEAR_FELL_BACK``: ``ctct_simple_loss`` swept a batch in the
+      linear domain, its check refused the result, and the log-domain kernels
+      computed the batch again (the results are right; see
+      ``joiner_linear_lattice``).
 
     Nothing in ``ctct_loss`` / ``ctct_simple_loss`` synchronises with the host;
     this call does (it waits for the device), so use it where a pipeline would
@@ -83,6 +87,17 @@ def status(reset: bool = True, device=None) -> int:
         return int(core.status(bool(reset)))
     with torch.cuda.device(device):
         return int(core.status(bool(reset)))
+
+
+def joiner_linear_lattice(from_frames: int = -1) -> int:
+    """From how many frames on ``ctct_simple_loss`` sweeps its lattices on path
+    masses instead of their logarithms (half the time per frame; the result is
+    checked on the GPU, and the log-domain kernels, queued behind, compute a
+    batch again whose check fails: ``STATUS_LINEAR_FELL_BACK``).  0: never,
+    1: always, negative: the defaults (512 frames, 1024 with normalisation).
+    One setting for the process; returns the previous one (negative: the
+    defaults).  The reference sweeps in the log domain only (csrc/simple.cu)."""
+    return int(core.joiner_linear_lattice(int(from_frames)))
 
 
 def label_range_violated(reset: bool = True, device=None) -> bool:
