@@ -377,6 +377,10 @@ def main():
     ap.add_argument("--graph", action="store_true",
                     help="capture one step in a HIP graph and time its replays (reduced line, "
                          "for any --config)")
+    ap.add_argument("--joiner-sweeps", choices=["default", "log", "linear"], default="default",
+                    help="domain of the log-add joiner's lattice sweeps (ctct_simple_loss): the "
+                         "library's choice by the number of frames, the log domain only, or the "
+                         "linear domain, checked, with the log domain as fall-back, for every input")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch one plain copy kernel of known size (1 GiB read + 1 GiB "
                          "written) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings can "
@@ -389,6 +393,8 @@ def main():
     import torch
     import warp_ctct
 
+    if args.joiner_sweeps != "default":
+        warp_ctct.joiner_linear_lattice({"log": 0, "linear": 1}[args.joiner_sweeps])
     if args.config != "c2" or args.graph:
         other_config(args, torch, warp_ctct)
         return
