@@ -31,8 +31,8 @@
 // recursion of the real lanes then needs nothing extra: the value arrives
 // through the same loads and the same DPP move as a neighbour's inside the
 // wavefront.  (For that the beta sweep sends its value already multiplied by
-// the receiver's unit, which the units array holds a second time, in the
-// sender's cell.)  The sender's S of a chunk travels in a spare field of the
+// the receiver's unit, which every lane reads from the cell of the context
+// below its own.)  The sender's S of a chunk travels in a spare field of the
 // chunk's first cell.  Nothing tells the receiver in advance that a value has
 // arrived: a field that has not been written holds a NaN pattern, the NaN
 // reaches the receiver's first real context within the chunk, and the receiver
@@ -104,21 +104,23 @@ static __device__ __forceinline__ double lane_value(double x) {
                             __builtin_amdgcn_readlane(__double2loint(x), from));
 }
 
-// Byte offset, inside a cell of units, of the third factor a sweep reads: the
-// next label's unit (alpha), or the next label's unit of the context below (beta).
-template <bool BETA>
-constexpr unsigned third_field() { return BETA ? 24u : 16u; }
+// Byte offset, inside a cell of units, of the next label's unit: the third
+// factor of the alpha sweep, and the field of a column in between that takes
+// the value handed over.  The beta sweep's third factor is the same field of the
+// cell of the context BELOW the lane's own (what it sends is multiplied with the
+// receiver's unit before it is sent).
+constexpr unsigned kNextField = 16u;
 // ... and of the field that carries the sender's S in the column it fills: one
 // that the lane playing the sender multiplies with a state that is always 0.
 template <bool BETA>
 constexpr unsigned scale_field() { return BETA ? 0u : 8u; }
 
-// One row of units for this lane: `at` is the row's byte offset in the sample's units.
-template <bool BETA>
+// One row of units for this lane: `at` is the row's byte offset in the sample's
+// units, lane_bytes the lane's own cell in a row, third_bytes its third factor.
 static __device__ __forceinline__ void row_load_lin(double (&lp)[3], __amdgpu_buffer_rsrc_t units,
-                                                    unsigned lane_bytes, unsigned at) {
+                                                    unsigned lane_bytes, unsigned third_bytes, unsigned at) {
     const v4u_lin w = __builtin_amdgcn_raw_buffer_load_b128(units, lane_bytes, at, 0);
-    const v2u_lin x = __builtin_amdgcn_raw_buffer_load_b64(units, lane_bytes + third_field<BETA>(), at, 0);
+    const v2u_lin x = __builtin_amdgcn_raw_buffer_load_b64(units, third_bytes, at, 0);
     lp[0] = __hiloint2double((int)w[1], (int)w[0]);
     lp[1] = __hiloint2double((int)w[3], (int)w[2]);
     lp[2] = as_double(x);
@@ -127,38 +129,38 @@ static __device__ __forceinline__ void row_load_lin(double (&lp)[3], __amdgpu_bu
 // The units of R frames from t_first on in sweep direction, frames clamped to the sample.
 template <bool BETA>
 static __device__ __forceinline__ void chunk_load_lin(ChunkL &c, __amdgpu_buffer_rsrc_t units,
-                                                      unsigned lane_bytes, unsigned step, int Tn,
-                                                      int t_first) {
+                                                      unsigned lane_bytes, unsigned third_bytes,
+                                                      unsigned step, int Tn, int t_first) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int t = min(max(t_first + (BETA ? -r : r), 0), Tn - 1);
-        row_load_lin<BETA>(c.lp[r], units, lane_bytes, (unsigned)t * step);
+        row_load_lin(c.lp[r], units, lane_bytes, third_bytes, (unsigned)t * step);
     }
 }
 
 // The units of R frames that all exist: `lowest` is the address of the chunk's
 // row with the lowest frame index, off[r] the byte offset of step r's row from
 // it (the same for every chunk, so no address arithmetic per frame).
-template <bool BETA>
 static __device__ __forceinline__ void chunk_load_whole_lin(ChunkL &c, const char *lowest,
-                                                            const unsigned (&off)[R], unsigned lane_bytes) {
+                                                            const unsigned (&off)[R], unsigned lane_bytes,
+                                                            unsigned third_bytes) {
     const __amdgpu_buffer_rsrc_t rows =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(lowest), 0, 0xffffffffu, 0x00020000);
 #pragma unroll
-    for (int r = 0; r < R; ++r) row_load_lin<BETA>(c.lp[r], rows, lane_bytes, off[r]);
+    for (int r = 0; r < R; ++r) row_load_lin(c.lp[r], rows, lane_bytes, third_bytes, off[r]);
 }
 
 // Only the fields another wavefront fills (the third factor of every frame and
 // the scale beside the first), fetched again past the caches.
 template <bool BETA>
 static __device__ __forceinline__ void chunk_reload_mail_lin(ChunkL &c, __amdgpu_buffer_rsrc_t units,
-                                                             unsigned lane_bytes, unsigned step, int Tn,
-                                                             int t_first) {
+                                                             unsigned lane_bytes, unsigned third_bytes,
+                                                             unsigned step, int Tn, int t_first) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int t = min(max(t_first + (BETA ? -r : r), 0), Tn - 1);
-        c.lp[r][2] = as_double(__builtin_amdgcn_raw_buffer_load_b64(units, lane_bytes + third_field<BETA>(),
-                                                                    (unsigned)t * step, kAgentScope));
+        c.lp[r][2] = as_double(
+            __builtin_amdgcn_raw_buffer_load_b64(units, third_bytes, (unsigned)t * step, kAgentScope));
     }
     const int t = min(max(t_first, 0), Tn - 1);
     c.lp[0][BETA ? 0 : 1] = as_double(__builtin_amdgcn_raw_buffer_load_b64(
@@ -240,9 +242,22 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
         const __amdgpu_buffer_rsrc_t rows_in = __builtin_amdgcn_make_buffer_rsrc(units_n, 0, 0xffffffffu, 0x00020000);
         const unsigned in_bytes = (unsigned)col * kCellBytes;
         const unsigned in_step = (unsigned)Pl * kCellBytes;
+        // Where the lane's third factor lies.  Alpha: the next label's unit of its
+        // own cell (for lane kGhost, the value handed over).  Beta: that of the
+        // context below, i.e. of the column before its own, or, for the first
+        // context of a wavefront, of the last context of the wavefront below, three
+        // columns before (the first context of all reads the 0 of the column in
+        // front of it); lane kGhost reads the value handed over from its own cell;
+        // lane 0, whose state is always 0, reads the 1 of its own cell.
+        unsigned third_bytes = in_bytes + kNextField;
+        if (BETA) {
+            if (lane == 0) third_bytes = in_bytes;
+            else if (lane == 1) third_bytes = in_bytes - (wave > 0 ? 3u : 1u) * kCellBytes + kNextField;
+            else if (lane != kGhost) third_bytes = in_bytes - kCellBytes + kNextField;
+        }
         // the column this wavefront fills for the next one: its lane kGhost's
         const unsigned send_bytes = (unsigned)((BETA ? wave - 1 : wave + 1) * 64 + kGhost) * kCellBytes;
-        chunk_load_lin<BETA>(a, rows_in, in_bytes, in_step, Tn, t_start);
+        chunk_load_lin<BETA>(a, rows_in, in_bytes, third_bytes, in_step, Tn, t_start);
         // byte offsets of a whole chunk's rows from its lowest one, in the units
         // and in the lattice: step r's row is the r-th from the bottom (alpha) or
         // from the top (beta)
@@ -333,7 +348,7 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
                 asm volatile("" : "+s"(t_again));
                 unsigned state = 0u;
                 for (int spins = 0;; ++spins) {
-                    chunk_reload_mail_lin<BETA>(c, rows_in, in_bytes, in_step, Tn, t_again);
+                    chunk_reload_mail_lin<BETA>(c, rows_in, in_bytes, third_bytes, in_step, Tn, t_again);
                     state = chunk_mail_state_lin<BETA, kGhost>(c, cnt);
                     if (state != 0u || spins >= max_spins) break;
                     __builtin_amdgcn_s_sleep(2);
@@ -357,7 +372,7 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     if (full || r < cnt)
-                        __builtin_amdgcn_raw_buffer_store_b64(as_words(mine[r]), to, send_bytes + third_field<BETA>(),
+                        __builtin_amdgcn_raw_buffer_store_b64(as_words(mine[r]), to, send_bytes + kNextField,
                                                               full ? in_off[r] : at, kAgentScope);
                     at = BETA ? at - in_step : at + in_step;
                 }
@@ -387,13 +402,13 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
             const ptrdiff_t onward = (ptrdiff_t)dir * R * (ptrdiff_t)in_step;
             int k = 0;
             do {
-                chunk_load_whole_lin<BETA>(b, lowest + onward, in_off, in_bytes);
+                chunk_load_whole_lin(b, lowest + onward, in_off, in_bytes, third_bytes);
                 run_chunk(a, k, R, true, false, lowest);
-                chunk_load_whole_lin<BETA>(a, lowest + 2 * onward, in_off, in_bytes);
+                chunk_load_whole_lin(a, lowest + 2 * onward, in_off, in_bytes, third_bytes);
                 run_chunk(b, k + 1, R, true, false, lowest + onward);
-                chunk_load_whole_lin<BETA>(b, lowest + 3 * onward, in_off, in_bytes);
+                chunk_load_whole_lin(b, lowest + 3 * onward, in_off, in_bytes, third_bytes);
                 run_chunk(a, k + 2, R, true, false, lowest + 2 * onward);
-                chunk_load_whole_lin<BETA>(a, lowest + 4 * onward, in_off, in_bytes);
+                chunk_load_whole_lin(a, lowest + 4 * onward, in_off, in_bytes, third_bytes);
                 run_chunk(b, k + 3, R, true, false, lowest + 3 * onward);
                 lowest += 4 * onward;
                 k += 4;
@@ -402,7 +417,7 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
         }
         // the rest (fewer than five chunks), one chunk per turn
         while (s0 < Tn) {
-            chunk_load_lin<BETA>(b, rows_in, in_bytes, in_step, Tn, t_start + dir * (s0 + R));
+            chunk_load_lin<BETA>(b, rows_in, in_bytes, third_bytes, in_step, Tn, t_start + dir * (s0 + R));
             run_chunk(a, s0 / R, min(Tn - s0, R), false, s0 + R >= Tn, nullptr);
             a = b;
             s0 += R;
@@ -417,7 +432,7 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
                 v2u_lin gone;
                 gone[0] = (unsigned)kLostBits, gone[1] = kLostHigh;
                 for (int t = 0; t < Tn; ++t) {
-                    __builtin_amdgcn_raw_buffer_store_b64(gone, rows_in, send_bytes + third_field<BETA>(),
+                    __builtin_amdgcn_raw_buffer_store_b64(gone, rows_in, send_bytes + kNextField,
                                                           (unsigned)t * in_step, kAgentScope);
                     __builtin_amdgcn_raw_buffer_store_b64(gone, rows_in, send_bytes + scale_field<BETA>(),
                                                           (unsigned)t * in_step, kAgentScope);

@@ -121,10 +121,10 @@ hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream, const unsign
 // its boundary value over THROUGH THE UNITS: context u lives in column
 // lin_column(u) of the lin_padded(U) columns that units, alphas and betas have
 // here, and the columns in between belong to those two lanes.
-//   units  (N,T,Pl,kLinUnit): {blank, label, next label, next label of the
-//          context below} as linear factors ({0,0,0,.} in padding and outside the
-//          band of complete alignments: mass that gets there is gone, instead of
-//          sitting there undiminished and dictating the wavefront's scale); written by
+//   units  (N,T,Pl,kLinUnit): {blank, label, next label} as linear factors
+//          ({0,0,0} in padding and outside the band of complete alignments: mass
+//          that gets there is gone, instead of sitting there undiminished and
+//          dictating the wavefront's scale); written by
 //          launch_simple_gather_units_lin, which also sets up the columns in
 //          between; the sweeps write what they hand over into them
 //   alphas, betas (N,T+1,Pl,2): pairs {o, e} of masses
@@ -137,7 +137,7 @@ hipError_t launch_lattice(const LatticeArgs &a, hipStream_t stream, const unsign
 // together with the check of the kernel that reads them (launch_simple_grads_lin).
 constexpr int kLinChunk = 12;
 constexpr int kLinReal = 62;
-constexpr int kLinUnit = 4;
+constexpr int kLinUnit = 3;
 __host__ __device__ inline int lin_chunks(int T) { return (T + kLinChunk - 1) / kLinChunk; }
 __host__ __device__ inline int lin_waves(int U) { return (U + kLinReal) / kLinReal; }   // U + 1 contexts
 __host__ __device__ inline int lin_padded(int U) { return 64 * lin_waves(U); }

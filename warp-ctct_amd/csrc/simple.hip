@@ -121,13 +121,11 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_kernel(
 // The units for the sweeps in the linear domain (lattice_lin.hip): one thread per
 // (frame, column); lanes 1..62 of a wavefront are the contexts 62 w .. 62 w + 61,
 // lane 0 and lane 63 the columns through which the wavefronts below / above hand
-// their boundary values over.  A context's cell holds {blank, label, next label,
-// next label of the context below} as linear factors; the
-// last one lets the beta sweep send what it hands down already multiplied.
-// Cells of the columns in between: lane 0 {1, 0, E, 0}, lane 63 {0, 1, 0, E},
-// E = "nothing there yet" where a wavefront will write, 0 where none does; the
-// zeros beside it take the sender's scale.  den, fmax, counter, status: as in
-// simple_gather_units_kernel; *flag is lowered.
+// their boundary values over.  A context's cell holds {blank, label, next label}
+// as linear factors.  Cells of the columns in between: lane 0 {1, 0, E}, lane 63
+// {0, 1, E}, E = "nothing there yet" where a wavefront will write, 0 where none
+// does; the 0 beside it takes the sender's scale.  den, fmax, counter, status: as
+// in simple_gather_units_kernel; *flag is lowered.
 template <bool DEFERRED>
 __global__ __launch_bounds__(kBlock) void simple_gather_units_lin_kernel(
     const float *__restrict__ f, const float *__restrict__ g, float *__restrict__ den,
@@ -175,10 +173,7 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_lin_kernel(
     const float f2 = wanted ? fr[c2] : 0.0f;
     float f1 = __shfl_up(f2, 1, 64);
     const int c1 = (in && u >= 1) ? clampi(y[u - 1], 0, V - 1) : 0;
-    // (lane 1's neighbour is in another wavefront; its unit is wanted for the
-    // fourth factor even where this cell itself is outside the band)
-    const bool below_live = in && u >= 1 && !outside_band(t, u - 1, Tn, Un);
-    if (lane == 1 && (live || below_live) && u >= 1) f1 = fr[c1];
+    if (lane == 1 && live && u >= 1) f1 = fr[c1];   // the neighbour is in another wavefront
     // Padding, and cells outside the band of complete alignments (their units
     // cannot influence costs or gradients): all 0.  The mass of alignments that
     // cannot be completed is then gone where it leaves the band; with factors of
@@ -200,36 +195,18 @@ __global__ __launch_bounds__(kBlock) void simple_gather_units_lin_kernel(
         v1 = unit_lin((cur != cur) ? neg_inf() : cur * kLog2e);
         v2 = unit_lin((nxt != nxt) ? neg_inf() : nxt);
     }
-    // what the context below stores as its next-label unit (0 where it stores
-    // none), whether this cell itself is inside the band or not: the step from
-    // (t, u-1) to (t+1, u) may be part of an alignment that cell (t, u) is not
-    double v3 = __hiloint2double(__shfl_up(__double2hiint(v2), 1, 64), __shfl_up(__double2loint(v2), 1, 64));
-    if (lane == 1) {
-        v3 = 0.0;
-        if (below_live) {
-            float den_b = 0.0f;
-            const float *gb = g + ((size_t)n * U1 + u - 1) * V;
-            if (DEFERRED) {
-                float row_max;
-                den_b = logmm_finish_cell(deferred, n, t, u - 1, fr, 1, gb, 1, V, row_max);
-            } else if (den) {
-                den_b = den[((size_t)n * T + t) * U1 + u - 1];
-            }
-            const double below = ((double)f1 + (double)gb[c1] - (double)den_b) * kLog2e;
-            v3 = unit_lin((below != below) ? neg_inf() : below);
-        }
-    }
     const double empty = __longlong_as_double((long long)kRelayEmpty);
     if (lane == 0) {
-        v0 = 1.0, v1 = 0.0, v3 = 0.0;
+        v0 = 1.0, v1 = 0.0;
         v2 = (w >= 1 && w * kLinReal <= Un) ? empty : 0.0;
     } else if (lane == 63) {
-        v0 = 0.0, v1 = 1.0, v2 = 0.0;
-        v3 = ((w + 1) * kLinReal <= Un) ? empty : 0.0;
+        v0 = 0.0, v1 = 1.0;
+        v2 = ((w + 1) * kLinReal <= Un) ? empty : 0.0;
     }
     double *o = units + (((size_t)n * T + t) * Pl + col) * kLinUnit;
-    *reinterpret_cast<double2 *>(o) = make_double2(v0, v1);
-    *reinterpret_cast<double2 *>(o + 2) = make_double2(v2, v3);
+    o[0] = v0;
+    o[1] = v1;
+    o[2] = v2;
 }
 
 // Per frame: grad_den[t,u] = -(g0+g1+g2), grad_f[t,u>=1] = g1[t,u] + g2[t,u-1],

@@ -76,8 +76,7 @@ __device__ __forceinline__ UnitGrad unit_grad_cell_lin(const double *units_n, co
     const double2 a = *reinterpret_cast<const double2 *>(alpha_n + ((size_t)t * Pl + col) * 2);
     const double2 b = *reinterpret_cast<const double2 *>(beta_n + ((size_t)(t + 1) * Pl + col) * 2);
     const double *lp = units_n + ((size_t)t * Pl + col) * kLinUnit;
-    const double2 lp01 = *reinterpret_cast<const double2 *>(lp);
-    const double lp0 = lp01.x, lp1 = lp01.y;
+    const double lp0 = lp[0], lp1 = lp[1];
     // a unit above 2^80 may overflow a chunk of frames (small ones can only lose
     // mass, which the sums of the posteriors show): such a batch is not for this form
     out_of_range = lp0 > 0x1p80 || (u >= 1 && lp1 > 0x1p80);
