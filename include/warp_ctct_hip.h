@@ -493,7 +493,7 @@ int warpctct_status(unsigned *bits, int clear);
  * WARPCTCT_STATUS_LINEAR_FELL_BACK is set.  No counterpart in the reference
  * (csrc/simple.cu sweeps in the log domain).  The linear sweeps save 35-45 ns
  * per frame and cost ~14 us per call (the launches that return at once, a
- * slower gather and gradient kernel), so they are used from T = 512 frames on,
+ * slower gather and gradient kernel), so they are used from T = 768 frames on,
  * with normalisation from T = 640 on.
  * warpctct_joiner_linear_lattice(n) sets one limit for both for later calls of
  * the process (0: never; 1: always; negative: back to those defaults) and

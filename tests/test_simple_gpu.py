@@ -874,14 +874,14 @@ def _loss_and_grads(f, g, ys, lx, ly, normalized, reduction="none", w=None):
 @pytest.mark.parametrize("normalized", [True, False])
 def test_linear_lattices_are_used_for_long_inputs_and_hold_on_ordinary_input(normalized, lattice_domain):
     """With the default setting the fused forward sweeps in the linear domain from
-    512 frames on, from 640 with normalisation (lattice_lin_kernel is launched, the
+    768 frames on, from 640 with normalisation (lattice_lin_kernel is launched, the
     log-domain kernels behind it return at once: the fall-back bit stays clear),
     and below that in the log domain; both agree with the oracle.  A chain of two
     workgroups per lattice."""
     import warp_ctct
     lib = hip_lib.lib()
     lib.warpctct_joiner_linear_lattice(-1)
-    for T, linear in (((650, True), (630, False)) if normalized else ((520, True), (500, False))):
+    for T, linear in (((650, True), (630, False)) if normalized else ((780, True), (760, False))):
         N, U, V = 2, 70, 24
         f, g, ys, lx, ly = make_simple_case(60 + T, N, T, U, V, lx=[T, T - 37], ly=[U, 41],
                                             normalized=normalized)

@@ -90,10 +90,14 @@ int forward_from_units(const Workspace &w, const int *ys, const int *lx, const i
 // defaults below).  The linear sweeps save 35-45 ns per frame and cost ~14 us
 // per call (three launches that return at once, a slower gather and gradient
 // kernel; the gather more so where it also finishes the denominators):
-// measured, they gain from about 450 frames on without the normalisation, and
-// with it from 400-600 frames on, later the more lattices are in flight (their
-// sweeps are then bound by the memory system, not by instructions).
-constexpr int kLinearFromFrames = 512, kLinearFromFramesNormalized = 640;
+// measured, they gain on the GPU from about 450 frames on without the
+// normalisation, and with it from 400-600 frames on, later the more lattices are
+// in flight (their sweeps are then bound by the memory system, not by
+// instructions).  Without the normalisation a step of that length has so little
+// other work that it may be bound by the host, which the three additional
+// launches cost ~9 us: the limit there lies where the step is bound by the GPU
+// on a slow host too.
+constexpr int kLinearFromFrames = 768, kLinearFromFramesNormalized = 640;
 std::atomic<int> g_linear_from{-1};
 
 struct SimpleWorkspace {
