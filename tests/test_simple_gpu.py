@@ -1011,3 +1011,41 @@ def test_linear_lattices_hold_on_peaked_scores(normalized, lattice_domain):
     np.testing.assert_allclose(got[0].cpu().numpy(), costs, rtol=LOSS_RTOL, atol=1e-5 if normalized else 0)
     np.testing.assert_allclose(got[1].cpu().numpy(), gf, atol=GRAD_ATOL, rtol=1e-5)
     np.testing.assert_allclose(got[2].cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
+
+
+def test_linear_lattices_with_several_wavefronts_on_every_simd(lattice_domain):
+    """1200 wavefronts of sweeps at once, more than one per SIMD: the state in which
+    a store of a lattice row whose data registers the next instruction overwrote
+    came out wrong now and then (the check then sent the whole call back to the
+    log domain).  The linear sweeps must hold, twice in a row with the same bits,
+    agree with the log-domain sweeps on every sample and with the oracle on a few."""
+    import warp_ctct
+    if lattice_domain != "linear_lattices":
+        pytest.skip("a test of the linear sweeps")
+    lib = hip_lib.lib()
+    N, T, U, V = 600, 260, 50, 16
+    rng = np.random.default_rng(11)
+    lx = rng.integers(T - 40, T + 1, size=N).astype(np.int32)
+    ly = rng.integers(U // 2, U + 1, size=N).astype(np.int32)
+    f, g, ys, lx, ly = make_simple_case(77, N, T, U, V, lx=lx, ly=ly, normalized=False)
+    w = rng.standard_normal(N)
+    runs = []
+    for domain in (1, 1, 0):
+        lib.warpctct_joiner_linear_lattice(domain)
+        warp_ctct.status(reset=True)
+        runs.append([x.cpu().numpy() for x in _loss_and_grads(f, g, ys, lx, ly, False, w=w)])
+        fell_back = warp_ctct.status(reset=True) & warp_ctct.STATUS_LINEAR_FELL_BACK
+        assert not fell_back, "the linear lattices were given up"
+    lib.warpctct_joiner_linear_lattice(1)
+    for a, b in zip(runs[0], runs[1]):
+        assert np.array_equal(a, b)
+    np.testing.assert_allclose(runs[0][0], runs[2][0], rtol=LOSS_RTOL)
+    np.testing.assert_allclose(runs[0][1], runs[2][1], atol=GRAD_ATOL, rtol=1e-5)
+    # (the gradient of g sums 260 frames)
+    np.testing.assert_allclose(runs[0][2], runs[2][2], atol=GRAD_ATOL * 2, rtol=1e-4)
+    some = [0, 255, 256, 311, 470, 599]
+    _, gf, gg, costs = O.ctct_simple_loss(f[some], g[some], ys[some], lx[some], ly[some], reduction="none",
+                                          normalized=False, grad_output=w[some])
+    np.testing.assert_allclose(runs[0][0][some], costs, rtol=LOSS_RTOL)
+    np.testing.assert_allclose(runs[0][1][some], gf, atol=GRAD_ATOL, rtol=1e-5)
+    np.testing.assert_allclose(runs[0][2][some], gg, atol=GRAD_ATOL * 2, rtol=1e-4)

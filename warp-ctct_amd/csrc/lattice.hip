@@ -92,7 +92,7 @@ __device__ __forceinline__ void front_store_at(__amdgpu_buffer_rsrc_t rows, unsi
     v4u w;
     w[0] = __double2loint(f.o), w[1] = __double2hiint(f.o);
     w[2] = __double2loint(f.e), w[3] = __double2hiint(f.e);
-    __builtin_amdgcn_raw_buffer_store_b128(w, rows, lane_bytes, at, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(w, rows, lane_bytes + at, 0, 0);
 }
 
 // ---- hand-over between the workgroups of one lattice -------------------------

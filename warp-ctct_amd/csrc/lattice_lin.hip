@@ -261,11 +261,11 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
         // byte offsets of a whole chunk's rows from its lowest one, in the units
         // and in the lattice: step r's row is the r-th from the bottom (alpha) or
         // from the top (beta)
-        unsigned in_off[R], out_off[R];
+        unsigned in_off[R], out_at[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             in_off[r] = (unsigned)(BETA ? R - 1 - r : r) * in_step;
-            out_off[r] = (unsigned)(BETA ? R - 1 - r : r) * out_step;
+            out_at[r] = out_lane + (unsigned)(BETA ? R - 1 - r : r) * out_step;
         }
         bool lost = false;     // the hand-over did not arrive in time, or its sender says so
         // whether a chunk has to find out that its hand-over was complete (not
@@ -323,7 +323,14 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
                         v4u_lin w;
                         w[0] = __double2loint(o), w[1] = __double2hiint(o);
                         w[2] = __double2loint(e), w[3] = __double2hiint(e);
-                        __builtin_amdgcn_raw_buffer_store_b128(w, rows, out_lane, full ? out_off[r] : at, 0);
+                        // (The row's offset goes into the lane's, not into the scalar offset
+                        // field.  With a scalar register there the compiler takes a store of
+                        // 16 bytes per lane to need no distance from an instruction that
+                        // overwrites its data registers, and lets the next frame's arithmetic
+                        // follow at once; on this hardware such a store then wrote, now and
+                        // then under load, what that arithmetic had put into the registers.
+                        // With a constant there it keeps the distance itself.)
+                        __builtin_amdgcn_raw_buffer_store_b128(w, rows, full ? out_at[r] : out_lane + at, 0, 0);
                         at = BETA ? at - out_step : at + out_step;
                     }
                 }
