@@ -1013,17 +1013,18 @@ def test_linear_lattices_hold_on_peaked_scores(normalized, lattice_domain):
     np.testing.assert_allclose(got[2].cpu().numpy(), gg, atol=GRAD_ATOL, rtol=1e-5)
 
 
-def test_linear_lattices_with_several_wavefronts_on_every_simd(lattice_domain):
-    """1200 wavefronts of sweeps at once, more than one per SIMD: the state in which
+@pytest.mark.parametrize("shape", [(600, 260, 50), (300, 200, 130)], ids=["lone_wavefronts", "chains_of_three"])
+def test_linear_lattices_with_several_wavefronts_on_every_simd(shape, lattice_domain):
+    """1200 or 1800 wavefronts of sweeps at once, more than one per SIMD: the state in which
     a store of a lattice row whose data registers the next instruction overwrote
     came out wrong now and then (the check then sent the whole call back to the
-    log domain).  The linear sweeps must hold, twice in a row with the same bits,
+    log domain).  The linear sweeps must hold, twice in a row with the same results,
     agree with the log-domain sweeps on every sample and with the oracle on a few."""
     import warp_ctct
     if lattice_domain != "linear_lattices":
         pytest.skip("a test of the linear sweeps")
     lib = hip_lib.lib()
-    N, T, U, V = 600, 260, 50, 16
+    (N, T, U), V = shape, 16
     rng = np.random.default_rng(11)
     lx = rng.integers(T - 40, T + 1, size=N).astype(np.int32)
     ly = rng.integers(U // 2, U + 1, size=N).astype(np.int32)
@@ -1037,13 +1038,16 @@ def test_linear_lattices_with_several_wavefronts_on_every_simd(lattice_domain):
         fell_back = warp_ctct.status(reset=True) & warp_ctct.STATUS_LINEAR_FELL_BACK
         assert not fell_back, "the linear lattices were given up"
     lib.warpctct_joiner_linear_lattice(1)
-    for a, b in zip(runs[0], runs[1]):
-        assert np.array_equal(a, b)
+    # (one wavefront per block of the gradient kernel adds in a fixed order; with
+    # several, the sums over the contexts take the order in which they arrive)
+    assert np.array_equal(runs[0][0], runs[1][0])
+    for a, b in zip(runs[0][1:], runs[1][1:]):
+        assert np.array_equal(a, b) if U < 62 else np.allclose(a, b, rtol=1e-5, atol=1e-6)
     np.testing.assert_allclose(runs[0][0], runs[2][0], rtol=LOSS_RTOL)
     np.testing.assert_allclose(runs[0][1], runs[2][1], atol=GRAD_ATOL, rtol=1e-5)
-    # (the gradient of g sums 260 frames)
+    # (the gradient of g sums all frames)
     np.testing.assert_allclose(runs[0][2], runs[2][2], atol=GRAD_ATOL * 2, rtol=1e-4)
-    some = [0, 255, 256, 311, 470, 599]
+    some = [0, 255, 256, N - 1]
     _, gf, gg, costs = O.ctct_simple_loss(f[some], g[some], ys[some], lx[some], ly[some], reduction="none",
                                           normalized=False, grad_output=w[some])
     np.testing.assert_allclose(runs[0][0][some], costs, rtol=LOSS_RTOL)
