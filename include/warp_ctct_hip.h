@@ -494,10 +494,14 @@ int warpctct_status(unsigned *bits, int clear);
  * (csrc/simple.cu sweeps in the log domain).  The linear sweeps save 35-45 ns
  * per frame and cost ~14 us per call (the launches that return at once, a
  * slower gather and gradient kernel), so they are used from T = 768 frames on,
- * with normalisation from T = 640 on.
- * warpctct_joiner_linear_lattice(n) sets one limit for both for later calls of
- * the process (0: never; 1: always; negative: back to those defaults) and
- * returns the previous setting (negative: the defaults). */
+ * with normalisation from T = 640 on, and only for batches of up to 256
+ * wavefronts of sweeps (2 N ceil((U+1)/62); up to 128 where a lattice needs one
+ * per direction): larger batches are bound by the memory system, where the
+ * linear form, with its units and states as doubles, is 3-12 % slower.
+ * warpctct_joiner_linear_lattice(n) sets one limit in frames for later calls of
+ * the process, which then holds for batches of any size (0: never; 1: always;
+ * negative: back to those defaults), and returns the previous setting (negative:
+ * the defaults). */
 int warpctct_joiner_linear_lattice(int from_frames);
 
 /* ---- measurement aid ------------------------------------------------------

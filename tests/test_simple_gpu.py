@@ -1053,3 +1053,21 @@ def test_linear_lattices_with_several_wavefronts_on_every_simd(shape, lattice_do
     np.testing.assert_allclose(runs[0][0][some], costs, rtol=LOSS_RTOL)
     np.testing.assert_allclose(runs[0][1][some], gf, atol=GRAD_ATOL, rtol=1e-5)
     np.testing.assert_allclose(runs[0][2][some], gg, atol=GRAD_ATOL * 2, rtol=1e-4)
+
+
+def test_linear_lattices_by_default_only_for_batches_bound_by_latency(lattice_domain):
+    """With the default setting, long inputs are swept in the linear domain only
+    up to 256 wavefronts of sweeps (128 where a lattice needs one per direction);
+    a limit set by the caller holds for every batch."""
+    import warp_ctct
+    if lattice_domain != "linear_lattices":
+        pytest.skip("a test of the linear sweeps")
+    lib = hip_lib.lib()
+    T, V = 780, 8
+    for N, U, linear in ((64, 50, True), (65, 50, False), (64, 123, True), (65, 123, False)):
+        f, g, ys, lx, ly = make_simple_case(N + U, N, T, U, V, normalized=False)
+        for setting, expected in ((-1, linear), (700, True)):
+            lib.warpctct_joiner_linear_lattice(setting)
+            names = _launched_kernels(lambda: _loss_and_grads(f, g, ys, lx, ly, False))
+            assert any("lattice_lin_kernel" in k for k in names) == expected, (N, U, setting, names)
+    lib.warpctct_joiner_linear_lattice(1)

@@ -100,6 +100,19 @@ int forward_from_units(const Workspace &w, const int *ys, const int *lx, const i
 constexpr int kLinearFromFrames = 768, kLinearFromFramesNormalized = 640;
 std::atomic<int> g_linear_from{-1};
 
+// With the default limits, only for batches whose sweeps are bound by the
+// latency of their instructions: up to 256 wavefronts (one per compute unit) for
+// chains, up to 128 for lattices of one wavefront per direction (which the log
+// domain sweeps faster than chains).  Beyond that the sweeps are bound by the
+// memory system, and the linear form moves more bytes (units and states as
+// doubles): measured at 800 frames, it gains 4-12 % per step inside these
+// bounds and loses 3-12 % from 1.5 times as many wavefronts on, up to 1024
+// lattices.
+bool linear_batch_fits(int N, int U) {
+    const long W = lin_waves(U), wavefronts = 2L * N * W;
+    return wavefronts <= (W == 1 ? 128 : 256);
+}
+
 struct SimpleWorkspace {
     Workspace lattice;
     float *unit_grads;   // (N,T,U+1,3)
@@ -796,8 +809,12 @@ int warpctct_simple_forward_reduced_f32(const float *f, const float *g, const in
             if (rc != WARPCTCT_OK) return rc;
         }
         int linear_from = g_linear_from.load(std::memory_order_relaxed);
-        if (linear_from < 0) linear_from = normalized ? kLinearFromFramesNormalized : kLinearFromFrames;
-        if (want_grad && linear_from > 0 && T >= linear_from && simple_grads_lin_applies(T, U)) {
+        bool batch_fits = true;   // a limit that the caller has set holds for every batch
+        if (linear_from < 0) {
+            linear_from = normalized ? kLinearFromFramesNormalized : kLinearFromFrames;
+            batch_fits = linear_batch_fits(N, U);
+        }
+        if (want_grad && linear_from > 0 && T >= linear_from && batch_fits && simple_grads_lin_applies(T, U)) {
             // The lattices in the linear domain (less than half the time per frame),
             // checked by the kernel that forms the gradients from them; the
             // log-domain kernels follow and return at once unless that check, or
