@@ -214,6 +214,7 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
     constexpr int kEdge = BETA ? 1 : 62;     // the context whose value is handed on
     const int lane = threadIdx.x & 63;
     const bool real = lane >= 1 && lane <= kLinReal;
+    const int real_bits = real ? -1 : 0;   // (a mask, not a condition: no branch in the renormalisation)
     const int u = wave * kLinReal + lane - 1;
     double omask = 1.0, skipf, e, o;
     skipf = (real && (u >= 1) && (u < Un) && (y[u] != y[u - 1])) ? 1.0 : 0.0;
@@ -392,7 +393,7 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
             // All states 0 (or below the normal range): nothing to scale; a state
             // that is not finite: the check behind the sweeps will say so.
             if (!last) {
-                const int top = wave_max_nonneg(real ? max(__double2hiint(e), __double2hiint(o)) : 0) >> 20;
+                const int top = wave_max_nonneg(max(__double2hiint(e), __double2hiint(o)) & real_bits) >> 20;
                 const int ex = (top > 0 && top < 0x7ff) ? top - 1022 : 0;
                 e = __builtin_amdgcn_ldexp(e, -ex);
                 o = __builtin_amdgcn_ldexp(o, -ex);
