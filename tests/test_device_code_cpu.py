@@ -1,8 +1,8 @@
 """What the compiler made of the kernels, read from its assembly output for
 gfx950 (the device pass alone, a few seconds per file; nothing is launched).
 
-Two rules that the sources are written to keep, and that a later edit could
-break without any test on a quiet GPU noticing:
+Rules that the sources are written to keep, and that a later edit could break
+without any test on a quiet GPU noticing:
 
 * A buffer store of more than 8 bytes per lane takes its row offset in the
   lane's offset register, never in the scalar offset field.  With a scalar
@@ -15,6 +15,7 @@ break without any test on a quiet GPU noticing:
   compiler keeps the distance itself; the second test checks that it does.
 * No packed single-precision arithmetic: the build switches the feature off,
   and no source asks for it by hand.
+* The lattice kernels stay within the registers that their occupancy rests on.
 """
 import glob
 import os
@@ -117,3 +118,26 @@ def test_no_packed_single_precision_arithmetic(listings):
             if re.match(r"v_pk_(add|mul|fma)_f32\b", text):
                 found.append("%s:%d: %s" % (name, at, text))
     assert not found, "\n".join(found[:20])
+
+
+def test_register_budgets_that_the_occupancy_rests_on(listings):
+    """lattice_fill_kernel's clearing workgroups carry the sweeps' register
+    allocation: up to 168 registers per lane three workgroups of 256 threads share
+    a compute unit, with more only two, and the clear that the typical batch's
+    step consists of takes 3 % longer.  The sweeping kernels must leave room for
+    two wavefronts per SIMD (256), and none of the three may spill to scratch
+    memory."""
+    budgets = {"lattice_fill_kernel": 168, "lattice_kernelE": 256, "lattice_lin_kernel": 256}
+    seen = {}
+    for name, lines in listings.items():
+        text = "\n".join(lines)
+        for block in text.split("  - .agpr_count")[1:]:
+            kernel = re.search(r"\.name:\s+(\S+)", block).group(1)
+            vgprs = int(re.search(r"\.vgpr_count:\s+(\d+)", block).group(1))
+            spilled = int(re.search(r"\.vgpr_spill_count:\s+(\d+)", block).group(1))
+            for key, most in budgets.items():
+                if key in kernel:
+                    seen[key] = vgprs
+                    assert vgprs <= most, (kernel, vgprs, most)
+                    assert spilled == 0, (kernel, spilled)
+    assert set(seen) == set(budgets), seen
