@@ -493,11 +493,13 @@ int warpctct_status(unsigned *bits, int clear);
  * WARPCTCT_STATUS_LINEAR_FELL_BACK is set.  No counterpart in the reference
  * (csrc/simple.cu sweeps in the log domain).  The linear sweeps save 35-45 ns
  * per frame and cost ~14 us per call (the launches that return at once, a
- * slower gather and gradient kernel), so they are used from T = 768 frames on,
- * with normalisation from T = 640 on, and only for batches of up to 256
- * wavefronts of sweeps (2 N ceil((U+1)/62); up to 128 where a lattice needs one
- * per direction): larger batches are bound by the memory system, where the
- * linear form, with its units and states as doubles, is 3-12 % slower.
+ * slower gather), so they are used from T = 768 frames on, with normalisation
+ * from T = 384 on, and only for batches of up to 768 wavefronts of sweeps
+ * (2 N ceil((U+1)/62); up to 256 where a lattice needs one per direction):
+ * larger batches are bound by the memory system, where the linear form has
+ * nothing to gain.  The rows of these lattices hold the states' high words
+ * (20 bits of mantissa): the posteriors formed from them carry a relative error
+ * of ~1e-6, the costs none (they come from the sweeps' registers).
  * warpctct_joiner_linear_lattice(n) sets one limit in frames for later calls of
  * the process, which then holds for batches of any size (0: never; 1: always;
  * negative: back to those defaults), and returns the previous setting (negative:

@@ -874,14 +874,14 @@ def _loss_and_grads(f, g, ys, lx, ly, normalized, reduction="none", w=None):
 @pytest.mark.parametrize("normalized", [True, False])
 def test_linear_lattices_are_used_for_long_inputs_and_hold_on_ordinary_input(normalized, lattice_domain):
     """With the default setting the fused forward sweeps in the linear domain from
-    768 frames on, from 640 with normalisation (lattice_lin_kernel is launched, the
+    768 frames on, from 384 with normalisation (lattice_lin_kernel is launched, the
     log-domain kernels behind it return at once: the fall-back bit stays clear),
     and below that in the log domain; both agree with the oracle.  A chain of two
     workgroups per lattice."""
     import warp_ctct
     lib = hip_lib.lib()
     lib.warpctct_joiner_linear_lattice(-1)
-    for T, linear in (((650, True), (630, False)) if normalized else ((780, True), (760, False))):
+    for T, linear in (((400, True), (380, False)) if normalized else ((780, True), (760, False))):
         N, U, V = 2, 70, 24
         f, g, ys, lx, ly = make_simple_case(60 + T, N, T, U, V, lx=[T, T - 37], ly=[U, 41],
                                             normalized=normalized)
@@ -1057,14 +1057,14 @@ def test_linear_lattices_with_several_wavefronts_on_every_simd(shape, lattice_do
 
 def test_linear_lattices_by_default_only_for_batches_bound_by_latency(lattice_domain):
     """With the default setting, long inputs are swept in the linear domain only
-    up to 256 wavefronts of sweeps (128 where a lattice needs one per direction);
+    up to 768 wavefronts of sweeps (256 where a lattice needs one per direction);
     a limit set by the caller holds for every batch."""
     import warp_ctct
     if lattice_domain != "linear_lattices":
         pytest.skip("a test of the linear sweeps")
     lib = hip_lib.lib()
     T, V = 780, 8
-    for N, U, linear in ((64, 50, True), (65, 50, False), (64, 123, True), (65, 123, False)):
+    for N, U, linear in ((128, 50, True), (129, 50, False), (192, 123, True), (193, 123, False)):
         f, g, ys, lx, ly = make_simple_case(N + U, N, T, U, V, normalized=False)
         for setting, expected in ((-1, linear), (700, True)):
             lib.warpctct_joiner_linear_lattice(setting)

@@ -87,30 +87,30 @@ int forward_from_units(const Workspace &w, const int *ys, const int *lx, const i
 
 // from how many frames on the fused joiner forward sweeps its lattices in the
 // linear domain first (warpctct_joiner_linear_lattice; 0: never; negative: the
-// defaults below).  The linear sweeps save 35-45 ns per frame and cost ~14 us
-// per call (three launches that return at once, a slower gather and gradient
-// kernel; the gather more so where it also finishes the denominators):
-// measured, they gain on the GPU from about 450 frames on without the
-// normalisation, and with it from 400-600 frames on, later the more lattices are
-// in flight (their sweeps are then bound by the memory system, not by
-// instructions).  Without the normalisation a step of that length has so little
-// other work that it may be bound by the host, which the three additional
-// launches cost ~9 us: the limit there lies where the step is bound by the GPU
-// on a slow host too.
-constexpr int kLinearFromFrames = 768, kLinearFromFramesNormalized = 640;
+// defaults below).  The linear sweeps save 35-50 ns per frame and cost ~10 us
+// per call (three launches that return at once, a slower gather; the gather
+// more so where it also finishes the denominators): measured, with the
+// normalisation they gain from 384 frames on (+0.6 to +2.9 % per step at 400
+// frames for 4 to 32 lattices of 81 contexts, V = 2048), and without it the GPU
+// gains from about 450 frames on.  Without the normalisation, though, a step of
+// that length has so little other work that it may be bound by the host, which
+// the three additional launches cost ~9 us (-4 to -10 % at 400 frames): the
+// limit there lies where the step is bound by the GPU on a slow host too.
+constexpr int kLinearFromFrames = 768, kLinearFromFramesNormalized = 384;
 std::atomic<int> g_linear_from{-1};
 
 // With the default limits, only for batches whose sweeps are bound by the
-// latency of their instructions: up to 256 wavefronts (one per compute unit) for
-// chains, up to 128 for lattices of one wavefront per direction (which the log
-// domain sweeps faster than chains).  Beyond that the sweeps are bound by the
-// memory system, and the linear form moves more bytes (units and states as
-// doubles): measured at 800 frames, it gains 4-12 % per step inside these
-// bounds and loses 3-12 % from 1.5 times as many wavefronts on, up to 1024
-// lattices.
+// latency of their instructions rather than by the memory system, where the
+// linear form has nothing to gain (it moves 24 + 8 bytes per column, direction
+// and frame, the log form 12 + 16): up to 256 wavefronts of sweeps (one per
+// compute unit) where a lattice needs one per direction, up to 768 for chains,
+// which the log domain sweeps more slowly.  Measured at 800 and 1500 frames: per
+// step +2 to +6 % for 64-128 lattices of one wavefront per direction, -1.6 %
+// for 192; chains of three +10 to +18 % for 32-64 lattices, +0.4 to +1 % for
+// 128-256; chains of five +7 to +10 % for 32-64, -0.4 % for 128.
 bool linear_batch_fits(int N, int U) {
     const long W = lin_waves(U), wavefronts = 2L * N * W;
-    return wavefronts <= (W == 1 ? 128 : 256);
+    return wavefronts <= (W == 1 ? 256 : 768);
 }
 
 struct SimpleWorkspace {
@@ -135,7 +135,7 @@ SimpleWorkspace carve_simple(void *base, int N, int T, int U) {
     const bool lin = simple_grads_lin_applies(T, U);
     const size_t Pl = (size_t)lin_padded(U);
     const size_t lin_units_b = lin ? align256((size_t)N * T * Pl * kLinUnit * sizeof(double)) : 0;
-    const size_t lin_lat_b = lin ? align256((size_t)N * (T + 1) * Pl * 2 * sizeof(double)) : 0;
+    const size_t lin_lat_b = lin ? align256((size_t)N * (T + 1) * Pl * 2 * sizeof(unsigned)) : 0;
     const uintptr_t b = reinterpret_cast<uintptr_t>(base);
     w.lin_units = reinterpret_cast<double *>(b);
     w.lin_alphas = reinterpret_cast<double *>(b + lin_units_b);

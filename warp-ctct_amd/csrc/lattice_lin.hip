@@ -81,8 +81,15 @@ __device__ __forceinline__ v2u_lin as_words(double x) {
     return w;
 }
 
-__device__ __forceinline__ void pair_store(double *dst, double o, double e) {
-    *reinterpret_cast<double2 *>(dst) = make_double2(o, e);
+// A row of a lattice holds, per column, the HIGH words of the pair {o, e}: sign,
+// exponent and 20 bits of mantissa, 8 bytes per lane.  The kernel that reads the
+// rows forms posteriors from them, which tolerate a relative error of 1e-6 (the
+// gradients are float32, compared at 1e-4); the sweeps carry the states as
+// doubles in registers, and the cost comes from those.  A store of 8 bytes per
+// lane costs the sweeping wavefront 12 cycles of a frame's ~100, one of 16 bytes
+// 27, and the rows are read back at half the traffic.
+__device__ __forceinline__ void pair_store(unsigned *dst, double o, double e) {
+    *reinterpret_cast<uint2 *>(dst) = make_uint2((unsigned)__double2hiint(o), (unsigned)__double2hiint(e));
 }
 
 // The largest of v >= 0 over the wavefront, as a scalar: four rotations inside
@@ -206,7 +213,7 @@ __device__ __forceinline__ double wave_shift_down_zero(double x) {
 // HAS_IN: a wavefront fills this one's column of hand-overs; has_out: this one
 // fills the next one's.
 template <bool BETA, bool HAS_IN>
-static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, int Pl, int wave, double *lat_n,
+static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, int Pl, int wave, unsigned *lat_n,
                                  int *scales, float *cost_n, bool has_out, int max_spins, unsigned *flag,
                                  unsigned *status) {
     constexpr int kGhost = BETA ? 63 : 0;    // plays the context next door
@@ -228,12 +235,12 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
     }
     const int col = wave * 64 + lane;
     const size_t srow = (size_t)Pl * 2;
-    double *out = lat_n + (size_t)col * 2;
+    unsigned *out = lat_n + (size_t)col * 2;
     pair_store(out + (size_t)(BETA ? Tn : 0) * srow, o, e);
     if (lane == 0) scales[0] = 0;
-    const unsigned out_lane = (unsigned)col * 2u * (unsigned)sizeof(double);
-    const unsigned out_step = (unsigned)(srow * sizeof(double));
-    char *out_row = reinterpret_cast<char *>(lat_n) + (size_t)(BETA ? Tn - 1 : 1) * srow * sizeof(double);
+    const unsigned out_lane = (unsigned)col * 2u * (unsigned)sizeof(unsigned);
+    const unsigned out_step = (unsigned)(srow * sizeof(unsigned));
+    char *out_row = reinterpret_cast<char *>(lat_n) + (size_t)(BETA ? Tn - 1 : 1) * srow * sizeof(unsigned);
     int S = 0;   // the states are mass / 2^S
 
     if (Tn > 0) {
@@ -321,17 +328,14 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
                             o = __builtin_fma(o, c.lp[r][1], recv);
                             e = sum * c.lp[r][0];
                         }
-                        v4u_lin w;
-                        w[0] = __double2loint(o), w[1] = __double2hiint(o);
-                        w[2] = __double2loint(e), w[3] = __double2hiint(e);
-                        // (The row's offset goes into the lane's, not into the scalar offset
-                        // field.  With a scalar register there the compiler takes a store of
-                        // 16 bytes per lane to need no distance from an instruction that
-                        // overwrites its data registers, and lets the next frame's arithmetic
-                        // follow at once; on this hardware such a store then wrote, now and
-                        // then under load, what that arithmetic had put into the registers.
-                        // With a constant there it keeps the distance itself.)
-                        __builtin_amdgcn_raw_buffer_store_b128(w, rows, full ? out_at[r] : out_lane + at, 0, 0);
+                        // (the row's offset in the lane's offset register, a constant in
+                        // the scalar offset field, as for every store of rows here: with a
+                        // scalar register there the compiler lets the next instruction
+                        // overwrite the data registers of a store of 16 bytes per lane,
+                        // which this hardware does not forgive)
+                        v2u_lin w;
+                        w[0] = (unsigned)__double2hiint(o), w[1] = (unsigned)__double2hiint(e);
+                        __builtin_amdgcn_raw_buffer_store_b64(w, rows, full ? out_at[r] : out_lane + at, 0, 0);
                         at = BETA ? at - out_step : at + out_step;
                     }
                 }
@@ -462,7 +466,7 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
 
 __global__ __launch_bounds__(64) void lattice_lin_kernel(
     double *__restrict__ units, const int *__restrict__ ys, const int *__restrict__ lx,
-    const int *__restrict__ ly, double *__restrict__ alphas, double *__restrict__ betas,
+    const int *__restrict__ ly, unsigned *__restrict__ alphas, unsigned *__restrict__ betas,
     int *__restrict__ scales, float *__restrict__ costs, int N, int T, int U, int W, int chains_pad,
     const CostReduce red, int max_spins, unsigned *__restrict__ flag, unsigned *__restrict__ status) {
     // workgroup index = link * chains_pad + chain, chain = n * 2 + d (d = 0: beta,
@@ -517,7 +521,8 @@ hipError_t launch_lattice_lin(const LatticeArgs &a, int *scales, unsigned *flag,
     if ((size_t)a.T * 64 * W * kCellBytes >= (1ULL << 31)) return hipErrorInvalidValue;
     const int max_spins = lattice_wait_limit_now();
     TIMED_LAUNCH(lattice_lin_kernel, dim3((unsigned)(chains_pad * W)), dim3(64), 0, stream,
-                 const_cast<double *>(a.units), a.ys, a.lx, a.ly, a.alphas, a.betas, scales, a.costs, a.N, a.T,
+                 const_cast<double *>(a.units), a.ys, a.lx, a.ly, reinterpret_cast<unsigned *>(a.alphas),
+                 reinterpret_cast<unsigned *>(a.betas), scales, a.costs, a.N, a.T,
                  a.U, W, (int)chains_pad, a.reduce, max_spins, flag, device_status_word());
     return hipGetLastError();
 }

@@ -304,6 +304,9 @@ __global__ __launch_bounds__(512) void simple_grads_kernel(
     const size_t lat = (size_t)(T + 1) * Pw * 2;
     const double *units_n = units + (size_t)n * T * Pw * (LIN ? kLinUnit : 3);
     const double *alpha_n = alphas + (size_t)n * lat, *beta_n = betas + (size_t)n * lat;
+    // LIN: rows of high words (lattice_lin.hip)
+    const unsigned *alpha_w = reinterpret_cast<const unsigned *>(alphas) + (size_t)n * lat;
+    const unsigned *beta_w = reinterpret_cast<const unsigned *>(betas) + (size_t)n * lat;
     const int *y = ys + (size_t)n * U;
     const int t_begin = blockIdx.x * F;
     // LIN: the scales of this context's wavefront (of the sweeps) and of the next
@@ -318,7 +321,7 @@ __global__ __launch_bounds__(512) void simple_grads_kernel(
         sc_beta = scales + (((size_t)n * 2 + 0) * lw + w_own) * chunks1;
         sc_beta_next = scales + (((size_t)n * 2 + 0) * lw + w_next) * chunks1;
         sc_alpha = scales + (((size_t)n * 2 + 1) * lw + w_own) * chunks1;
-        const double ll = beta_n[lin_column(0) * 2 + 1];
+        const double ll = __hiloint2double((int)beta_w[lin_column(0) * 2 + 1], 0);
         const int ex = (ll > 0.0 && ll < __builtin_huge_val()) ? __builtin_amdgcn_frexp_exp(ll) : 0;
         inv_ll = 1.0 / __builtin_amdgcn_ldexp(ll, -ex);   // (0 or inf: NaN below, caught by the check)
         // row 0 of beta was stored by step Tn - 1 of context 0's wavefront
@@ -339,7 +342,7 @@ __global__ __launch_bounds__(512) void simple_grads_kernel(
                 const int ia = t > 0 ? 1 + (t - 1) / kLinChunk : 0;
                 const int ib = t + 1 < Tn ? 1 + (Tn - 2 - t) / kLinChunk : 0;
                 bool bad;
-                g[f] = unit_grad_cell_lin(units_n, alpha_n, beta_n, y, t, u, Un, Pw, sc_alpha[ia],
+                g[f] = unit_grad_cell_lin(units_n, alpha_w, beta_w, y, t, u, Un, Pw, sc_alpha[ia],
                                           sc_beta[ib], sc_beta_next[ib], inv_ll, s_ll, bad);
                 bad_unit = bad_unit || bad;
             } else {

@@ -63,18 +63,21 @@ __device__ __forceinline__ UnitGrad unit_grad_cell(const double *units_n, const 
 
 // The same from lattices in the linear domain (lattice_lin.hip): alpha / beta
 // rows are masses relative to 2^scale, one scale per (direction, wavefront of
-// kLinReal contexts, chunk of frames); units are linear; Pl columns per row,
+// kLinReal contexts, chunk of frames), of which a row holds the high words
+// (20 bits of mantissa); units are linear; Pl columns per row,
 // context u in column lin_column(u).  sa / sb / sb_next: the scales of row t of
 // alpha, and of row t+1 of beta for context u and for context u+1; inv_ll and
 // s_ll: 1 / mantissa and exponent of the lattice's total mass beta(0, state 0).
-__device__ __forceinline__ UnitGrad unit_grad_cell_lin(const double *units_n, const double *alpha_n,
-                                                       const double *beta_n, const int *y, int t,
+__device__ __forceinline__ UnitGrad unit_grad_cell_lin(const double *units_n, const unsigned *alpha_n,
+                                                       const unsigned *beta_n, const int *y, int t,
                                                        int u, int Un, int Pl, int sa, int sb,
                                                        int sb_next, double inv_ll, int s_ll,
                                                        bool &out_of_range) {
     const int col = lin_column(u);
-    const double2 a = *reinterpret_cast<const double2 *>(alpha_n + ((size_t)t * Pl + col) * 2);
-    const double2 b = *reinterpret_cast<const double2 *>(beta_n + ((size_t)(t + 1) * Pl + col) * 2);
+    const uint2 aw = *reinterpret_cast<const uint2 *>(alpha_n + ((size_t)t * Pl + col) * 2);
+    const uint2 bw = *reinterpret_cast<const uint2 *>(beta_n + ((size_t)(t + 1) * Pl + col) * 2);
+    const double2 a = make_double2(__hiloint2double((int)aw.x, 0), __hiloint2double((int)aw.y, 0));
+    const double2 b = make_double2(__hiloint2double((int)bw.x, 0), __hiloint2double((int)bw.y, 0));
     const double *lp = units_n + ((size_t)t * Pl + col) * kLinUnit;
     const double lp0 = lp[0], lp1 = lp[1];
     // a unit above 2^80 may overflow a chunk of frames (small ones can only lose
@@ -94,7 +97,7 @@ __device__ __forceinline__ UnitGrad unit_grad_cell_lin(const double *units_n, co
         const double lp2 = lp[2];
         out_of_range = out_of_range || lp2 > 0x1p80;
         const int k2 = sa + sb_next - s_ll;
-        const double bo_next = __builtin_amdgcn_ldexp(beta_n[((size_t)(t + 1) * Pl + lin_column(u + 1)) * 2], k2 - ka) * inv_ll;
+        const double bo_next = __builtin_amdgcn_ldexp(__hiloint2double((int)beta_n[((size_t)(t + 1) * Pl + lin_column(u + 1)) * 2], 0), k2 - ka) * inv_ll;
         const double from = (u >= 1 && y[u - 1] != y[u]) ? as.y + as.x : as.y;
         r.g2 = -(float)((from * lp2) * bo_next);
     }

@@ -94,10 +94,10 @@ def joiner_linear_lattice(from_frames: int = -1) -> int:
     masses instead of their logarithms (half the time per frame; the result is
     checked on the GPU, and the log-domain kernels, queued behind, compute a
     batch again whose check fails: ``STATUS_LINEAR_FELL_BACK``).  0: never,
-    1: always, negative: the defaults (768 frames, 640 with normalisation, and
-    only batches of up to 256 wavefronts of sweeps, 2 N ceil((U+1)/62), or 128
+    1: always, negative: the defaults (768 frames, 384 with normalisation, and
+    only batches of up to 768 wavefronts of sweeps, 2 N ceil((U+1)/62), or 256
     where a lattice needs one per direction: larger batches are bound by the
-    memory system, where the log domain moves fewer bytes).  A limit set here
+    memory system, where the linear form has nothing to gain).  A limit set here
     holds for batches of any size.  One setting for the process; returns the
     previous one (negative: the defaults).  The reference sweeps in the log domain only (csrc/simple.cu)."""
     return int(core.joiner_linear_lattice(int(from_frames)))
