@@ -286,8 +286,11 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
             const int S_kept = S;
             double mine[R];
             // (written so that the ordinary way through a chunk is one straight run
-            // of instructions: a lone wavefront pays for every taken branch)
-            for (bool again = false;; again = true) {
+            // of instructions: a lone wavefront pays for every taken branch.  The
+            // pass through the chunk's frames therefore exists twice for a wavefront
+            // that receives: once in that run, once behind the wait for a hand-over
+            // that had not arrived, out of the way.)
+            auto pass = [&]() {
                 double coded = 1.0;
                 if (HAS_IN) {
                     coded = lane_value<kGhost>(c.lp[0][BETA ? 0 : 1]);
@@ -339,18 +342,15 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
                         at = BETA ? at - out_step : at + out_step;
                     }
                 }
-                if (!HAS_IN) break;
                 // a field that had not been written is a NaN, and by now it sits in
                 // the context next to the lane that plays the sender; a scale that
                 // had not been written is 0
                 const double probe = BETA ? e : o;
                 const bool nan_in = ((__ballot(probe != probe) >> kProbe) & 1ULL) != 0ULL;
-                const bool incomplete = nan_in | !(coded > 0.0);
-                if (__builtin_expect(!(watch & incomplete), 1)) break;
-                if (again) {   // all was there: the NaN is the sender's own
-                    watch = false;
-                    break;
-                }
+                return nan_in | !(coded > 0.0);
+            };
+            const bool incomplete = pass();
+            if (HAS_IN && __builtin_expect(watch & incomplete, 0)) {
                 // Back to the states kept; wait for the chunk's hand-over and fetch
                 // it again, then once more through the chunk.
                 e = e_kept, o = o_kept, S = S_kept;
@@ -370,6 +370,8 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
                 // Fetching it again here instead would cost every chunk a wait for
                 // all loads in flight where the two versions of it meet.)
                 if (state <= 1u) lost = true, watch = false;
+                // all was there now: a NaN that is still found is the sender's own
+                if (pass()) watch = false;
             }
             out_row = BETA ? out_row - (size_t)(full ? R : cnt) * out_step
                            : out_row + (size_t)(full ? R : cnt) * out_step;
