@@ -84,8 +84,9 @@ __device__ __forceinline__ v2u_lin as_words(double x) {
 // A row of a lattice holds, per column, the HIGH words of the pair {o, e}: sign,
 // exponent and 20 bits of mantissa, 8 bytes per lane.  The kernel that reads the
 // rows forms posteriors from them, which tolerate a relative error of 1e-6 (the
-// gradients are float32, compared at 1e-4); the sweeps carry the states as
-// doubles in registers, and the cost comes from those.  A store of 8 bytes per
+// gradients are float32, compared at 1e-4), and takes the middle of what the
+// missing low word can have been (lin_state in unit_grad.h); the sweeps carry
+// the states as doubles in registers, and the cost comes from those.  A store of 8 bytes per
 // lane costs the sweeping wavefront 12 cycles of a frame's ~100, one of 16 bytes
 // 27, and the rows are read back at half the traffic.
 __device__ __forceinline__ void pair_store(unsigned *dst, double o, double e) {

@@ -321,7 +321,7 @@ __global__ __launch_bounds__(512) void simple_grads_kernel(
         sc_beta = scales + (((size_t)n * 2 + 0) * lw + w_own) * chunks1;
         sc_beta_next = scales + (((size_t)n * 2 + 0) * lw + w_next) * chunks1;
         sc_alpha = scales + (((size_t)n * 2 + 1) * lw + w_own) * chunks1;
-        const double ll = __hiloint2double((int)beta_w[lin_column(0) * 2 + 1], 0);
+        const double ll = lin_state(beta_w[lin_column(0) * 2 + 1]);
         const int ex = (ll > 0.0 && ll < __builtin_huge_val()) ? __builtin_amdgcn_frexp_exp(ll) : 0;
         inv_ll = 1.0 / __builtin_amdgcn_ldexp(ll, -ex);   // (0 or inf: NaN below, caught by the check)
         // row 0 of beta was stored by step Tn - 1 of context 0's wavefront

@@ -68,6 +68,15 @@ __device__ __forceinline__ UnitGrad unit_grad_cell(const double *units_n, const 
 // context u in column lin_column(u).  sa / sb / sb_next: the scales of row t of
 // alpha, and of row t+1 of beta for context u and for context u+1; inv_ll and
 // s_ll: 1 / mantissa and exponent of the lattice's total mass beta(0, state 0).
+// A state from the high word that its row holds: the low word was cut off, so
+// the middle of what it can have been is taken (the error of a posterior is
+// then 2.4e-7 at most and has no sign of its own; with 0 for the low word every
+// posterior came out low, and a gradient that sums 1500 of them 1e-6 low).  A
+// state of exactly 0 becomes 1e-314, which no product notices.
+__device__ __forceinline__ double lin_state(unsigned high) {
+    return __hiloint2double((int)high, (int)0x80000000u);
+}
+
 __device__ __forceinline__ UnitGrad unit_grad_cell_lin(const double *units_n, const unsigned *alpha_n,
                                                        const unsigned *beta_n, const int *y, int t,
                                                        int u, int Un, int Pl, int sa, int sb,
@@ -76,8 +85,8 @@ __device__ __forceinline__ UnitGrad unit_grad_cell_lin(const double *units_n, co
     const int col = lin_column(u);
     const uint2 aw = *reinterpret_cast<const uint2 *>(alpha_n + ((size_t)t * Pl + col) * 2);
     const uint2 bw = *reinterpret_cast<const uint2 *>(beta_n + ((size_t)(t + 1) * Pl + col) * 2);
-    const double2 a = make_double2(__hiloint2double((int)aw.x, 0), __hiloint2double((int)aw.y, 0));
-    const double2 b = make_double2(__hiloint2double((int)bw.x, 0), __hiloint2double((int)bw.y, 0));
+    const double2 a = make_double2(lin_state(aw.x), lin_state(aw.y));
+    const double2 b = make_double2(lin_state(bw.x), lin_state(bw.y));
     const double *lp = units_n + ((size_t)t * Pl + col) * kLinUnit;
     const double lp0 = lp[0], lp1 = lp[1];
     // a unit above 2^80 may overflow a chunk of frames (small ones can only lose
@@ -97,7 +106,7 @@ __device__ __forceinline__ UnitGrad unit_grad_cell_lin(const double *units_n, co
         const double lp2 = lp[2];
         out_of_range = out_of_range || lp2 > 0x1p80;
         const int k2 = sa + sb_next - s_ll;
-        const double bo_next = __builtin_amdgcn_ldexp(__hiloint2double((int)beta_n[((size_t)(t + 1) * Pl + lin_column(u + 1)) * 2], 0), k2 - ka) * inv_ll;
+        const double bo_next = __builtin_amdgcn_ldexp(lin_state(beta_n[((size_t)(t + 1) * Pl + lin_column(u + 1)) * 2]), k2 - ka) * inv_ll;
         const double from = (u >= 1 && y[u - 1] != y[u]) ? as.y + as.x : as.y;
         r.g2 = -(float)((from * lp2) * bo_next);
     }
