@@ -492,7 +492,7 @@ int warpctct_status(unsigned *bits, int clear);
  * batch again (they return at once otherwise), and
  * WARPCTCT_STATUS_LINEAR_FELL_BACK is set.  No counterpart in the reference
  * (csrc/simple.cu sweeps in the log domain).  The linear sweeps save 35-45 ns
- * per frame and cost ~14 us per call (the launches that return at once, a
+ * per frame and cost ~10 us per call (the launches that return at once, a
  * slower gather), so they are used from T = 768 frames on, with normalisation
  * from T = 384 on, and only for batches of up to 768 wavefronts of sweeps
  * (2 N ceil((U+1)/62); up to 256 where a lattice needs one per direction):
