@@ -86,9 +86,9 @@ __device__ __forceinline__ v2u_lin as_words(double x) {
 // rows forms posteriors from them, which tolerate a relative error of 1e-6 (the
 // gradients are float32, compared at 1e-4), and takes the middle of what the
 // missing low word can have been (lin_state in unit_grad.h); the sweeps carry
-// the states as doubles in registers, and the cost comes from those.  A store of 8 bytes per
-// lane costs the sweeping wavefront 12 cycles of a frame's ~100, one of 16 bytes
-// 27, and the rows are read back at half the traffic.
+// the states as doubles in registers, and the cost comes from those.  Half the
+// traffic of the rows, written here and read back by that kernel: what bounds
+// the sweeps of more than a few dozen lattices.
 __device__ __forceinline__ void pair_store(unsigned *dst, double o, double e) {
     *reinterpret_cast<uint2 *>(dst) = make_uint2((unsigned)__double2hiint(o), (unsigned)__double2hiint(e));
 }
