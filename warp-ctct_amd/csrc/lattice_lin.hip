@@ -337,9 +337,12 @@ static __device__ void sweep_lin(double *units_n, const int *y, int Tn, int Un, 
                         // scalar register there the compiler lets the next instruction
                         // overwrite the data registers of a store of 16 bytes per lane,
                         // which this hardware does not forgive)
-                        v2u_lin w;
-                        w[0] = (unsigned)__double2hiint(o), w[1] = (unsigned)__double2hiint(e);
-                        __builtin_amdgcn_raw_buffer_store_b64(w, rows, full ? out_at[r] : out_lane + at, 0, 0);
+                        // (two stores of a word each: the two high words lie in registers
+                        // that are not neighbours, and to put them side by side for one
+                        // store of 8 bytes takes two moves, which cost more than the store)
+                        const unsigned to = full ? out_at[r] : out_lane + at;
+                        __builtin_amdgcn_raw_buffer_store_b32((unsigned)__double2hiint(o), rows, to, 0, 0);
+                        __builtin_amdgcn_raw_buffer_store_b32((unsigned)__double2hiint(e), rows, to + 4u, 0, 0);
                         at = BETA ? at - out_step : at + out_step;
                     }
                 }
