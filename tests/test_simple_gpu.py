@@ -1018,8 +1018,9 @@ def test_linear_lattices_with_several_wavefronts_on_every_simd(shape, lattice_do
     """1200 or 1800 wavefronts of sweeps at once, more than one per SIMD: the state in which
     a store of a lattice row whose data registers the next instruction overwrote
     came out wrong now and then (the check then sent the whole call back to the
-    log domain).  The linear sweeps must hold, twice in a row with the same results,
-    agree with the log-domain sweeps on every sample and with the oracle on a few."""
+    log domain).  The linear sweeps must hold, twice in a row with the same results (and
+    so must the log-domain sweeps, whose rows are stored the same way), agree with
+    the log-domain sweeps on every sample and with the oracle on a few."""
     import warp_ctct
     if lattice_domain != "linear_lattices":
         pytest.skip("a test of the linear sweeps")
@@ -1031,7 +1032,7 @@ def test_linear_lattices_with_several_wavefronts_on_every_simd(shape, lattice_do
     f, g, ys, lx, ly = make_simple_case(77, N, T, U, V, lx=lx, ly=ly, normalized=False)
     w = rng.standard_normal(N)
     runs = []
-    for domain in (1, 1, 0):
+    for domain in (1, 1, 0, 0):
         lib.warpctct_joiner_linear_lattice(domain)
         warp_ctct.status(reset=True)
         runs.append([x.cpu().numpy() for x in _loss_and_grads(f, g, ys, lx, ly, False, w=w)])
@@ -1040,9 +1041,10 @@ def test_linear_lattices_with_several_wavefronts_on_every_simd(shape, lattice_do
     lib.warpctct_joiner_linear_lattice(1)
     # (one wavefront per block of the gradient kernel adds in a fixed order; with
     # several, the sums over the contexts take the order in which they arrive)
-    assert np.array_equal(runs[0][0], runs[1][0])
-    for a, b in zip(runs[0][1:], runs[1][1:]):
-        assert np.array_equal(a, b) if U < 62 else np.allclose(a, b, rtol=1e-5, atol=1e-6)
+    for first, second in ((runs[0], runs[1]), (runs[2], runs[3])):   # linear twice, log domain twice
+        assert np.array_equal(first[0], second[0])
+        for a, b in zip(first[1:], second[1:]):
+            assert np.array_equal(a, b) if U < 62 else np.allclose(a, b, rtol=1e-5, atol=1e-6)
     np.testing.assert_allclose(runs[0][0], runs[2][0], rtol=LOSS_RTOL)
     np.testing.assert_allclose(runs[0][1], runs[2][1], atol=GRAD_ATOL, rtol=1e-5)
     # (the gradient of g sums all frames)
