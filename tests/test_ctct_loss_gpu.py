@@ -1079,3 +1079,39 @@ def test_full_size_typical_batch_in_half_precision(dtype, logits):
     ulp = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
     assert np.all(np.abs(got - ref_grad) <= GRAD_ATOL / N + ulp * np.abs(ref_grad))
     assert np.all(got[ref_grad == 0] == 0)
+
+
+@pytest.mark.parametrize("shape", [(800, 96, 40), (300, 96, 100)], ids=["lone_wavefronts", "chains_of_two"])
+def test_many_lattices_at_once_repeat_bit_for_bit(shape):
+    """1600 or 1200 wavefronts of sweeps in one launch, several per SIMD, in both
+    launches that sweep (with the clear of the gradient riding along, and
+    without): the rows of the lattices are stored 16 bytes per lane, and a store
+    like that whose data registers the next instruction overwrites came out
+    wrong now and then on a full chip.  Two calls must agree bit for bit, and with
+    the oracle on a few samples."""
+    import warp_ctct
+    (N, T, U), V = shape, 4
+    rng = np.random.default_rng(3)
+    lx = rng.integers(T - 30, T + 1, size=N)
+    ly = rng.integers(U // 2, U + 1, size=N)
+    joint, ys, lx, ly = make_joint_case(31, N, T, U, V, lx=lx, ly=ly)
+    w = rng.standard_normal(N)
+    some = [0, 1, N // 2, N - 1]
+    _, ref_dense, ref_costs = O.ctct_loss(joint[some], ys[some], lx[some], ly[some], reduction="none",
+                                          grad_output=w[some])
+    before = warp_ctct.CLEAR_GRADIENT_IN_FORWARD
+    try:
+        for clear_in_forward in (True, False):
+            warp_ctct.CLEAR_GRADIENT_IN_FORWARD = clear_in_forward
+            runs = []
+            for _ in range(2):
+                x = dev(joint).requires_grad_(True)
+                costs = warp_ctct.ctct_loss(x, dev(ys), dev(lx), dev(ly), reduction="none")
+                (costs * dev(w, torch.float32)).sum().backward()
+                runs.append((costs.detach().cpu().numpy(), x.grad.cpu().numpy()))
+            assert np.array_equal(runs[0][0], runs[1][0])
+            assert np.array_equal(runs[0][1], runs[1][1])
+            np.testing.assert_allclose(runs[0][0][some], ref_costs, rtol=LOSS_RTOL)
+            np.testing.assert_allclose(runs[0][1][some], ref_dense, atol=GRAD_ATOL * np.abs(w).max(), rtol=0)
+    finally:
+        warp_ctct.CLEAR_GRADIENT_IN_FORWARD = before
