@@ -5,7 +5,9 @@ public API.  Every case prints its parameters before it runs, so a failure or
 a fault names its case.
 
 WARPCTCT_RANDOM_CASES_SCALE=k in the environment runs k times as many cases per
-test (the same seeds, longer streams) for an occasional long run."""
+test (the same seeds, longer streams) for an occasional long run;
+WARPCTCT_RANDOM_SEED_OFFSET=m adds m to every seed, for other cases than the
+committed ones."""
 import os
 
 import numpy as np
@@ -20,6 +22,7 @@ from oracle import ctct_oracle as O
 pytestmark = pytest.mark.gpu
 
 SCALE = max(1, int(os.environ.get("WARPCTCT_RANDOM_CASES_SCALE", "1")))
+SEED_OFFSET = int(os.environ.get("WARPCTCT_RANDOM_SEED_OFFSET", "0"))
 LOSS_RTOL = 1e-5     # loss: relative
 GRAD_ATOL = 1e-4     # gradients: absolute
 
@@ -41,7 +44,7 @@ def test_random_joint_and_logits_cases(seed):
     """ctct_loss and ctct_loss_with_logits: all three element types, views,
     reductions, average_frames, weights per sample."""
     import warp_ctct
-    rng = np.random.default_rng(seed)
+    rng = np.random.default_rng(seed + SEED_OFFSET)
     Ts = [1, 2, 7, 8, 9, 11, 12, 13, 23, 24, 25, 36, 37, 70, 140]
     Us = [0, 1, 2, 5, 62, 63, 64, 65, 127, 128, 129, 200]
     Vs = [2, 3, 4, 5, 8, 31, 32, 33, 64, 100]
@@ -100,7 +103,7 @@ def test_random_joiner_cases(seed):
     -inf vocabulary entries and a frame far below the others in a quarter of
     the cases; the lattices swept in the linear domain in half of them."""
     import warp_ctct
-    rng = np.random.default_rng(seed)
+    rng = np.random.default_rng(seed + SEED_OFFSET)
     # (the long ones for the sweeps in the linear domain: whole turns of their
     # chunks, and chains of up to five workgroups that run into one another)
     Ts = [1, 17, 96, 127, 128, 129, 143, 144, 160, 333, 700]
@@ -171,7 +174,7 @@ def test_random_log_matmul_cases(seed):
     operands views into wider tensors; rows
     and columns of -inf and maxima 300 apart in a quarter of the cases."""
     from warp_ctct import _C
-    rng = np.random.default_rng(seed)
+    rng = np.random.default_rng(seed + SEED_OFFSET)
     Ms = [1, 3, 15, 16, 17, 31, 33, 64, 95, 96, 97, 127, 128, 129, 144, 200, 260]
     Ks = [1, 2, 31, 32, 33, 64, 255, 256, 257, 300, 511, 512, 544, 800, 1024, 2047, 2048, 2049, 2304]
     Ns = [1, 2, 15, 16, 17, 32, 33, 48, 64, 80, 96, 97, 130, 200]
@@ -241,7 +244,7 @@ def test_random_cases_of_the_operators_on_gathered_inputs(seed):
     surface): up to 601 contexts (chains of ten workgroups; beyond 512 the
     joiner's reductions take their own kernels), with and without gradients."""
     from warp_ctct import _C
-    rng = np.random.default_rng(seed)
+    rng = np.random.default_rng(seed + SEED_OFFSET)
     Ts = [1, 2, 7, 8, 9, 12, 13, 24, 25, 37, 70, 140, 300]
     Us = [0, 1, 2, 5, 62, 63, 64, 65, 127, 128, 129, 200, 511, 512, 513, 600]
     done = 0
