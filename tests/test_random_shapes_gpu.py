@@ -154,9 +154,15 @@ def test_random_joiner_cases(seed):
         if same_costs(np.atleast_1d(out.detach().cpu().numpy()), np.atleast_1d(loss),
                       atol=1e-4 if (mask and normalized) else 1e-5):
             scale = max(1.0, float(np.abs(w).max()))
-            # dense gradients sum up to T (resp. U+1) unit gradients per entry
-            np.testing.assert_allclose(tf.grad.cpu().numpy(), gf, atol=GRAD_ATOL * scale, rtol=1e-5)
-            np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=GRAD_ATOL * scale, rtol=1e-5)
+            # dense gradients sum up to T (resp. U+1) unit gradients per entry.  With the
+            # normalisation, the denominators are float32 here as in the reference (the
+            # oracle's are float64): their rounding, ~5e-7 per frame, moves the weight of
+            # an alignment against one that dwells elsewhere by ~1e-5 over some hundred
+            # frames (333 frames in 17 contexts: 7-13e-6 on the entries that sum a
+            # context's ~100 posteriors, in either domain of the sweeps)
+            rtol = 2e-5 if normalized else 1e-5
+            np.testing.assert_allclose(tf.grad.cpu().numpy(), gf, atol=GRAD_ATOL * scale, rtol=rtol)
+            np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=GRAD_ATOL * scale, rtol=rtol)
         # (ordinary input: the linear sweeps hold on their own; a sample that has no
         # alignment at all -- too few frames for its labels and their repeats, or,
         # with masked columns, a label without any mass -- sends them back to the
