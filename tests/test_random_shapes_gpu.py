@@ -162,7 +162,13 @@ def test_random_joiner_cases(seed):
             # context's ~100 posteriors, in either domain of the sweeps)
             rtol = 2e-5 if normalized else 1e-5
             np.testing.assert_allclose(tf.grad.cpu().numpy(), gf, atol=GRAD_ATOL * scale, rtol=rtol)
-            np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=GRAD_ATOL * scale, rtol=rtol)
+            # (with masked columns a row may be left with one admissible entry, whose
+            # probability is 1: its gradient wrt g is the sum over the frames of
+            # posterior - probability = 1 - 1, formed in float32 from factors that
+            # are each good to ~4e-6, and 700 such frames leave 3e-3 where the oracle
+            # has 1e-12)
+            atol_g = GRAD_ATOL * scale * (max(1.0, T / 20.0) if (mask and normalized) else 1.0)
+            np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=atol_g, rtol=rtol)
         # (ordinary input: the linear sweeps hold on their own; a sample that has no
         # alignment at all -- too few frames for its labels and their repeats, or,
         # with masked columns, a label without any mass -- sends them back to the
