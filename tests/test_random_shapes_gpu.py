@@ -165,9 +165,9 @@ def test_random_joiner_cases(seed):
             # (with masked columns a row may be left with one admissible entry, whose
             # probability is 1: its gradient wrt g is the sum over the frames of
             # posterior - probability = 1 - 1, formed in float32 from factors that
-            # are each good to ~4e-6, and 700 such frames leave 3e-3 where the oracle
+            # are each good to ~4e-6, and 700 such frames leave 3e-3 (allowed: 1e-5 per frame) where the oracle
             # has 1e-12)
-            atol_g = GRAD_ATOL * scale * (max(1.0, T / 20.0) if (mask and normalized) else 1.0)
+            atol_g = GRAD_ATOL * scale * (max(1.0, T / 10.0) if (mask and normalized) else 1.0)
             np.testing.assert_allclose(tg.grad.cpu().numpy(), gg, atol=atol_g, rtol=rtol)
         # (ordinary input: the linear sweeps hold on their own; a sample that has no
         # alignment at all -- too few frames for its labels and their repeats, or,
